@@ -1,0 +1,53 @@
+"""CPU oracle for the per-token RL loss path.  TEST INFRASTRUCTURE ONLY.
+
+This package is a plain torch/numpy restatement, on the CPU, of the arithmetic that the
+reference (sii-research/siiRL) performs on its per-token loss path.  It exists so that the
+HIP kernels in ``siirl_amd`` can be checked against an independent statement of the same
+maths on the same seeded inputs.  It is never part of the product:
+
+* only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py``
+  may import it, and there only as the checker (or as the thing timed on the host cores);
+* nothing under ``siirl_amd/`` imports it, and ``siirl_amd`` has no CPU fallback: without the
+  HIP library its ops raise.
+
+Every function cites the reference ``file:line`` it follows.  The reference package itself is
+not importable in the build container (its dependencies ``loguru``, ``omegaconf``, ``hydra``,
+``tensordict`` and ``ray`` are absent), so nothing here imports it.
+
+How each function is pinned (see ``tests/test_oracle_*.py``):
+
+=====================================  ==========================================================
+function                               pinned by
+=====================================  ==========================================================
+logprobs_from_logits                   ``-F.cross_entropy``; ``log_softmax().gather()``; fp64
+                                       brute force; shift invariance; uniform row -> -log V
+entropy_from_logits                    ``torch.distributions.Categorical.entropy``; uniform ->
+                                       log V; two equal logits -> log 2; bounds 0 <= H <= log V
+logprob_entropy_backward               ``torch.autograd.grad`` on the fp64 forward;
+                                       ``gradcheck``; rows of the gradient sum to zero
+masked_sum / masked_mean               direct arithmetic on hand-written cases
+compute_grpo_outcome_advantage         brute-force dict loop; unbiased-std known answers
+                                       1.78885 / -0.73030 logged in the reference's quickstart
+                                       (docs/start/quickstart.rst:137); group sums are zero
+agg_loss                               four closed forms on hand-written cases
+compute_policy_loss_vanilla / _gspo    hand-computed cases at ratio = 1, 1 +- eps, c, |d| = 20;
+                                       closed-form gradient vs autograd; GSPO with L = 1 == PPO
+kl_penalty                             closed forms per mode; k3 >= 0; straight-through identities
+apply_kl_penalty / KL controllers      hand-computed controller step
+dynamic_sampling_keep_indices          worked example of the reference's docs
+                                       (docs/user_interface/filter_interface.rst:72-77); brute force
+make_uid / filter_by_indices           uid layout and ordered index select pinned by the
+                                       reference's tests (tests/dag_worker/test_dapo_pipeline.py:14-49,
+                                       tests/dag_worker/test_dapo_merge.py:90-120)
+fused_linear_for_ppo_fwd / _bwd        equals logprob/entropy of ``(h @ W.T)/T`` in fp64 and
+                                       autograd through that expression
+=====================================  ==========================================================
+
+Parity unpinned (third-party arithmetic absent from the reference tree, no fixture in the
+reference's tests): the exact rounding of flash-attn's Triton ``cross_entropy_loss`` (the
+reference's CUDA dispatch target for ``logprobs_from_logits``) and of the Triton kernels in
+``siirl/utils/kernel/kernels.py``.  The oracle states their published algorithm (fp32
+log-softmax / online softmax) instead.
+"""
+
+from . import torch_functional, core_algos, dapo_filter, fused_linear, actor_step  # noqa: F401

@@ -1,0 +1,122 @@
+"""Oracle (test infrastructure): log-prob / entropy from logits and the masked reductions.
+
+Restates ``siirl/utils/model_utils/torch_functional.py:41-168`` of the reference on the CPU.
+
+Precision policy.  The reference's fp32 branch (``torch_functional.py:103-107``) is
+``gather(x) - logsumexp(x)``; for 16-bit logits the deployed path is flash-attn's fp32
+cross-entropy (``:73-79,85-90``) and the chunked entropy upcasts with ``.float()``
+(``:139-142``).  The oracle therefore upcasts 16-bit logits and applies the fp32 (or, on
+request, fp64) formula.  ``literal_bf16=True`` reproduces the reference's no-flash-attn
+16-bit branch (``:108-115``, ``:128-132``), whose results are rounded to the input dtype;
+it is a side note, not the parity target.
+"""
+
+from __future__ import annotations
+
+import torch
+import torch.nn.functional as F
+
+
+def _work_dtype(x: torch.Tensor, dtype):
+    if dtype is not None:
+        return dtype
+    return torch.float64 if x.dtype == torch.float64 else torch.float32
+
+
+def gather_from_labels(data: torch.Tensor, label: torch.Tensor) -> torch.Tensor:
+    """``data[..., label]`` along the last axis (reference ``torch_functional.py:41-53``)."""
+    return data.gather(-1, label.unsqueeze(-1)).squeeze(-1)
+
+
+def logprobs_from_logits(logits, labels, inplace_backward=True, *, dtype=None, literal_bf16=False):
+    """Per-row ``x[y] - logsumexp(x)`` (reference ``torch_functional.py:56-82,99-116``).
+
+    ``inplace_backward`` is accepted for signature parity and has no effect on values.
+    """
+    if literal_bf16 and logits.dtype in (torch.bfloat16, torch.float16):
+        # reference :108-115 -- row-wise log_softmax in the input dtype, then gather
+        flat = logits.reshape(-1, logits.shape[-1])
+        lab = labels.reshape(-1)
+        rows = [F.log_softmax(r, dim=-1)[y] for r, y in zip(flat, lab)]
+        return torch.stack(rows).reshape(labels.shape)
+    x = logits.to(_work_dtype(logits, dtype))
+    picked = gather_from_labels(x, labels)
+    return picked - torch.logsumexp(x, dim=-1)
+
+
+def entropy_from_logits(logits, *, dtype=None, literal_bf16=False):
+    """``H = logsumexp(x) - sum(softmax(x) * x)`` (reference ``torch_functional.py:128-132``)."""
+    if literal_bf16:
+        p = torch.softmax(logits, dim=-1)
+        return torch.logsumexp(logits, dim=-1) - (p * logits).sum(-1)
+    x = logits.to(_work_dtype(logits, dtype))
+    p = torch.softmax(x, dim=-1)
+    return torch.logsumexp(x, dim=-1) - (p * x).sum(-1)
+
+
+def entropy_from_logits_with_chunking(logits, chunk_size: int = 2048):
+    """Row-chunked fp32 entropy of a 2-D tensor (reference ``torch_functional.py:135-143``)."""
+    out = torch.zeros(logits.shape[0], dtype=torch.float32)
+    for lo in range(0, logits.shape[0], chunk_size):
+        out[lo : lo + chunk_size] = entropy_from_logits(logits[lo : lo + chunk_size].float())
+    return out
+
+
+def logprob_entropy_forward(logits, labels, temperature: float = 1.0, *, dtype=None):
+    """Both outputs of the actor's post-logits step with the in-place ``logits / T`` of
+    ``siirl/engine/actor/dp_actor.py:176`` folded in.  Returns ``(logprob, entropy, lse, ex)``
+    where ``lse = logsumexp(z)`` and ``ex = E_p[z]`` for ``z = x / T``."""
+    z = logits.to(_work_dtype(logits, dtype)) / temperature
+    lse = torch.logsumexp(z, dim=-1)
+    p = torch.exp(z - lse.unsqueeze(-1))
+    ex = (p * z).sum(-1)
+    return gather_from_labels(z, labels) - lse, lse - ex, lse, ex
+
+
+def logprob_entropy_backward(logits, labels, g_logprob, g_entropy, temperature: float = 1.0, *, dtype=None):
+    """Closed-form gradient of ``sum(g_lp * logprob) + sum(g_H * entropy)`` w.r.t. the logits.
+
+    ``dx = (1/T) * [ g_lp * (onehot(y) - p) - g_H * p * (z - E_p[z]) ]`` with ``z = x/T``,
+    ``p = softmax(z)``: the explicit form of ``siirl/utils/experimental/torch_functional.py:49-62``
+    (``log p + H == z - E_p[z]``) and of ``siirl/utils/kernel/kernels.py:828-835``.
+    Either upstream gradient may be ``None``.  Returned in the working dtype (not rounded)."""
+    wd = _work_dtype(logits, dtype)
+    z = logits.to(wd) / temperature
+    lse = torch.logsumexp(z, dim=-1, keepdim=True)
+    p = torch.exp(z - lse)
+    dz = torch.zeros_like(z)
+    if g_logprob is not None:
+        g = g_logprob.to(wd).unsqueeze(-1)
+        onehot = torch.zeros_like(z).scatter_(-1, labels.unsqueeze(-1), 1.0)
+        dz += g * (onehot - p)
+    if g_entropy is not None:
+        gh = g_entropy.to(wd).unsqueeze(-1)
+        ex = (p * z).sum(-1, keepdim=True)
+        dz -= gh * p * (z - ex)
+    return dz / temperature
+
+
+def logprob_entropy_backward_autograd(logits, labels, g_logprob, g_entropy, temperature: float = 1.0, *, dtype=None):
+    """Same gradient obtained the way the reference obtains it: autograd through the forward."""
+    wd = _work_dtype(logits, dtype)
+    x = logits.to(wd).detach().clone().requires_grad_(True)
+    z = x / temperature
+    total = x.new_zeros(())
+    if g_logprob is not None:
+        total = total + (g_logprob.to(wd) * logprobs_from_logits(z, labels, dtype=wd)).sum()
+    if g_entropy is not None:
+        total = total + (g_entropy.to(wd) * entropy_from_logits(z, dtype=wd)).sum()
+    (grad,) = torch.autograd.grad(total, x)
+    return grad
+
+
+def masked_sum(values, mask, axis=None):
+    """``sum(where(mask, v, 0) * mask)`` (reference ``torch_functional.py:146-151``): values outside
+    the mask, NaN included, do not contribute."""
+    kept = torch.where(mask.bool(), values, torch.zeros((), dtype=values.dtype))
+    return (kept * mask).sum(axis)
+
+
+def masked_mean(values, mask, axis=None):
+    """``masked_sum / (sum(mask) + 1e-8)`` (reference ``torch_functional.py:154-168``)."""
+    return masked_sum(values, mask, axis) / (mask.sum(axis) + 1e-8)

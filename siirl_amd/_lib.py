@@ -1,0 +1,84 @@
+"""ctypes binding of ``libsiirl_hip.so`` (the C ABI declared in ``include/siirl_hip.h``).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised."""
+
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsiirl_hip.so"
+
+# dtype codes of siirl_dtype
+F32, BF16, F16, F64, I64, I32, U8 = range(7)
+BWD_SKIP_ZERO_ROWS = 1
+
+_p, _i64, _i32, _f32, _u32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint32, C.c_size_t
+
+# name -> (restype, argtypes); one entry per function declared in include/siirl_hip.h
+SIGNATURES = {
+    "siirl_hip_abi_version": (_i32, []),
+    "siirl_hip_last_error": (C.c_char_p, []),
+    "siirl_logprob_entropy_fwd": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p]),
+    "siirl_logprob_entropy_bwd": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p, _i64, _u32, _p]),
+}
+
+_lock = threading.Lock()
+_lib = None
+
+
+class SiirlHipError(RuntimeError):
+    pass
+
+
+def lib():
+    """The loaded library.  torch must be imported first so that the HIP runtime torch uses is the
+    one this library binds to (both carry the soname libamdhip64.so.7)."""
+    global _lib
+    if _lib is None:
+        with _lock:
+            if _lib is None:
+                import torch  # noqa: F401  (loads torch's libamdhip64 before ours is resolved)
+
+                if not LIB_PATH.exists():
+                    raise SiirlHipError(
+                        f"{LIB_PATH} is missing: build it with `python -m siirl_amd.build` "
+                        "(hipcc, gfx950).  siirl_amd has no CPU or eager fallback.")
+                h = C.CDLL(str(LIB_PATH))
+                for name, (res, args) in SIGNATURES.items():
+                    fn = getattr(h, name)  # AttributeError if the symbol is not exported
+                    fn.restype, fn.argtypes = res, args
+                _lib = h
+    return _lib
+
+
+def check(rc: int, what: str):
+    if rc != 0:
+        msg = lib().siirl_hip_last_error().decode("utf-8", "replace")
+        if rc == -1:
+            raise ValueError(f"{what}: {msg}")
+        if rc == -2:
+            raise NotImplementedError(f"{what}: {msg}")
+        raise SiirlHipError(f"{what} failed (status {rc}): {msg}")
+
+
+def dtype_code(torch_dtype) -> int:
+    import torch
+
+    table = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16, torch.float64: F64,
+             torch.int64: I64, torch.int32: I32, torch.uint8: U8, torch.bool: U8}
+    if torch_dtype not in table:
+        raise TypeError(f"dtype {torch_dtype} is not supported by libsiirl_hip")
+    return table[torch_dtype]
+
+
+def ptr(t):
+    """Device pointer of a tensor (or NULL for None)."""
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def current_stream(device):
+    import torch
+
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)

@@ -1,0 +1,403 @@
+// Log-prob and entropy from logits[T, V]: forward (one read of the row) and backward (one read of the
+// row, one write of the gradient).  HBM-bound streaming kernels for gfx950; one workgroup per row.
+//
+// Replaces logprobs_from_logits / entropy_from_logits and their autograd backward:
+//   siirl/utils/model_utils/torch_functional.py:56-116,128-143
+//   siirl/utils/experimental/torch_functional.py:49-62 (closed form of the gradient)
+//
+// Forward keeps, per lane, an online-softmax state in base-2 arithmetic
+//     mx = running max of raw x,   s = sum 2^{(x - mx) k},   t = sum x * 2^{(x - mx) k},   k = log2(e)/T
+// so that each element costs one fma, one v_exp_f32 and two accumulations; the running max is
+// refreshed once per UNROLL 16-byte loads (v_max3 chains), the rescale is a rarely-taken branch.
+// States are merged across the wave with shuffles and across waves through LDS.
+#include "common.hpp"
+
+namespace siirl {
+namespace {
+
+constexpr int kThreads = 256;  // 4 waves per row
+constexpr int kUnroll = 4;     // 16-byte loads in flight per lane
+
+// ------------------------------------------------------------------ element traits (16-byte vectors)
+
+struct ElemBF16 {
+  using elem_t = uint16_t;
+  static constexpr int VEC = 8;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float* v) {
+    v[0] = bf16_lo(r.x); v[1] = bf16_hi(r.x); v[2] = bf16_lo(r.y); v[3] = bf16_hi(r.y);
+    v[4] = bf16_lo(r.z); v[5] = bf16_hi(r.z); v[6] = bf16_lo(r.w); v[7] = bf16_hi(r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* v) {
+    return mk4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+  }
+  static __device__ __forceinline__ float load1(const elem_t* p) { return u2f(((uint32_t)*p) << 16); }
+  static __device__ __forceinline__ void store1(elem_t* p, float f) { *p = (elem_t)(pack_bf16(f, 0.f) & 0xffffu); }
+};
+
+struct ElemF16 {
+  using elem_t = uint16_t;
+  static constexpr int VEC = 8;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float* v) {
+    v[0] = f16_lo(r.x); v[1] = f16_hi(r.x); v[2] = f16_lo(r.y); v[3] = f16_hi(r.y);
+    v[4] = f16_lo(r.z); v[5] = f16_hi(r.z); v[6] = f16_lo(r.w); v[7] = f16_hi(r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* v) {
+    return mk4(pack_f16(v[0], v[1]), pack_f16(v[2], v[3]), pack_f16(v[4], v[5]), pack_f16(v[6], v[7]));
+  }
+  static __device__ __forceinline__ float load1(const elem_t* p) { return f16_lo((uint32_t)*p); }
+  static __device__ __forceinline__ void store1(elem_t* p, float f) { *p = (elem_t)(pack_f16(f, 0.f) & 0xffffu); }
+};
+
+struct ElemF32 {
+  using elem_t = float;
+  static constexpr int VEC = 4;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float* v) {
+    v[0] = u2f(r.x); v[1] = u2f(r.y); v[2] = u2f(r.z); v[3] = u2f(r.w);
+  }
+  static __device__ __forceinline__ u32x4 pack(const float* v) {
+    return mk4(f2u(v[0]), f2u(v[1]), f2u(v[2]), f2u(v[3]));
+  }
+  static __device__ __forceinline__ float load1(const elem_t* p) { return *p; }
+  static __device__ __forceinline__ void store1(elem_t* p, float f) { *p = f; }
+};
+
+// A row is split into [0, head) scalars up to the first 16-byte boundary, nvec 16-byte vectors, and
+// the scalars left over.  When the source and destination rows do not share their alignment the
+// whole row is scalar (head = V).
+template <class E>
+struct RowSplit {
+  int head, nvec, tail0;
+  __device__ __forceinline__ RowSplit(const void* a, const void* b, int V) {
+    const uintptr_t pa = (uintptr_t)a, pb = b ? (uintptr_t)b : pa;
+    constexpr int ES = sizeof(typename E::elem_t);
+    int h = (int)(((16u - (unsigned)(pa & 15u)) & 15u) / ES);
+    if ((pa & 15u) != (pb & 15u)) h = V;
+    head = h < V ? h : V;
+    nvec = (V - head) / E::VEC;
+    tail0 = head + nvec * E::VEC;
+  }
+};
+
+// ----------------------------------------------------------------------------------- forward
+
+struct SoftState {
+  float mx, s, t;
+};
+
+__device__ __forceinline__ void merge(SoftState& a, float omx, float os, float ot, float k) {
+  const float M = fmaxf(a.mx, omx);
+  const float fa = fast_exp2((a.mx - M) * k), fb = fast_exp2((omx - M) * k);
+  a.s = a.s * fa + os * fb;
+  a.t = a.t * fa + ot * fb;
+  a.mx = M;
+}
+
+template <bool ENT>
+__device__ __forceinline__ void absorb1(SoftState& st, float v, float k) {
+  if (v > st.mx) {
+    const float sc = fast_exp2((st.mx - v) * k);
+    st.s *= sc;
+    st.t *= sc;
+    st.mx = v;
+  }
+  const float e = fast_exp2((v - st.mx) * k);
+  st.s += e;
+  if (ENT) st.t = fmaf(v, e, st.t);
+}
+
+template <class E, bool ENT, int N>
+__device__ __forceinline__ void absorb_vecs(SoftState& st, const u32x4* buf, float k) {
+  float v[N][E::VEC];
+#pragma unroll
+  for (int u = 0; u < N; ++u) E::unpack(buf[u], v[u]);
+  float cm = v[0][0];
+#pragma unroll
+  for (int u = 0; u < N; ++u)
+#pragma unroll
+    for (int j = 0; j < E::VEC; ++j) cm = fmaxf(cm, v[u][j]);
+  if (cm > st.mx) {
+    const float sc = fast_exp2((st.mx - cm) * k);
+    st.s *= sc;
+    st.t *= sc;
+    st.mx = cm;
+  }
+  const float nmk = -st.mx * k;
+  float s = st.s, t = st.t;
+#pragma unroll
+  for (int u = 0; u < N; ++u)
+#pragma unroll
+    for (int j = 0; j < E::VEC; ++j) {
+      const float e = fast_exp2(fmaf(v[u][j], k, nmk));
+      s += e;
+      if (ENT) t = fmaf(v[u][j], e, t);
+    }
+  st.s = s;
+  st.t = t;
+}
+
+template <class E, bool ENT>
+__global__ __launch_bounds__(kThreads) void lpe_fwd_kernel(const typename E::elem_t* __restrict__ logits,
+                                                           int64_t row_stride, int V,
+                                                           const int64_t* __restrict__ labels, float inv_T,
+                                                           float* __restrict__ logprob, float* __restrict__ entropy,
+                                                           float* __restrict__ lse_out, float* __restrict__ ex_out) {
+  using elem_t = typename E::elem_t;
+  const int64_t row = blockIdx.x;
+  const elem_t* __restrict__ x = logits + row * row_stride;
+  const int tid = threadIdx.x;
+  const float k = inv_T * kLog2e;
+  const RowSplit<E> sp(x, nullptr, V);
+
+  SoftState st{-1e30f, 0.f, 0.f};
+
+  for (int i = tid; i < sp.head; i += kThreads) absorb1<ENT>(st, E::load1(x + i), k);
+  for (int i = sp.tail0 + tid; i < V; i += kThreads) absorb1<ENT>(st, E::load1(x + i), k);
+
+  const u32x4* __restrict__ xv = reinterpret_cast<const u32x4*>(x + sp.head);
+  constexpr int kTile = kThreads * kUnroll;
+  const int nfull = sp.nvec / kTile * kTile;
+  for (int base = 0; base < nfull; base += kTile) {
+    u32x4 buf[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) buf[u] = __builtin_nontemporal_load(xv + base + u * kThreads + tid);
+    absorb_vecs<E, ENT, kUnroll>(st, buf, k);
+  }
+  for (int i = nfull + tid; i < sp.nvec; i += kThreads) {
+    u32x4 b = __builtin_nontemporal_load(xv + i);
+    absorb_vecs<E, ENT, 1>(st, &b, k);
+  }
+
+  // wave merge
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const float omx = __shfl_xor(st.mx, o, kWave);
+    const float os = __shfl_xor(st.s, o, kWave);
+    const float ot = __shfl_xor(st.t, o, kWave);
+    merge(st, omx, os, ot, k);
+  }
+  __shared__ float sm[3 * (kThreads / kWave)];
+  const int lane = tid & (kWave - 1), wid = tid / kWave;
+  if (lane == 0) {
+    sm[wid * 3 + 0] = st.mx;
+    sm[wid * 3 + 1] = st.s;
+    sm[wid * 3 + 2] = st.t;
+  }
+  __syncthreads();
+  if (tid == 0) {
+#pragma unroll
+    for (int w = 1; w < kThreads / kWave; ++w) merge(st, sm[w * 3], sm[w * 3 + 1], sm[w * 3 + 2], k);
+    const float lse = st.mx * inv_T + logf(st.s);
+    lse_out[row] = lse;
+    if (ENT) {
+      const float exv = inv_T * (st.t / st.s);
+      ex_out[row] = exv;
+      entropy[row] = lse - exv;
+    }
+    if (logprob != nullptr) {
+      const int64_t y = labels[row];
+      float lp = __builtin_nanf("");
+      if (y >= 0 && y < (int64_t)V) lp = E::load1(x + y) * inv_T - lse;
+      logprob[row] = lp;
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------------- backward
+
+struct BwdCoef {
+  float k, nl, c0, c1;
+};
+
+template <bool HAS_ENT>
+__device__ __forceinline__ float grad1(float x, const BwdCoef& c) {
+  const float p = fast_exp2(fmaf(x, c.k, c.nl));
+  return HAS_ENT ? p * fmaf(x, c.c1, c.c0) : p * c.c0;
+}
+
+template <class E, bool HAS_ENT>
+__global__ __launch_bounds__(kThreads) void lpe_bwd_kernel(const typename E::elem_t* logits, int64_t row_stride,
+                                                           int V, const int64_t* __restrict__ labels, float inv_T,
+                                                           const float* __restrict__ lse,
+                                                           const float* __restrict__ ex,
+                                                           const float* __restrict__ g_lp,
+                                                           const float* __restrict__ g_ent,
+                                                           typename E::elem_t* dlogits, int64_t d_stride,
+                                                           uint32_t flags) {
+  using elem_t = typename E::elem_t;
+  const int64_t row = blockIdx.x;
+  const elem_t* x = logits + row * row_stride;
+  elem_t* d = dlogits + row * d_stride;
+  const int tid = threadIdx.x;
+  const RowSplit<E> sp(x, d, V);
+
+  const float g1 = g_lp ? g_lp[row] : 0.f;
+  const float g2 = HAS_ENT ? g_ent[row] : 0.f;
+  const u32x4* xv = reinterpret_cast<const u32x4*>(x + sp.head);
+  u32x4* dv = reinterpret_cast<u32x4*>(d + sp.head);
+
+  if ((flags & SIIRL_BWD_SKIP_ZERO_ROWS) && g1 == 0.f && g2 == 0.f) {
+    for (int i = tid; i < sp.head; i += kThreads) E::store1(d + i, 0.f);
+    for (int i = sp.tail0 + tid; i < V; i += kThreads) E::store1(d + i, 0.f);
+    const u32x4 z = u32x4{0u, 0u, 0u, 0u};
+    for (int i = tid; i < sp.nvec; i += kThreads) __builtin_nontemporal_store(z, dv + i);
+    return;
+  }
+
+  BwdCoef c;
+  c.k = inv_T * kLog2e;
+  c.nl = -lse[row] * kLog2e;
+  c.c0 = inv_T * ((HAS_ENT ? g2 * ex[row] : 0.f) - g1);
+  c.c1 = -g2 * inv_T * inv_T;
+  const float hot = g1 * inv_T;
+  int y = -1;
+  if (g_lp) {
+    const int64_t yl = labels[row];
+    if (yl >= 0 && yl < (int64_t)V) y = (int)yl;
+  }
+  // position of the label inside the vector body, or -1
+  const int yb = (y >= sp.head && y < sp.tail0) ? (y - sp.head) : -1;
+  const int yvec = yb >= 0 ? yb / E::VEC : -1;
+  const int yj = yb >= 0 ? yb % E::VEC : 0;
+
+  for (int i = tid; i < sp.head; i += kThreads) {
+    float g = grad1<HAS_ENT>(E::load1(x + i), c);
+    if (i == y) g += hot;
+    E::store1(d + i, g);
+  }
+  for (int i = sp.tail0 + tid; i < V; i += kThreads) {
+    float g = grad1<HAS_ENT>(E::load1(x + i), c);
+    if (i == y) g += hot;
+    E::store1(d + i, g);
+  }
+
+  auto do_vec = [&](const u32x4& in, int idx) {
+    float v[E::VEC], g[E::VEC];
+    E::unpack(in, v);
+#pragma unroll
+    for (int j = 0; j < E::VEC; ++j) g[j] = grad1<HAS_ENT>(v[j], c);
+    if (idx == yvec) {
+#pragma unroll
+      for (int j = 0; j < E::VEC; ++j) g[j] += (j == yj) ? hot : 0.f;
+    }
+    __builtin_nontemporal_store(E::pack(g), dv + idx);
+  };
+
+  constexpr int kTile = kThreads * kUnroll;
+  const int nfull = sp.nvec / kTile * kTile;
+  for (int base = 0; base < nfull; base += kTile) {
+    u32x4 buf[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) buf[u] = __builtin_nontemporal_load(xv + base + u * kThreads + tid);
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) do_vec(buf[u], base + u * kThreads + tid);
+  }
+  for (int i = nfull + tid; i < sp.nvec; i += kThreads) {
+    const u32x4 b = __builtin_nontemporal_load(xv + i);
+    do_vec(b, i);
+  }
+}
+
+template <class E>
+int launch_fwd(const void* logits, int64_t T, int V, int64_t row_stride, const int64_t* labels, float inv_T,
+               float* logprob, float* entropy, float* lse, float* ex, hipStream_t st) {
+  using elem_t = typename E::elem_t;
+  dim3 grid((unsigned)T), block(kThreads);
+  if (entropy)
+    lpe_fwd_kernel<E, true><<<grid, block, 0, st>>>((const elem_t*)logits, row_stride, V, labels, inv_T, logprob,
+                                                    entropy, lse, ex);
+  else
+    lpe_fwd_kernel<E, false><<<grid, block, 0, st>>>((const elem_t*)logits, row_stride, V, labels, inv_T, logprob,
+                                                     nullptr, lse, nullptr);
+  SIIRL_LAUNCH_CHECK("lpe_fwd_kernel");
+  return SIIRL_OK;
+}
+
+template <class E>
+int launch_bwd(const void* logits, int64_t T, int V, int64_t row_stride, const int64_t* labels, float inv_T,
+               const float* lse, const float* ex, const float* g_lp, const float* g_ent, void* dlogits,
+               int64_t d_stride, uint32_t flags, hipStream_t st) {
+  using elem_t = typename E::elem_t;
+  dim3 grid((unsigned)T), block(kThreads);
+  if (g_ent)
+    lpe_bwd_kernel<E, true><<<grid, block, 0, st>>>((const elem_t*)logits, row_stride, V, labels, inv_T, lse, ex,
+                                                    g_lp, g_ent, (elem_t*)dlogits, d_stride, flags);
+  else
+    lpe_bwd_kernel<E, false><<<grid, block, 0, st>>>((const elem_t*)logits, row_stride, V, labels, inv_T, lse,
+                                                     nullptr, g_lp, nullptr, (elem_t*)dlogits, d_stride, flags);
+  SIIRL_LAUNCH_CHECK("lpe_bwd_kernel");
+  return SIIRL_OK;
+}
+
+int check_common(const void* logits, int dt, int64_t T, int64_t V, int64_t row_stride, float inv_T) {
+  SIIRL_REQUIRE(dt == SIIRL_F32 || dt == SIIRL_BF16 || dt == SIIRL_F16,
+                "logits dtype %d not supported (f32, bf16, f16)", dt);
+  SIIRL_REQUIRE(T >= 0 && T <= 0x7fffffffLL, "T=%lld out of range", (long long)T);
+  SIIRL_REQUIRE(V >= 1 && V <= 0x3fffffffLL, "V=%lld out of range", (long long)V);
+  SIIRL_REQUIRE(row_stride >= V, "row_stride %lld < V %lld", (long long)row_stride, (long long)V);
+  SIIRL_REQUIRE(inv_T > 0.f && inv_T < 1e30f, "inv_temperature must be positive and finite");
+  SIIRL_REQUIRE(T == 0 || logits != nullptr, "logits is NULL");
+  SIIRL_REQUIRE(((uintptr_t)logits % dtype_size(dt)) == 0, "logits not aligned to its element size");
+  return SIIRL_OK;
+}
+
+}  // namespace
+}  // namespace siirl
+
+using namespace siirl;
+
+extern "C" int siirl_logprob_entropy_fwd(const void* logits, int logits_dtype, int64_t T, int64_t V,
+                                         int64_t row_stride, const int64_t* labels, float inv_temperature,
+                                         float* logprob, float* entropy, float* lse, float* ex,
+                                         siirl_stream_t stream) {
+  if (int rc = check_common(logits, logits_dtype, T, V, row_stride, inv_temperature)) return rc;
+  if (T == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(lse != nullptr, "lse is NULL");
+  SIIRL_REQUIRE((logprob == nullptr) == (labels == nullptr), "labels and logprob must be given together");
+  SIIRL_REQUIRE(entropy == nullptr || ex != nullptr, "ex is required when entropy is requested");
+  SIIRL_REQUIRE(logprob != nullptr || entropy != nullptr, "nothing requested: logprob and entropy are both NULL");
+  hipStream_t st = (hipStream_t)stream;
+  switch (logits_dtype) {
+    case SIIRL_BF16:
+      return launch_fwd<ElemBF16>(logits, T, (int)V, row_stride, labels, inv_temperature, logprob, entropy, lse, ex, st);
+    case SIIRL_F16:
+      return launch_fwd<ElemF16>(logits, T, (int)V, row_stride, labels, inv_temperature, logprob, entropy, lse, ex, st);
+    default:
+      return launch_fwd<ElemF32>(logits, T, (int)V, row_stride, labels, inv_temperature, logprob, entropy, lse, ex, st);
+  }
+}
+
+extern "C" int siirl_logprob_entropy_bwd(const void* logits, int logits_dtype, int64_t T, int64_t V,
+                                         int64_t row_stride, const int64_t* labels, float inv_temperature,
+                                         const float* lse, const float* ex, const float* g_logprob,
+                                         const float* g_entropy, void* dlogits, int64_t dlogits_row_stride,
+                                         uint32_t flags, siirl_stream_t stream) {
+  if (int rc = check_common(logits, logits_dtype, T, V, row_stride, inv_temperature)) return rc;
+  if (T == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(dlogits != nullptr && lse != nullptr, "dlogits / lse is NULL");
+  SIIRL_REQUIRE(dlogits_row_stride >= V, "dlogits_row_stride %lld < V", (long long)dlogits_row_stride);
+  SIIRL_REQUIRE(g_logprob != nullptr || g_entropy != nullptr, "no upstream gradient given");
+  SIIRL_REQUIRE(g_logprob == nullptr || labels != nullptr, "labels is required with g_logprob");
+  SIIRL_REQUIRE(g_entropy == nullptr || ex != nullptr, "ex is required with g_entropy");
+  SIIRL_REQUIRE((flags & ~SIIRL_BWD_SKIP_ZERO_ROWS) == 0, "unknown flags 0x%x", flags);
+  SIIRL_REQUIRE(((uintptr_t)dlogits % dtype_size(logits_dtype)) == 0, "dlogits not aligned to its element size");
+  if (dlogits == logits) {
+    SIIRL_REQUIRE(dlogits_row_stride == row_stride, "in-place backward needs equal row strides");
+  } else {
+    const size_t es = dtype_size(logits_dtype);
+    const uintptr_t a0 = (uintptr_t)logits, a1 = a0 + (size_t)((T - 1) * row_stride + V) * es;
+    const uintptr_t b0 = (uintptr_t)dlogits, b1 = b0 + (size_t)((T - 1) * dlogits_row_stride + V) * es;
+    SIIRL_REQUIRE(a1 <= b0 || b1 <= a0, "dlogits overlaps logits without being the same buffer");
+  }
+  hipStream_t st = (hipStream_t)stream;
+  switch (logits_dtype) {
+    case SIIRL_BF16:
+      return launch_bwd<ElemBF16>(logits, T, (int)V, row_stride, labels, inv_temperature, lse, ex, g_logprob,
+                                  g_entropy, dlogits, dlogits_row_stride, flags, st);
+    case SIIRL_F16:
+      return launch_bwd<ElemF16>(logits, T, (int)V, row_stride, labels, inv_temperature, lse, ex, g_logprob,
+                                 g_entropy, dlogits, dlogits_row_stride, flags, st);
+    default:
+      return launch_bwd<ElemF32>(logits, T, (int)V, row_stride, labels, inv_temperature, lse, ex, g_logprob,
+                                 g_entropy, dlogits, dlogits_row_stride, flags, st);
+  }
+}

@@ -1,0 +1,166 @@
+"""Log-prob / entropy from logits and masked reductions, with the reference's Python signatures.
+
+Mirror of ``siirl/utils/model_utils/torch_functional.py:41-168`` of the reference: same names, same
+argument meaning.  The arithmetic runs in ``libsiirl_hip.so``; tensors must live on the GPU.
+
+Differences a caller can observe, all deliberate:
+
+* results for 16-bit logits are fp32 (what the reference returns on its flash-attn dispatch,
+  ``torch_functional.py:73-79,85-90``); accumulation is always fp32;
+* ``logprobs_from_logits(..., inplace_backward=False)`` also computes the entropy in the same pass over
+  the row and parks it, so that the ``entropy_from_logits(logits)`` call that the actor issues next on
+  the same tensor (``siirl/engine/actor/dp_actor.py:179-195``) costs no second pass and both gradients
+  are written by one backward kernel.  ``set_pairing(False)`` turns this off.
+"""
+
+from __future__ import annotations
+
+import weakref
+from typing import Optional
+
+import torch
+
+from . import ops  # noqa: F401  (registers torch.ops.siirl_hip.*)
+
+_fwd = torch.ops.siirl_hip.logprob_entropy_fwd
+_bwd = torch.ops.siirl_hip.logprob_entropy_bwd
+_bwd_ = torch.ops.siirl_hip.logprob_entropy_bwd_
+
+_SKIP_ZERO_ROWS = True
+
+
+def set_skip_zero_rows(flag: bool) -> None:
+    """Backward writes zeros, without reading the row, where both upstream gradients are zero
+    (padding rows).  On by default; identical results for finite logits."""
+    global _SKIP_ZERO_ROWS
+    _SKIP_ZERO_ROWS = bool(flag)
+
+
+class _LogprobEntropy(torch.autograd.Function):
+    """(logits, labels) -> (logprob, entropy) with one forward pass and one backward pass over the rows."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, inv_temperature, want_entropy, inplace_backward):
+        lp, ent, lse, ex = _fwd(logits, labels, inv_temperature, want_entropy)
+        ctx.save_for_backward(logits, labels if labels is not None else lse.new_empty(0), lse, ex)
+        ctx.has_labels = labels is not None
+        ctx.want_entropy = want_entropy
+        ctx.inv_temperature = inv_temperature
+        ctx.inplace = inplace_backward
+        ctx.set_materialize_grads(False)
+        if labels is None:
+            ctx.mark_non_differentiable(lp)
+        if not want_entropy:
+            ctx.mark_non_differentiable(ent)
+        return lp, ent
+
+    @staticmethod
+    def backward(ctx, g_lp, g_ent):
+        logits, labels, lse, ex = ctx.saved_tensors
+        if not ctx.has_labels:
+            labels, g_lp = None, None
+        if not ctx.want_entropy:
+            g_ent = None
+        if g_lp is None and g_ent is None:
+            return None, None, None, None, None
+        args = (logits, labels if g_lp is not None else None, ctx.inv_temperature, lse,
+                ex if g_ent is not None else None, g_lp, g_ent, _SKIP_ZERO_ROWS)
+        if ctx.inplace:
+            _bwd_(*args)
+            return logits, None, None, None, None
+        return _bwd(*args), None, None, None, None
+
+
+def _check_logits(logits):
+    if not isinstance(logits, torch.Tensor) or logits.dim() < 1:
+        raise TypeError("logits must be a tensor of shape (..., vocab_size)")
+    if logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise TypeError(f"logits dtype {logits.dtype} is not supported (float32, bfloat16, float16)")
+    if logits.shape[-1] > 1 and logits.stride(-1) != 1:
+        logits = logits.contiguous()
+    return logits
+
+
+def logprobs_and_entropy_from_logits(logits: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
+                                     inplace_backward: bool = False):
+    """Both per-token outputs of the actor's post-logits step in one pass: ``(logprob, entropy)`` of
+    ``logits / temperature``.  The division is folded into the kernels, ``logits`` is left untouched
+    (the reference divides in place first, ``siirl/engine/actor/dp_actor.py:176``)."""
+    logits = _check_logits(logits)
+    return _LogprobEntropy.apply(logits, labels, 1.0 / float(temperature), True, inplace_backward)
+
+
+# ------------------------------------------------------------------------------ pairing slot
+
+_PAIRING = True
+_slot = None  # (weakref to logits, _version, grad_enabled, entropy)
+
+
+def set_pairing(flag: bool) -> None:
+    global _PAIRING, _slot
+    _PAIRING, _slot = bool(flag), None
+
+
+def _park(logits, entropy):
+    global _slot
+    _slot = (weakref.ref(logits), logits._version, torch.is_grad_enabled(), entropy)
+
+
+def _claim(logits):
+    global _slot
+    if _slot is None:
+        return None
+    ref, version, grad_mode, entropy = _slot
+    if ref() is logits and logits._version == version and torch.is_grad_enabled() == grad_mode:
+        _slot = None
+        return entropy
+    if ref() is None:
+        _slot = None
+    return None
+
+
+# ------------------------------------------------------------------------------ reference API
+
+
+def gather_from_labels(data: torch.Tensor, label: torch.Tensor) -> torch.Tensor:
+    """reference ``torch_functional.py:41-53`` (plain indexing; not a hot op)."""
+    return torch.gather(data, -1, label.unsqueeze(-1)).squeeze(-1)
+
+
+def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True):
+    """Log-probability of ``labels`` under ``softmax(logits)``, shape ``logits.shape[:-1]``
+    (reference ``torch_functional.py:56-82``).  With ``inplace_backward=True`` the backward pass
+    overwrites ``logits`` with its gradient, as the reference's flash-attn path does (``:85-90``)."""
+    logits = _check_logits(logits)
+    if _PAIRING and not inplace_backward:
+        lp, ent = _LogprobEntropy.apply(logits, labels, 1.0, True, False)
+        _park(logits, ent)
+        return lp
+    lp, _ = _LogprobEntropy.apply(logits, labels, 1.0, False, bool(inplace_backward))
+    return lp
+
+
+def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor):
+    """reference ``torch_functional.py:99-116``; same kernel, never in place."""
+    return logprobs_from_logits(logits, labels, inplace_backward=False)
+
+
+logprobs_from_logits_naive = logprobs_from_logits_v2  # reference :93-96
+
+
+def entropy_from_logits(logits: torch.Tensor):
+    """Entropy of ``softmax(logits)`` per row (reference ``torch_functional.py:128-132``)."""
+    logits = _check_logits(logits)
+    parked = _claim(logits) if _PAIRING else None
+    if parked is not None:
+        return parked
+    _, ent = _LogprobEntropy.apply(logits, None, 1.0, True, False)
+    return ent
+
+
+def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 2048):
+    """reference ``torch_functional.py:135-143``.  The chunking there bounds the fp32 temporaries; the
+    kernel has none, so the whole tensor goes in one launch.  2-D input, fp32 output, as there."""
+    if logits.dim() != 2:
+        raise ValueError("entropy_from_logits_with_chunking expects a 2-D tensor")
+    return entropy_from_logits(logits)

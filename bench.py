@@ -1,0 +1,210 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-token RL loss hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one pass of the hot path over one batch: log-prob + entropy forward over bf16 logits
+``[32768, 152064]`` (8 sequences x 4096 tokens, Qwen2.5-7B vocabulary), then the backward pass that
+writes ``dlogits`` -- the "logprob+entropy fwd+bwd" workload the headline metric is quoted on.  Inputs are
+synthetic and resident in HBM before the timed region.  One JSON line is printed at the end.
+
+``roofline`` describes the dominant kernel (the backward): algorithmic bytes per launch (read the row,
+write the gradient: 4 * V bytes per token for bf16) over its average duration, measured with events on
+the launch stream inside the timed region.  ``cpu_baseline`` times the CPU oracle (a torch restatement
+of the reference's eager ops) on a bounded row sample of the same tensor on the host cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "logprob+entropy fwd+bwd tokens/sec @vocab152k bf16; % HBM roofline"
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
+
+# Config 2 of the baseline: 8 sequences x 4096 tokens, vocab 152064, bf16 logits ~ N(0, 3) with one +15
+# spike in 1% of the rows, uniform labels, upstream gradients ~ N(0, 1e-2) zeroed on padded rows
+# (sequence lengths uniform in [512, 4096]).
+SEQS, SEQ_LEN, VOCAB = 8, 4096, 152064
+SEED = 20250602
+
+# HBM bytes per launch of the dominant kernel (lpe_bwd_kernel at the default workload) from two
+# rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same
+# counter reads for a plain 2 GiB device copy (FETCH_SIZE reads half the bytes fetched: factor 2.0;
+# WRITE_SIZE factor 1.0).  Figures and commands: profiles/lpe_config2_hbm_traffic.md
+MEASURED_TRAFFIC_BYTES = int((4872501.73 * 2.0 + 9732197.53) * 1024)
+
+
+def make_workload(dev, seqs=SEQS, seq_len=SEQ_LEN, vocab=VOCAB, seed=SEED):
+    import torch
+
+    T = seqs * seq_len
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    logits = torch.empty(T, vocab, dtype=torch.bfloat16, device=dev)
+    for lo in range(0, T, 2048):  # chunked so that the fp32 staging stays small
+        n = min(2048, T - lo)
+        logits[lo : lo + n] = (torch.randn(n, vocab, device=dev, generator=gen) * 3.0).to(torch.bfloat16)
+    n_spike = max(1, T // 100)
+    rows = torch.randperm(T, device=dev, generator=gen)[:n_spike]
+    cols = torch.randint(0, vocab, (n_spike,), device=dev, generator=gen)
+    logits[rows, cols] = (logits[rows, cols].float() + 15.0).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (T,), device=dev, generator=gen)
+    lengths = torch.randint(512, seq_len + 1, (seqs,), device=dev, generator=gen)
+    mask = (torch.arange(seq_len, device=dev)[None, :] < lengths[:, None]).reshape(T).float()
+    g_lp = torch.randn(T, device=dev, generator=gen) * 1e-2 * mask
+    g_ent = torch.randn(T, device=dev, generator=gen) * 1e-2 * mask
+    return logits, labels, g_lp, g_ent, mask
+
+
+def cpu_baseline(logits, labels, g_lp, g_ent, rows=4096, iters=5):
+    """Oracle (``kind: port``): the reference's eager ops on fp32-upcast rows, forward + autograd backward."""
+    import torch
+
+    from oracle import torch_functional as OF
+
+    x = logits[:rows].float().cpu()
+    y, a, b = labels[:rows].cpu(), g_lp[:rows].cpu(), g_ent[:rows].cpu()
+    times = []
+    for it in range(iters + 1):
+        xr = x.clone().requires_grad_(True)
+        t0 = time.perf_counter()
+        lp = OF.logprobs_from_logits(xr, y)
+        ent = OF.entropy_from_logits(xr)
+        torch.autograd.grad([lp, ent], [xr], [a, b])
+        dt = time.perf_counter() - t0
+        if it:  # first pass is the warm-up
+            times.append(dt)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first {rows} of {logits.shape[0]} rows of the same tensor, upcast to fp32; "
+                      f"median of {iters} fwd+bwd passes ({med:.2f} s each)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--with-row-skip", action="store_true",
+                    help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 2 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--seqs", type=int, default=SEQS, help="sequences of 4096 tokens (8 = the baseline's config)")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the hot path needs no collective; every row is "
+              "independent); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import siirl_amd.torch_functional as SF
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    SF.set_skip_zero_rows(False)  # dense: every row is read and written, as the algorithmic byte count assumes
+
+    logits, labels, g_lp, g_ent, mask = make_workload(dev, seqs=args.seqs)
+    T, V = logits.shape
+    x = logits.requires_grad_(True)
+
+    def step():
+        lp, ent = SF.logprobs_and_entropy_from_logits(x, labels)
+        (dx,) = torch.autograd.grad([lp, ent], [x], [g_lp, g_ent])
+        return lp, ent, dx
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        lp, ent = SF.logprobs_and_entropy_from_logits(x, labels)
+        ev[k][1].record()
+        (dx,) = torch.autograd.grad([lp, ent], [x], [g_lp, g_ent])
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    ms_per_step = wall * 1e3 / args.steps
+    tokens_per_s = T * args.steps / wall
+
+    es = logits.element_size()
+    fwd_bytes, bwd_bytes = es * V * T, 2 * es * V * T
+    bwd_gbs = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+    fwd_gbs = fwd_bytes / (fwd_ms * 1e-3) / 1e9
+    step_gbs = (fwd_bytes + bwd_bytes) / (ms_per_step * 1e-3) / 1e9
+
+    row_skip = None
+    if args.with_row_skip:  # padding rows written as zeros unread; reported beside the dense headline
+        SF.set_skip_zero_rows(True)
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        skip_wall = time.perf_counter() - t1
+        SF.set_skip_zero_rows(False)
+        n_valid = int(mask.sum().item())
+        row_skip = {"tokens_per_s": T * args.steps / skip_wall, "valid_tokens": n_valid,
+                    "algorithmic_bytes": es * V * (3 * n_valid + (T - n_valid))}
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.bfloat16, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
+    out = {
+        "metric": METRIC,
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"config2: logprob+entropy fwd+bwd, bf16 logits [{args.seqs}x{SEQ_LEN}, {V}] ~N(0,3), "
+                               "1% spiked rows, uniform labels, grads ~N(0,1e-2) zeroed on padding; dense rows",
+                   "tokens": T, "vocab": V, "seed": SEED},
+        "hbm_roofline_pct_step": 100.0 * step_gbs / HBM_PEAK_GBS,
+        "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
+        "kernels": {"lpe_fwd_kernel": {"ms": fwd_ms, "GB/s": fwd_gbs, "bytes": fwd_bytes},
+                    "lpe_bwd_kernel": {"ms": bwd_ms, "GB/s": bwd_gbs, "bytes": bwd_bytes}},
+        "roofline": {"bound": "hbm", "kernel": "lpe_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES if args.seqs == SEQS else None},
+        "row_skip_variant": row_skip,
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(logits.detach(), labels, g_lp, g_ent)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

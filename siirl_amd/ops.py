@@ -115,9 +115,15 @@ def _bwd_launch(logits, labels, inv_temperature, lse, ex, g_logprob, g_entropy, 
     if labels is not None:
         labels = labels.to(device=dev, dtype=torch.int64).contiguous()
     in_blocks = list(row_blocks(logits))
-    out_blocks = in_blocks if out is logits else list(row_blocks(out))
-    if [b[1] for b in in_blocks] != [b[1] for b in out_blocks]:
-        raise ValueError("siirl_amd: dlogits layout is incompatible with logits")
+    if out is logits:
+        out_blocks = in_blocks
+    else:  # a fresh contiguous tensor: rows follow one another whatever the blocking of the input
+        if not out.is_contiguous() or out.shape != logits.shape:
+            raise ValueError("siirl_amd: dlogits must be contiguous and shaped like logits")
+        out_blocks, r = [], 0
+        for _, rows, _ in in_blocks:
+            out_blocks.append((r * V, rows, V))
+            r += rows
     flags = _lib.BWD_SKIP_ZERO_ROWS if skip_zero_rows else 0
     done = 0
     with torch.cuda.device(dev):

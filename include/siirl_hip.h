@@ -114,6 +114,133 @@ int siirl_logprob_entropy_bwd(const void* logits, int logits_dtype, int64_t T, i
                               const float* g_logprob, const float* g_entropy, void* dlogits,
                               int64_t dlogits_row_stride, uint32_t flags, siirl_stream_t stream);
 
+/* ------------------------------------------------------------ [B, L] loss arithmetic of the actor */
+
+/* Bytes of scratch the *_fwd entry points below need for a [B, L] problem. */
+size_t siirl_loss_workspace_bytes(int64_t B, int64_t L);
+
+/* Layout of the 16-float result block `out16` written by siirl_agg_loss_fwd / siirl_actor_loss_fwd. */
+#define SIIRL_OUT_LOSS 0         /* (policy_loss) * loss_scale, the scalar that is back-propagated      */
+#define SIIRL_OUT_PG_LOSS 1      /* pg_loss (for siirl_agg_loss_fwd: the aggregated value)              */
+#define SIIRL_OUT_PG_CLIPFRAC 2  /* masked_mean(l2 > l1)                                                */
+#define SIIRL_OUT_PPO_KL 3       /* masked_mean(-(log_prob - old_log_prob))                             */
+#define SIIRL_OUT_PG_CLIPFRAC_LOWER 4
+#define SIIRL_OUT_ENTROPY_LOSS 5 /* agg_loss(entropy)            (0 when entropy is NULL)               */
+#define SIIRL_OUT_KL_LOSS 6      /* agg_loss(kl_penalty(lp,ref)) (0 when ref_log_prob is NULL)          */
+#define SIIRL_OUT_RATIO_MEAN 7   /* mean / min / max over ALL B*L tokens of exp(log_prob - old_log_prob) */
+#define SIIRL_OUT_RATIO_MIN 8
+#define SIIRL_OUT_RATIO_MAX 9
+#define SIIRL_OUT_MASK_TOTAL 10  /* sum of the mask                                                     */
+#define SIIRL_OUT_POLICY_LOSS 11 /* pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss          */
+
+/*
+ * agg_loss(loss_mat, loss_mask, loss_agg_mode): scalar aggregation of a [B, L] fp32 matrix.
+ * mask_dtype: U8 (bool), I32, I64, F32, BF16 or F16.  out16[SIIRL_OUT_PG_LOSS] receives the value,
+ * row_msum[B] the per-row mask sums (saved for the backward).  token-mean is
+ * sum(where(mask, v, 0) * mask) / (sum(mask) + 1e-8); seq-mean-token-mean has no epsilon, so a row with
+ * an empty mask yields NaN, as in the reference.
+ * Replaces: agg_loss siirl/dag_worker/core_algos.py:536-569; masked_sum / masked_mean
+ *           siirl/utils/model_utils/torch_functional.py:146-168 (token-mean numerator and value).
+ */
+int siirl_agg_loss_fwd(const float* loss_mat, const void* mask, int mask_dtype, int64_t B, int64_t L,
+                       int agg_mode, float* out16, float* row_msum, void* workspace, size_t workspace_bytes,
+                       siirl_stream_t stream);
+
+/* d(loss_mat) = g_out[0] * d(agg)/d(loss_mat).  g_out is a device scalar. */
+int siirl_agg_loss_bwd(const float* g_out, const void* mask, int mask_dtype, const float* out16,
+                       const float* row_msum, int64_t B, int64_t L, int agg_mode, float* d_loss_mat,
+                       siirl_stream_t stream);
+
+/*
+ * The actor's loss for one micro-batch in one pass over [B, L] fp32 operands:
+ *   pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower  = policy loss `loss_mode` (vanilla: PPO/GRPO/DAPO clip
+ *        with dual clip `clip_c`; gspo: sequence-level ratio, always seq-mean-token-mean),
+ *   entropy_loss = agg_loss(entropy)                       when entropy != NULL,
+ *   kl_loss      = agg_loss(kl_penalty(log_prob, ref))     when ref_log_prob != NULL,
+ *   loss = (pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss) * loss_scale,
+ * plus the ratio statistics the actor logs.  is_weights (rollout importance weights) may be NULL.
+ * row_msum[B] and row_s[B] (GSPO's per-sequence mean log-ratio; may be NULL for vanilla) are saved for
+ * the backward.  Called with entropy = ref_log_prob = NULL and loss_scale = 1 this is exactly
+ * compute_policy_loss_vanilla / compute_policy_loss_gspo.  log_ratio_clamp bounds |log_prob - old_log_prob|
+ * before the exponential in the vanilla loss: 20 as in core_algos.py:758, +infinity for the legacy
+ * compute_policy_loss (core_algos.py:631-707) which does not clamp.
+ * Replaces: siirl/dag_worker/core_algos.py:710-792 (vanilla), :795-862 (gspo), :1215-1276 (kl_penalty),
+ *           and the composition in siirl/engine/actor/dp_actor.py:455-513.
+ */
+int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_prob, const float* advantages,
+                         const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
+                         const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
+                         float clip_high, float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff,
+                         int kl_mode, int kl_straight_through, float kl_coef, float loss_scale, float* out16, float* row_msum,
+                         float* row_s, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
+
+/*
+ * Backward of the above for an upstream gradient g_loss[0] (device scalar) on out16[SIIRL_OUT_LOSS]:
+ * d_log_prob[B, L] and, when entropy was given, d_entropy[B, L].  Ties follow autograd: maximum / minimum
+ * split the gradient 1/2 : 1/2, clamp passes it on the closed interval.
+ */
+int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const float* log_prob,
+                         const float* advantages, const void* mask, int mask_dtype, const float* is_weights,
+                         const float* entropy, const float* ref_log_prob, int64_t B, int64_t L, int loss_mode,
+                         float clip_low, float clip_high, float clip_c, float log_ratio_clamp, int agg_mode,
+                         float entropy_coeff, int kl_mode, int kl_straight_through, float kl_coef, float loss_scale,
+                         const float* out16,
+                         const float* row_msum, const float* row_s, float* d_log_prob, float* d_entropy,
+                         siirl_stream_t stream);
+
+/*
+ * kl_penalty, elementwise over n fp32 values.  straight_through != 0 gives the k2 gradient
+ * (log_prob - ref) whatever the estimator.  d_logprob or d_ref_logprob may be NULL.
+ * Replaces: kl_penalty / kl_penalty_forward siirl/dag_worker/core_algos.py:1215-1276.
+ */
+int siirl_kl_penalty_fwd(const float* logprob, const float* ref_logprob, int64_t n, int kl_mode, float* out,
+                         siirl_stream_t stream);
+int siirl_kl_penalty_bwd(const float* g, const float* logprob, const float* ref_logprob, int64_t n, int kl_mode,
+                         int straight_through, float* d_logprob, float* d_ref_logprob, siirl_stream_t stream);
+
+/*
+ * masked_sum / masked_mean over a [B, L] fp32 matrix: row_sum[b] = sum_t where(mask, v, 0) * mask,
+ * row_mean[b] = row_sum[b] / (sum_t mask + 1e-8), total2 = {sum over all, sum / (sum(mask) + 1e-8)}.
+ * Any of the three outputs may be NULL.  Workspace as for the loss entry points.
+ * Replaces: masked_sum / masked_mean siirl/utils/model_utils/torch_functional.py:146-168 (axis None or -1).
+ */
+int siirl_masked_reduce(const float* values, const void* mask, int mask_dtype, int64_t B, int64_t L, float* row_sum,
+                        float* row_mean, float* total2, void* workspace, size_t workspace_bytes,
+                        siirl_stream_t stream);
+
+/*
+ * KL penalty folded into the reward: kld = kl_penalty(old_log_prob, ref_log_prob) * mask,
+ * token_level_rewards = token_level_scores - beta * kld, row_kl[b] = masked_mean(kld, mask) of row b,
+ * current_kl[0] = mean_b row_kl[b] (device scalar; the controller update stays on the host).
+ * Replaces: apply_kl_penalty siirl/dag_worker/core_algos.py:1358-1397 (device arithmetic).
+ */
+int siirl_kl_in_reward(const float* token_level_scores, const float* old_log_prob, const float* ref_log_prob,
+                       const void* mask, int mask_dtype, int64_t B, int64_t L, int kl_mode, float beta,
+                       float* token_level_rewards, float* row_kl, float* current_kl, siirl_stream_t stream);
+
+/* ------------------------------------------------------------------- per-prompt group statistics */
+
+/*
+ * GRPO outcome advantage: s_i = sum_t rewards[i, t]; per group of equal uid the mean and the unbiased
+ * (N-1) standard deviation (a group of one: mean 0, std 1); a_i = (s_i - mean) / (std + epsilon), or
+ * s_i - mean when norm_adv_by_std == 0; advantages[i, t] = a_i * mask[i, t].  uid values are arbitrary.
+ * scratch_2B: 2*B floats of scratch; on return scratch_2B[0..B) holds the scores s_i and [B..2B) the a_i.
+ * Replaces: compute_grpo_outcome_advantage siirl/dag_worker/core_algos.py:279-348.
+ */
+int siirl_grpo_outcome_advantage(const float* token_level_rewards, const void* mask, int mask_dtype,
+                                 const int64_t* uid, int64_t B, int64_t L, float epsilon, int norm_adv_by_std,
+                                 float* advantages, float* scratch_2B, siirl_stream_t stream);
+
+/*
+ * DAPO dynamic sampling: keep[i] = 1 iff the uid-group of trajectory i has a single member or
+ * np.std(metric of the group) > 0, with numpy's arithmetic (population std, pairwise summation, in the
+ * dtype of the metric: SIIRL_F32 or SIIRL_F64) reproduced bit for bit.  group_size (int32[B], may be
+ * NULL) receives each trajectory's group size.  The kept indices are the positions of the ones, ascending.
+ * Replaces: the group test of dynamic_sampling siirl/user_interface/filter_interface/dapo.py:66-93.
+ */
+int siirl_group_keep_mask(const void* metric, int metric_dtype, const int64_t* uid, int64_t B, uint8_t* keep,
+                          int32_t* group_size, siirl_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

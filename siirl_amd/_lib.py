@@ -22,6 +22,19 @@ SIGNATURES = {
     "siirl_hip_last_error": (C.c_char_p, []),
     "siirl_logprob_entropy_fwd": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p]),
     "siirl_logprob_entropy_bwd": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p, _i64, _u32, _p]),
+    "siirl_loss_workspace_bytes": (_sz, [_i64, _i64]),
+    "siirl_agg_loss_fwd": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
+    "siirl_agg_loss_bwd": (_i32, [_p, _p, _i32, _p, _p, _i64, _i64, _i32, _p, _p]),
+    "siirl_actor_loss_fwd": (_i32, [_p, _p, _p, _p, _i32, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _f32, _f32, _i32,
+                                    _f32, _i32, _i32, _f32, _f32, _p, _p, _p, _p, _sz, _p]),
+    "siirl_actor_loss_bwd": (_i32, [_p, _p, _p, _p, _p, _i32, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _f32, _f32,
+                                    _i32, _f32, _i32, _i32, _f32, _f32, _p, _p, _p, _p, _p, _p]),
+    "siirl_kl_penalty_fwd": (_i32, [_p, _p, _i64, _i32, _p, _p]),
+    "siirl_kl_penalty_bwd": (_i32, [_p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
+    "siirl_masked_reduce": (_i32, [_p, _p, _i32, _i64, _i64, _p, _p, _p, _p, _sz, _p]),
+    "siirl_kl_in_reward": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i32, _f32, _p, _p, _p, _p]),
+    "siirl_grpo_outcome_advantage": (_i32, [_p, _p, _i32, _p, _i64, _i64, _f32, _i32, _p, _p, _p]),
+    "siirl_group_keep_mask": (_i32, [_p, _i32, _p, _i64, _p, _p, _p]),
 }
 
 _lock = threading.Lock()

@@ -1,0 +1,631 @@
+"""Advantages, policy losses, aggregation and KL penalty with the reference's Python signatures.
+
+Mirror of the in-scope part of ``siirl/dag_worker/core_algos.py``: the two registries (``:51-86``,
+``:127-164``), ``compute_grpo_outcome_advantage`` (``:279-348``), ``agg_loss`` (``:536-569``),
+``compute_policy_loss`` (``:631-707``), ``compute_policy_loss_vanilla`` (``:710-792``),
+``compute_policy_loss_gspo`` (``:795-862``), ``kl_penalty`` (``:1215-1276``), the KL controllers
+(``:167-226``), ``apply_kl_penalty`` (``:1358-1397``) and the GRPO branch of ``compute_advantage``
+(``:1400-1471``).  Same names, keyword arguments, return order and exception types; the arithmetic
+runs in ``libsiirl_hip.so``.  ``actor_loss`` is an addition: the whole loss of one micro-batch
+(policy loss, entropy bonus, KL loss, scaling, logged metrics) in one fused launch.
+
+Tensors must be on the GPU, except in ``compute_grpo_outcome_advantage`` / ``apply_kl_penalty`` /
+``compute_advantage``, which the reference runs on host tensors: host inputs are staged to the
+current GPU and the results returned on the host.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from enum import Enum
+from typing import Any, Callable, Optional
+
+import numpy as np
+import torch
+
+from . import _lib
+from . import torch_functional as siirl_F
+
+__all__ = [
+    "register_policy_loss", "get_policy_loss_fn", "register_adv_est", "get_adv_estimator_fn", "AdvantageEstimator",
+    "AdaptiveKLController", "FixedKLController", "get_kl_controller", "compute_response_mask",
+    "compute_grpo_outcome_advantage", "compute_rewards", "agg_loss", "compute_policy_loss",
+    "compute_policy_loss_vanilla", "compute_policy_loss_gspo", "kl_penalty", "kl_penalty_forward",
+    "apply_kl_penalty", "compute_advantage", "actor_loss", "ActorLossOutput",
+]
+
+AGG_MODES = {"token-mean": 0, "seq-mean-token-sum": 1, "seq-mean-token-mean": 2, "seq-mean-token-sum-norm": 3}
+KL_MODES = {"kl": 0, "k1": 0, "abs": 1, "mse": 2, "k2": 2, "low_var_kl": 3, "k3": 3}
+LOSS_VANILLA, LOSS_GSPO = 0, 1
+# indices into the 16-float result block (SIIRL_OUT_* of include/siirl_hip.h)
+O_LOSS, O_PG, O_CLIPFRAC, O_PPOKL, O_CLIPLOWER, O_ENT, O_KL, O_RMEAN, O_RMIN, O_RMAX, O_MTOTAL, O_POLICY = range(12)
+
+
+class AdvantageEstimator(str, Enum):
+    """reference ``siirl/execution/scheduler/enums.py:20-30``"""
+
+    GAE = "gae"
+    GRPO = "grpo"
+    CPGD = "cpgd"
+    GAE_MARFT = "gae_marft"
+
+
+# ------------------------------------------------------------------------------------ registries
+
+PolicyLossFn = Callable[..., tuple]
+POLICY_LOSS_REGISTRY: dict[str, PolicyLossFn] = {}
+ADV_ESTIMATOR_REGISTRY: dict[str, Any] = {}
+
+
+def register_policy_loss(name: str):
+    """Decorator: file a policy-loss function under ``name`` (reference ``core_algos.py:54-68``)."""
+
+    def decorator(func):
+        POLICY_LOSS_REGISTRY[name] = func
+        return func
+
+    return decorator
+
+
+def get_policy_loss_fn(name):
+    """reference ``core_algos.py:71-86``: unknown names raise ``ValueError`` listing what exists."""
+    if name not in POLICY_LOSS_REGISTRY:
+        raise ValueError(f"Unsupported loss mode: {name}. Supported modes are: {list(POLICY_LOSS_REGISTRY.keys())}")
+    return POLICY_LOSS_REGISTRY[name]
+
+
+def register_adv_est(name_or_enum):
+    """reference ``core_algos.py:130-148``: a taken name may only be re-registered with the same function."""
+
+    def decorator(fn):
+        name = name_or_enum.value if isinstance(name_or_enum, Enum) else name_or_enum
+        if name in ADV_ESTIMATOR_REGISTRY and ADV_ESTIMATOR_REGISTRY[name] != fn:
+            raise ValueError(f"Adv estimator {name} has already been registered: {ADV_ESTIMATOR_REGISTRY[name]} vs {fn}")
+        ADV_ESTIMATOR_REGISTRY[name] = fn
+        return fn
+
+    return decorator
+
+
+def get_adv_estimator_fn(name_or_enum):
+    """reference ``core_algos.py:151-164``"""
+    name = name_or_enum.value if isinstance(name_or_enum, Enum) else name_or_enum
+    if name not in ADV_ESTIMATOR_REGISTRY:
+        raise ValueError(f"Unknown advantage estimator simply: {name}")
+    return ADV_ESTIMATOR_REGISTRY[name]
+
+
+# ------------------------------------------------------------------------------------ plumbing
+
+
+def _f32(t: torch.Tensor, dev) -> torch.Tensor:
+    return t.detach().to(device=dev, dtype=torch.float32).contiguous()
+
+
+def _mask_arg(mask: torch.Tensor, dev):
+    m = mask.detach().to(device=dev)
+    if m.dtype not in (torch.bool, torch.uint8, torch.int32, torch.int64, torch.float32, torch.bfloat16, torch.float16):
+        m = m.to(torch.float32)
+    m = m.contiguous()
+    return m, _lib.dtype_code(m.dtype)
+
+
+def _as_2d(t: torch.Tensor):
+    if t.dim() == 2:
+        return t
+    if t.dim() == 1:
+        return t.unsqueeze(0)
+    return t.reshape(-1, t.shape[-1])
+
+
+def _gpu_of(*tensors):
+    for t in tensors:
+        if isinstance(t, torch.Tensor) and t.is_cuda:
+            return t.device
+    raise RuntimeError("siirl_amd: these ops run on the GPU only (no CPU fallback); move the tensors to the device")
+
+
+def _staging_device(*tensors):
+    """Device to compute on for the ops the reference runs on host tensors, and whether to copy back."""
+    for t in tensors:
+        if isinstance(t, torch.Tensor) and t.is_cuda:
+            return t.device, False
+    if not torch.cuda.is_available():
+        raise RuntimeError("siirl_amd: no GPU visible; there is no CPU fallback")
+    return torch.device("cuda", torch.cuda.current_device()), True
+
+
+def _workspace(B, L, dev):
+    n = _lib.lib().siirl_loss_workspace_bytes(B, L)
+    return torch.empty(n, dtype=torch.uint8, device=dev), n
+
+
+def _agg_code(loss_agg_mode: str) -> int:
+    if loss_agg_mode not in AGG_MODES:
+        raise ValueError(f"Invalid loss_agg_mode: {loss_agg_mode}")
+    return AGG_MODES[loss_agg_mode]
+
+
+# ------------------------------------------------------------------------------------ KL controllers
+
+
+class AdaptiveKLController:
+    """reference ``core_algos.py:167-189`` (https://arxiv.org/pdf/1909.08593.pdf)"""
+
+    def __init__(self, init_kl_coef, target_kl, horizon):
+        self.value = init_kl_coef
+        self.target = target_kl
+        self.horizon = horizon
+
+    def update(self, current_kl, n_steps):
+        proportional_error = np.clip(current_kl / self.target - 1, -0.2, 0.2)
+        self.value *= 1 + proportional_error * n_steps / self.horizon
+
+
+class FixedKLController:
+    """reference ``core_algos.py:192-206``"""
+
+    def __init__(self, kl_coef):
+        self.value = kl_coef
+
+    def update(self, current_kl, n_steps):
+        pass
+
+
+def get_kl_controller(kl_ctrl):
+    """reference ``core_algos.py:209-226``"""
+    if kl_ctrl.type == "fixed":
+        return FixedKLController(kl_coef=kl_ctrl.kl_coef)
+    if kl_ctrl.type == "adaptive":
+        assert kl_ctrl.horizon > 0, f"horizon must be larger than 0. Got {kl_ctrl.horizon}"
+        return AdaptiveKLController(init_kl_coef=kl_ctrl.kl_coef, target_kl=kl_ctrl.target_kl, horizon=kl_ctrl.horizon)
+    raise NotImplementedError
+
+
+# ------------------------------------------------------------------------------------ advantages
+
+
+def compute_response_mask(data):
+    """``attention_mask[:, -response_length:]``, 3-D embodied responses flattened (reference
+    ``core_algos.py:89-125``).  Pure indexing."""
+    responses, attention_mask = data["responses"], data["attention_mask"]
+    if responses.ndim == 3:
+        if attention_mask.ndim == 3:
+            return attention_mask[:, :, -responses.size(2):].reshape(responses.size(0), -1)
+        return attention_mask[:, -(responses.size(1) * responses.size(2)):]
+    if responses.ndim == 2:
+        return attention_mask[:, -responses.size(1):]
+    raise ValueError(f"Unexpected responses shape: {responses.shape}, ndim={responses.ndim}")
+
+
+def _uid_tensor(index, n, dev) -> torch.Tensor:
+    if isinstance(index, torch.Tensor):
+        out = index.detach().reshape(-1).to(device=dev, dtype=torch.int64)
+    else:
+        arr = np.asarray(index)
+        if arr.dtype.kind not in "iu":
+            arr = np.asarray([int(v) for v in arr.reshape(-1)], dtype=np.int64)  # numeric strings, floats
+        out = torch.from_numpy(np.ascontiguousarray(arr.reshape(-1).astype(np.int64))).to(dev)
+    if out.numel() != n:
+        raise ValueError(f"index has {out.numel()} entries for a batch of {n}")
+    return out.contiguous()
+
+
+@register_adv_est(AdvantageEstimator.GRPO)
+def compute_grpo_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
+                                   epsilon: float = 1e-6, norm_adv_by_std_in_grpo: bool = True, config=None):
+    """Group-normalised outcome advantage (reference ``core_algos.py:279-348``): the sequence score is
+    normalised by the mean and unbiased std of its ``index`` group (a group of one: mean 0, std 1),
+    broadcast over the tokens and masked.  Returns the same ``[B, L]`` fp32 tensor twice."""
+    dev, back = _staging_device(token_level_rewards, response_mask)
+    B, L = token_level_rewards.shape
+    r = _f32(token_level_rewards, dev)
+    m, mcode = _mask_arg(response_mask, dev)
+    uid = _uid_tensor(index, B, dev)
+    adv = torch.empty(B, L, dtype=torch.float32, device=dev)
+    scratch = torch.empty(2 * max(B, 1), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().siirl_grpo_outcome_advantage(_lib.ptr(r), _lib.ptr(m), mcode, _lib.ptr(uid), B, L,
+                                                     float(epsilon), int(bool(norm_adv_by_std_in_grpo)),
+                                                     _lib.ptr(adv), _lib.ptr(scratch), _lib.current_stream(dev))
+    _lib.check(rc, "siirl_grpo_outcome_advantage")
+    if back:
+        adv = adv.to(token_level_rewards.device)
+    return adv, adv
+
+
+def compute_rewards(token_level_scores, old_log_prob, ref_log_prob, kl_ratio):
+    """reference ``core_algos.py:520-533``: ``scores - (old - ref) * kl_ratio`` (k1 estimator, no mask)."""
+    dev = _gpu_of(token_level_scores, old_log_prob, ref_log_prob)
+    ones = torch.ones(token_level_scores.shape, dtype=torch.uint8, device=dev)
+    rewards, _ = _kl_in_reward(token_level_scores, old_log_prob, ref_log_prob, ones, "kl", float(kl_ratio), dev)
+    return rewards
+
+
+def _kl_in_reward(scores, old, ref, mask, kl_type, beta, dev):
+    if kl_type not in KL_MODES:
+        raise NotImplementedError
+    s2 = _as_2d(_f32(scores, dev))
+    B, L = s2.shape
+    o2, r2 = _as_2d(_f32(old, dev)), _as_2d(_f32(ref, dev))
+    m, mcode = _mask_arg(_as_2d(mask), dev)
+    rewards = torch.empty_like(s2)
+    row_kl = torch.empty(B, dtype=torch.float32, device=dev)
+    cur = torch.empty(1, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().siirl_kl_in_reward(_lib.ptr(s2), _lib.ptr(o2), _lib.ptr(r2), _lib.ptr(m), mcode, B, L,
+                                           KL_MODES[kl_type], float(beta), _lib.ptr(rewards), _lib.ptr(row_kl),
+                                           _lib.ptr(cur), _lib.current_stream(dev))
+    _lib.check(rc, "siirl_kl_in_reward")
+    return rewards.reshape(scores.shape), cur
+
+
+def _td_set(data, key, value):
+    target = data.batch if hasattr(data, "batch") and not callable(getattr(data, "batch")) else data
+    target[key] = value
+
+
+def apply_kl_penalty(data, kl_ctrl, kl_penalty="kl", multi_turn=False):
+    """KL-in-reward (reference ``core_algos.py:1358-1397``): ``token_level_rewards = token_level_scores -
+    beta * kl_penalty(old_log_probs, ref_log_prob) * response_mask``; the controller is then updated with
+    the batch mean of the per-sequence masked mean.  ``data`` is any mapping of tensors."""
+    scores = data["token_level_scores"]
+    dev, back = _staging_device(scores, data["old_log_probs"])
+    beta = kl_ctrl.value
+    rewards, cur = _kl_in_reward(scores, data["old_log_probs"], data["ref_log_prob"], data["response_mask"],
+                                 kl_penalty, beta, dev)
+    current_kl = cur.item()
+    batch_size = data.batch_size[0] if hasattr(data, "batch_size") else scores.shape[0]
+    kl_ctrl.update(current_kl=current_kl, n_steps=batch_size)
+    _td_set(data, "token_level_rewards", rewards.to(scores.device) if back else rewards)
+    return data, {"actor/reward_kl_penalty": current_kl, "actor/reward_kl_penalty_coeff": beta}
+
+
+def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_in_grpo=True,
+                      weight_factor_in_cpgd="STD_weight", **kwargs):
+    """Dispatcher (reference ``core_algos.py:1400-1492``).  Only the GRPO branch (``:1440-1471``) is in scope;
+    GAE / MARFT raise ``NotImplementedError`` here, and the CPGD branch fails with the reference's own
+    ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a keyword it does not take, ``:1475-1480``)."""
+    if "response_mask" not in data.keys():
+        _td_set(data, "response_mask", compute_response_mask(data))
+    est = adv_estimator.value if isinstance(adv_estimator, Enum) else adv_estimator
+    if est == "grpo":
+        if "finish_step" in data.keys() and data["responses"].ndim == 3:
+            responses = data["responses"]
+            length = responses.size(1) * responses.size(2)
+            finish = data["finish_step"] * responses.size(2)
+            steps = torch.arange(length, device=responses.device).unsqueeze(0).expand(responses.size(0), -1)
+            calc_mask = steps < finish.unsqueeze(1)
+        else:
+            calc_mask = data["response_mask"]
+        advantages, returns = compute_grpo_outcome_advantage(
+            token_level_rewards=data["token_level_rewards"], response_mask=calc_mask, index=data["uid"],
+            norm_adv_by_std_in_grpo=norm_adv_by_std_in_grpo)
+        data["advantages"] = advantages
+        data["returns"] = returns
+        data["response_mask"] = calc_mask
+        return data
+    if est == "cpgd":
+        compute_grpo_outcome_advantage(token_level_rewards=data["token_level_rewards"],
+                                       response_mask=data["response_mask"], index=data["uid"],
+                                       weight_factor_in_cpgd=weight_factor_in_cpgd)
+    raise NotImplementedError(f"advantage estimator {est!r} is outside this build (GRPO only)")
+
+
+# ------------------------------------------------------------------------------------ aggregation
+
+
+class _AggLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, loss_mat, loss_mask, agg_code):
+        dev = loss_mat.device
+        v = _as_2d(_f32(loss_mat, dev))
+        B, L = v.shape
+        m, mcode = _mask_arg(_as_2d(loss_mask), dev)
+        out16 = torch.empty(16, dtype=torch.float32, device=dev)
+        row_msum = torch.empty(B, dtype=torch.float32, device=dev)
+        ws, nws = _workspace(B, L, dev)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().siirl_agg_loss_fwd(_lib.ptr(v), _lib.ptr(m), mcode, B, L, agg_code, _lib.ptr(out16),
+                                               _lib.ptr(row_msum), _lib.ptr(ws), nws, _lib.current_stream(dev))
+        _lib.check(rc, "siirl_agg_loss_fwd")
+        ctx.save_for_backward(m, out16, row_msum)
+        ctx.meta = (mcode, B, L, agg_code, loss_mat.shape, loss_mat.dtype)
+        return out16[O_PG]
+
+    @staticmethod
+    def backward(ctx, g):
+        m, out16, row_msum = ctx.saved_tensors
+        mcode, B, L, agg_code, shape, dtype = ctx.meta
+        dev = out16.device
+        g = g.detach().to(torch.float32).reshape(1).contiguous()
+        d = torch.empty(B, L, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().siirl_agg_loss_bwd(_lib.ptr(g), _lib.ptr(m), mcode, _lib.ptr(out16), _lib.ptr(row_msum),
+                                               B, L, agg_code, _lib.ptr(d), _lib.current_stream(dev))
+        _lib.check(rc, "siirl_agg_loss_bwd")
+        return d.reshape(shape).to(dtype), None, None
+
+
+def agg_loss(loss_mat: torch.Tensor, loss_mask: torch.Tensor, loss_agg_mode: str):
+    """Aggregate a ``[B, L]`` loss into a scalar (reference ``core_algos.py:536-569``); unknown modes raise
+    ``ValueError``.  ``seq-mean-token-mean`` of a row with an empty mask is NaN, as in the reference."""
+    code = _agg_code(loss_agg_mode)
+    _gpu_of(loss_mat)
+    return _AggLoss.apply(loss_mat, loss_mask, code)
+
+
+# ------------------------------------------------------------------------------------ policy loss
+
+
+class _ActorLoss(torch.autograd.Function):
+    """One fused forward (partials + finish) and one elementwise backward for the whole micro-batch loss.
+    ``policy_only``: the four policy-loss scalars are the outputs and the gradient enters through pg_loss;
+    otherwise the scaled total enters through ``loss``.  The other scalars are metrics (no gradient)."""
+
+    @staticmethod
+    def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, ref_log_prob, cfg):
+        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, scale,
+         policy_only) = cfg
+        dev = log_prob.device
+        lp = _as_2d(_f32(log_prob, dev))
+        B, L = lp.shape
+        old = _as_2d(_f32(old_log_prob, dev))
+        adv = _as_2d(_f32(advantages, dev))
+        m, mcode = _mask_arg(_as_2d(response_mask), dev)
+        isw = None if is_weights is None else _as_2d(_f32(is_weights, dev))
+        ent = None if entropy is None else _as_2d(_f32(entropy, dev))
+        ref = None if ref_log_prob is None else _as_2d(_f32(ref_log_prob, dev))
+        for name, t in (("old_log_prob", old), ("advantages", adv), ("response_mask", m), ("rollout_is_weights", isw),
+                        ("entropy", ent), ("ref_log_prob", ref)):
+            if t is not None and tuple(t.shape) != (B, L):
+                raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {(B, L)}")
+        out16 = torch.empty(16, dtype=torch.float32, device=dev)
+        row_msum = torch.empty(B, dtype=torch.float32, device=dev)
+        row_s = torch.empty(B, dtype=torch.float32, device=dev)
+        ws, nws = _workspace(B, L, dev)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().siirl_actor_loss_fwd(
+                _lib.ptr(old), _lib.ptr(lp), _lib.ptr(adv), _lib.ptr(m), mcode, _lib.ptr(isw), _lib.ptr(ent),
+                _lib.ptr(ref), B, L, loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st,
+                kl_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s), _lib.ptr(ws), nws,
+                _lib.current_stream(dev))
+        _lib.check(rc, "siirl_actor_loss_fwd")
+        ctx.save_for_backward(lp, old, adv, m, out16, row_msum, row_s,
+                              *(t for t in (isw, ent, ref) if t is not None))
+        ctx.flags = (isw is not None, ent is not None, ref is not None)
+        ctx.meta = (mcode, B, L, cfg, log_prob.shape, log_prob.dtype,
+                    None if entropy is None else (entropy.shape, entropy.dtype))
+        ctx.set_materialize_grads(False)
+        outs = tuple(out16[i] for i in range(12))
+        diff = (O_PG,) if policy_only else (O_LOSS,)
+        ctx.mark_non_differentiable(*(o for i, o in enumerate(outs) if i not in diff))
+        ctx.diff_index = diff[0]
+        return outs
+
+    @staticmethod
+    def backward(ctx, *grads):
+        g = grads[ctx.diff_index]
+        if g is None:
+            return (None,) * 8
+        lp, old, adv, m, out16, row_msum, row_s, *rest = ctx.saved_tensors
+        has_isw, has_ent, has_ref = ctx.flags
+        rest = list(rest)
+        isw = rest.pop(0) if has_isw else None
+        ent = rest.pop(0) if has_ent else None
+        ref = rest.pop(0) if has_ref else None
+        mcode, B, L, cfg, lp_shape, lp_dtype, ent_meta = ctx.meta
+        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, scale, _) = cfg
+        dev = lp.device
+        g = g.detach().to(torch.float32).reshape(1).contiguous()
+        d_lp = torch.empty(B, L, dtype=torch.float32, device=dev)
+        d_ent = torch.empty(B, L, dtype=torch.float32, device=dev) if has_ent else None
+        with torch.cuda.device(dev):
+            rc = _lib.lib().siirl_actor_loss_bwd(
+                _lib.ptr(g), _lib.ptr(old), _lib.ptr(lp), _lib.ptr(adv), _lib.ptr(m), mcode, _lib.ptr(isw),
+                _lib.ptr(ent), _lib.ptr(ref), B, L, loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef,
+                kl_code, kl_st, kl_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s), _lib.ptr(d_lp),
+                _lib.ptr(d_ent), _lib.current_stream(dev))
+        _lib.check(rc, "siirl_actor_loss_bwd")
+        g_lp = d_lp.reshape(lp_shape).to(lp_dtype)
+        g_ent = None if d_ent is None else d_ent.reshape(ent_meta[0]).to(ent_meta[1])
+        return g_lp, g_ent, None, None, None, None, None, None
+
+
+def _clip_params(config):
+    clip_ratio = config.clip_ratio
+    lo = config.clip_ratio_low if getattr(config, "clip_ratio_low", None) is not None else clip_ratio
+    hi = config.clip_ratio_high if getattr(config, "clip_ratio_high", None) is not None else clip_ratio
+    return float(lo), float(hi)
+
+
+def _policy_only(loss_mode, old_log_prob, log_prob, advantages, response_mask, agg_code, lo, hi, c, dclamp,
+                 rollout_is_weights):
+    _gpu_of(log_prob)
+    cfg = (loss_mode, lo, hi, float(c), float(dclamp), agg_code, 0.0, 0, 0, 0.0, 1.0, True)
+    outs = _ActorLoss.apply(log_prob, None, old_log_prob, advantages, response_mask, rollout_is_weights, None, cfg)
+    return outs[O_PG], outs[O_CLIPFRAC], outs[O_PPOKL], outs[O_CLIPLOWER]
+
+
+@register_policy_loss("vanilla")
+def compute_policy_loss_vanilla(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                response_mask: torch.Tensor, loss_agg_mode: str = "token-mean", config=None,
+                                rollout_is_weights: Optional[torch.Tensor] = None):
+    """Clipped PPO / GRPO / DAPO objective with dual clip (reference ``core_algos.py:710-792``).
+    ``config`` is any object with ``clip_ratio``, ``clip_ratio_low``, ``clip_ratio_high``, ``clip_ratio_c``.
+    Returns ``(pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower)`` as 0-d device tensors; only ``pg_loss``
+    carries a gradient (to ``log_prob``)."""
+    assert config is not None
+    assert type(config).__name__ != "AlgorithmArguments"  # reference :744
+    lo, hi = _clip_params(config)
+    clip_ratio_c = config.clip_ratio_c
+    assert clip_ratio_c > 1.0, (
+        "The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0,"
+        + f" but get the value: {clip_ratio_c}."
+    )
+    return _policy_only(LOSS_VANILLA, old_log_prob, log_prob, advantages, response_mask, _agg_code(loss_agg_mode),
+                        lo, hi, clip_ratio_c, 20.0, rollout_is_weights)
+
+
+@register_policy_loss("gspo")
+def compute_policy_loss_gspo(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                             response_mask: torch.Tensor, loss_agg_mode: str = "seq-mean-token-mean", config=None,
+                             rollout_is_weights: Optional[torch.Tensor] = None):
+    """GSPO (reference ``core_algos.py:795-862``): sequence-level importance ratio, token-level gradient,
+    always aggregated ``seq-mean-token-mean`` whatever ``loss_agg_mode`` says (``:854``);
+    ``pg_clipfrac_lower`` is zero."""
+    assert config is not None
+    assert all(hasattr(config, k) for k in ("clip_ratio", "clip_ratio_low", "clip_ratio_high"))  # reference :824
+    lo, hi = _clip_params(config)
+    return _policy_only(LOSS_GSPO, old_log_prob, log_prob, advantages, response_mask,
+                        AGG_MODES["seq-mean-token-mean"], lo, hi, 3.0, 20.0, rollout_is_weights)
+
+
+def compute_policy_loss(old_log_prob, log_prob, advantages, response_mask, cliprange=None, cliprange_low=None,
+                        cliprange_high=None, clip_ratio_c=3.0, loss_agg_mode: str = "token-mean", use_cpgd_loss=False):
+    """The legacy entry (reference ``core_algos.py:631-707``): as ``vanilla`` but the log-ratio is not clamped
+    to +-20.  The CPGD variant (``use_cpgd_loss=True``) is outside this build."""
+    assert clip_ratio_c > 1.0, (
+        "The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0,"
+        + f" but get the value: {clip_ratio_c}."
+    )
+    if use_cpgd_loss:
+        raise NotImplementedError("the CPGD loss is outside this build")
+    lo = cliprange if cliprange_low is None else cliprange_low
+    hi = cliprange if cliprange_high is None else cliprange_high
+    return _policy_only(LOSS_VANILLA, old_log_prob, log_prob, advantages, response_mask, _agg_code(loss_agg_mode),
+                        float(lo), float(hi), clip_ratio_c, float("inf"), None)
+
+
+# ------------------------------------------------------------------------------------ KL penalty
+
+
+class _KlPenalty(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logprob, ref_logprob, code, straight_through):
+        dev = logprob.device
+        lp, ref = _f32(logprob, dev), _f32(ref_logprob, dev)
+        if ref.shape != lp.shape:
+            ref = ref.expand(lp.shape).contiguous()
+        out = torch.empty_like(lp)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().siirl_kl_penalty_fwd(_lib.ptr(lp), _lib.ptr(ref), lp.numel(), code, _lib.ptr(out),
+                                                 _lib.current_stream(dev))
+        _lib.check(rc, "siirl_kl_penalty_fwd")
+        ctx.save_for_backward(lp, ref)
+        ctx.meta = (code, straight_through, logprob.dtype, ref_logprob.dtype, ref_logprob.shape)
+        return out.to(logprob.dtype) if logprob.dtype != torch.float32 else out
+
+    @staticmethod
+    def backward(ctx, g):
+        lp, ref = ctx.saved_tensors
+        code, st, lp_dtype, ref_dtype, ref_shape = ctx.meta
+        dev = lp.device
+        g = _f32(g, dev)
+        need_lp, need_ref = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        d_lp = torch.empty_like(lp) if need_lp else None
+        d_ref = torch.empty_like(lp) if need_ref else None
+        if need_lp or need_ref:
+            with torch.cuda.device(dev):
+                rc = _lib.lib().siirl_kl_penalty_bwd(_lib.ptr(g), _lib.ptr(lp), _lib.ptr(ref), lp.numel(), code,
+                                                     int(st), _lib.ptr(d_lp), _lib.ptr(d_ref),
+                                                     _lib.current_stream(dev))
+            _lib.check(rc, "siirl_kl_penalty_bwd")
+        if d_ref is not None and tuple(ref_shape) != tuple(lp.shape):
+            d_ref = d_ref.sum_to_size(ref_shape)
+        return (None if d_lp is None else d_lp.to(lp_dtype), None if d_ref is None else d_ref.to(ref_dtype),
+                None, None)
+
+
+def kl_penalty_forward(logprob: torch.Tensor, ref_logprob: torch.Tensor, kl_penalty) -> torch.Tensor:
+    """Per-token KL estimator (reference ``core_algos.py:1241-1276``): ``kl``/``k1``, ``abs``, ``mse``/``k2``,
+    ``low_var_kl``/``k3``; anything else, ``full`` included, raises ``NotImplementedError``."""
+    if kl_penalty not in KL_MODES:
+        raise NotImplementedError
+    _gpu_of(logprob, ref_logprob)
+    return _KlPenalty.apply(logprob, ref_logprob, KL_MODES[kl_penalty], False)
+
+
+def kl_penalty(logprob: torch.Tensor, ref_logprob: torch.Tensor, kl_penalty) -> torch.Tensor:
+    """reference ``core_algos.py:1215-1238``.  The reference hands the name, ``+`` suffix included, to
+    ``kl_penalty_forward`` first (``:1227``), which knows no suffixed name: ``k1+``, ``k3+`` ... therefore
+    raise ``NotImplementedError`` there, and do so here.  The straight-through estimator those names were
+    meant to select (value of the estimator, gradient of k2) is ``kl_penalty_straight_through``."""
+    return kl_penalty_forward(logprob, ref_logprob, kl_penalty)
+
+
+def kl_penalty_straight_through(logprob: torch.Tensor, ref_logprob: torch.Tensor, kl_penalty: str) -> torch.Tensor:
+    """Value of estimator ``kl_penalty`` (without the ``+``) with the gradient of k2,
+    ``0.5 * (logprob - ref)^2`` -- the intent of reference ``core_algos.py:1231-1238``."""
+    name = kl_penalty[:-1] if kl_penalty.endswith("+") else kl_penalty
+    if name not in KL_MODES:
+        raise NotImplementedError
+    _gpu_of(logprob, ref_logprob)
+    return _KlPenalty.apply(logprob, ref_logprob, KL_MODES[name], True)
+
+
+# ------------------------------------------------------------------------------------ fused actor loss
+
+
+class ActorLossOutput:
+    """Result of ``actor_loss``: ``loss`` (0-d, differentiable) and the scalars the actor logs, all still on
+    the device; ``metrics()`` fetches them with a single device-to-host copy."""
+
+    _NAMES = ("loss", "pg_loss", "pg_clipfrac", "ppo_kl", "pg_clipfrac_lower", "entropy_loss", "kl_loss",
+              "ratio_mean", "ratio_min", "ratio_max", "mask_total", "policy_loss")
+
+    def __init__(self, outs, loss_scale, kl_coef, has_kl, has_entropy):
+        self._outs = outs
+        for i, n in enumerate(self._NAMES):
+            setattr(self, n, outs[i])
+        self._scale, self._kl_coef, self._has_kl, self._has_entropy = loss_scale, kl_coef, has_kl, has_entropy
+
+    def metrics(self) -> dict:
+        """The per-micro-batch metrics of reference ``dp_actor.py:485-513`` under the same names."""
+        v = torch.stack([o.detach() for o in self._outs]).tolist()
+        out = {
+            "actor/pg_clip_mean": v[O_RMEAN], "actor/pg_clip_min": v[O_RMIN], "actor/pg_clip_max": v[O_RMAX],
+            "actor/pg_loss": v[O_PG] * self._scale, "actor/pg_clipfrac": v[O_CLIPFRAC], "actor/ppo_kl": v[O_PPOKL],
+            "actor/pg_clipfrac_lower": v[O_CLIPLOWER],
+        }
+        if self._has_kl:
+            out["actor/kl_loss"] = v[O_KL] * self._scale
+            out["actor/kl_coef"] = self._kl_coef
+        if self._has_entropy:
+            out["actor/entropy_loss"] = v[O_ENT]
+        return out
+
+
+def actor_loss(old_log_prob, log_prob, advantages, response_mask, config, entropy=None, ref_log_prob=None,
+               loss_scale_factor: float = 1.0, rollout_is_weights=None) -> ActorLossOutput:
+    """The loss of one micro-batch as ``DataParallelPPOActor.update_policy`` composes it (reference
+    ``siirl/engine/actor/dp_actor.py:455-500``), fused:
+    ``loss = (pg_loss - entropy_coeff * agg(entropy) + kl_loss_coef * agg(kl_penalty(log_prob, ref))) * scale``.
+    ``config`` carries ``clip_ratio*``, ``entropy_coeff``, ``use_kl_loss``, ``kl_loss_coef``, ``kl_loss_type``,
+    ``loss_agg_mode`` and ``policy_loss.loss_mode`` (or ``loss_mode``).  The entropy term is used when
+    ``entropy`` is given and ``entropy_coeff != 0``; the KL term when ``config.use_kl_loss``."""
+    _gpu_of(log_prob)
+    mode = getattr(getattr(config, "policy_loss", None), "loss_mode", None) or getattr(config, "loss_mode", "vanilla")
+    if mode not in ("vanilla", "gspo"):
+        raise ValueError(f"Unsupported loss mode: {mode}. Supported modes are: ['vanilla', 'gspo']")
+    lo, hi = _clip_params(config)
+    c = float(getattr(config, "clip_ratio_c", 3.0))
+    if mode == "vanilla":
+        assert c > 1.0, f"The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0, but get the value: {c}."
+    agg_code = _agg_code(getattr(config, "loss_agg_mode", "token-mean"))
+    ent_coef = float(getattr(config, "entropy_coeff", 0.0))
+    use_ent = entropy is not None and ent_coef != 0
+    use_kl = bool(getattr(config, "use_kl_loss", False))
+    kl_code, kl_coef = 0, 0.0
+    if use_kl:
+        if ref_log_prob is None:
+            raise ValueError("config.use_kl_loss is set but ref_log_prob is None")
+        kl_type = getattr(config, "kl_loss_type", "low_var_kl")
+        if kl_type not in KL_MODES:
+            raise NotImplementedError
+        kl_code, kl_coef = KL_MODES[kl_type], float(getattr(config, "kl_loss_coef", 0.001))
+    cfg = (LOSS_GSPO if mode == "gspo" else LOSS_VANILLA, lo, hi, c, 20.0, agg_code, ent_coef if use_ent else 0.0,
+           kl_code, 0, kl_coef, float(loss_scale_factor), False)
+    outs = _ActorLoss.apply(log_prob, entropy if use_ent else None, old_log_prob, advantages, response_mask,
+                            rollout_is_weights, ref_log_prob if use_kl else None, cfg)
+    return ActorLossOutput(outs, float(loss_scale_factor), kl_coef, use_kl, use_ent)

@@ -1,0 +1,306 @@
+// Per-prompt group statistics: GRPO outcome advantage and the DAPO dynamic-sampling keep mask.
+//
+// Replaces compute_grpo_outcome_advantage (siirl/dag_worker/core_algos.py:279-348) and the group test of
+// dynamic_sampling (siirl/user_interface/filter_interface/dapo.py:66-93).
+//
+// Groups are defined by equal uid; uids are arbitrary int64 and need not be contiguous.  Each thread owns
+// one trajectory i and scans all trajectories j in batch order through LDS tiles, picking those with
+// uid[j] == uid[i]: O(B^2) compares, exact integer bookkeeping, no atomics, and every group statistic is
+// accumulated in the batch order the reference uses.  B is a rollout batch (10^3..10^5): at 8192 rows a
+// scan costs ~30 us.
+//
+// The keep mask reproduces np.std(values) > 0 bit for bit: numpy sums with an 8-accumulator pairwise
+// scheme in the dtype of the values, so e.g. three equal fp64 values 0.1 have std 1.4e-17 > 0.  This
+// file is compiled with -ffp-contract=off so that (v - mean)^2 is rounded as numpy rounds it.
+#include "common.hpp"
+
+namespace siirl {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kTile = 1024;
+
+// ---------------------------------------------------------------------------- row sums
+
+// scores[b] = sum_t x[b, t]  (double accumulation, one workgroup per row)
+__global__ __launch_bounds__(kThreads) void row_sum_kernel(const float* __restrict__ x, int64_t L,
+                                                           float* __restrict__ out) {
+  const int64_t b = blockIdx.x;
+  const float* r = x + b * L;
+  double s = 0.0;
+  for (int64_t t = threadIdx.x; t < L; t += kThreads) s += (double)r[t];
+  __shared__ double sh[kThreads / kWave + 1];
+  s = block_sum(s, sh);
+  if (threadIdx.x == 0) out[b] = (float)s;
+}
+
+// ---------------------------------------------------------------------------- GRPO advantage
+
+// a[i] = (s_i - mean_g) / (std_g + eps), unbiased std; a group of one uses mean 0, std 1.
+__global__ __launch_bounds__(kThreads) void grpo_group_kernel(const float* __restrict__ scores,
+                                                              const int64_t* __restrict__ uid, int64_t B, float eps,
+                                                              int norm_by_std, float* __restrict__ a_out) {
+  __shared__ int64_t s_uid[kTile];
+  __shared__ float s_val[kTile];
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const bool live = i < B;
+  const int64_t my = live ? uid[i] : 0;
+  int n = 0;
+  double sum = 0.0;
+  for (int64_t base = 0; base < B; base += kTile) {
+    __syncthreads();
+    for (int k = threadIdx.x; k < kTile; k += kThreads) {
+      const int64_t j = base + k;
+      s_uid[k] = j < B ? uid[j] : 0;
+      s_val[k] = j < B ? scores[j] : 0.f;
+    }
+    __syncthreads();
+    const int lim = (int)((B - base) < kTile ? (B - base) : kTile);
+    if (live)
+      for (int k = 0; k < lim; ++k)
+        if (s_uid[k] == my) {
+          ++n;
+          sum += (double)s_val[k];
+        }
+  }
+  const double mean = n > 1 ? sum / (double)n : 0.0;
+  double ss = 0.0;
+  for (int64_t base = 0; base < B; base += kTile) {
+    __syncthreads();
+    for (int k = threadIdx.x; k < kTile; k += kThreads) {
+      const int64_t j = base + k;
+      s_uid[k] = j < B ? uid[j] : 0;
+      s_val[k] = j < B ? scores[j] : 0.f;
+    }
+    __syncthreads();
+    const int lim = (int)((B - base) < kTile ? (B - base) : kTile);
+    if (live && n > 1)
+      for (int k = 0; k < lim; ++k)
+        if (s_uid[k] == my) {
+          const double d = (double)s_val[k] - mean;
+          ss += d * d;
+        }
+  }
+  if (!live) return;
+  const double sd = n > 1 ? sqrt(ss / (double)(n - 1)) : 1.0;
+  const double s = (double)scores[i];
+  // the reference evaluates (s - mean) / (std + eps) on fp32 0-d tensors; round the pieces likewise
+  const float num = (float)s - (float)mean;
+  a_out[i] = norm_by_std ? num / ((float)sd + eps) : num;
+}
+
+__global__ __launch_bounds__(kThreads) void broadcast_mask_kernel(const float* __restrict__ a, const void* mask,
+                                                                  int mask_dtype, int64_t B, int64_t L,
+                                                                  float* __restrict__ out) {
+  const int64_t n = B * L;
+  for (int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * kThreads)
+    out[idx] = a[idx / L] * load_mask(mask, mask_dtype, idx);
+}
+
+// ---------------------------------------------------------------------------- numpy pairwise sum
+
+// Streaming restatement of numpy's pairwise_sum for one block of n <= 128 values fed in order.
+template <typename T>
+struct NpBlock {
+  T r0, r1, r2, r3, r4, r5, r6, r7, res;
+  int n, nb, k;
+  __device__ void begin(int n_) {
+    n = n_;
+    nb = n < 8 ? 0 : n - (n % 8);
+    k = 0;
+    r0 = r1 = r2 = r3 = r4 = r5 = r6 = r7 = T(0);
+    res = T(0);
+  }
+  __device__ T fold() const { return ((r0 + r1) + (r2 + r3)) + ((r4 + r5) + (r6 + r7)); }
+  __device__ void push(T v) {
+    if (k < nb) {
+      switch (k & 7) {
+        case 0: r0 += v; break;
+        case 1: r1 += v; break;
+        case 2: r2 += v; break;
+        case 3: r3 += v; break;
+        case 4: r4 += v; break;
+        case 5: r5 += v; break;
+        case 6: r6 += v; break;
+        default: r7 += v;
+      }
+    } else {
+      if (k == nb && nb > 0) res = fold();
+      res += v;
+    }
+    ++k;
+  }
+  __device__ T finish() const { return (nb > 0 && n == nb) ? fold() : res; }
+};
+
+// Pull-style iterator over the members of uid `my`, in batch order, from global memory.
+template <typename T>
+struct MemberCursor {
+  const int64_t* uid;
+  const T* val;
+  int64_t B, j;
+  int64_t my;
+  __device__ T next() {
+    while (j < B && uid[j] != my) ++j;
+    return val[j++];
+  }
+};
+
+// numpy's pairwise_sum over n members with an optional transform (v - mean)^2; explicit stack instead of
+// recursion.  Leaves hold at most 128 values; n2 = n/2 rounded down to a multiple of 8.
+template <typename T, bool SQDEV>
+__device__ T np_pairwise(MemberCursor<T>& cur, int n, T mean) {
+  struct Frame {
+    int n, stage;
+    T left;
+  };
+  Frame st[40];
+  int sp = 0;
+  st[0] = {n, 0, T(0)};
+  T ret = T(0);
+  while (sp >= 0) {
+    Frame& f = st[sp];
+    if (f.n <= 128) {
+      NpBlock<T> blk;
+      blk.begin(f.n);
+      for (int q = 0; q < f.n; ++q) {
+        T v = cur.next();
+        if (SQDEV) {
+          const T d = v - mean;
+          v = d * d;
+        }
+        blk.push(v);
+      }
+      ret = blk.finish();
+      --sp;
+      while (sp >= 0) {
+        Frame& p = st[sp];
+        if (p.stage == 1) {  // left child done: run the right child
+          p.left = ret;
+          p.stage = 2;
+          int n2 = p.n / 2;
+          n2 -= n2 % 8;
+          st[++sp] = {p.n - n2, 0, T(0)};
+          break;
+        }
+        ret = p.left + ret;  // right child done
+        --sp;
+      }
+    } else {
+      f.stage = 1;
+      int n2 = f.n / 2;
+      n2 -= n2 % 8;
+      st[++sp] = {n2, 0, T(0)};
+    }
+  }
+  return ret;
+}
+
+// keep[i] = group of i has one member, or np.std(group values) > 0
+template <typename T>
+__global__ __launch_bounds__(kThreads) void keep_mask_kernel(const T* __restrict__ val, const int64_t* __restrict__ uid,
+                                                             int64_t B, uint8_t* __restrict__ keep,
+                                                             int32_t* __restrict__ group_size) {
+  __shared__ int64_t s_uid[kTile];
+  __shared__ T s_val[kTile];
+  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const bool live = i < B;
+  const int64_t my = live ? uid[i] : 0;
+  auto stage = [&](int64_t base) {
+    __syncthreads();
+    for (int k = threadIdx.x; k < kTile; k += kThreads) {
+      const int64_t j = base + k;
+      s_uid[k] = j < B ? uid[j] : 0;
+      s_val[k] = j < B ? val[j] : T(0);
+    }
+    __syncthreads();
+    return (int)((B - base) < kTile ? (B - base) : kTile);
+  };
+  int n = 0;
+  for (int64_t base = 0; base < B; base += kTile) {
+    const int lim = stage(base);
+    if (live)
+      for (int k = 0; k < lim; ++k) n += (s_uid[k] == my) ? 1 : 0;
+  }
+  const bool small = n <= 128;
+  // mean
+  NpBlock<T> blk;
+  blk.begin(small ? n : 0);
+  for (int64_t base = 0; base < B; base += kTile) {
+    const int lim = stage(base);
+    if (live && small && n > 1)
+      for (int k = 0; k < lim; ++k)
+        if (s_uid[k] == my) blk.push(s_val[k]);
+  }
+  T mean = blk.finish() / (T)n;
+  // sum of squared deviations
+  blk.begin(small ? n : 0);
+  for (int64_t base = 0; base < B; base += kTile) {
+    const int lim = stage(base);
+    if (live && small && n > 1)
+      for (int k = 0; k < lim; ++k)
+        if (s_uid[k] == my) {
+          const T d = s_val[k] - mean;
+          blk.push(d * d);
+        }
+  }
+  T ssq = blk.finish();
+  if (live && !small) {  // rare: groups of more than 128, numpy recurses
+    MemberCursor<T> c1{uid, val, B, 0, my};
+    mean = np_pairwise<T, false>(c1, n, T(0)) / (T)n;
+    MemberCursor<T> c2{uid, val, B, 0, my};
+    ssq = np_pairwise<T, true>(c2, n, mean);
+  }
+  if (!live) return;
+  const T sd = sqrt(ssq / (T)n);
+  keep[i] = (n == 1 || sd > T(0)) ? 1 : 0;
+  if (group_size) group_size[i] = n;
+}
+
+}  // namespace
+}  // namespace siirl
+
+using namespace siirl;
+
+extern "C" int siirl_grpo_outcome_advantage(const float* token_level_rewards, const void* mask, int mask_dtype,
+                                            const int64_t* uid, int64_t B, int64_t L, float epsilon,
+                                            int norm_adv_by_std, float* advantages, float* scratch_2B,
+                                            siirl_stream_t stream) {
+  SIIRL_REQUIRE(B >= 0 && L >= 1, "B=%lld L=%lld out of range", (long long)B, (long long)L);
+  if (B == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(B <= 0x7fffffffLL, "B too large");
+  SIIRL_REQUIRE(token_level_rewards && mask && uid && advantages && scratch_2B, "NULL operand");
+  SIIRL_REQUIRE(mask_dtype == SIIRL_U8 || mask_dtype == SIIRL_I64 || mask_dtype == SIIRL_I32 ||
+                    mask_dtype == SIIRL_F32 || mask_dtype == SIIRL_BF16 || mask_dtype == SIIRL_F16,
+                "mask dtype %d not supported", mask_dtype);
+  hipStream_t st = (hipStream_t)stream;
+  float* scores = scratch_2B;
+  float* a = scratch_2B + B;
+  row_sum_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(token_level_rewards, L, scores);
+  SIIRL_LAUNCH_CHECK("row_sum_kernel");
+  grpo_group_kernel<<<dim3((unsigned)((B + kThreads - 1) / kThreads)), dim3(kThreads), 0, st>>>(
+      scores, uid, B, epsilon, norm_adv_by_std, a);
+  SIIRL_LAUNCH_CHECK("grpo_group_kernel");
+  const int64_t n = B * L;
+  const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads < 16384 ? (n + kThreads - 1) / kThreads : 16384);
+  broadcast_mask_kernel<<<dim3(blocks), dim3(kThreads), 0, st>>>(a, mask, mask_dtype, B, L, advantages);
+  SIIRL_LAUNCH_CHECK("broadcast_mask_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_group_keep_mask(const void* metric, int metric_dtype, const int64_t* uid, int64_t B,
+                                     uint8_t* keep, int32_t* group_size, siirl_stream_t stream) {
+  SIIRL_REQUIRE(B >= 0 && B <= 0x7fffffffLL, "B=%lld out of range", (long long)B);
+  if (B == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(metric && uid && keep, "NULL operand");
+  SIIRL_REQUIRE(metric_dtype == SIIRL_F32 || metric_dtype == SIIRL_F64, "metric dtype %d not supported (f32, f64)",
+                metric_dtype);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)((B + kThreads - 1) / kThreads)), block(kThreads);
+  if (metric_dtype == SIIRL_F32)
+    keep_mask_kernel<float><<<grid, block, 0, st>>>((const float*)metric, uid, B, keep, group_size);
+  else
+    keep_mask_kernel<double><<<grid, block, 0, st>>>((const double*)metric, uid, B, keep, group_size);
+  SIIRL_LAUNCH_CHECK("keep_mask_kernel");
+  return SIIRL_OK;
+}

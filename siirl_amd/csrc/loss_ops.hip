@@ -1,0 +1,686 @@
+// [B, L] loss arithmetic of the actor update: clipped policy-gradient loss (PPO / GRPO / DAPO "vanilla",
+// GSPO), KL penalty, masked aggregation, and their hand-written backward.
+//
+// Replaces, of siirl/dag_worker/core_algos.py:  agg_loss :536-569, compute_policy_loss_vanilla :710-792,
+// compute_policy_loss_gspo :795-862, kl_penalty :1215-1276; of siirl/utils/model_utils/torch_functional.py:
+// masked_sum / masked_mean :146-168; and the composition of siirl/engine/actor/dp_actor.py:455-513.
+//
+// Shape of the computation: one workgroup reduces a segment of kSeg tokens of one row into kNP partial
+// sums (LDS tree per partial), a single-workgroup finish kernel folds segments into rows and rows into
+// the scalars in double precision.  No atomics: results are reproducible run to run.  The backward is a
+// plain elementwise kernel that re-evaluates the token and applies autograd's tie rules by hand.
+#include "common.hpp"
+
+namespace siirl {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kSeg = 2048;  // tokens per workgroup
+constexpr int kNP = 12;     // partials per segment (see enum P)
+
+enum P { P_PG = 0, P_M, P_CLIP, P_NEGD, P_LOWER, P_ENT, P_KL, P_RSUM, P_RMIN, P_RMAX, P_AUX0, P_AUX1 };
+// out[] of the finish kernel
+enum O { O_LOSS = 0, O_PG, O_CLIPFRAC, O_PPOKL, O_CLIPLOWER, O_ENTLOSS, O_KLLOSS, O_RMEAN, O_RMIN, O_RMAX,
+         O_MTOTAL, O_POLICY, O_COUNT = 16 };
+
+struct LossArgs {
+  const float* old_lp;   // [B,L] or null (kind == KIND_AGG)
+  const float* lp;       // [B,L]  (kind == KIND_AGG: the loss matrix to aggregate)
+  const float* adv;      // [B,L]
+  const void* mask;      // [B,L]
+  const float* isw;      // [B,L] or null
+  const float* ent;      // [B,L] or null
+  const float* ref;      // [B,L] or null
+  int mask_dtype;
+  int kind;              // KIND_*
+  int agg_mode;          // aggregation of the policy term (GSPO: forced to seq-mean-token-mean)
+  int aux_agg_mode;      // aggregation of the entropy and KL terms
+  int kl_mode, kl_st;
+  float eps_lo, eps_hi, clip_c, dclamp;
+  float ent_coef, kl_coef, scale;
+  int64_t B, L;
+  int nseg;
+};
+enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2 };
+
+// torch.clamp / torch.maximum / torch.minimum semantics (NaN propagates)
+__device__ __forceinline__ float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
+__device__ __forceinline__ float clamp_max(float x, float hi) { return x > hi ? hi : x; }
+__device__ __forceinline__ float tmax(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
+__device__ __forceinline__ float tmin(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+
+// masked contribution.  token-mean goes through masked_mean: where(mask, v, 0) * mask; the other modes
+// multiply directly (a NaN under a zero mask poisons them, as in the reference).
+__device__ __forceinline__ float contrib_where(float v, float m) { return m != 0.f ? v * m : 0.f; }
+__device__ __forceinline__ float contrib(float v, float m, int agg) {
+  return agg == SIIRL_AGG_TOKEN_MEAN ? contrib_where(v, m) : v * m;
+}
+
+struct KlOut {
+  float v, g;  // value and d value / d logprob
+};
+__device__ __forceinline__ KlOut kl_token(float lp, float ref, int mode, int straight_through) {
+  const float x = lp - ref;
+  KlOut o;
+  switch (mode) {
+    case SIIRL_KL_K1: o.v = x; o.g = 1.f; break;
+    case SIIRL_KL_ABS: o.v = fabsf(x); o.g = x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f); break;
+    case SIIRL_KL_K2: o.v = 0.5f * x * x; o.g = x; break;
+    default: {  // K3
+      const float kr = ref - lp;
+      const float k = clampf(kr, -20.f, 20.f);
+      const float e = expf(k);
+      const float raw = e - k - 1.f;
+      o.v = clampf(raw, -10.f, 10.f);
+      const bool pass = (kr >= -20.f && kr <= 20.f) && (raw >= -10.f && raw <= 10.f);
+      o.g = pass ? -(e - 1.f) : 0.f;
+    }
+  }
+  if (straight_through) o.g = x;  // value of the estimator, gradient of k2
+  return o;
+}
+
+struct PgOut {
+  float tok, dtok;  // per-token loss and d tok / d logprob (before the aggregation weight)
+  float clip, lower, negd, r_raw;
+};
+
+// seq_s: GSPO's sequence-level mean log-ratio (unused for vanilla)
+__device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A, float isw, float seq_s,
+                                          float eps_lo, float eps_hi, float clip_c, float dclamp) {
+  PgOut o;
+  const float raw = lp - old;
+  o.r_raw = expf(raw);
+  const float lo = 1.f - eps_lo, hi = 1.f + eps_hi;
+  if (kind == KIND_VANILLA) {
+    const float d = clampf(raw, -dclamp, dclamp);
+    const float r = expf(d);
+    const float dr = (raw >= -dclamp && raw <= dclamp) ? r : 0.f;  // d r / d lp
+    o.negd = -d;
+    const float l1 = -A * r;
+    const float rc = clampf(r, lo, hi);
+    const float l2 = -A * rc;
+    const float c1 = tmax(l1, l2);
+    o.clip = l2 > l1 ? 1.f : 0.f;
+    const float l3 = -A * clip_c;
+    const float c2 = tmin(l3, c1);
+    o.lower = (c1 > l3 && A < 0.f) ? 1.f : 0.f;
+    o.tok = A < 0.f ? c2 : c1;
+    // autograd: maximum / minimum give each side 1, 1/2 (tie) or 0; clamp passes inside [lo, hi] inclusive
+    const float dl1 = -A * dr;
+    const float dl2 = (r >= lo && r <= hi) ? -A * dr : 0.f;
+    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float dc1 = w1 * dl1 + w2 * dl2;
+    const float wc = c1 < l3 ? 1.f : (c1 == l3 ? 0.5f : 0.f);
+    o.dtok = A < 0.f ? wc * dc1 : dc1;
+  } else {  // GSPO
+    o.negd = -raw;
+    const float l = clamp_max(seq_s, 10.f);  // lp - lp.detach() == 0
+    const float r = expf(l);
+    const float dr = (seq_s <= 10.f) ? r : 0.f;
+    const float l1 = -A * r;
+    const float rc = clampf(r, lo, hi);
+    const float l2 = -A * rc;
+    o.tok = tmax(l1, l2);
+    o.clip = l2 > l1 ? 1.f : 0.f;
+    o.lower = 0.f;
+    const float dl1 = -A * dr;
+    const float dl2 = (r >= lo && r <= hi) ? -A * dr : 0.f;
+    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    o.dtok = w1 * dl1 + w2 * dl2;
+  }
+  o.tok *= isw;  // importance weights multiply value and gradient alike
+  o.dtok *= isw;
+  return o;
+}
+
+// ---------------------------------------------------------------------------- row pre-pass (GSPO)
+
+// rowstat[b] = { sum_t (lp - old) * m , sum_t m } per segment -> partials[b][seg][AUX0/AUX1]
+__global__ __launch_bounds__(kThreads) void gspo_prepass_kernel(LossArgs a, float* __restrict__ pre) {
+  const int64_t b = blockIdx.x / a.nseg;
+  const int seg = blockIdx.x % a.nseg;
+  const int64_t t0 = (int64_t)seg * kSeg;
+  float sd = 0.f, sm = 0.f;
+  for (int i = threadIdx.x; i < kSeg; i += kThreads) {
+    const int64_t t = t0 + i;
+    if (t < a.L) {
+      const int64_t idx = b * a.L + t;
+      const float m = load_mask(a.mask, a.mask_dtype, idx);
+      sd += (a.lp[idx] - a.old_lp[idx]) * m;
+      sm += m;
+    }
+  }
+  __shared__ float sh[kThreads / kWave + 1];
+  sd = block_sum(sd, sh);
+  sm = block_sum(sm, sh);
+  if (threadIdx.x == 0) {
+    pre[(b * a.nseg + seg) * 2 + 0] = sd;
+    pre[(b * a.nseg + seg) * 2 + 1] = sm;
+  }
+}
+
+// folds the pre-pass segments of each row: row_s[b] = sum d*m / max(sum m, 1)
+__global__ __launch_bounds__(kThreads) void gspo_rowfinish_kernel(const float* __restrict__ pre, int nseg, int64_t B,
+                                                                  float* __restrict__ row_s) {
+  const int64_t b = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (b >= B) return;
+  double sd = 0.0, sm = 0.0;
+  for (int s = 0; s < nseg; ++s) {
+    sd += pre[(b * nseg + s) * 2 + 0];
+    sm += pre[(b * nseg + s) * 2 + 1];
+  }
+  const float n = fmaxf((float)sm, 1.f);  // .clamp(min=1)
+  row_s[b] = (float)sd / n;
+}
+
+// ---------------------------------------------------------------------------- segment partials
+
+__global__ __launch_bounds__(kThreads) void loss_partials_kernel(LossArgs a, const float* __restrict__ row_s,
+                                                                 float* __restrict__ partials) {
+  const int64_t b = blockIdx.x / a.nseg;
+  const int seg = blockIdx.x % a.nseg;
+  const int64_t t0 = (int64_t)seg * kSeg;
+  float acc[kNP];
+#pragma unroll
+  for (int k = 0; k < kNP; ++k) acc[k] = 0.f;
+  acc[P_RMIN] = __builtin_inff();
+  acc[P_RMAX] = -__builtin_inff();
+  const float seq_s = (a.kind == KIND_GSPO) ? row_s[b] : 0.f;
+
+  for (int i = threadIdx.x; i < kSeg; i += kThreads) {
+    const int64_t t = t0 + i;
+    if (t >= a.L) break;
+    const int64_t idx = b * a.L + t;
+    const float m = load_mask(a.mask, a.mask_dtype, idx);
+    acc[P_M] += m;
+    if (a.kind == KIND_AGG) {
+      acc[P_PG] += contrib(a.lp[idx], m, a.agg_mode);
+      continue;
+    }
+    const float lp = a.lp[idx];
+    const float isw = a.isw ? a.isw[idx] : 1.f;
+    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a.eps_lo, a.eps_hi, a.clip_c, a.dclamp);
+    acc[P_PG] += contrib(o.tok, m, a.agg_mode);
+    acc[P_CLIP] += contrib_where(o.clip, m);
+    acc[P_NEGD] += contrib_where(o.negd, m);
+    acc[P_LOWER] += contrib_where(o.lower, m);
+    acc[P_RSUM] += o.r_raw;
+    acc[P_RMIN] = fminf(acc[P_RMIN], o.r_raw);
+    acc[P_RMAX] = fmaxf(acc[P_RMAX], o.r_raw);
+    if (a.ent) acc[P_ENT] += contrib(a.ent[idx], m, a.aux_agg_mode);
+    if (a.ref) acc[P_KL] += contrib(kl_token(lp, a.ref[idx], a.kl_mode, 0).v, m, a.aux_agg_mode);
+  }
+
+  __shared__ float sh[kThreads / kWave + 1];
+  float* out = partials + (b * a.nseg + seg) * kNP;
+#pragma unroll
+  for (int k = 0; k < kNP; ++k) {
+    if (k == P_RMIN || k == P_RMAX) continue;
+    const float v = block_sum(acc[k], sh);
+    if (threadIdx.x == 0) out[k] = v;
+  }
+  // min / max of the raw ratio
+  float mn = acc[P_RMIN], mx = acc[P_RMAX];
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    mn = fminf(mn, __shfl_xor(mn, o, kWave));
+    mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+  }
+  __shared__ float shm[2 * (kThreads / kWave)];
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
+  if (lane == 0) {
+    shm[wid] = mn;
+    shm[kThreads / kWave + wid] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / kWave; ++w) {
+      mn = fminf(mn, shm[w]);
+      mx = fmaxf(mx, shm[kThreads / kWave + w]);
+    }
+    out[P_RMIN] = mn;
+    out[P_RMAX] = mx;
+  }
+}
+
+// ---------------------------------------------------------------------------- finish
+
+__device__ __forceinline__ double block_sum_d(double v, double* sh) { return block_sum(v, sh); }
+
+// Aggregates a per-row numerator given the mode.  num/msum are row sums; returns this row's term of
+// the batch sum whose final normaliser is applied by the caller.
+__device__ __forceinline__ double row_term(double num, double msum, int agg) {
+  return agg == SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN ? num / msum : num;  // 0/0 -> NaN, as the reference
+}
+__device__ __forceinline__ double finish_term(double total, double mtotal, int agg, int64_t B, int64_t L) {
+  switch (agg) {
+    case SIIRL_AGG_TOKEN_MEAN: return total / (mtotal + 1e-8);
+    case SIIRL_AGG_SEQ_MEAN_TOKEN_SUM: return total / (double)B;
+    case SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN: return total / (double)B;
+    default: return total / (double)L;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const float* __restrict__ partials,
+                                                               float* __restrict__ out,
+                                                               float* __restrict__ row_msum) {
+  double t_pg = 0, t_m = 0, t_clip = 0, t_negd = 0, t_lower = 0, t_ent = 0, t_kl = 0, t_rsum = 0;
+  float rmin = __builtin_inff(), rmax = -__builtin_inff();
+  for (int64_t b = threadIdx.x; b < a.B; b += kThreads) {
+    double r[kNP];
+    for (int k = 0; k < kNP; ++k) r[k] = 0.0;
+    for (int s = 0; s < a.nseg; ++s) {
+      const float* p = partials + (b * a.nseg + s) * kNP;
+      for (int k = 0; k < kNP; ++k) {
+        if (k == P_RMIN) rmin = fminf(rmin, p[k]);
+        else if (k == P_RMAX) rmax = fmaxf(rmax, p[k]);
+        else r[k] += p[k];
+      }
+    }
+    row_msum[b] = (float)r[P_M];
+    t_m += r[P_M];
+    t_pg += row_term(r[P_PG], r[P_M], a.agg_mode);
+    t_ent += row_term(r[P_ENT], r[P_M], a.aux_agg_mode);
+    t_kl += row_term(r[P_KL], r[P_M], a.aux_agg_mode);
+    t_clip += r[P_CLIP];
+    t_negd += r[P_NEGD];
+    t_lower += r[P_LOWER];
+    t_rsum += r[P_RSUM];
+  }
+  __shared__ double sh[kThreads / kWave + 1];
+  t_pg = block_sum_d(t_pg, sh);
+  t_m = block_sum_d(t_m, sh);
+  t_clip = block_sum_d(t_clip, sh);
+  t_negd = block_sum_d(t_negd, sh);
+  t_lower = block_sum_d(t_lower, sh);
+  t_ent = block_sum_d(t_ent, sh);
+  t_kl = block_sum_d(t_kl, sh);
+  t_rsum = block_sum_d(t_rsum, sh);
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    rmin = fminf(rmin, __shfl_xor(rmin, o, kWave));
+    rmax = fmaxf(rmax, __shfl_xor(rmax, o, kWave));
+  }
+  __shared__ float shm[2 * (kThreads / kWave)];
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
+  if (lane == 0) {
+    shm[wid] = rmin;
+    shm[kThreads / kWave + wid] = rmax;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kThreads / kWave; ++w) {
+      rmin = fminf(rmin, shm[w]);
+      rmax = fmaxf(rmax, shm[kThreads / kWave + w]);
+    }
+    const double pg = finish_term(t_pg, t_m, a.agg_mode, a.B, a.L);
+    const double den = t_m + 1e-8;
+    double policy = pg;
+    double entl = 0.0, kll = 0.0;
+    if (a.ent) {
+      entl = finish_term(t_ent, t_m, a.aux_agg_mode, a.B, a.L);
+      policy = policy - entl * (double)a.ent_coef;
+    }
+    if (a.ref) {
+      kll = finish_term(t_kl, t_m, a.aux_agg_mode, a.B, a.L);
+      policy = policy + kll * (double)a.kl_coef;
+    }
+    for (int k = 0; k < O_COUNT; ++k) out[k] = 0.f;
+    out[O_PG] = (float)pg;
+    out[O_POLICY] = (float)policy;
+    out[O_LOSS] = (float)(policy * (double)a.scale);
+    out[O_MTOTAL] = (float)t_m;
+    if (a.kind != KIND_AGG) {
+      out[O_CLIPFRAC] = (float)(t_clip / den);
+      out[O_PPOKL] = (float)(t_negd / den);
+      out[O_CLIPLOWER] = (float)(t_lower / den);
+      out[O_ENTLOSS] = (float)entl;
+      out[O_KLLOSS] = (float)kll;
+      out[O_RMEAN] = (float)(t_rsum / (double)(a.B * a.L));
+      out[O_RMIN] = rmin;
+      out[O_RMAX] = rmax;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------- backward
+
+// aggregation weight of token (b, t): d (aggregate) / d (loss_mat[b, t])
+__device__ __forceinline__ float agg_weight(int agg, float m, float mtotal, float mrow, int64_t B, int64_t L) {
+  switch (agg) {
+    case SIIRL_AGG_TOKEN_MEAN: return m != 0.f ? m / (mtotal + 1e-8f) : 0.f;
+    case SIIRL_AGG_SEQ_MEAN_TOKEN_SUM: return m / (float)B;
+    case SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN: return m / mrow / (float)B;
+    default: return m / (float)L;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void loss_bwd_kernel(LossArgs a, const float* __restrict__ g_out,
+                                                            const float* __restrict__ saved_out,
+                                                            const float* __restrict__ row_msum,
+                                                            const float* __restrict__ row_s,
+                                                            float* __restrict__ d_lp, float* __restrict__ d_ent) {
+  const int64_t b = blockIdx.x / a.nseg;
+  const int64_t t0 = (int64_t)(blockIdx.x % a.nseg) * kSeg;
+  const float g = g_out[0] * a.scale;
+  const float mtotal = saved_out[O_MTOTAL];
+  const float mrow = row_msum[b];
+  const float seq_s = (a.kind == KIND_GSPO) ? row_s[b] : 0.f;
+  for (int i = threadIdx.x; i < kSeg; i += kThreads) {
+    const int64_t t = t0 + i;
+    if (t >= a.L) break;
+    const int64_t idx = b * a.L + t;
+    const float m = load_mask(a.mask, a.mask_dtype, idx);
+    if (a.kind == KIND_AGG) {
+      d_lp[idx] = g * agg_weight(a.agg_mode, m, mtotal, mrow, a.B, a.L);
+      continue;
+    }
+    const float lp = a.lp[idx];
+    const float isw = a.isw ? a.isw[idx] : 1.f;
+    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a.eps_lo, a.eps_hi, a.clip_c, a.dclamp);
+    float d = agg_weight(a.agg_mode, m, mtotal, mrow, a.B, a.L) * o.dtok;
+    if (a.ent || a.ref) {
+      const float wa = agg_weight(a.aux_agg_mode, m, mtotal, mrow, a.B, a.L);
+      if (a.ref) d += a.kl_coef * wa * kl_token(lp, a.ref[idx], a.kl_mode, a.kl_st).g;
+      if (a.ent && d_ent) d_ent[idx] = -g * a.ent_coef * wa;
+    }
+    d_lp[idx] = g * d;
+  }
+}
+
+// ---------------------------------------------------------------------------- KL penalty (elementwise)
+
+__global__ __launch_bounds__(kThreads) void kl_fwd_kernel(const float* __restrict__ lp, const float* __restrict__ ref,
+                                                          int64_t n, int mode, float* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads)
+    out[i] = kl_token(lp[i], ref[i], mode, 0).v;
+}
+__global__ __launch_bounds__(kThreads) void kl_bwd_kernel(const float* __restrict__ g, const float* __restrict__ lp,
+                                                          const float* __restrict__ ref, int64_t n, int mode, int st,
+                                                          float* __restrict__ d_lp, float* __restrict__ d_ref) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+    const float d = g[i] * kl_token(lp[i], ref[i], mode, st).g;
+    if (d_lp) d_lp[i] = d;
+    if (d_ref) d_ref[i] = -d;  // every estimator depends on lp - ref only
+  }
+}
+
+// ---------------------------------------------------------------------------- masked_sum / masked_mean
+
+// row_sum[b] = sum_t where(m, v, 0) * m ; row_mean[b] = row_sum / (sum_t m + 1e-8); total2 = {sum, mean} over all
+__global__ __launch_bounds__(kThreads) void masked_finish_kernel(const float* __restrict__ partials, int nseg,
+                                                                 int64_t B, float* __restrict__ row_sum,
+                                                                 float* __restrict__ row_mean,
+                                                                 float* __restrict__ total2) {
+  double tv = 0, tm = 0;
+  for (int64_t b = threadIdx.x; b < B; b += kThreads) {
+    double v = 0, m = 0;
+    for (int s = 0; s < nseg; ++s) {
+      v += partials[(b * nseg + s) * kNP + P_PG];
+      m += partials[(b * nseg + s) * kNP + P_M];
+    }
+    if (row_sum) row_sum[b] = (float)v;
+    if (row_mean) row_mean[b] = (float)(v / (m + 1e-8));
+    tv += v;
+    tm += m;
+  }
+  __shared__ double sh[kThreads / kWave + 1];
+  tv = block_sum_d(tv, sh);
+  tm = block_sum_d(tm, sh);
+  if (threadIdx.x == 0 && total2) {
+    total2[0] = (float)tv;
+    total2[1] = (float)(tv / (tm + 1e-8));
+  }
+}
+
+// ---------------------------------------------------------------------------- KL penalty in the reward
+
+// rewards = scores - beta * kld,  kld = kl(old, ref) * m ; row_kl[b] = masked_mean(kld, m) of the row
+__global__ __launch_bounds__(kThreads) void kl_reward_kernel(const float* __restrict__ scores,
+                                                             const float* __restrict__ old_lp,
+                                                             const float* __restrict__ ref, const void* mask,
+                                                             int mask_dtype, int64_t L, int kl_mode, float beta,
+                                                             float* __restrict__ rewards, float* __restrict__ row_kl) {
+  const int64_t b = blockIdx.x;
+  float sv = 0.f, sm = 0.f;
+  for (int64_t t = threadIdx.x; t < L; t += kThreads) {
+    const int64_t idx = b * L + t;
+    const float m = load_mask(mask, mask_dtype, idx);
+    const float kld = kl_token(old_lp[idx], ref[idx], kl_mode, 0).v * m;
+    rewards[idx] = scores[idx] - beta * kld;
+    sv += contrib_where(kld, m);
+    sm += m;
+  }
+  __shared__ float sh[kThreads / kWave + 1];
+  sv = block_sum(sv, sh);
+  sm = block_sum(sm, sh);
+  if (threadIdx.x == 0) row_kl[b] = sv / (sm + 1e-8f);
+}
+__global__ __launch_bounds__(kThreads) void mean_rows_kernel(const float* __restrict__ row, int64_t B,
+                                                             float* __restrict__ out) {
+  double s = 0;
+  for (int64_t b = threadIdx.x; b < B; b += kThreads) s += row[b];
+  __shared__ double sh[kThreads / kWave + 1];
+  s = block_sum_d(s, sh);
+  if (threadIdx.x == 0) out[0] = (float)(s / (double)B);
+}
+
+// ---------------------------------------------------------------------------- host
+
+int nseg_of(int64_t L) { return (int)((L + kSeg - 1) / kSeg); }
+
+size_t ws_bytes_of(int64_t B, int64_t L) {
+  const size_t ns = (size_t)nseg_of(L);
+  return (size_t)B * ns * kNP * sizeof(float) + (size_t)B * ns * 2 * sizeof(float) + 256;
+}
+
+int check_dims(int64_t B, int64_t L) {
+  SIIRL_REQUIRE(B >= 1 && L >= 1, "B=%lld L=%lld must be positive", (long long)B, (long long)L);
+  SIIRL_REQUIRE(L <= (1LL << 40) && B * (int64_t)nseg_of(L) <= 0x7fffffffLL, "B=%lld x L=%lld exceeds the launch grid",
+                (long long)B, (long long)L);
+  return SIIRL_OK;
+}
+int check_mask_dtype(int dt) {
+  SIIRL_REQUIRE(dt == SIIRL_U8 || dt == SIIRL_I64 || dt == SIIRL_I32 || dt == SIIRL_F32 || dt == SIIRL_BF16 ||
+                    dt == SIIRL_F16, "mask dtype %d not supported", dt);
+  return SIIRL_OK;
+}
+int check_agg(int agg) {
+  SIIRL_REQUIRE(agg >= 0 && agg <= 3, "Invalid loss_agg_mode: %d", agg);
+  return SIIRL_OK;
+}
+
+int run_forward(LossArgs& a, float* out16, float* row_msum, float* row_s, void* ws, size_t ws_bytes,
+                hipStream_t st) {
+  a.nseg = nseg_of(a.L);
+  if (ws_bytes < ws_bytes_of(a.B, a.L) || ws == nullptr)
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed for B=%lld L=%lld",
+                ws_bytes, ws_bytes_of(a.B, a.L), (long long)a.B, (long long)a.L);
+  float* partials = (float*)ws;
+  float* pre = partials + (size_t)a.B * a.nseg * kNP;
+  dim3 grid((unsigned)(a.B * a.nseg)), block(kThreads);
+  if (a.kind == KIND_GSPO) {
+    gspo_prepass_kernel<<<grid, block, 0, st>>>(a, pre);
+    SIIRL_LAUNCH_CHECK("gspo_prepass_kernel");
+    gspo_rowfinish_kernel<<<dim3((unsigned)((a.B + kThreads - 1) / kThreads)), block, 0, st>>>(pre, a.nseg, a.B, row_s);
+    SIIRL_LAUNCH_CHECK("gspo_rowfinish_kernel");
+  }
+  loss_partials_kernel<<<grid, block, 0, st>>>(a, row_s, partials);
+  SIIRL_LAUNCH_CHECK("loss_partials_kernel");
+  loss_finish_kernel<<<1, block, 0, st>>>(a, partials, out16, row_msum);
+  SIIRL_LAUNCH_CHECK("loss_finish_kernel");
+  return SIIRL_OK;
+}
+
+}  // namespace
+}  // namespace siirl
+
+using namespace siirl;
+
+extern "C" size_t siirl_loss_workspace_bytes(int64_t B, int64_t L) {
+  if (B < 1 || L < 1) return 0;
+  return ws_bytes_of(B, L);
+}
+
+extern "C" int siirl_agg_loss_fwd(const float* loss_mat, const void* mask, int mask_dtype, int64_t B, int64_t L,
+                                  int agg_mode, float* out16, float* row_msum, void* workspace,
+                                  size_t workspace_bytes, siirl_stream_t stream) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  if (int rc = check_agg(agg_mode)) return rc;
+  SIIRL_REQUIRE(loss_mat && mask && out16 && row_msum, "NULL operand");
+  LossArgs a{};
+  a.lp = loss_mat; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode;
+  a.aux_agg_mode = agg_mode; a.scale = 1.f; a.B = B; a.L = L;
+  return run_forward(a, out16, row_msum, nullptr, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int siirl_agg_loss_bwd(const float* g_out, const void* mask, int mask_dtype, const float* out16,
+                                  const float* row_msum, int64_t B, int64_t L, int agg_mode, float* d_loss_mat,
+                                  siirl_stream_t stream) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  if (int rc = check_agg(agg_mode)) return rc;
+  SIIRL_REQUIRE(g_out && mask && out16 && row_msum && d_loss_mat, "NULL operand");
+  LossArgs a{};
+  a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode; a.aux_agg_mode = agg_mode;
+  a.scale = 1.f; a.B = B; a.L = L; a.nseg = nseg_of(L);
+  loss_bwd_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, (hipStream_t)stream>>>(a, g_out, out16, row_msum,
+                                                                                       nullptr, d_loss_mat, nullptr);
+  SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
+  return SIIRL_OK;
+}
+
+static int fill_actor_args(LossArgs& a, const float* old_log_prob, const float* log_prob, const float* advantages,
+                           const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
+                           const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
+                           float clip_high, float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode,
+                           int kl_straight_through, float kl_coef, float loss_scale) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  if (int rc = check_agg(agg_mode)) return rc;
+  SIIRL_REQUIRE(loss_mode == SIIRL_LOSS_VANILLA || loss_mode == SIIRL_LOSS_GSPO, "Unsupported loss mode: %d", loss_mode);
+  SIIRL_REQUIRE(old_log_prob && log_prob && advantages && mask, "NULL operand");
+  if (loss_mode == SIIRL_LOSS_VANILLA)
+    SIIRL_REQUIRE(clip_c > 1.0f, "clip_ratio_c must be greater than 1.0, got %f", (double)clip_c);
+  SIIRL_REQUIRE(log_ratio_clamp > 0.f, "log_ratio_clamp must be positive (20 in the reference, +inf for none)");
+  if (ref_log_prob) SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
+  a.old_lp = old_log_prob; a.lp = log_prob; a.adv = advantages; a.mask = mask; a.mask_dtype = mask_dtype;
+  a.isw = is_weights; a.ent = entropy; a.ref = ref_log_prob;
+  a.kind = loss_mode == SIIRL_LOSS_GSPO ? KIND_GSPO : KIND_VANILLA;
+  a.agg_mode = loss_mode == SIIRL_LOSS_GSPO ? SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN : agg_mode;
+  a.aux_agg_mode = agg_mode;
+  a.kl_mode = kl_mode; a.kl_st = kl_straight_through;
+  a.eps_lo = clip_low; a.eps_hi = clip_high; a.clip_c = clip_c; a.dclamp = log_ratio_clamp;
+  a.ent_coef = entropy_coeff; a.kl_coef = kl_coef; a.scale = loss_scale;
+  a.B = B; a.L = L; a.nseg = nseg_of(L);
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_prob, const float* advantages,
+                                    const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
+                                    const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
+                                    float clip_high, float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode,
+                                    int kl_straight_through, float kl_coef, float loss_scale, float* out16,
+                                    float* row_msum, float* row_s, void* workspace, size_t workspace_bytes,
+                                    siirl_stream_t stream) {
+  LossArgs a{};
+  if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
+                               ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff,
+                               kl_mode, kl_straight_through, kl_coef, loss_scale))
+    return rc;
+  SIIRL_REQUIRE(out16 && row_msum, "NULL output");
+  SIIRL_REQUIRE(loss_mode != SIIRL_LOSS_GSPO || row_s, "row_s is required for GSPO");
+  return run_forward(a, out16, row_msum, row_s, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const float* log_prob,
+                                    const float* advantages, const void* mask, int mask_dtype,
+                                    const float* is_weights, const float* entropy, const float* ref_log_prob,
+                                    int64_t B, int64_t L, int loss_mode, float clip_low, float clip_high, float clip_c,
+                                    float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode, int kl_straight_through,
+                                    float kl_coef, float loss_scale, const float* out16, const float* row_msum,
+                                    const float* row_s, float* d_log_prob, float* d_entropy, siirl_stream_t stream) {
+  LossArgs a{};
+  if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
+                               ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff,
+                               kl_mode, kl_straight_through, kl_coef, loss_scale))
+    return rc;
+  SIIRL_REQUIRE(g_loss && out16 && row_msum && d_log_prob, "NULL operand");
+  SIIRL_REQUIRE(loss_mode != SIIRL_LOSS_GSPO || row_s, "row_s is required for GSPO");
+  SIIRL_REQUIRE(entropy == nullptr || d_entropy != nullptr, "d_entropy is required when entropy is given");
+  loss_bwd_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, (hipStream_t)stream>>>(a, g_loss, out16, row_msum,
+                                                                                       row_s, d_log_prob, d_entropy);
+  SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_kl_penalty_fwd(const float* logprob, const float* ref_logprob, int64_t n, int kl_mode, float* out,
+                                    siirl_stream_t stream) {
+  SIIRL_REQUIRE(n >= 0, "n < 0");
+  SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
+  if (n == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(logprob && ref_logprob && out, "NULL operand");
+  const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads < 8192 ? (n + kThreads - 1) / kThreads : 8192);
+  kl_fwd_kernel<<<dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream>>>(logprob, ref_logprob, n, kl_mode, out);
+  SIIRL_LAUNCH_CHECK("kl_fwd_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_kl_penalty_bwd(const float* g, const float* logprob, const float* ref_logprob, int64_t n,
+                                    int kl_mode, int straight_through, float* d_logprob, float* d_ref_logprob,
+                                    siirl_stream_t stream) {
+  SIIRL_REQUIRE(n >= 0, "n < 0");
+  SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
+  if (n == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(g && logprob && ref_logprob && (d_logprob || d_ref_logprob), "NULL operand");
+  const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads < 8192 ? (n + kThreads - 1) / kThreads : 8192);
+  kl_bwd_kernel<<<dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream>>>(g, logprob, ref_logprob, n, kl_mode,
+                                                                        straight_through, d_logprob, d_ref_logprob);
+  SIIRL_LAUNCH_CHECK("kl_bwd_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_masked_reduce(const float* values, const void* mask, int mask_dtype, int64_t B, int64_t L,
+                                   float* row_sum, float* row_mean, float* total2, void* workspace,
+                                   size_t workspace_bytes, siirl_stream_t stream) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  SIIRL_REQUIRE(values && mask, "NULL operand");
+  SIIRL_REQUIRE(row_sum || row_mean || total2, "no output requested");
+  LossArgs a{};
+  a.lp = values; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = SIIRL_AGG_TOKEN_MEAN;
+  a.aux_agg_mode = a.agg_mode; a.scale = 1.f; a.B = B; a.L = L; a.nseg = nseg_of(L);
+  if (workspace_bytes < ws_bytes_of(B, L) || workspace == nullptr)
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes,
+                ws_bytes_of(B, L));
+  hipStream_t st = (hipStream_t)stream;
+  float* partials = (float*)workspace;
+  loss_partials_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, st>>>(a, nullptr, partials);
+  SIIRL_LAUNCH_CHECK("loss_partials_kernel");
+  masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, total2);
+  SIIRL_LAUNCH_CHECK("masked_finish_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_kl_in_reward(const float* token_level_scores, const float* old_log_prob,
+                                  const float* ref_log_prob, const void* mask, int mask_dtype, int64_t B, int64_t L,
+                                  int kl_mode, float beta, float* token_level_rewards, float* row_kl,
+                                  float* current_kl, siirl_stream_t stream) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
+  SIIRL_REQUIRE(token_level_scores && old_log_prob && ref_log_prob && mask && token_level_rewards && row_kl &&
+                    current_kl, "NULL operand");
+  hipStream_t st = (hipStream_t)stream;
+  kl_reward_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(token_level_scores, old_log_prob, ref_log_prob, mask,
+                                                                mask_dtype, L, kl_mode, beta, token_level_rewards,
+                                                                row_kl);
+  SIIRL_LAUNCH_CHECK("kl_reward_kernel");
+  mean_rows_kernel<<<1, dim3(kThreads), 0, st>>>(row_kl, B, current_kl);
+  SIIRL_LAUNCH_CHECK("mean_rows_kernel");
+  return SIIRL_OK;
+}

@@ -164,3 +164,52 @@ def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 20
     if logits.dim() != 2:
         raise ValueError("entropy_from_logits_with_chunking expects a 2-D tensor")
     return entropy_from_logits(logits)
+
+
+# ------------------------------------------------------------------------------ masked reductions
+
+
+def _masked_reduce(values: torch.Tensor, mask: torch.Tensor, axis, want_mean: bool):
+    from . import _lib
+    from . import core_algos as CA
+
+    if not values.is_cuda:
+        raise RuntimeError("siirl_amd: masked reductions run on the GPU only (no CPU fallback)")
+    nd = values.dim()
+    if isinstance(axis, (tuple, list)):
+        axis = axis[0] if len(axis) == 1 else (None if sorted(a % nd for a in axis) == list(range(nd)) else axis)
+    per_row = axis is not None
+    if per_row and (not isinstance(axis, int) or axis % nd != nd - 1):
+        raise NotImplementedError("siirl_amd: masked_sum / masked_mean reduce over all elements or over the last axis")
+    if values.requires_grad and torch.is_grad_enabled():
+        if want_mean and not per_row:  # identical arithmetic to agg_loss(..., 'token-mean'), which has a backward
+            return CA.agg_loss(values, mask.expand_as(values), "token-mean")
+        raise NotImplementedError("siirl_amd: only masked_mean over all elements is differentiable here")
+    dev = values.device
+    mask = mask.expand_as(values)
+    v = CA._as_2d(CA._f32(values, dev)) if nd >= 1 else CA._f32(values, dev).reshape(1, 1)
+    m, mcode = CA._mask_arg(CA._as_2d(mask) if nd >= 1 else mask.reshape(1, 1), dev)
+    B, L = v.shape
+    ws, nws = CA._workspace(B, L, dev)
+    row = torch.empty(B, dtype=torch.float32, device=dev) if per_row else None
+    tot = None if per_row else torch.empty(2, dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().siirl_masked_reduce(_lib.ptr(v), _lib.ptr(m), mcode, B, L,
+                                            _lib.ptr(row) if (per_row and not want_mean) else None,
+                                            _lib.ptr(row) if (per_row and want_mean) else None, _lib.ptr(tot),
+                                            _lib.ptr(ws), nws, _lib.current_stream(dev))
+    _lib.check(rc, "siirl_masked_reduce")
+    if per_row:
+        return row.reshape(values.shape[:-1])
+    return tot[1] if want_mean else tot[0]
+
+
+def masked_sum(values: torch.Tensor, mask: torch.Tensor, axis=None):
+    """``sum(where(mask, values, 0) * mask)`` over everything or over the last axis (reference
+    ``torch_functional.py:146-151``); fp32 result."""
+    return _masked_reduce(values, mask, axis, want_mean=False)
+
+
+def masked_mean(values: torch.Tensor, mask: torch.Tensor, axis=None):
+    """``masked_sum / (mask.sum + 1e-8)`` (reference ``torch_functional.py:154-168``)."""
+    return _masked_reduce(values, mask, axis, want_mean=True)

@@ -1,0 +1,355 @@
+"""GPU parity: [B, L] loss arithmetic (through the C ABI) vs the CPU oracle.
+
+Tolerances: scalars (losses, clip fractions, KL) within 1e-3 absolute of the fp32 oracle as the task states,
+and within 2e-5 of the fp64 oracle on the same fp32 inputs; per-token gradients within 1e-6 + 1e-5 relative
+of autograd through the fp64 oracle."""
+
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from oracle import core_algos as OC
+from oracle import torch_functional as OF
+
+pytestmark = pytest.mark.gpu
+
+AGGS = ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"]
+
+
+def _batch(B, L, seed, min_len=1, dtype_mask=torch.int64):
+    g = torch.Generator().manual_seed(seed)
+    lp = torch.randn(B, L, generator=g) - 1.5
+    old = lp + 0.3 * torch.randn(B, L, generator=g)
+    ref = lp + 0.2 * torch.randn(B, L, generator=g)
+    adv = torch.randn(B, 1, generator=g).expand(B, L).contiguous()
+    lens = torch.randint(min_len, L + 1, (B,), generator=g)
+    mask = (torch.arange(L)[None, :] < lens[:, None]).to(dtype_mask)
+    ent = torch.rand(B, L, generator=g) * 3
+    return lp, old, ref, adv, mask, ent
+
+
+def _close(got, want64, tol=2e-5):
+    return abs(float(got) - float(want64)) <= tol + 1e-5 * abs(float(want64))
+
+
+def _grad_close(got, want64):
+    err = (got.double() - want64).abs()
+    return bool((err <= 1e-6 + 1e-5 * want64.abs()).all()), err.max().item()
+
+
+@pytest.mark.parametrize("mode", AGGS)
+@pytest.mark.parametrize("B,L", [(1, 1), (3, 5), (8, 256), (5, 2049), (2, 6000), (1, 32768)])
+@pytest.mark.parametrize("mdt", [torch.int64, torch.bool, torch.float32])
+def test_agg_loss(dev, mode, B, L, mdt):
+    import siirl_amd.core_algos as CA
+
+    lp, _, _, _, mask, _ = _batch(B, L, seed=B * 31 + L, dtype_mask=mdt)
+    x = lp.to(dev).requires_grad_(True)
+    out = CA.agg_loss(loss_mat=x, loss_mask=mask.to(dev), loss_agg_mode=mode)
+    assert out.dim() == 0 and out.is_cuda
+    x64 = lp.double().requires_grad_(True)
+    m_o = mask.to(torch.float64) if mdt != torch.int64 else mask
+    want = OC.agg_loss(x64, m_o, mode)
+    assert _close(out, want), (float(out), float(want))
+    assert abs(float(out) - float(OC.agg_loss(lp, mask if mdt != torch.bool else mask.float(), mode))) < 1e-3
+    out.backward()
+    want.backward()
+    ok, err = _grad_close(x.grad.cpu(), x64.grad)
+    assert ok, err
+
+
+def test_agg_loss_nan_semantics_and_errors(dev):
+    import siirl_amd.core_algos as CA
+
+    v = torch.tensor([[1.0, float("nan"), 3.0], [4.0, 5.0, 6.0]])
+    m = torch.tensor([[1, 0, 1], [0, 0, 0]])
+    # token-mean goes through where(): NaN outside the mask is harmless
+    got = CA.agg_loss(v.to(dev), m.to(dev), "token-mean")
+    assert _close(got, OC.agg_loss(v.double(), m, "token-mean")) and _close(got, 2.0)
+    # the other modes multiply: NaN * 0 poisons them, and an empty row is 0/0 in seq-mean-token-mean
+    for mode in AGGS[1:]:
+        assert math.isnan(float(CA.agg_loss(v.to(dev), m.to(dev), mode))) and math.isnan(float(OC.agg_loss(v, m, mode)))
+    v2 = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+    assert math.isnan(float(CA.agg_loss(v2.to(dev), m.to(dev), "seq-mean-token-mean")))
+    assert _close(CA.agg_loss(v2.to(dev), m.to(dev), "seq-mean-token-sum"), 2.0)
+    with pytest.raises(ValueError, match="Invalid loss_agg_mode"):
+        CA.agg_loss(v2.to(dev), m.to(dev), "mean")
+
+
+def _cfg(lo=0.2, hi=0.2, c=3.0, **kw):
+    return SimpleNamespace(clip_ratio=0.2, clip_ratio_low=lo, clip_ratio_high=hi, clip_ratio_c=c, **kw)
+
+
+@pytest.mark.parametrize("mode", AGGS)
+@pytest.mark.parametrize("B,L,lo,hi,c", [(4, 7, 0.2, 0.2, 3.0), (8, 256, 0.2, 0.28, 10.0), (3, 4100, 0.1, 0.3, 1.5)])
+@pytest.mark.parametrize("use_isw", [False, True])
+def test_policy_loss_vanilla(dev, mode, B, L, lo, hi, c, use_isw):
+    import siirl_amd.core_algos as CA
+
+    lp, old, _, adv, mask, _ = _batch(B, L, seed=7 * B + L)
+    lp[0, 0] = old[0, 0] + 25.0  # beyond the +-20 clamp
+    if L > 2:
+        lp[1, 1] = old[1, 1]  # ratio exactly 1: both branches of the maximum tie
+        adv[1] = 0.0  # zero advantage row
+    isw = (torch.rand(B, L, generator=torch.Generator().manual_seed(1)) + 0.5) if use_isw else None
+    cfg = _cfg(lo, hi, c)
+    x = lp.to(dev).requires_grad_(True)
+    got = CA.compute_policy_loss_vanilla(old_log_prob=old.to(dev), log_prob=x, advantages=adv.to(dev),
+                                         response_mask=mask.to(dev), loss_agg_mode=mode, config=cfg,
+                                         rollout_is_weights=None if isw is None else isw.to(dev))
+    x64 = lp.double().requires_grad_(True)
+    want = OC.compute_policy_loss_vanilla(old.double(), x64, adv.double(), mask, mode, cfg,
+                                          None if isw is None else isw.double())
+    want32 = OC.compute_policy_loss_vanilla(old, lp, adv, mask, mode, cfg, isw)
+    assert len(got) == 4
+    for g_, w_, w32 in zip(got, want, want32):
+        assert g_.dim() == 0 and g_.is_cuda
+        assert _close(g_, w_), (float(g_), float(w_))
+        assert abs(float(g_) - float(w32)) < 1e-3
+    got[0].backward()
+    want[0].backward()
+    ok, err = _grad_close(x.grad.cpu(), x64.grad)
+    assert ok, err
+    # and the hand-written closed form agrees with autograd away from exact ties
+    cf = OC.policy_loss_grad_closed_form(old.double(), lp.double(), adv.double(), mask, mode, cfg,
+                                         None if isw is None else isw.double())
+    assert (cf - x64.grad).abs().max() < 1e-9  # the 1e-8 of masked_mean vanishes in fp32 for an integer mask
+
+
+def test_policy_loss_vanilla_known_cases(dev):
+    """Hand-computed: lp == old gives ratio 1, pg_loss = agg(-A), no clipping, zero KL; saturation at the
+    clip edges; the dual clip caps the loss at -A*c for negative advantages."""
+    import siirl_amd.core_algos as CA
+
+    cfg = _cfg(0.2, 0.28, 3.0)
+    old = torch.zeros(1, 6)
+    mask = torch.ones(1, 6, dtype=torch.int64)
+    A = torch.tensor([[1.0, -1.0, 2.0, -2.0, 0.5, -0.5]])
+    out = CA.compute_policy_loss_vanilla(old.to(dev), old.clone().to(dev), A.to(dev), mask.to(dev), "token-mean", cfg)
+    assert _close(out[0], -A.mean()) and float(out[1]) == 0.0 and abs(float(out[2])) < 1e-9 and float(out[3]) == 0.0
+    # ratios: 1.5 (clipped high, A>0), 0.5 (clipped low, A<0), 4 (dual clip, A<0), 1.1 (inside)
+    lp = torch.log(torch.tensor([[1.5, 0.5, 4.0, 1.1, 1.5, 4.0]]))
+    A2 = torch.tensor([[2.0, -1.0, -1.0, 1.0, -1.0, 1.0]])
+    x = lp.to(dev).requires_grad_(True)
+    out = CA.compute_policy_loss_vanilla(old.to(dev), x, A2.to(dev), mask.to(dev), "seq-mean-token-sum", cfg)
+    tok = [-2 * 1.28, 0.8, 3.0, -1.1, 1.5, -1.28]  # max(-A r, -A clip(r)); A<0: min(., -A c)
+    assert _close(out[0], sum(tok), 1e-5)
+    assert _close(out[1], (1 + 1 + 0 + 0 + 0 + 1) / 6) and _close(out[3], 1 / 6)
+    out[0].backward()
+    want_g = torch.tensor([[0.0, 0.0, 0.0, -1.1, 1.5, 0.0]])  # gradient only through the unclipped branch
+    assert (x.grad.cpu() - want_g).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("B,L", [(1, 1), (4, 9), (2, 4100), (1, 32768)])
+@pytest.mark.parametrize("eps", [(0.2, 0.2), (3e-4, 4e-4)])
+def test_policy_loss_gspo(dev, B, L, eps):
+    import siirl_amd.core_algos as CA
+
+    lp, old, _, adv, mask, _ = _batch(B, L, seed=B + L)
+    old = lp + 0.02 * (old - lp)  # token log-ratios ~ N(0, small), as in GSPO's regime
+    cfg = _cfg(*eps)
+    isw = torch.rand(B, L, generator=torch.Generator().manual_seed(3)) + 0.5
+    x = lp.to(dev).requires_grad_(True)
+    got = CA.compute_policy_loss_gspo(old_log_prob=old.to(dev), log_prob=x, advantages=adv.to(dev),
+                                      response_mask=mask.to(dev), loss_agg_mode="token-mean", config=cfg,
+                                      rollout_is_weights=isw.to(dev))
+    x64 = lp.double().requires_grad_(True)
+    want = OC.compute_policy_loss_gspo(old.double(), x64, adv.double(), mask, "token-mean", cfg, isw.double())
+    want32 = OC.compute_policy_loss_gspo(old, lp, adv, mask, "token-mean", cfg, isw)
+    for g_, w_, w32 in zip(got, want, want32):
+        assert _close(g_, w_, 5e-5), (float(g_), float(w_))
+        assert abs(float(g_) - float(w32)) < 1e-3
+    assert float(got[3]) == 0.0
+    got[0].backward()
+    want[0].backward()
+    # the sequence ratio sits within 1e-3 of the clip edges here, where fp32 vs fp64 can pick different sides:
+    # compare tokens whose fp64 ratio is clear of the edges
+    n = mask.sum(-1).clamp(min=1)
+    s = ((lp.double() - old.double()) * mask).sum(-1) / n
+    rho = torch.exp(s)
+    clear = ((rho - (1 - eps[0])).abs() > 1e-6) & ((rho - (1 + eps[1])).abs() > 1e-6)
+    ok, err = _grad_close(x.grad.cpu()[clear], x64.grad[clear])
+    assert ok, err
+
+
+def test_gspo_length_one_is_ppo_without_dual_clip(dev):
+    import siirl_amd.core_algos as CA
+
+    lp, old, _, adv, mask, _ = _batch(16, 1, seed=5)
+    mask = torch.ones_like(mask)
+    cfg = _cfg(0.2, 0.2, 1e9)
+    a = CA.compute_policy_loss_gspo(old.to(dev), lp.to(dev), adv.to(dev), mask.to(dev), config=cfg)
+    b = CA.compute_policy_loss_vanilla(old.to(dev), lp.to(dev), adv.to(dev), mask.to(dev), "seq-mean-token-mean", cfg)
+    assert _close(a[0], float(b[0])) and _close(a[1], float(b[1])) and _close(a[2], float(b[2]))
+
+
+def test_legacy_compute_policy_loss(dev):
+    import siirl_amd.core_algos as CA
+
+    lp, old, _, adv, mask, _ = _batch(6, 33, seed=9)
+    got = CA.compute_policy_loss(old.to(dev), lp.to(dev), adv.to(dev), mask.to(dev), cliprange=0.2,
+                                 clip_ratio_c=3.0, loss_agg_mode="token-mean")
+    want = OC.compute_policy_loss_vanilla(old.double(), lp.double(), adv.double(), mask, "token-mean", _cfg())
+    for g_, w_ in zip(got, want):  # |d| < 20 everywhere here, so the clamp of the vanilla loss is inactive
+        assert _close(g_, w_)
+    with pytest.raises(AssertionError):
+        CA.compute_policy_loss(old.to(dev), lp.to(dev), adv.to(dev), mask.to(dev), cliprange=0.2, clip_ratio_c=1.0)
+
+
+def test_policy_loss_errors(dev):
+    import siirl_amd.core_algos as CA
+
+    lp, old, _, adv, mask, _ = _batch(2, 4, seed=1)
+    args = (old.to(dev), lp.to(dev), adv.to(dev), mask.to(dev))
+    with pytest.raises(AssertionError):
+        CA.compute_policy_loss_vanilla(*args, config=None)
+    with pytest.raises(AssertionError, match="clip_ratio_c"):
+        CA.compute_policy_loss_vanilla(*args, config=_cfg(c=1.0))
+    with pytest.raises(ValueError, match="Invalid loss_agg_mode"):
+        CA.compute_policy_loss_vanilla(*args, loss_agg_mode="bogus", config=_cfg())
+    with pytest.raises(ValueError, match="Unsupported loss mode"):
+        CA.get_policy_loss_fn("clip_cov")
+    assert CA.get_policy_loss_fn("vanilla") is CA.compute_policy_loss_vanilla
+    assert CA.get_policy_loss_fn("gspo") is CA.compute_policy_loss_gspo
+    with pytest.raises(RuntimeError, match="GPU only"):
+        CA.compute_policy_loss_vanilla(old, lp, adv, mask, config=_cfg())
+
+
+@pytest.mark.parametrize("kind", ["kl", "k1", "abs", "mse", "k2", "low_var_kl", "k3"])
+def test_kl_penalty(dev, kind):
+    import siirl_amd.core_algos as CA
+
+    lp, _, ref, _, _, _ = _batch(5, 300, seed=2)
+    ref[0, 0] = lp[0, 0] + 30.0  # beyond the clamp of k3
+    ref[0, 1] = lp[0, 1] - 30.0
+    ref[0, 2] = lp[0, 2]  # zero difference (abs: zero gradient)
+    x = lp.to(dev).requires_grad_(True)
+    out = CA.kl_penalty(logprob=x, ref_logprob=ref.to(dev), kl_penalty=kind)
+    x64 = lp.double().requires_grad_(True)
+    want = OC.kl_penalty(x64, ref.double(), kind)
+    assert ((out.cpu().double() - want).abs() <= 2e-5 + 1e-6 * want.abs()).all()
+    assert ((out.cpu() - OC.kl_penalty(lp, ref, kind)).abs() <= 1e-3 + 1e-6 * want.abs()).all()
+    g = torch.randn(5, 300, generator=torch.Generator().manual_seed(4))
+    out.backward(g.to(dev))
+    want.backward(g.double())
+    ok, err = _grad_close(x.grad.cpu(), x64.grad)
+    assert ok, err
+    if kind in ("low_var_kl", "k3"):
+        assert float(out.min()) >= 0.0 and float(out[0, 2]) == 0.0 and float(out[0, 1]) == 10.0
+
+
+def test_kl_penalty_names(dev):
+    import siirl_amd.core_algos as CA
+
+    a, b = torch.zeros(3, device=dev), torch.ones(3, device=dev)
+    for bad in ("full", "k3+", "k1+", "low_var_kl+", "nope"):
+        with pytest.raises(NotImplementedError):
+            CA.kl_penalty(a, b, bad)
+        with pytest.raises(NotImplementedError):
+            OC.kl_penalty(a.cpu(), b.cpu(), bad)
+    # the straight-through estimator: value of k3, gradient of k2
+    lp, _, ref, _, _, _ = _batch(3, 50, seed=6)
+    x = lp.to(dev).requires_grad_(True)
+    out = CA.kl_penalty_straight_through(x, ref.to(dev), "k3+")
+    assert (out.cpu() - OC.kl_penalty_forward(lp, ref, "k3")).abs().max() < 2e-5
+    out.sum().backward()
+    assert (x.grad.cpu() - (lp - ref)).abs().max() < 1e-6
+
+
+@pytest.mark.parametrize("loss_mode", ["vanilla", "gspo"])
+@pytest.mark.parametrize("mode", AGGS)
+@pytest.mark.parametrize("ent_coef,use_kl", [(0.0, False), (0.01, False), (0.0, True), (0.003, True)])
+def test_actor_loss_fused_matches_composition(dev, loss_mode, mode, ent_coef, use_kl):
+    """The fused launch equals the reference's composition: pg_loss - c_e * agg(entropy) + c_k * agg(kl), scaled."""
+    import siirl_amd.core_algos as CA
+
+    B, L = 6, 700
+    lp, old, ref, adv, mask, ent = _batch(B, L, seed=13)
+    cfg = _cfg(0.2, 0.28, 10.0, entropy_coeff=ent_coef, use_kl_loss=use_kl, kl_loss_coef=0.001,
+               kl_loss_type="low_var_kl", loss_agg_mode=mode, loss_mode=loss_mode)
+    scale = 0.25
+    x = lp.to(dev).requires_grad_(True)
+    e = ent.to(dev).requires_grad_(True)
+    res = CA.actor_loss(old.to(dev), x, adv.to(dev), mask.to(dev), cfg, entropy=e, ref_log_prob=ref.to(dev),
+                        loss_scale_factor=scale)
+    x64, e64 = lp.double().requires_grad_(True), ent.double().requires_grad_(True)
+    fn = OC.compute_policy_loss_vanilla if loss_mode == "vanilla" else OC.compute_policy_loss_gspo
+    pg, cf, kl, cfl = fn(old.double(), x64, adv.double(), mask, mode, cfg)
+    policy = pg
+    ent_loss = OC.agg_loss(e64, mask, mode)
+    if ent_coef != 0:
+        policy = policy - ent_loss * ent_coef
+    kl_loss = OC.agg_loss(OC.kl_penalty(x64, ref.double(), "low_var_kl"), mask, mode)
+    if use_kl:
+        policy = policy + kl_loss * 0.001
+    loss = policy * scale
+    assert _close(res.loss, loss) and _close(res.pg_loss, pg) and _close(res.pg_clipfrac, cf)
+    assert _close(res.ppo_kl, kl) and _close(res.pg_clipfrac_lower, cfl)
+    if ent_coef != 0:
+        assert _close(res.entropy_loss, ent_loss)
+    if use_kl:
+        assert _close(res.kl_loss, kl_loss)
+    ratio = (lp.double() - old.double()).exp()
+    mt = res.metrics()
+    assert _close(mt["actor/pg_clip_mean"], ratio.mean(), 1e-4) and _close(mt["actor/pg_clip_max"], ratio.max(), 1e-3)
+    assert _close(mt["actor/pg_clip_min"], ratio.min()) and _close(mt["actor/pg_loss"], pg * scale)
+    res.loss.backward()
+    loss.backward()
+    ok, err = _grad_close(x.grad.cpu(), x64.grad)
+    assert ok, err
+    if ent_coef != 0:
+        ok, err = _grad_close(e.grad.cpu(), e64.grad)
+        assert ok, err
+    else:
+        assert e.grad is None
+
+
+def test_masked_reductions(dev):
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(3)
+    v = torch.randn(7, 2500, generator=g)
+    m = (torch.rand(7, 2500, generator=g) > 0.4).long()
+    v[0, 0] = float("nan")
+    m[0, 0] = 0
+    m[3] = 0  # empty row: mean 0 / 1e-8 = 0
+    assert _close(SF.masked_sum(v.to(dev), m.to(dev)), OF.masked_sum(v.double(), m))
+    assert _close(SF.masked_mean(v.to(dev), m.to(dev)), OF.masked_mean(v.double(), m))
+    got = SF.masked_mean(v.to(dev), m.to(dev), axis=-1).cpu().double()
+    assert (got - OF.masked_mean(v.double(), m, axis=-1)).abs().max() < 2e-5 and float(got[3]) == 0.0
+    got = SF.masked_sum(v.to(dev), m.to(dev), axis=-1).cpu().double()
+    assert (got - OF.masked_sum(v.double(), m, axis=-1)).abs().max() < 2e-4
+
+
+def test_apply_kl_penalty_and_controllers(dev):
+    import siirl_amd.core_algos as CA
+
+    B, L = 12, 40
+    lp, old, ref, _, mask, _ = _batch(B, L, seed=17)
+    scores = torch.zeros(B, L)
+    scores[torch.arange(B), mask.sum(-1) - 1] = 1.0
+    for kind in ("kl", "low_var_kl", "abs", "mse"):
+        mk = lambda t: t.clone()  # noqa: E731
+        data = {"token_level_scores": mk(scores).to(dev), "old_log_probs": mk(old).to(dev),
+                "ref_log_prob": mk(ref).to(dev), "response_mask": mask.to(dev), "responses": torch.zeros(B, L)}
+        ctrl = CA.AdaptiveKLController(init_kl_coef=0.05, target_kl=0.1, horizon=100)
+        data, metrics = CA.apply_kl_penalty(data, ctrl, kl_penalty=kind)
+        odata = {"token_level_scores": scores.clone(), "old_log_probs": old, "ref_log_prob": ref, "response_mask": mask}
+        octrl = OC.AdaptiveKLController(0.05, 0.1, 100)
+        odata, ometrics = OC.apply_kl_penalty(odata, octrl, kind)
+        assert (data["token_level_rewards"].cpu() - odata["token_level_rewards"]).abs().max() < 1e-5
+        assert abs(metrics["actor/reward_kl_penalty"] - ometrics["actor/reward_kl_penalty"]) < 1e-5
+        assert metrics["actor/reward_kl_penalty_coeff"] == 0.05 and abs(ctrl.value - octrl.value) < 1e-8
+    # controller step by hand: kl/target - 1 = 1 clipped to 0.2; value *= 1 + 0.2 * 50 / 100
+    c = CA.AdaptiveKLController(0.1, 0.05, 100)
+    c.update(current_kl=0.1, n_steps=50)
+    assert abs(c.value - 0.11) < 1e-12
+    f = CA.get_kl_controller(SimpleNamespace(type="fixed", kl_coef=0.3))
+    f.update(1.0, 10)
+    assert f.value == 0.3
+    with pytest.raises(NotImplementedError):
+        CA.get_kl_controller(SimpleNamespace(type="pid", kl_coef=0.3))
+    r = CA.compute_rewards(scores.to(dev), old.to(dev), ref.to(dev), 0.1)
+    assert (r.cpu() - OC.compute_rewards(scores, old, ref, 0.1)).abs().max() < 1e-6

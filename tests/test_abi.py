@@ -1,0 +1,83 @@
+"""The C ABI (CPU only, no kernel is launched): libsiirl_hip.so loads, exports every function that
+include/siirl_hip.h declares, the ctypes table covers exactly those, and argument validation reports errors."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "siirl_hip.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(siirl_[a-z0-9_]+)\s*\(", text)))
+
+
+def _lib():
+    from siirl_amd import _lib
+
+    if not _lib.LIB_PATH.exists():
+        from siirl_amd import build
+
+        build.build()
+    return _lib
+
+
+def test_header_symbols_are_exported_and_bound():
+    L = _lib()
+    names = _declared()
+    assert len(names) >= 14
+    h = L.lib()
+    for n in names:
+        assert hasattr(h, n), f"{n} is declared in siirl_hip.h but not exported"
+    assert sorted(L.SIGNATURES) == names, "ctypes table and header disagree"
+    assert h.siirl_hip_abi_version() >= 1000
+
+
+def test_every_entry_point_cites_the_reference():
+    text = open(HEADER).read()
+    for n in _declared():
+        if n in ("siirl_hip_abi_version", "siirl_hip_last_error", "siirl_loss_workspace_bytes", "siirl_agg_loss_bwd",
+                 "siirl_actor_loss_bwd", "siirl_kl_penalty_bwd"):
+            continue
+        pos = text.index(n + "(")
+        comment = text[text.rfind("/*", 0, pos):pos]
+        assert "Replaces:" in comment and re.search(r"siirl/[\w/]+\.py:\d+", comment), f"{n} lacks a reference citation"
+
+
+def test_argument_validation_without_gpu():
+    L = _lib()
+    h = L.lib()
+    buf = (ctypes.c_float * 64)()
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # V = 0
+    assert h.siirl_logprob_entropy_fwd(p, L.BF16, 4, 0, 0, p, 1.0, p, p, p, p, None) == -1
+    assert b"V=0" in h.siirl_hip_last_error()
+    # unsupported logits dtype
+    assert h.siirl_logprob_entropy_fwd(p, L.I64, 4, 8, 8, p, 1.0, p, p, p, p, None) == -1
+    # labels without logprob
+    assert h.siirl_logprob_entropy_fwd(p, L.F32, 1, 8, 8, p, 1.0, None, p, p, p, None) == -1
+    # backward: overlapping but distinct buffers
+    q = ctypes.c_void_p(p.value + 8)
+    assert h.siirl_logprob_entropy_bwd(p, L.F32, 1, 8, 8, p, 1.0, p, p, p, p, q, 8, 0, None) == -1
+    assert b"overlaps" in h.siirl_hip_last_error()
+    # loss: bad aggregation mode / clip_ratio_c / workspace
+    assert h.siirl_agg_loss_fwd(p, p, L.F32, 2, 4, 9, p, p, p, 1 << 20, None) == -1
+    assert b"Invalid loss_agg_mode" in h.siirl_hip_last_error()
+    assert h.siirl_actor_loss_fwd(p, p, p, p, L.F32, None, None, None, 2, 4, 0, 0.2, 0.2, 1.0, 20.0, 0, 0.0, 0, 0, 0.0,
+                                  1.0, p, p, p, p, 1 << 20, None) == -1
+    assert b"clip_ratio_c" in h.siirl_hip_last_error()
+    assert h.siirl_agg_loss_fwd(p, p, L.F32, 2, 4, 0, p, p, p, 8, None) == -4
+    assert h.siirl_loss_workspace_bytes(2, 4) > 0 and h.siirl_loss_workspace_bytes(0, 4) == 0
+    assert h.siirl_kl_penalty_fwd(p, p, 4, 7, p, None) == -1
+    assert h.siirl_group_keep_mask(p, L.BF16, p, 4, p, None, None) == -1
+    with pytest.raises(ValueError):
+        L.check(-1, "x")
+    with pytest.raises(NotImplementedError):
+        L.check(-2, "x")
+    with pytest.raises(L.SiirlHipError):
+        L.check(-3, "x")

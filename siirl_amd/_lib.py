@@ -35,6 +35,12 @@ SIGNATURES = {
     "siirl_kl_in_reward": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i32, _f32, _p, _p, _p, _p]),
     "siirl_grpo_outcome_advantage": (_i32, [_p, _p, _i32, _p, _i64, _i64, _f32, _i32, _p, _p, _p]),
     "siirl_group_keep_mask": (_i32, [_p, _i32, _p, _i64, _p, _p, _p]),
+    "siirl_fused_linear_fwd_workspace_bytes": (_sz, [_i64, _i64, _i64]),
+    "siirl_fused_linear_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32, _i32]),
+    "siirl_fused_linear_logprob_entropy_fwd": (_i32, [_p, _p, _i32, _p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _p, _sz,
+                                                      _p]),
+    "siirl_fused_linear_logprob_entropy_bwd": (_i32, [_p, _p, _i32, _p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _p, _p,
+                                                      _p, _sz, _p]),
 }
 
 _lock = threading.Lock()

@@ -1,0 +1,562 @@
+// lm_head projection fused with log-prob / entropy: logits = hidden[T,H] . W[V,H]^T are produced tile by tile on
+// the matrix cores and consumed in the epilogue, never written to memory.
+//
+// Replaces FusedLinearForPPO (siirl/utils/experimental/torch_functional.py:20-211) and linear_cross_entropy
+// (siirl/utils/kernel/linear_cross_entropy.py:40-117 -> siirl/utils/kernel/kernels.py:507-696,1378-1586); the
+// per-tile online-softmax state (max, sum exp, sum x*exp) is the one of kernels.py:254-266,343-350.
+//
+// One GEMM core, C[M,N] = A[M,K] . B[N,K]^T with both operands K-major bf16 and fp32 accumulation:
+//   256 x 256 x 64 workgroup tile, 4 waves of 128 x 128 (4 x 4 MFMA 32x32x16 bf16 tiles, 256 accumulator
+//   registers), double-buffered LDS (rows padded to 144 B so that ds_read_b128 fragments are conflict-free),
+//   global loads of the next K-step issued before the MFMAs of the current one.
+// Four epilogues: softmax partials (forward), dlogits in both layouts (backward), fp32 accumulate (d hidden),
+// bf16 store (d weight).  The backward walks the vocabulary in slabs: recompute the slab's logits, write
+// dlogits[T, slab] and its transpose, then dH += dlogits . W_slab and dW_slab = dlogits^T . hidden as two more
+// runs of the same core against transposed copies of W and hidden.
+#include "common.hpp"
+
+namespace siirl {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int kThreads = 256;
+constexpr int kRowBytes = BK * 2 + 16;        // 128 B of data + 16 B pad
+constexpr int kTileBytes = BM * kRowBytes;    // 36864
+constexpr int kStageBytes = 2 * kTileBytes;   // A tile + B tile
+constexpr int kSmemBytes = 2 * kStageBytes;   // 147456 of the 160 KB
+constexpr int kGroupN = 8;                    // N-tiles per rasterisation group
+constexpr int kSlab = 8192;                   // vocabulary columns per backward slab
+
+struct GemmArgs {
+  const uint16_t* A;
+  int64_t lda;
+  const uint16_t* B;
+  int64_t ldb;
+  int M, N, K;  // K is a multiple of BK; rows beyond M / N are clamped on load and masked by the epilogue
+  int tiles_m, tiles_n;
+};
+
+struct TileCoord {
+  int tm, tn;
+};
+__device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int id) {
+  const int group_sz = kGroupN * g.tiles_m;
+  const int grp = id / group_sz;
+  const int first_n = grp * kGroupN;
+  const int gn = (g.tiles_n - first_n) < kGroupN ? (g.tiles_n - first_n) : kGroupN;
+  const int in = id % group_sz;
+  return {in / gn, first_n + in % gn};
+}
+
+// Accumulator coordinates of lane `lane` in wave (wm, wn): element r of acc[i][j] is
+//   row = wm*128 + i*32 + (r/4)*8 + (lane/32)*4 + r%4 ,  col = wn*128 + j*32 + lane%32   (tile-relative)
+__device__ __forceinline__ int acc_row(int wm, int i, int r, int lane) {
+  return wm * 128 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+}
+__device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * 128 + j * 32 + (lane & 31); }
+
+template <class Epi>
+__global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(GemmArgs g, Epi epi) {
+  extern __shared__ __align__(16) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int wm = w >> 1, wn = w & 1;
+  const TileCoord tc = tile_of(g, blockIdx.x);
+  const int m0 = tc.tm * BM, n0 = tc.tn * BN;
+
+  // global -> LDS mapping: 16-byte chunk c of rows r0 + 32 j.  Rows past the matrix edge are clamped to the
+  // last row; offsets are relative to the tile's first row so that they fit 32 bits.
+  const int c = tid & 7, r0 = tid >> 3;
+  const uint16_t* baseA = g.A + (int64_t)m0 * g.lda + c * 8;
+  const uint16_t* baseB = g.B + (int64_t)n0 * g.ldb + c * 8;
+  int offA[8], offB[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    int ra = r0 + 32 * j, rb = r0 + 32 * j;
+    ra = (m0 + ra < g.M) ? ra : g.M - 1 - m0;
+    rb = (n0 + rb < g.N) ? rb : g.N - 1 - n0;
+    offA[j] = ra * (int)g.lda;
+    offB[j] = rb * (int)g.ldb;
+  }
+  const int lds_w = r0 * kRowBytes + c * 16;
+
+  floatx16 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  u32x4 ga[8], gb[8];
+  auto gload = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      ga[j] = *reinterpret_cast<const u32x4*>(baseA + kt * BK + offA[j]);
+      gb[j] = *reinterpret_cast<const u32x4*>(baseB + kt * BK + offB[j]);
+    }
+  };
+  auto swrite = [&](char* st) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      *reinterpret_cast<u32x4*>(st + lds_w + 32 * j * kRowBytes) = ga[j];
+      *reinterpret_cast<u32x4*>(st + kTileBytes + lds_w + 32 * j * kRowBytes) = gb[j];
+    }
+  };
+
+  const int KT = g.K / BK;
+  gload(0);
+  swrite(smem);
+  __syncthreads();
+
+  const int frag_a = (wm * 128 + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
+  const int frag_b = kTileBytes + (wn * 128 + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
+
+  for (int kt = 0; kt < KT; ++kt) {
+    char* cur = smem + (kt & 1) * kStageBytes;
+    const bool more = kt + 1 < KT;
+    if (more) gload(kt + 1);
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8 af[4], bfr[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        af[i] = *reinterpret_cast<const bf16x8*>(cur + frag_a + i * 32 * kRowBytes + kk * 32);
+        bfr[i] = *reinterpret_cast<const bf16x8*>(cur + frag_b + i * 32 * kRowBytes + kk * 32);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+    if (more) swrite(smem + ((kt + 1) & 1) * kStageBytes);
+    __syncthreads();
+  }
+  epi(acc, m0, n0, tc.tn, wm, wn, lane, tid, smem);
+}
+
+// ------------------------------------------------------------------------------ epilogue: softmax partials
+
+// Per row of the tile: mx = max_v z, s = sum exp(z - mx), t = sum z * exp(z - mx) over the tile's 256 columns,
+// z = acc * inv_T.  Row reductions run across the 32 lanes that share a row; the two column halves of the
+// workgroup are merged through LDS and one (mx, s, t) per row is written to part[tn][row].
+struct SoftmaxPartialsEpi {
+  float inv_T;
+  int T, V;
+  float* part;  // [tiles_n][3][T]
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
+                             char* smem) const {
+    float* sh = reinterpret_cast<float*>(smem);  // [2][256][3]; the main loop's last barrier freed the LDS
+    const float k = kLog2e;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        float x[4];
+        float mx = -__builtin_inff();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const bool ok = n0 + acc_col(wn, j, lane) < V;
+          x[j] = ok ? acc[i][j][r] * inv_T : -__builtin_inff();
+          mx = fmaxf(mx, x[j]);
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
+        float s = 0.f, t = 0.f;
+        if (mx > -__builtin_inff()) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float e = fast_exp2((x[j] - mx) * k);  // 0 for masked columns
+            s += e;
+            t += (x[j] > -__builtin_inff()) ? x[j] * e : 0.f;
+          }
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) {
+          s += __shfl_xor(s, o, kWave);
+          t += __shfl_xor(t, o, kWave);
+        }
+        if ((lane & 31) == 0) {
+          float* d = sh + (wn * BM + acc_row(wm, i, r, lane)) * 3;
+          d[0] = mx;
+          d[1] = s;
+          d[2] = t;
+        }
+      }
+    }
+    __syncthreads();
+    const int row = m0 + tid;
+    if (row < T) {
+      const float* a = sh + tid * 3;
+      const float* b = sh + (BM + tid) * 3;
+      const float M = fmaxf(a[0], b[0]);
+      const float fa = a[0] > -__builtin_inff() ? fast_exp2((a[0] - M) * k) : 0.f;
+      const float fb = b[0] > -__builtin_inff() ? fast_exp2((b[0] - M) * k) : 0.f;
+      float* o = part + (int64_t)tn * 3 * T;
+      o[row] = M;
+      o[(int64_t)T + row] = a[1] * fa + b[1] * fb;
+      o[2 * (int64_t)T + row] = a[2] * fa + b[2] * fb;
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------ epilogue: dlogits
+
+// d raw_logit = inv_T * ( g_lp * (1[v == y] - p) - g_h * p * (z - ex) ),  p = exp(z - lse), z = acc * inv_T,
+// written as bf16 to D[row][col] (ld = ldd) and to Dt[col][row] (ld = ldt); col is slab-relative.  Columns in
+// [N, Npad) are written as zeros: they are K-padding of the GEMMs that consume the buffers.
+struct DlogitsEpi {
+  float inv_T;
+  int T, N, Npad;
+  int64_t v0;  // first vocabulary column of the slab
+  const float* lse;
+  const float* ex;
+  const float* g_lp;  // may be null
+  const float* g_h;   // may be null
+  const int64_t* labels;
+  uint16_t* D;
+  int64_t ldd;
+  uint16_t* Dt;
+  int64_t ldt;
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
+                             char* smem) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + acc_row(wm, i, r, lane);
+        if (row >= T) continue;
+        const float g1 = g_lp ? g_lp[row] : 0.f;
+        const float g2 = g_h ? g_h[row] : 0.f;
+        const float nl = -lse[row] * kLog2e;
+        const float exv = g_h ? ex[row] : 0.f;
+        const int64_t y = g_lp ? labels[row] - v0 : -1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int col = n0 + acc_col(wn, j, lane);
+          if (col >= Npad) continue;
+          float d = 0.f;
+          if (col < N) {
+            const float z = acc[i][j][r] * inv_T;
+            const float p = fast_exp2(fmaf(z, kLog2e, nl));
+            d = p * (-g1 - g2 * (z - exv));
+            if ((int64_t)col == y) d += g1;
+            d *= inv_T;
+          }
+          const uint16_t h = (uint16_t)(pack_bf16(d, 0.f) & 0xffffu);
+          D[(int64_t)row * ldd + col] = h;
+          Dt[(int64_t)col * ldt + row] = h;
+        }
+      }
+    }
+  }
+};
+
+// ------------------------------------------------------------------------------ epilogues: plain stores
+
+struct AccumF32Epi {  // C[row][col] = (beta ? C : 0) + acc
+  float* C;
+  int64_t ldc;
+  int M, N, beta;
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
+                             char* smem) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + acc_row(wm, i, r, lane);
+        if (row >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int col = n0 + acc_col(wn, j, lane);
+          if (col >= N) continue;
+          float* p = C + (int64_t)row * ldc + col;
+          *p = beta ? *p + acc[i][j][r] : acc[i][j][r];
+        }
+      }
+  }
+};
+
+struct StoreBf16Epi {  // C[row][col] = bf16(acc)
+  uint16_t* C;
+  int64_t ldc;
+  int M, N;
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
+                             char* smem) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = m0 + acc_row(wm, i, r, lane);
+        if (row >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int col = n0 + acc_col(wn, j, lane);
+          if (col >= N) continue;
+          C[(int64_t)row * ldc + col] = (uint16_t)(pack_bf16(acc[i][j][r], 0.f) & 0xffffu);
+        }
+      }
+  }
+};
+
+// ------------------------------------------------------------------------------ small kernels
+
+// out[c][r] = in[r][c] for r < R, c < C; out has ld_out >= R columns, columns [R, ld_out) are zero-filled
+// for every row c < C_out (rows c in [C, C_out) are zero too).
+__global__ __launch_bounds__(256) void transpose_pad_kernel(const uint16_t* __restrict__ in, int64_t ld_in, int R,
+                                                            int C, uint16_t* __restrict__ out, int64_t ld_out,
+                                                            int C_out) {
+  __shared__ uint16_t tile[64][66];
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  for (int rr = ty; rr < 64; rr += 4) {
+    const int r = r0 + rr, cc = c0 + tx;
+    tile[rr][tx] = (r < R && cc < C) ? in[(int64_t)r * ld_in + cc] : (uint16_t)0;
+  }
+  __syncthreads();
+  for (int cc = ty; cc < 64; cc += 4) {
+    const int cidx = c0 + cc, r = r0 + tx;
+    if (cidx < C_out && r < ld_out) out[(int64_t)cidx * ld_out + r] = tile[tx][cc];
+  }
+}
+
+// label_logit[row] = inv_T * <hidden[row], W[labels[row]]>, one wave per row (NaN for a label outside [0, V))
+__global__ __launch_bounds__(256) void label_logit_kernel(const uint16_t* __restrict__ hidden,
+                                                          const uint16_t* __restrict__ W,
+                                                          const int64_t* __restrict__ labels, int T, int H, int64_t V,
+                                                          float inv_T, float* __restrict__ out) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= T) return;
+  const int64_t y = labels[row];
+  if (y < 0 || y >= V) {
+    if (lane == 0) out[row] = __builtin_nanf("");
+    return;
+  }
+  const u32x4* a = reinterpret_cast<const u32x4*>(hidden + (int64_t)row * H);
+  const u32x4* b = reinterpret_cast<const u32x4*>(W + y * (int64_t)H);
+  float s = 0.f;
+  for (int i = lane; i < H / 8; i += kWave) {
+    const u32x4 u = a[i], v = b[i];
+    s += bf16_lo(u.x) * bf16_lo(v.x) + bf16_hi(u.x) * bf16_hi(v.x) + bf16_lo(u.y) * bf16_lo(v.y) +
+         bf16_hi(u.y) * bf16_hi(v.y) + bf16_lo(u.z) * bf16_lo(v.z) + bf16_hi(u.z) * bf16_hi(v.z) +
+         bf16_lo(u.w) * bf16_lo(v.w) + bf16_hi(u.w) * bf16_hi(v.w);
+  }
+  s = wave_sum(s);
+  if (lane == 0) out[row] = s * inv_T;
+}
+
+// folds the per-tile partials of each row: lse, ex, entropy, logprob
+__global__ __launch_bounds__(256) void merge_partials_kernel(const float* __restrict__ part, int nparts, int T,
+                                                             const float* __restrict__ label_logit,
+                                                             float* __restrict__ logprob, float* __restrict__ entropy,
+                                                             float* __restrict__ lse_out, float* __restrict__ ex_out) {
+  const int row = blockIdx.x * 256 + threadIdx.x;
+  if (row >= T) return;
+  float M = -__builtin_inff();
+  for (int p = 0; p < nparts; ++p) M = fmaxf(M, part[(int64_t)p * 3 * T + row]);
+  double s = 0.0, t = 0.0;
+  for (int p = 0; p < nparts; ++p) {
+    const float* q = part + (int64_t)p * 3 * T;
+    const float m = q[row];
+    if (m > -__builtin_inff()) {
+      const float f = fast_exp2((m - M) * kLog2e);
+      s += (double)(q[(int64_t)T + row] * f);
+      t += (double)(q[2 * (int64_t)T + row] * f);
+    }
+  }
+  const float lse = M + logf((float)s);
+  const float exv = (float)(t / s);
+  lse_out[row] = lse;
+  if (ex_out) ex_out[row] = exv;
+  if (entropy) entropy[row] = lse - exv;
+  if (logprob) logprob[row] = label_logit[row] - lse;
+}
+
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, uint16_t* __restrict__ out,
+                                                          int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+    out[i] = (uint16_t)(pack_bf16(in[i], 0.f) & 0xffffu);
+}
+
+// ------------------------------------------------------------------------------ host
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+template <class Epi>
+int launch_gemm(const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, int M, int N, int K, const Epi& epi,
+                hipStream_t st, const char* what) {
+  static bool attr_set = false;  // one flag per instantiation
+  if (!attr_set) {
+    SIIRL_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi>),
+                                        hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
+    attr_set = true;
+  }
+  GemmArgs g{A, lda, B, ldb, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN};
+  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  gemm_nt_kernel<Epi><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
+  SIIRL_LAUNCH_CHECK(what);
+  return SIIRL_OK;
+}
+
+int check_fused(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V, float inv_T, int dtype) {
+  SIIRL_REQUIRE(dtype == SIIRL_BF16, "fused lm_head path takes bf16 operands (dtype %d given)", dtype);
+  SIIRL_REQUIRE(T >= 1 && T < (1LL << 30) && V >= 1 && V < (1LL << 30), "T=%lld V=%lld out of range", (long long)T,
+                (long long)V);
+  SIIRL_REQUIRE(H >= BK && H % BK == 0 && H < (1 << 22), "hidden size %lld must be a positive multiple of %d",
+                (long long)H, BK);
+  SIIRL_REQUIRE(hidden && weight, "NULL operand");
+  SIIRL_REQUIRE(((uintptr_t)hidden & 15) == 0 && ((uintptr_t)weight & 15) == 0, "operands must be 16-byte aligned");
+  SIIRL_REQUIRE(inv_T > 0.f && inv_T < 1e30f, "inv_temperature must be positive and finite");
+  return SIIRL_OK;
+}
+int check_ws_align(const void* ws) {
+  SIIRL_REQUIRE(((uintptr_t)ws & 255) == 0, "workspace must be 256-byte aligned");
+  return SIIRL_OK;
+}
+
+struct FwdWs {
+  size_t part, label, total;
+};
+FwdWs fwd_ws(int64_t T, int64_t V) {
+  FwdWs w;
+  const int64_t tiles_n = (V + BN - 1) / BN;
+  w.part = 0;
+  w.label = round_up((size_t)tiles_n * 3 * T * 4, 256);
+  w.total = w.label + round_up((size_t)T * 4, 256);
+  return w;
+}
+
+struct BwdWs {
+  size_t wt, ht, d, dt, dh32, total;
+  int64_t ldwt, ldt;
+};
+BwdWs bwd_ws(int64_t T, int64_t H, int64_t V, bool want_dh, bool want_dw) {
+  BwdWs w;
+  w.ldwt = round_up(V, BK);
+  w.ldt = round_up(T, BK);
+  size_t off = 0;
+  w.wt = off; off += want_dh ? round_up((size_t)H * w.ldwt * 2, 256) : 0;
+  w.ht = off; off += want_dw ? round_up((size_t)H * w.ldt * 2, 256) : 0;
+  w.d = off; off += round_up((size_t)T * kSlab * 2, 256);
+  w.dt = off; off += round_up((size_t)kSlab * w.ldt * 2, 256);
+  w.dh32 = off; off += want_dh ? round_up((size_t)T * H * 4, 256) : 0;
+  w.total = off;
+  return w;
+}
+
+}  // namespace
+}  // namespace siirl
+
+using namespace siirl;
+
+extern "C" size_t siirl_fused_linear_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
+  if (T < 1 || V < 1) return 0;
+  return fwd_ws(T, V).total;
+}
+
+extern "C" size_t siirl_fused_linear_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int want_d_hidden,
+                                                         int want_d_weight) {
+  if (T < 1 || V < 1 || H < 1) return 0;
+  return bwd_ws(T, H, V, want_d_hidden != 0, want_d_weight != 0).total;
+}
+
+extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype,
+                                                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
+                                                      float inv_temperature, float* logprob, float* entropy, float* lse,
+                                                      float* ex, void* workspace, size_t workspace_bytes,
+                                                      siirl_stream_t stream) {
+  if (int rc = check_fused(hidden, weight, T, H, V, inv_temperature, dtype)) return rc;
+  SIIRL_REQUIRE(lse != nullptr, "lse is NULL");
+  SIIRL_REQUIRE((logprob == nullptr) == (labels == nullptr), "labels and logprob must be given together");
+  SIIRL_REQUIRE(entropy == nullptr || ex != nullptr, "ex is required when entropy is requested");
+  const FwdWs ws = fwd_ws(T, V);
+  if (workspace == nullptr || workspace_bytes < ws.total)
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, ws.total);
+  if (int rc = check_ws_align(workspace)) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  float* part = reinterpret_cast<float*>((char*)workspace + ws.part);
+  float* label_logit = reinterpret_cast<float*>((char*)workspace + ws.label);
+  const uint16_t* h = (const uint16_t*)hidden;
+  const uint16_t* w = (const uint16_t*)weight;
+  if (labels) {
+    label_logit_kernel<<<dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st>>>(h, w, labels, (int)T, (int)H, V,
+                                                                          inv_temperature, label_logit);
+    SIIRL_LAUNCH_CHECK("label_logit_kernel");
+  }
+  SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part};
+  if (int rc = launch_gemm(h, H, w, H, (int)T, (int)V, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
+  const int tiles_n = (int)((V + BN - 1) / BN);
+  merge_partials_kernel<<<dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st>>>(part, tiles_n, (int)T, label_logit,
+                                                                               logprob, entropy, lse, ex);
+  SIIRL_LAUNCH_CHECK("merge_partials_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const void* weight, int dtype,
+                                                      const int64_t* labels, int64_t T, int64_t H, int64_t V,
+                                                      float inv_temperature, const float* lse, const float* ex,
+                                                      const float* g_logprob, const float* g_entropy, void* d_hidden,
+                                                      void* d_weight, void* workspace, size_t workspace_bytes,
+                                                      siirl_stream_t stream) {
+  if (int rc = check_fused(hidden, weight, T, H, V, inv_temperature, dtype)) return rc;
+  SIIRL_REQUIRE(lse != nullptr, "lse is NULL");
+  SIIRL_REQUIRE(g_logprob != nullptr || g_entropy != nullptr, "no upstream gradient given");
+  SIIRL_REQUIRE(g_logprob == nullptr || labels != nullptr, "labels is required with g_logprob");
+  SIIRL_REQUIRE(g_entropy == nullptr || ex != nullptr, "ex is required with g_entropy");
+  SIIRL_REQUIRE(d_hidden != nullptr || d_weight != nullptr, "neither d_hidden nor d_weight requested");
+  const bool want_dh = d_hidden != nullptr, want_dw = d_weight != nullptr;
+  const BwdWs ws = bwd_ws(T, H, V, want_dh, want_dw);
+  if (workspace == nullptr || workspace_bytes < ws.total)
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, ws.total);
+  if (int rc = check_ws_align(workspace)) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char* base = (char*)workspace;
+  uint16_t* Wt = (uint16_t*)(base + ws.wt);    // [H][ldwt]
+  uint16_t* Ht = (uint16_t*)(base + ws.ht);    // [H][ldt]
+  uint16_t* D = (uint16_t*)(base + ws.d);      // [T][kSlab]
+  uint16_t* Dt = (uint16_t*)(base + ws.dt);    // [kSlab][ldt]
+  float* dH32 = (float*)(base + ws.dh32);      // [T][H]
+  const uint16_t* h = (const uint16_t*)hidden;
+  const uint16_t* w = (const uint16_t*)weight;
+
+  if (want_dh) {
+    transpose_pad_kernel<<<dim3((unsigned)((ws.ldwt + 63) / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st>>>(
+        w, H, (int)V, (int)H, Wt, ws.ldwt, (int)H);
+    SIIRL_LAUNCH_CHECK("transpose_pad_kernel(W)");
+  }
+  if (want_dw) {
+    transpose_pad_kernel<<<dim3((unsigned)((ws.ldt + 63) / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st>>>(
+        h, H, (int)T, (int)H, Ht, ws.ldt, (int)H);
+    SIIRL_LAUNCH_CHECK("transpose_pad_kernel(hidden)");
+  }
+  // K-padding rows of Dt (token index in [T, ldt)) are never written by the epilogue: clear once
+  SIIRL_HIP_CHECK(hipMemsetAsync(Dt, 0, (size_t)kSlab * ws.ldt * 2, st));
+
+  int slab_idx = 0;
+  for (int64_t v0 = 0; v0 < V; v0 += kSlab, ++slab_idx) {
+    const int N = (int)((V - v0) < kSlab ? (V - v0) : kSlab);
+    const int Npad = (int)round_up(N, BK);
+    DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels, D, kSlab, Dt, ws.ldt};
+    if (int rc = launch_gemm(h, H, w + v0 * H, H, (int)T, N, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
+    if (want_dh) {  // dH[T, H] += D[T, Npad] . Wt[H, v0 : v0 + Npad]^T
+      AccumF32Epi acc{dH32, H, (int)T, (int)H, slab_idx > 0 ? 1 : 0};
+      if (int rc = launch_gemm(D, kSlab, Wt + v0, ws.ldwt, (int)T, (int)H, Npad, acc, st, "gemm_nt_kernel<AccumF32Epi>"))
+        return rc;
+    }
+    if (want_dw) {  // dW[v0 : v0 + N, H] = Dt[N, ldt] . Ht[H, ldt]^T
+      StoreBf16Epi sto{(uint16_t*)d_weight + v0 * H, H, N, (int)H};
+      if (int rc = launch_gemm(Dt, ws.ldt, Ht, ws.ldt, N, (int)H, (int)ws.ldt, sto, st, "gemm_nt_kernel<StoreBf16Epi>"))
+        return rc;
+    }
+  }
+  if (want_dh) {
+    const int64_t n = T * H;
+    const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
+    f32_to_bf16_kernel<<<dim3(blocks), dim3(256), 0, st>>>(dH32, (uint16_t*)d_hidden, n);
+    SIIRL_LAUNCH_CHECK("f32_to_bf16_kernel");
+  }
+  return SIIRL_OK;
+}

@@ -34,11 +34,11 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published peak
 SEQS, SEQ_LEN, VOCAB = 8, 4096, 152064
 SEED = 20250602
 
-# HBM bytes per launch of the dominant kernel (lpe_bwd_kernel at the default workload) from two
+# HBM bytes per launch of the dominant kernel (lpe_bwd_flat_kernel at the default workload) from two
 # rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same
 # counter reads for a plain 2 GiB device copy (FETCH_SIZE reads half the bytes fetched: factor 2.0;
 # WRITE_SIZE factor 1.0).  Figures and commands: profiles/lpe_config2_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES = int((4872501.73 * 2.0 + 9732197.53) * 1024)
+MEASURED_TRAFFIC_BYTES = int((4872295.36 * 2.0 + 9733447.5) * 1024)
 
 
 def make_workload(dev, seqs=SEQS, seq_len=SEQ_LEN, vocab=VOCAB, seed=SEED):
@@ -193,8 +193,8 @@ def main():
         "hbm_roofline_pct_step": 100.0 * step_gbs / HBM_PEAK_GBS,
         "step_algorithmic_bytes": fwd_bytes + bwd_bytes,
         "kernels": {"lpe_fwd_kernel": {"ms": fwd_ms, "GB/s": fwd_gbs, "bytes": fwd_bytes},
-                    "lpe_bwd_kernel": {"ms": bwd_ms, "GB/s": bwd_gbs, "bytes": bwd_bytes}},
-        "roofline": {"bound": "hbm", "kernel": "lpe_bwd_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
+                    "lpe_bwd_flat_kernel": {"ms": bwd_ms, "GB/s": bwd_gbs, "bytes": bwd_bytes}},
+        "roofline": {"bound": "hbm", "kernel": "lpe_bwd_flat_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES if args.seqs == SEQS else None},
         "row_skip_variant": row_skip,

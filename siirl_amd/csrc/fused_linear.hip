@@ -22,12 +22,18 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int kThreads = 256;
+#ifndef SIIRL_GEMM_WAVES_N
+#define SIIRL_GEMM_WAVES_N 4
+#endif
+constexpr int WM = 2, WN = SIIRL_GEMM_WAVES_N;  // wave grid over the workgroup tile
+constexpr int kThreads = WM * WN * 64;
+constexpr int MI = BM / (WM * 32), NJ = BN / (WN * 32);  // 32x32 MFMA tiles per wave
+constexpr int kLoadsPerThread = (BM * BK / 8) / kThreads;  // 16-byte chunks per operand tile per thread
+constexpr int kLoadRowStep = kThreads / 8;
 constexpr int kRowBytes = BK * 2 + 16;        // 128 B of data + 16 B pad
 constexpr int kTileBytes = BM * kRowBytes;    // 36864
 constexpr int kStageBytes = 2 * kTileBytes;   // A tile + B tile
 constexpr int kSmemBytes = 2 * kStageBytes;   // 147456 of the 160 KB
-constexpr int kGroupN = 8;                    // N-tiles per rasterisation group
 constexpr int kSlab = 8192;                   // vocabulary columns per backward slab
 
 struct GemmArgs {
@@ -41,29 +47,42 @@ struct GemmArgs {
 
 struct TileCoord {
   int tm, tn;
+  bool valid;
 };
+// XCD-aware rasterisation.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2, so
+// workgroup id runs on XCD id % 8 as that XCD's (id / 8)-th workgroup.  The tile grid is cut into blocks of
+// kBlkM x kBlkN tiles (32 tiles: one XCD's resident set); block b goes to XCD b % 8 and its tiles to 32
+// consecutive workgroups of that XCD, so the workgroups sharing an L2 at any time share 8 A-tiles and 4
+// B-tiles instead of streaming 32 different A-tiles.  Blocks sweep M fastest inside a strip of kBlkN N-tiles,
+// which keeps a strip's B-tiles hot across the 8 XCDs.
+constexpr int kXcd = 8, kBlkM = 8, kBlkN = 4;
+__host__ __device__ inline int64_t raster_grid(int tiles_m, int tiles_n) {
+  const int64_t blocks = (int64_t)((tiles_m + kBlkM - 1) / kBlkM) * ((tiles_n + kBlkN - 1) / kBlkN);
+  return (blocks + kXcd - 1) / kXcd * kXcd * (kBlkM * kBlkN);
+}
 __device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int id) {
-  const int group_sz = kGroupN * g.tiles_m;
-  const int grp = id / group_sz;
-  const int first_n = grp * kGroupN;
-  const int gn = (g.tiles_n - first_n) < kGroupN ? (g.tiles_n - first_n) : kGroupN;
-  const int in = id % group_sz;
-  return {in / gn, first_n + in % gn};
+  const int xcd = id % kXcd, l = id / kXcd;
+  const int blk = (l / (kBlkM * kBlkN)) * kXcd + xcd, j = l % (kBlkM * kBlkN);
+  const int mb = (g.tiles_m + kBlkM - 1) / kBlkM;
+  const int tm = (blk % mb) * kBlkM + j % kBlkM;
+  const int tn = (blk / mb) * kBlkN + j / kBlkM;
+  return {tm, tn, tm < g.tiles_m && tn < g.tiles_n};
 }
 
 // Accumulator coordinates of lane `lane` in wave (wm, wn): element r of acc[i][j] is
-//   row = wm*128 + i*32 + (r/4)*8 + (lane/32)*4 + r%4 ,  col = wn*128 + j*32 + lane%32   (tile-relative)
+//   row = wm*MI*32 + i*32 + (r/4)*8 + (lane/32)*4 + r%4 ,  col = wn*NJ*32 + j*32 + lane%32   (tile-relative)
 __device__ __forceinline__ int acc_row(int wm, int i, int r, int lane) {
-  return wm * 128 + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+  return wm * (MI * 32) + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
 }
-__device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * 128 + j * 32 + (lane & 31); }
+__device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (NJ * 32) + j * 32 + (lane & 31); }
 
 template <class Epi>
-__global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(GemmArgs g, Epi epi) {
+__global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int wm = w >> 1, wn = w & 1;
+  const int wm = w / WN, wn = w % WN;
   const TileCoord tc = tile_of(g, blockIdx.x);
+  if (!tc.valid) return;
   const int m0 = tc.tm * BM, n0 = tc.tn * BN;
 
   // global -> LDS mapping: 16-byte chunk c of rows r0 + 32 j.  Rows past the matrix edge are clamped to the
@@ -71,10 +90,10 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(GemmArgs g, Epi ep
   const int c = tid & 7, r0 = tid >> 3;
   const uint16_t* baseA = g.A + (int64_t)m0 * g.lda + c * 8;
   const uint16_t* baseB = g.B + (int64_t)n0 * g.ldb + c * 8;
-  int offA[8], offB[8];
+  int offA[kLoadsPerThread], offB[kLoadsPerThread];
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    int ra = r0 + 32 * j, rb = r0 + 32 * j;
+  for (int j = 0; j < kLoadsPerThread; ++j) {
+    int ra = r0 + kLoadRowStep * j, rb = r0 + kLoadRowStep * j;
     ra = (m0 + ra < g.M) ? ra : g.M - 1 - m0;
     rb = (n0 + rb < g.N) ? rb : g.N - 1 - n0;
     offA[j] = ra * (int)g.lda;
@@ -82,27 +101,27 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(GemmArgs g, Epi ep
   }
   const int lds_w = r0 * kRowBytes + c * 16;
 
-  floatx16 acc[4][4];
+  floatx16 acc[MI][NJ];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  u32x4 ga[8], gb[8];
+  u32x4 ga[kLoadsPerThread], gb[kLoadsPerThread];
   auto gload = [&](int kt) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int j = 0; j < kLoadsPerThread; ++j) {
       ga[j] = *reinterpret_cast<const u32x4*>(baseA + kt * BK + offA[j]);
       gb[j] = *reinterpret_cast<const u32x4*>(baseB + kt * BK + offB[j]);
     }
   };
   auto swrite = [&](char* st) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      *reinterpret_cast<u32x4*>(st + lds_w + 32 * j * kRowBytes) = ga[j];
-      *reinterpret_cast<u32x4*>(st + kTileBytes + lds_w + 32 * j * kRowBytes) = gb[j];
+    for (int j = 0; j < kLoadsPerThread; ++j) {
+      *reinterpret_cast<u32x4*>(st + lds_w + kLoadRowStep * j * kRowBytes) = ga[j];
+      *reinterpret_cast<u32x4*>(st + kTileBytes + lds_w + kLoadRowStep * j * kRowBytes) = gb[j];
     }
   };
 
@@ -111,8 +130,8 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(GemmArgs g, Epi ep
   swrite(smem);
   __syncthreads();
 
-  const int frag_a = (wm * 128 + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
-  const int frag_b = kTileBytes + (wn * 128 + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
+  const int frag_a = (wm * (MI * 32) + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
+  const int frag_b = kTileBytes + (wn * (NJ * 32) + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
 
   for (int kt = 0; kt < KT; ++kt) {
     char* cur = smem + (kt & 1) * kStageBytes;
@@ -120,84 +139,95 @@ __global__ __launch_bounds__(kThreads, 1) void gemm_nt_kernel(GemmArgs g, Epi ep
     if (more) gload(kt + 1);
 #pragma unroll
     for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 af[4], bfr[4];
+      bf16x8 af[MI], bfr[NJ];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < MI; ++i)
         af[i] = *reinterpret_cast<const bf16x8*>(cur + frag_a + i * 32 * kRowBytes + kk * 32);
-        bfr[i] = *reinterpret_cast<const bf16x8*>(cur + frag_b + i * 32 * kRowBytes + kk * 32);
-      }
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int j = 0; j < NJ; ++j)
+        bfr[j] = *reinterpret_cast<const bf16x8*>(cur + frag_b + j * 32 * kRowBytes + kk * 32);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
     }
     if (more) swrite(smem + ((kt + 1) & 1) * kStageBytes);
     __syncthreads();
   }
-  epi(acc, m0, n0, tc.tn, wm, wn, lane, tid, smem);
+  epi(acc, m0, n0, tc.tm, wm, wn, lane, tid, smem);
 }
 
 // ------------------------------------------------------------------------------ epilogue: softmax partials
 
-// Per row of the tile: mx = max_v z, s = sum exp(z - mx), t = sum z * exp(z - mx) over the tile's 256 columns,
-// z = acc * inv_T.  Row reductions run across the 32 lanes that share a row; the two column halves of the
-// workgroup are merged through LDS and one (mx, s, t) per row is written to part[tn][row].
+// The two fused GEMMs run "transposed": M is the vocabulary (A = W), N the tokens (B = hidden).  In the MFMA
+// accumulator layout a lane then owns one token (column) and its registers run over vocabulary rows, so the
+// softmax reductions over the vocabulary are in-register, followed by one exchange between the two lane halves
+// and a merge of the WM waves through LDS -- no 32-lane butterfly per row.
+//
+// Per token of the tile: mx = max_v z, s = sum exp(z - mx), t = sum z * exp(z - mx) over the tile's 256
+// vocabulary rows, z = acc * inv_T; one (mx, s, t) per token is written to part[tm][.][token].
 struct SoftmaxPartialsEpi {
   float inv_T;
   int T, V;
-  float* part;  // [tiles_n][3][T]
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
-                             char* smem) const {
-    float* sh = reinterpret_cast<float*>(smem);  // [2][256][3]; the main loop's last barrier freed the LDS
+  float* part;  // [tiles_m][3][T]
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn,
+                                             int lane, int tid, char* smem) const {
+    float* sh = reinterpret_cast<float*>(smem);  // [WM][BN][3]; the main loop's last barrier freed the LDS
     const float k = kLog2e;
+    const float ninf = -__builtin_inff();
+    const bool full = m0 + BM <= V;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int j = 0; j < NJ; ++j) {
+      float mx = ninf;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float x[4];
-        float mx = -__builtin_inff();
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const bool ok = n0 + acc_col(wn, j, lane) < V;
-          x[j] = ok ? acc[i][j][r] * inv_T : -__builtin_inff();
-          mx = fmaxf(mx, x[j]);
+        for (int r = 0; r < 16; ++r) {
+          const bool ok = full || (m0 + acc_row(wm, i, r, lane) < V);
+          mx = fmaxf(mx, ok ? acc[i][j][r] * inv_T : ninf);
         }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      float s = 0.f, t = 0.f;
+      if (mx > ninf) {
+        const float nmk = -mx * k;
 #pragma unroll
-        for (int o = 16; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
-        float s = 0.f, t = 0.f;
-        if (mx > -__builtin_inff()) {
+        for (int i = 0; i < MI; ++i)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float e = fast_exp2((x[j] - mx) * k);  // 0 for masked columns
+          for (int r = 0; r < 16; ++r) {
+            const bool ok = full || (m0 + acc_row(wm, i, r, lane) < V);
+            const float x = acc[i][j][r] * inv_T;
+            const float e = ok ? fast_exp2(fmaf(x, k, nmk)) : 0.f;
             s += e;
-            t += (x[j] > -__builtin_inff()) ? x[j] * e : 0.f;
+            t = fmaf(ok ? x : 0.f, e, t);
           }
-        }
-#pragma unroll
-        for (int o = 16; o > 0; o >>= 1) {
-          s += __shfl_xor(s, o, kWave);
-          t += __shfl_xor(t, o, kWave);
-        }
-        if ((lane & 31) == 0) {
-          float* d = sh + (wn * BM + acc_row(wm, i, r, lane)) * 3;
-          d[0] = mx;
-          d[1] = s;
-          d[2] = t;
-        }
+      }
+      s += __shfl_xor(s, 32, kWave);
+      t += __shfl_xor(t, 32, kWave);
+      if (lane < 32) {
+        float* d = sh + (wm * BN + acc_col(wn, j, lane)) * 3;
+        d[0] = mx;
+        d[1] = s;
+        d[2] = t;
       }
     }
     __syncthreads();
-    const int row = m0 + tid;
-    if (row < T) {
-      const float* a = sh + tid * 3;
-      const float* b = sh + (BM + tid) * 3;
-      const float M = fmaxf(a[0], b[0]);
-      const float fa = a[0] > -__builtin_inff() ? fast_exp2((a[0] - M) * k) : 0.f;
-      const float fb = b[0] > -__builtin_inff() ? fast_exp2((b[0] - M) * k) : 0.f;
-      float* o = part + (int64_t)tn * 3 * T;
-      o[row] = M;
-      o[(int64_t)T + row] = a[1] * fa + b[1] * fb;
-      o[2 * (int64_t)T + row] = a[2] * fa + b[2] * fb;
+    const int tok = n0 + tid;
+    if (tid < BN && tok < T) {
+      float M = ninf;
+#pragma unroll
+      for (int q = 0; q < WM; ++q) M = fmaxf(M, sh[(q * BN + tid) * 3]);
+      float ss = 0.f, tt = 0.f;
+#pragma unroll
+      for (int q = 0; q < WM; ++q) {
+        const float* a = sh + (q * BN + tid) * 3;
+        const float f = a[0] > ninf ? fast_exp2((a[0] - M) * k) : 0.f;
+        ss += a[1] * f;
+        tt += a[2] * f;
+      }
+      float* o = part + (int64_t)tm * 3 * T;
+      o[tok] = M;
+      o[(int64_t)T + tok] = ss;
+      o[2 * (int64_t)T + tok] = tt;
     }
   }
 };
@@ -205,11 +235,12 @@ struct SoftmaxPartialsEpi {
 // ------------------------------------------------------------------------------ epilogue: dlogits
 
 // d raw_logit = inv_T * ( g_lp * (1[v == y] - p) - g_h * p * (z - ex) ),  p = exp(z - lse), z = acc * inv_T,
-// written as bf16 to D[row][col] (ld = ldd) and to Dt[col][row] (ld = ldt); col is slab-relative.  Columns in
-// [N, Npad) are written as zeros: they are K-padding of the GEMMs that consume the buffers.
+// written as bf16 to D[token][v] (ld = ldd) and to Dt[v][token] (ld = ldt); v is slab-relative and is the M
+// dimension of this GEMM.  Rows v in [Vs, Vpad) are written as zeros: they are K-padding of the GEMM that
+// consumes D.  A lane owns one token, so the per-token coefficients are loaded once per lane.
 struct DlogitsEpi {
   float inv_T;
-  int T, N, Npad;
+  int T, Vs, Vpad;
   int64_t v0;  // first vocabulary column of the slab
   const float* lse;
   const float* ex;
@@ -220,36 +251,43 @@ struct DlogitsEpi {
   int64_t ldd;
   uint16_t* Dt;
   int64_t ldt;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
-                             char* smem) const {
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn,
+                                             int lane, int tid, char* smem) const {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int j = 0; j < NJ; ++j) {
+      const int tok = n0 + acc_col(wn, j, lane);
+      if (tok >= T) continue;
+      const float g1 = g_lp ? g_lp[tok] : 0.f;
+      const float g2 = g_h ? g_h[tok] : 0.f;
+      const float nl = -lse[tok] * kLog2e;
+      const float exv = g_h ? ex[tok] : 0.f;
+      const int y = g_lp ? (int)((labels[tok] - v0 >= 0 && labels[tok] - v0 < Vs) ? labels[tok] - v0 : -1) : -1;
+      uint16_t* drow = D + (int64_t)tok * ldd;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = m0 + acc_row(wm, i, r, lane);
-        if (row >= T) continue;
-        const float g1 = g_lp ? g_lp[row] : 0.f;
-        const float g2 = g_h ? g_h[row] : 0.f;
-        const float nl = -lse[row] * kLog2e;
-        const float exv = g_h ? ex[row] : 0.f;
-        const int64_t y = g_lp ? labels[row] - v0 : -1;
+      for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int col = n0 + acc_col(wn, j, lane);
-          if (col >= Npad) continue;
-          float d = 0.f;
-          if (col < N) {
-            const float z = acc[i][j][r] * inv_T;
-            const float p = fast_exp2(fmaf(z, kLog2e, nl));
-            d = p * (-g1 - g2 * (z - exv));
-            if ((int64_t)col == y) d += g1;
-            d *= inv_T;
+        for (int q = 0; q < 4; ++q) {
+          const int v = m0 + acc_row(wm, i, q * 4, lane);  // 4 consecutive vocabulary rows v .. v+3
+          if (v >= Vpad) continue;
+          float d[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            d[e] = 0.f;
+            if (v + e < Vs) {
+              const float z = acc[i][j][q * 4 + e] * inv_T;
+              const float p = fast_exp2(fmaf(z, kLog2e, nl));
+              float g = p * (-g1 - g2 * (z - exv));
+              if (v + e == y) g += g1;
+              d[e] = g * inv_T;
+            }
           }
-          const uint16_t h = (uint16_t)(pack_bf16(d, 0.f) & 0xffffu);
-          D[(int64_t)row * ldd + col] = h;
-          Dt[(int64_t)col * ldt + row] = h;
+          const uint32_t lo = pack_bf16(d[0], d[1]), hi = pack_bf16(d[2], d[3]);
+          *reinterpret_cast<uint2*>(drow + v) = make_uint2(lo, hi);  // v % 4 == 0, ldd % 4 == 0: 8-byte aligned
+          Dt[(int64_t)(v + 0) * ldt + tok] = (uint16_t)(lo & 0xffffu);
+          Dt[(int64_t)(v + 1) * ldt + tok] = (uint16_t)(lo >> 16);
+          Dt[(int64_t)(v + 2) * ldt + tok] = (uint16_t)(hi & 0xffffu);
+          Dt[(int64_t)(v + 3) * ldt + tok] = (uint16_t)(hi >> 16);
         }
-      }
     }
   }
 };
@@ -260,16 +298,16 @@ struct AccumF32Epi {  // C[row][col] = (beta ? C : 0) + acc
   float* C;
   int64_t ldc;
   int M, N, beta;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn, int lane, int tid,
                              char* smem) const {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + acc_row(wm, i, r, lane);
         if (row >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
           const int col = n0 + acc_col(wn, j, lane);
           if (col >= N) continue;
           float* p = C + (int64_t)row * ldc + col;
@@ -283,16 +321,16 @@ struct StoreBf16Epi {  // C[row][col] = bf16(acc)
   uint16_t* C;
   int64_t ldc;
   int M, N;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[4][4], int m0, int n0, int tn, int wm, int wn, int lane, int tid,
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn, int lane, int tid,
                              char* smem) const {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int row = m0 + acc_row(wm, i, r, lane);
         if (row >= M) continue;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NJ; ++j) {
           const int col = n0 + acc_col(wn, j, lane);
           if (col >= N) continue;
           C[(int64_t)row * ldc + col] = (uint16_t)(pack_bf16(acc[i][j][r], 0.f) & 0xffffu);
@@ -395,7 +433,7 @@ int launch_gemm(const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, 
     attr_set = true;
   }
   GemmArgs g{A, lda, B, ldb, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN};
-  const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+  const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n);
   gemm_nt_kernel<Epi><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
   SIIRL_LAUNCH_CHECK(what);
   return SIIRL_OK;
@@ -422,9 +460,9 @@ struct FwdWs {
 };
 FwdWs fwd_ws(int64_t T, int64_t V) {
   FwdWs w;
-  const int64_t tiles_n = (V + BN - 1) / BN;
+  const int64_t tiles_v = (V + BM - 1) / BM;
   w.part = 0;
-  w.label = round_up((size_t)tiles_n * 3 * T * 4, 256);
+  w.label = round_up((size_t)tiles_v * 3 * T * 4, 256);
   w.total = w.label + round_up((size_t)T * 4, 256);
   return w;
 }
@@ -487,9 +525,9 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
     SIIRL_LAUNCH_CHECK("label_logit_kernel");
   }
   SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part};
-  if (int rc = launch_gemm(h, H, w, H, (int)T, (int)V, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
-  const int tiles_n = (int)((V + BN - 1) / BN);
-  merge_partials_kernel<<<dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st>>>(part, tiles_n, (int)T, label_logit,
+  if (int rc = launch_gemm(w, H, h, H, (int)V, (int)T, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
+  const int tiles_v = (int)((V + BM - 1) / BM);
+  merge_partials_kernel<<<dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
                                                                                logprob, entropy, lse, ex);
   SIIRL_LAUNCH_CHECK("merge_partials_kernel");
   return SIIRL_OK;
@@ -540,7 +578,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
     const int N = (int)((V - v0) < kSlab ? (V - v0) : kSlab);
     const int Npad = (int)round_up(N, BK);
     DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels, D, kSlab, Dt, ws.ldt};
-    if (int rc = launch_gemm(h, H, w + v0 * H, H, (int)T, N, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
+    if (int rc = launch_gemm(w + v0 * H, H, h, H, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
     if (want_dh) {  // dH[T, H] += D[T, Npad] . Wt[H, v0 : v0 + Npad]^T
       AccumF32Epi acc{dH32, H, (int)T, (int)H, slab_idx > 0 ? 1 : 0};
       if (int rc = launch_gemm(D, kSlab, Wt + v0, ws.ldwt, (int)T, (int)H, Npad, acc, st, "gemm_nt_kernel<AccumF32Epi>"))

@@ -386,27 +386,49 @@ __global__ __launch_bounds__(256) void label_logit_kernel(const uint16_t* __rest
   if (lane == 0) out[row] = s * inv_T;
 }
 
-// folds the per-tile partials of each row: lse, ex, entropy, logprob
+// folds the per-tile partials of each token: lse, ex, entropy, logprob.  A workgroup handles 64 tokens; four
+// thread groups each merge every fourth tile online, then the four states are merged through LDS.
 __global__ __launch_bounds__(256) void merge_partials_kernel(const float* __restrict__ part, int nparts, int T,
                                                              const float* __restrict__ label_logit,
                                                              float* __restrict__ logprob, float* __restrict__ entropy,
                                                              float* __restrict__ lse_out, float* __restrict__ ex_out) {
-  const int row = blockIdx.x * 256 + threadIdx.x;
-  if (row >= T) return;
-  float M = -__builtin_inff();
-  for (int p = 0; p < nparts; ++p) M = fmaxf(M, part[(int64_t)p * 3 * T + row]);
-  double s = 0.0, t = 0.0;
-  for (int p = 0; p < nparts; ++p) {
-    const float* q = part + (int64_t)p * 3 * T;
-    const float m = q[row];
-    if (m > -__builtin_inff()) {
-      const float f = fast_exp2((m - M) * kLog2e);
-      s += (double)(q[(int64_t)T + row] * f);
-      t += (double)(q[2 * (int64_t)T + row] * f);
+  __shared__ float sh[4][64][3];
+  const int tl = threadIdx.x & 63, grp = threadIdx.x >> 6;
+  const int row = blockIdx.x * 64 + tl;
+  float M = -__builtin_inff(), s = 0.f, t = 0.f;
+  if (row < T) {
+    for (int p = grp; p < nparts; p += 4) {
+      const float* q = part + (int64_t)p * 3 * T;
+      const float m = q[row];
+      if (m > -__builtin_inff()) {
+        const float Mn = fmaxf(M, m);
+        const float fo = fast_exp2((M - Mn) * kLog2e), fn = fast_exp2((m - Mn) * kLog2e);
+        s = s * fo + q[(int64_t)T + row] * fn;
+        t = t * fo + q[2 * (int64_t)T + row] * fn;
+        M = Mn;
+      }
     }
   }
-  const float lse = M + logf((float)s);
-  const float exv = (float)(t / s);
+  sh[grp][tl][0] = M;
+  sh[grp][tl][1] = s;
+  sh[grp][tl][2] = t;
+  __syncthreads();
+  if (grp != 0 || row >= T) return;
+  float Mx = M;
+#pragma unroll
+  for (int g = 1; g < 4; ++g) Mx = fmaxf(Mx, sh[g][tl][0]);
+  double ss = 0.0, tt = 0.0;
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const float m = sh[g][tl][0];
+    if (m > -__builtin_inff()) {
+      const float f = fast_exp2((m - Mx) * kLog2e);
+      ss += (double)(sh[g][tl][1] * f);
+      tt += (double)(sh[g][tl][2] * f);
+    }
+  }
+  const float lse = Mx + logf((float)ss);
+  const float exv = (float)(tt / ss);
   lse_out[row] = lse;
   if (ex_out) ex_out[row] = exv;
   if (entropy) entropy[row] = lse - exv;
@@ -527,7 +549,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part};
   if (int rc = launch_gemm(w, H, h, H, (int)V, (int)T, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
   const int tiles_v = (int)((V + BM - 1) / BM);
-  merge_partials_kernel<<<dim3((unsigned)((T + 255) / 256)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
+  merge_partials_kernel<<<dim3((unsigned)((T + 63) / 64)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
                                                                                logprob, entropy, lse, ex);
   SIIRL_LAUNCH_CHECK("merge_partials_kernel");
   return SIIRL_OK;

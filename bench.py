@@ -87,6 +87,67 @@ def cpu_baseline(logits, labels, g_lp, g_ent, rows=4096, iters=5):
                       f"median of {iters} fwd+bwd passes ({med:.2f} s each)"}
 
 
+def bench_config5(args, dev):
+    """Fused lm_head + log-prob/entropy (MFMA path): hidden [16384, 3584] ~ N(0,1), W [152064, 3584] ~ N(0, 0.02),
+    bf16, uniform labels, forward + backward to hidden and W.  Not the headline; same JSON shape."""
+    import torch
+
+    from siirl_amd.fused_linear import fused_linear_logprob_entropy
+
+    T, H, V = 16384, 3584, 152064
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    h = torch.randn(T, H, device=dev, generator=gen).to(torch.bfloat16).requires_grad_(True)
+    w = torch.empty(V, H, dtype=torch.bfloat16, device=dev)
+    for lo in range(0, V, 16384):
+        n = min(16384, V - lo)
+        w[lo:lo + n] = (torch.randn(n, H, device=dev, generator=gen) * 0.02).to(torch.bfloat16)
+    w.requires_grad_(True)
+    y = torch.randint(0, V, (T,), device=dev, generator=gen)
+    g_lp = torch.randn(T, device=dev, generator=gen) * 1e-2
+    g_h = torch.randn(T, device=dev, generator=gen) * 1e-2
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        lp, ent = fused_linear_logprob_entropy(h, w, y)
+        if ev:
+            ev[1].record()
+        torch.autograd.backward([lp, ent], [g_lp, g_h])
+        if ev:
+            ev[2].record()
+        h.grad = w.grad = None
+
+    steps, warm = min(args.steps, 10), min(args.warmup, 2)
+    for _ in range(warm):
+        step()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for k in range(steps):
+        step(evs[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    gemm = 2.0 * T * H * V
+    tf_step = 3 * gemm / (wall / steps) / 1e12
+    out = {
+        "metric": "fused lm_head+logprob/entropy fwd+bwd tokens/sec @vocab152k bf16; % MFMA roofline",
+        "value": T * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": wall * 1e3 / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config5: fused lm_head + logprob/entropy, hidden [{T}, {H}], W [{V}, {H}], fwd + bwd to "
+                               "hidden and W", "tokens": T, "hidden": H, "vocab": V, "seed": SEED},
+        "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
+                    "backward (3 x gemm_nt_kernel per 8192-column slab)": {"ms": bwd_ms, "TFLOP/s executed": 3 * gemm / bwd_ms / 1e9}},
+        "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel", "achieved": tf_step, "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": tf_step / 2500.0, "traffic": None,
+                     "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step; the backward's recompute is not counted"},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -97,6 +158,8 @@ def main():
                     help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 2 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--workload", default="config2", choices=["config2", "config5"],
+                    help="config2 (default): the headline logprob+entropy fwd+bwd; config5: fused lm_head variant")
     ap.add_argument("--seqs", type=int, default=SEQS, help="sequences of 4096 tokens (8 = the baseline's config)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -113,6 +176,8 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "config5":
+        return bench_config5(args, dev)
     SF.set_skip_zero_rows(False)  # dense: every row is read and written, as the algorithmic byte count assumes
 
     logits, labels, g_lp, g_ent, mask = make_workload(dev, seqs=args.seqs)

@@ -6,8 +6,7 @@
 // Groups are defined by equal uid; uids are arbitrary int64 and need not be contiguous.  Each thread owns
 // one trajectory i and scans all trajectories j in batch order through LDS tiles, picking those with
 // uid[j] == uid[i]: O(B^2) compares, exact integer bookkeeping, no atomics, and every group statistic is
-// accumulated in the batch order the reference uses.  B is a rollout batch (10^3..10^5): at 8192 rows a
-// scan costs ~30 us.
+// accumulated in the batch order the reference uses.  B is a rollout batch (10^3..10^5).
 //
 // The keep mask reproduces np.std(values) > 0 bit for bit: numpy sums with an 8-accumulator pairwise
 // scheme in the dtype of the values, so e.g. three equal fp64 values 0.1 have std 1.4e-17 > 0.  This
@@ -17,7 +16,8 @@
 namespace siirl {
 namespace {
 
-constexpr int kThreads = 256;
+constexpr int kThreads = 256;   // streaming kernels (row sums, broadcast)
+constexpr int kGroupThreads = 64;  // all-pairs kernels: one wave per workgroup, so B = 8192 already fills 128 CUs
 constexpr int kTile = 1024;
 
 // ---------------------------------------------------------------------------- row sums
@@ -37,19 +37,19 @@ __global__ __launch_bounds__(kThreads) void row_sum_kernel(const float* __restri
 // ---------------------------------------------------------------------------- GRPO advantage
 
 // a[i] = (s_i - mean_g) / (std_g + eps), unbiased std; a group of one uses mean 0, std 1.
-__global__ __launch_bounds__(kThreads) void grpo_group_kernel(const float* __restrict__ scores,
+__global__ __launch_bounds__(kGroupThreads) void grpo_group_kernel(const float* __restrict__ scores,
                                                               const int64_t* __restrict__ uid, int64_t B, float eps,
                                                               int norm_by_std, float* __restrict__ a_out) {
   __shared__ int64_t s_uid[kTile];
   __shared__ float s_val[kTile];
-  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t i = (int64_t)blockIdx.x * kGroupThreads + threadIdx.x;
   const bool live = i < B;
   const int64_t my = live ? uid[i] : 0;
   int n = 0;
   double sum = 0.0;
   for (int64_t base = 0; base < B; base += kTile) {
     __syncthreads();
-    for (int k = threadIdx.x; k < kTile; k += kThreads) {
+    for (int k = threadIdx.x; k < kTile; k += kGroupThreads) {
       const int64_t j = base + k;
       s_uid[k] = j < B ? uid[j] : 0;
       s_val[k] = j < B ? scores[j] : 0.f;
@@ -67,7 +67,7 @@ __global__ __launch_bounds__(kThreads) void grpo_group_kernel(const float* __res
   double ss = 0.0;
   for (int64_t base = 0; base < B; base += kTile) {
     __syncthreads();
-    for (int k = threadIdx.x; k < kTile; k += kThreads) {
+    for (int k = threadIdx.x; k < kTile; k += kGroupThreads) {
       const int64_t j = base + k;
       s_uid[k] = j < B ? uid[j] : 0;
       s_val[k] = j < B ? scores[j] : 0.f;
@@ -198,17 +198,17 @@ __device__ T np_pairwise(MemberCursor<T>& cur, int n, T mean) {
 
 // keep[i] = group of i has one member, or np.std(group values) > 0
 template <typename T>
-__global__ __launch_bounds__(kThreads) void keep_mask_kernel(const T* __restrict__ val, const int64_t* __restrict__ uid,
+__global__ __launch_bounds__(kGroupThreads) void keep_mask_kernel(const T* __restrict__ val, const int64_t* __restrict__ uid,
                                                              int64_t B, uint8_t* __restrict__ keep,
                                                              int32_t* __restrict__ group_size) {
   __shared__ int64_t s_uid[kTile];
   __shared__ T s_val[kTile];
-  const int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t i = (int64_t)blockIdx.x * kGroupThreads + threadIdx.x;
   const bool live = i < B;
   const int64_t my = live ? uid[i] : 0;
   auto stage = [&](int64_t base) {
     __syncthreads();
-    for (int k = threadIdx.x; k < kTile; k += kThreads) {
+    for (int k = threadIdx.x; k < kTile; k += kGroupThreads) {
       const int64_t j = base + k;
       s_uid[k] = j < B ? uid[j] : 0;
       s_val[k] = j < B ? val[j] : T(0);
@@ -278,7 +278,7 @@ extern "C" int siirl_grpo_outcome_advantage(const float* token_level_rewards, co
   float* a = scratch_2B + B;
   row_sum_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(token_level_rewards, L, scores);
   SIIRL_LAUNCH_CHECK("row_sum_kernel");
-  grpo_group_kernel<<<dim3((unsigned)((B + kThreads - 1) / kThreads)), dim3(kThreads), 0, st>>>(
+  grpo_group_kernel<<<dim3((unsigned)((B + kGroupThreads - 1) / kGroupThreads)), dim3(kGroupThreads), 0, st>>>(
       scores, uid, B, epsilon, norm_adv_by_std, a);
   SIIRL_LAUNCH_CHECK("grpo_group_kernel");
   const int64_t n = B * L;
@@ -296,7 +296,7 @@ extern "C" int siirl_group_keep_mask(const void* metric, int metric_dtype, const
   SIIRL_REQUIRE(metric_dtype == SIIRL_F32 || metric_dtype == SIIRL_F64, "metric dtype %d not supported (f32, f64)",
                 metric_dtype);
   hipStream_t st = (hipStream_t)stream;
-  const dim3 grid((unsigned)((B + kThreads - 1) / kThreads)), block(kThreads);
+  const dim3 grid((unsigned)((B + kGroupThreads - 1) / kGroupThreads)), block(kGroupThreads);
   if (metric_dtype == SIIRL_F32)
     keep_mask_kernel<float><<<grid, block, 0, st>>>((const float*)metric, uid, B, keep, group_size);
   else

@@ -5,14 +5,21 @@
 // (siirl/utils/kernel/linear_cross_entropy.py:40-117 -> siirl/utils/kernel/kernels.py:507-696,1378-1586); the
 // per-tile online-softmax state (max, sum exp, sum x*exp) is the one of kernels.py:254-266,343-350.
 //
-// One GEMM core, C[M,N] = A[M,K] . B[N,K]^T with both operands K-major bf16 and fp32 accumulation:
-//   256 x 256 x 64 workgroup tile, 4 waves of 128 x 128 (4 x 4 MFMA 32x32x16 bf16 tiles, 256 accumulator
-//   registers), double-buffered LDS (rows padded to 144 B so that ds_read_b128 fragments are conflict-free),
-//   global loads of the next K-step issued before the MFMAs of the current one.
+// One GEMM core, C[M,N] = A[M,K] . B[N,K]^T, bf16 operands, fp32 accumulation, 256 x 256 x 64 workgroup tile,
+// 8 waves (2 x 4) of 128 x 64 (4 x 2 MFMA 32x32x16 bf16 tiles, 128 accumulator registers each):
+//   * A (K-major rows) goes global -> LDS by DMA (global_load_lds_dwordx4, no staging registers, no ds_write)
+//     into a ring of four 32 KB stages.  Rows are unpadded; 16-byte chunks are XOR-swizzled by (row / 2) % 8 so
+//     that the ds_read_b128 fragment reads are conflict-free.  A stage is issued three K-steps before it is read
+//     and published (barrier) one step before, so the first fragments of the next step are read ahead of the
+//     barrier and the matrix cores do not drain at it.
+//   * B never touches the LDS: it is prepared once per call in the MFMA operand's lane order ("fragment-packed")
+//     and each lane loads its 16-byte operands straight into registers, one K-step ahead.
+//   * all loads of the main loop are inline asm with hand-placed s_waitcnt vmcnt: the compiler's own tracking
+//     would wait for every outstanding DMA before each LDS read.
 // Four epilogues: softmax partials (forward), dlogits in both layouts (backward), fp32 accumulate (d hidden),
 // bf16 store (d weight).  The backward walks the vocabulary in slabs: recompute the slab's logits, write
 // dlogits[T, slab] and its transpose, then dH += dlogits . W_slab and dW_slab = dlogits^T . hidden as two more
-// runs of the same core against transposed copies of W and hidden.
+// runs of the same core against packed transposed copies of W and hidden.
 #include "common.hpp"
 
 namespace siirl {
@@ -30,18 +37,22 @@ constexpr int kThreads = WM * WN * 64;
 constexpr int MI = BM / (WM * 32), NJ = BN / (WN * 32);  // 32x32 MFMA tiles per wave
 constexpr int kLoadsPerThread = (BM * BK / 8) / kThreads;  // 16-byte chunks per operand tile per thread
 constexpr int kLoadRowStep = kThreads / 8;
-constexpr int kRowBytes = BK * 2 + 16;        // 128 B of data + 16 B pad
-constexpr int kTileBytes = BM * kRowBytes;    // 36864
-constexpr int kStageBytes = 2 * kTileBytes;   // A tile + B tile
-constexpr int kSmemBytes = 2 * kStageBytes;   // 147456 of the 160 KB
+constexpr int kRowBytes = BK * 2;             // unpadded rows, 16-byte chunks XOR-swizzled by (row / 2) % 8
+constexpr int kTileBytes = BM * kRowBytes;    // 32768
+constexpr int kStageBytes = kTileBytes;       // A tile only: B goes global -> registers
+constexpr int kStages = 4;
+constexpr int kSmemBytes = kStages * kStageBytes;  // 131072
+constexpr int kDmaPerWave = kTileBytes / 1024 / (kThreads / 64);  // 1 KB per wave instruction
 constexpr int kSlab = 8192;                   // vocabulary columns per backward slab
+constexpr int kLdPad = 64;                    // extra elements per row of D / Dt: keeps a tile's 256 rows off a
+                                              // power-of-two stride, which would put them all in one memory channel
 
 struct GemmArgs {
   const uint16_t* A;
   int64_t lda;
-  const uint16_t* B;
-  int64_t ldb;
-  int M, N, K;  // K is a multiple of BK; rows beyond M / N are clamped on load and masked by the epilogue
+  const u32x4* Bp;  // fragment-packed B (see pack layout), already offset to the first K block of this GEMM
+  int64_t kb_total; // 16-wide K blocks per 32-row block of the packed buffer
+  int M, N, K;  // K is a multiple of BK; rows beyond M are clamped on load and masked by the epilogue
   int tiles_m, tiles_n;
 };
 
@@ -76,6 +87,9 @@ __device__ __forceinline__ int acc_row(int wm, int i, int r, int lane) {
 }
 __device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (NJ * 32) + j * 32 + (lane & 31); }
 
+// m0 (the DMA's LDS base) is a reserved register: naming it in a clobber list is right but draws a warning
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
 template <class Epi>
 __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) {
   extern __shared__ __align__(16) char smem[];
@@ -84,22 +98,28 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
   const TileCoord tc = tile_of(g, blockIdx.x);
   if (!tc.valid) return;
   const int m0 = tc.tm * BM, n0 = tc.tn * BN;
+  const int KT = g.K / BK;
 
-  // global -> LDS mapping: 16-byte chunk c of rows r0 + 32 j.  Rows past the matrix edge are clamped to the
-  // last row; offsets are relative to the tile's first row so that they fit 32 bits.
-  const int c = tid & 7, r0 = tid >> 3;
-  const uint16_t* baseA = g.A + (int64_t)m0 * g.lda + c * 8;
-  const uint16_t* baseB = g.B + (int64_t)n0 * g.ldb + c * 8;
-  int offA[kLoadsPerThread], offB[kLoadsPerThread];
+  // A: global -> LDS by DMA (global_load_lds_dwordx4): wave instruction I = w * kDmaPerWave + i fills the 1 KB
+  // [I * 1024, I * 1024 + 1024) of the stage; 16-byte slot sl = I * 64 + lane holds row sl / 8, chunk
+  // (sl % 8) ^ ((row / 2) % 8).  Rows past the matrix edge are clamped to the last row.
+  const int wu = __builtin_amdgcn_readfirstlane(w);
+  const char* gA = reinterpret_cast<const char*>(g.A + (int64_t)m0 * g.lda);
+  uint32_t offA[kDmaPerWave];
 #pragma unroll
-  for (int j = 0; j < kLoadsPerThread; ++j) {
-    int ra = r0 + kLoadRowStep * j, rb = r0 + kLoadRowStep * j;
-    ra = (m0 + ra < g.M) ? ra : g.M - 1 - m0;
-    rb = (n0 + rb < g.N) ? rb : g.N - 1 - n0;
-    offA[j] = ra * (int)g.lda;
-    offB[j] = rb * (int)g.ldb;
+  for (int i = 0; i < kDmaPerWave; ++i) {
+    const int sl = (wu * kDmaPerWave + i) * 64 + lane;
+    int row = sl >> 3;
+    const int ch = (sl & 7) ^ ((row >> 1) & 7);
+    row = (m0 + row < g.M) ? row : g.M - 1 - m0;
+    offA[i] = (uint32_t)row * (uint32_t)g.lda * 2u + ch * 16;
   }
-  const int lds_w = r0 * kRowBytes + c * 16;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
+  // B: fragment-packed, one 16-byte load per lane per MFMA operand, no LDS
+  const char* gB = reinterpret_cast<const char*>(g.Bp + (int64_t)(n0 >> 5) * g.kb_total * 64);
+  uint32_t offB[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) offB[j] = (uint32_t)(((wn * NJ + j) * g.kb_total * 64 + lane) * 16);
 
   floatx16 acc[MI][NJ];
 #pragma unroll
@@ -109,53 +129,92 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  u32x4 ga[kLoadsPerThread], gb[kLoadsPerThread];
-  auto gload = [&](int kt) {
+  u32x4 b0[NJ][BK / 16], b1[NJ][BK / 16];
+  auto dma = [&](int stage, int kt) {
+    const char* base = gA + (int64_t)kt * (BK * 2);
 #pragma unroll
-    for (int j = 0; j < kLoadsPerThread; ++j) {
-      ga[j] = *reinterpret_cast<const u32x4*>(baseA + kt * BK + offA[j]);
-      gb[j] = *reinterpret_cast<const u32x4*>(baseB + kt * BK + offB[j]);
+    for (int i = 0; i < kDmaPerWave; ++i) {
+      const uint32_t dst = lds0 + stage * kStageBytes + (wu * kDmaPerWave + i) * 1024;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(offA[i]), "s"(base) : "m0", "memory");
     }
   };
-  auto swrite = [&](char* st) {
+  auto bload = [&](u32x4 (&b)[NJ][BK / 16], int kt) {
+    const char* base = gB + (int64_t)kt * (BK / 16 * 1024);
 #pragma unroll
-    for (int j = 0; j < kLoadsPerThread; ++j) {
-      *reinterpret_cast<u32x4*>(st + lds_w + kLoadRowStep * j * kRowBytes) = ga[j];
-      *reinterpret_cast<u32x4*>(st + kTileBytes + lds_w + kLoadRowStep * j * kRowBytes) = gb[j];
+    for (int j = 0; j < NJ; ++j) {
+      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(b[j][0]) : "v"(offB[j]), "s"(base));
+      asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(b[j][1]) : "v"(offB[j]), "s"(base));
+      asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(b[j][2]) : "v"(offB[j]), "s"(base));
+      asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(b[j][3]) : "v"(offB[j]), "s"(base));
     }
   };
+  // waits until at most `n` of this wave's loads are in flight and ties the B registers to the wait
+#define SIIRL_BWAIT(n, b)                                                                                              \
+  asm volatile("s_waitcnt vmcnt(" #n ")"                                                                              \
+               : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[0][3]), "+v"(b[1][0]), "+v"(b[1][1]),            \
+                 "+v"(b[1][2]), "+v"(b[1][3])::"memory")
+  static_assert(NJ == 2 && BK == 64 && kDmaPerWave == 4, "the wait counts below assume 8 B loads and 4 DMA per step");
 
-  const int KT = g.K / BK;
-  gload(0);
-  swrite(smem);
+  bload(b0, 0);
+  dma(0, 0);
+  dma(1, KT > 1 ? 1 : 0);
+  dma(2, KT > 2 ? 2 : 0);
+  SIIRL_BWAIT(4, b0);
   __syncthreads();
 
-  const int frag_a = (wm * (MI * 32) + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
-  const int frag_b = kTileBytes + (wn * (NJ * 32) + (lane & 31)) * kRowBytes + (lane >> 5) * 16;
+  const int m31 = lane & 31, gsel = lane >> 5, sw = (m31 >> 1) & 7;
+  const int frag_row = (wm * (MI * 32) + m31) * kRowBytes;
+  int xk[BK / 16];
+#pragma unroll
+  for (int kk = 0; kk < BK / 16; ++kk) xk[kk] = frag_row + (((kk * 2 + gsel) ^ sw) << 4);
 
-  for (int kt = 0; kt < KT; ++kt) {
-    char* cur = smem + (kt & 1) * kStageBytes;
-    const bool more = kt + 1 < KT;
-    if (more) gload(kt + 1);
+  // step kt: stage kt % 4 is read; B(kt + 1) and DMA(kt + 3) are issued (K-steps past the end are clamped to the
+  // last one: they land in stages that are not read again); the barrier at the end publishes stage
+  // (kt + 2) % 4, whose DMA was issued one step earlier, and frees stage kt % 4 for DMA(kt + 4).
+  // A fragments are read one MFMA K-slice ahead; the slice after the last one of a step is the first of the next
+  // step, whose stage was published by the previous barrier, so the reads cross the barrier.
+  bf16x8 afa[MI], afb[MI];
+  auto fread = [&](bf16x8 (&af)[MI], int stage, int kk) {
+    const char* cur = smem + stage * kStageBytes;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8 af[MI], bfr[NJ];
+    for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + xk[kk] + i * 32 * kRowBytes);
+  };
+  auto mma = [&](bf16x8 (&af)[MI], u32x4 (&bc)[NJ][BK / 16], int kk) {
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
-        af[i] = *reinterpret_cast<const bf16x8*>(cur + frag_a + i * 32 * kRowBytes + kk * 32);
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j)
-        bfr[j] = *reinterpret_cast<const bf16x8*>(cur + frag_b + j * 32 * kRowBytes + kk * 32);
-#pragma unroll
-      for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-    }
-    if (more) swrite(smem + ((kt + 1) & 1) * kStageBytes);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], __builtin_bit_cast(bf16x8, bc[j][kk]), acc[i][j], 0, 0, 0);
+  };
+  fread(afa, 0, 0);
+  auto step = [&](int kt, u32x4 (&bc)[NJ][BK / 16], u32x4 (&bn)[NJ][BK / 16]) {
+    const int stage = kt & 3;
+    bload(bn, kt + 1 < KT ? kt + 1 : KT - 1);
+    dma((stage + 3) & 3, kt + 3 < KT ? kt + 3 : KT - 1);
+    fread(afb, stage, 1);
+    mma(afa, bc, 0);
+    fread(afa, stage, 2);
+    mma(afb, bc, 1);
+    fread(afb, stage, 3);
+    mma(afa, bc, 2);
+    fread(afa, (stage + 1) & 3, 0);
+    mma(afb, bc, 3);
+    SIIRL_BWAIT(4, bn);
     __syncthreads();
+  };
+  int kt = 0;
+  for (; kt + 2 <= KT; kt += 2) {
+    step(kt, b0, b1);
+    step(kt + 1, b1, b0);
   }
+  if (kt < KT) step(kt, b0, b1);
+  // the clamped DMA of the last steps may still be in flight and the epilogue reuses the LDS
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+#undef SIIRL_BWAIT
   epi(acc, m0, n0, tc.tm, wm, wn, lane, tid, smem);
 }
+#pragma clang diagnostic pop
 
 // ------------------------------------------------------------------------------ epilogue: softmax partials
 
@@ -341,22 +400,42 @@ struct StoreBf16Epi {  // C[row][col] = bf16(acc)
 
 // ------------------------------------------------------------------------------ small kernels
 
-// out[c][r] = in[r][c] for r < R, c < C; out has ld_out >= R columns, columns [R, ld_out) are zero-filled
-// for every row c < C_out (rows c in [C, C_out) are zero too).
-__global__ __launch_bounds__(256) void transpose_pad_kernel(const uint16_t* __restrict__ in, int64_t ld_in, int R,
-                                                            int C, uint16_t* __restrict__ out, int64_t ld_out,
-                                                            int C_out) {
+// Fragment-packed B operand.  For a K-major matrix B[n][k] the packed buffer holds, for each block of 32 rows nb
+// and each block of 16 columns kb, the 64 x 16 bytes that one 32x32x16 MFMA takes as its B operand, in lane order:
+//   chunk index ((nb * KB + kb) * 64 + l),  l = (n % 32) + 32 * ((k % 16) / 8),  8 consecutive k per chunk.
+// Rows n >= N and columns k >= K are zero.  One thread per chunk.
+__global__ __launch_bounds__(256) void pack_b_kernel(const uint16_t* __restrict__ in, int64_t ld_in, int N, int K,
+                                                     u32x4* __restrict__ out, int64_t KB, int64_t chunks) {
+  const int64_t ch = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (ch >= chunks) return;
+  const int l = (int)(ch & 63);
+  const int64_t blk = ch >> 6, kb = blk % KB, nb = blk / KB;
+  const int64_t n = nb * 32 + (l & 31), k = kb * 16 + (l >> 5) * 8;
+  u32x4 v = {0u, 0u, 0u, 0u};
+  if (n < N && k < K) v = *reinterpret_cast<const u32x4*>(in + n * ld_in + k);  // K % 8 == 0
+  out[ch] = v;
+}
+
+// The same packing of the transpose: B[n][k] = in[k][n] with in of shape [R = K][C = N].  A workgroup stages a
+// 64 x 64 tile through LDS and emits its 512 chunks.
+__global__ __launch_bounds__(256) void transpose_pack_b_kernel(const uint16_t* __restrict__ in, int64_t ld_in, int R,
+                                                               int C, u32x4* __restrict__ out, int64_t KB) {
   __shared__ uint16_t tile[64][66];
-  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 x 4
+  const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;  // r = k, c = n
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   for (int rr = ty; rr < 64; rr += 4) {
     const int r = r0 + rr, cc = c0 + tx;
     tile[rr][tx] = (r < R && cc < C) ? in[(int64_t)r * ld_in + cc] : (uint16_t)0;
   }
   __syncthreads();
-  for (int cc = ty; cc < 64; cc += 4) {
-    const int cidx = c0 + cc, r = r0 + tx;
-    if (cidx < C_out && r < ld_out) out[(int64_t)cidx * ld_out + r] = tile[tx][cc];
+  for (int q = threadIdx.x; q < 512; q += 256) {
+    const int nl = q & 63, kc = q >> 6;  // local n, local chunk of 8 k
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) w[e] = (uint32_t)tile[kc * 8 + 2 * e][nl] | ((uint32_t)tile[kc * 8 + 2 * e + 1][nl] << 16);
+    const int64_t n = c0 + nl, k = r0 + kc * 8;
+    const int64_t ch = ((n >> 5) * KB + (k >> 4)) * 64 + (n & 31) + 32 * ((k >> 3) & 1);
+    out[ch] = u32x4{w[0], w[1], w[2], w[3]};
   }
 }
 
@@ -435,6 +514,12 @@ __global__ __launch_bounds__(256) void merge_partials_kernel(const float* __rest
   if (logprob) logprob[row] = label_logit[row] - lse;
 }
 
+// p[r][c] = 0 for c in [c0, c1), four rows per workgroup (c1 - c0 < 64)
+__global__ __launch_bounds__(256) void zero_cols_kernel(uint16_t* __restrict__ p, int64_t ld, int c0, int c1) {
+  const int r = blockIdx.x * 4 + (threadIdx.x >> 6), c = c0 + (threadIdx.x & 63);
+  if (c < c1) p[(int64_t)r * ld + c] = 0;
+}
+
 __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, uint16_t* __restrict__ out,
                                                           int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
@@ -446,7 +531,7 @@ __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restric
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 template <class Epi>
-int launch_gemm(const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, int M, int N, int K, const Epi& epi,
+int launch_gemm(const uint16_t* A, int64_t lda, const u32x4* Bp, int64_t kb_total, int M, int N, int K, const Epi& epi,
                 hipStream_t st, const char* what) {
   static bool attr_set = false;  // one flag per instantiation
   if (!attr_set) {
@@ -454,7 +539,7 @@ int launch_gemm(const uint16_t* A, int64_t lda, const uint16_t* B, int64_t ldb, 
                                         hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     attr_set = true;
   }
-  GemmArgs g{A, lda, B, ldb, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN};
+  GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN};
   const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n);
   gemm_nt_kernel<Epi><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
   SIIRL_LAUNCH_CHECK(what);
@@ -478,33 +563,46 @@ int check_ws_align(const void* ws) {
 }
 
 struct FwdWs {
-  size_t part, label, total;
+  size_t part, label, hp, total;
 };
-FwdWs fwd_ws(int64_t T, int64_t V) {
+FwdWs fwd_ws(int64_t T, int64_t H, int64_t V) {
   FwdWs w;
   const int64_t tiles_v = (V + BM - 1) / BM;
-  w.part = 0;
-  w.label = round_up((size_t)tiles_v * 3 * T * 4, 256);
-  w.total = w.label + round_up((size_t)T * 4, 256);
+  size_t off = 0;
+  w.part = off; off += round_up((size_t)tiles_v * 3 * T * 4, 256);
+  w.label = off; off += round_up((size_t)T * 4, 256);
+  w.hp = off; off += (size_t)round_up(T, BN) * H * 2;
+  w.total = off;
   return w;
 }
 
 struct BwdWs {
-  size_t wt, ht, d, dt, dh32, total;
-  int64_t ldwt, ldt;
+  size_t hp, wtp, htp, d, dt, dh32, total;
+  int64_t ldwt, ldt, hpad, ldd_row, ldt_row;  // ldt: token count padded to BK (a GEMM K); *_row: row strides
 };
 BwdWs bwd_ws(int64_t T, int64_t H, int64_t V, bool want_dh, bool want_dw) {
   BwdWs w;
   w.ldwt = round_up(V, BK);
   w.ldt = round_up(T, BK);
+  w.ldd_row = kSlab + kLdPad;
+  w.ldt_row = w.ldt + kLdPad;
+  w.hpad = round_up(H, BN);
   size_t off = 0;
-  w.wt = off; off += want_dh ? round_up((size_t)H * w.ldwt * 2, 256) : 0;
-  w.ht = off; off += want_dw ? round_up((size_t)H * w.ldt * 2, 256) : 0;
-  w.d = off; off += round_up((size_t)T * kSlab * 2, 256);
-  w.dt = off; off += round_up((size_t)kSlab * w.ldt * 2, 256);
+  w.hp = off; off += (size_t)round_up(T, BN) * H * 2;
+  w.wtp = off; off += want_dh ? (size_t)w.hpad * w.ldwt * 2 : 0;
+  w.htp = off; off += want_dw ? (size_t)w.hpad * w.ldt * 2 : 0;
+  w.d = off; off += round_up((size_t)T * w.ldd_row * 2, 256);
+  w.dt = off; off += round_up((size_t)kSlab * w.ldt_row * 2, 256);
   w.dh32 = off; off += want_dh ? round_up((size_t)T * H * 4, 256) : 0;
   w.total = off;
   return w;
+}
+
+int pack_hidden(const uint16_t* h, int64_t T, int64_t H, u32x4* out, hipStream_t st) {
+  const int64_t chunks = round_up(T, BN) * H / 8;
+  pack_b_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(h, H, (int)T, (int)H, out, H / 16, chunks);
+  SIIRL_LAUNCH_CHECK("pack_b_kernel");
+  return SIIRL_OK;
 }
 
 }  // namespace
@@ -514,7 +612,7 @@ using namespace siirl;
 
 extern "C" size_t siirl_fused_linear_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
   if (T < 1 || V < 1) return 0;
-  return fwd_ws(T, V).total;
+  return fwd_ws(T, H, V).total;
 }
 
 extern "C" size_t siirl_fused_linear_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int want_d_hidden,
@@ -532,7 +630,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   SIIRL_REQUIRE(lse != nullptr, "lse is NULL");
   SIIRL_REQUIRE((logprob == nullptr) == (labels == nullptr), "labels and logprob must be given together");
   SIIRL_REQUIRE(entropy == nullptr || ex != nullptr, "ex is required when entropy is requested");
-  const FwdWs ws = fwd_ws(T, V);
+  const FwdWs ws = fwd_ws(T, H, V);
   if (workspace == nullptr || workspace_bytes < ws.total)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, ws.total);
   if (int rc = check_ws_align(workspace)) return rc;
@@ -546,8 +644,10 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
                                                                           inv_temperature, label_logit);
     SIIRL_LAUNCH_CHECK("label_logit_kernel");
   }
+  u32x4* hp = reinterpret_cast<u32x4*>((char*)workspace + ws.hp);
+  if (int rc = pack_hidden(h, T, H, hp, st)) return rc;
   SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part};
-  if (int rc = launch_gemm(w, H, h, H, (int)V, (int)T, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
+  if (int rc = launch_gemm(w, H, hp, H / 16, (int)V, (int)T, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
   const int tiles_v = (int)((V + BM - 1) / BM);
   merge_partials_kernel<<<dim3((unsigned)((T + 63) / 64)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
                                                                                logprob, entropy, lse, ex);
@@ -574,41 +674,48 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
   if (int rc = check_ws_align(workspace)) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* base = (char*)workspace;
-  uint16_t* Wt = (uint16_t*)(base + ws.wt);    // [H][ldwt]
-  uint16_t* Ht = (uint16_t*)(base + ws.ht);    // [H][ldt]
-  uint16_t* D = (uint16_t*)(base + ws.d);      // [T][kSlab]
-  uint16_t* Dt = (uint16_t*)(base + ws.dt);    // [kSlab][ldt]
+  u32x4* hp = (u32x4*)(base + ws.hp);          // packed hidden: B[n = token][k = H]
+  u32x4* Wtp = (u32x4*)(base + ws.wtp);        // packed W^T:    B[n = H][k = vocabulary]
+  u32x4* Htp = (u32x4*)(base + ws.htp);        // packed hidden^T: B[n = H][k = token]
+  uint16_t* D = (uint16_t*)(base + ws.d);      // [T][ldd_row]
+  uint16_t* Dt = (uint16_t*)(base + ws.dt);    // [kSlab][ldt_row]
   float* dH32 = (float*)(base + ws.dh32);      // [T][H]
   const uint16_t* h = (const uint16_t*)hidden;
   const uint16_t* w = (const uint16_t*)weight;
 
+  if (int rc = pack_hidden(h, T, H, hp, st)) return rc;
   if (want_dh) {
-    transpose_pad_kernel<<<dim3((unsigned)((ws.ldwt + 63) / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st>>>(
-        w, H, (int)V, (int)H, Wt, ws.ldwt, (int)H);
-    SIIRL_LAUNCH_CHECK("transpose_pad_kernel(W)");
+    transpose_pack_b_kernel<<<dim3((unsigned)(ws.ldwt / 64), (unsigned)(ws.hpad / 64)), dim3(256), 0, st>>>(
+        w, H, (int)V, (int)H, Wtp, ws.ldwt / 16);
+    SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(W)");
   }
   if (want_dw) {
-    transpose_pad_kernel<<<dim3((unsigned)((ws.ldt + 63) / 64), (unsigned)((H + 63) / 64)), dim3(256), 0, st>>>(
-        h, H, (int)T, (int)H, Ht, ws.ldt, (int)H);
-    SIIRL_LAUNCH_CHECK("transpose_pad_kernel(hidden)");
+    transpose_pack_b_kernel<<<dim3((unsigned)(ws.ldt / 64), (unsigned)(ws.hpad / 64)), dim3(256), 0, st>>>(
+        h, H, (int)T, (int)H, Htp, ws.ldt / 16);
+    SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(hidden)");
   }
-  // K-padding rows of Dt (token index in [T, ldt)) are never written by the epilogue: clear once
-  SIIRL_HIP_CHECK(hipMemsetAsync(Dt, 0, (size_t)kSlab * ws.ldt * 2, st));
+  // K-padding columns of Dt (token index in [T, ldt)) are never written by the epilogue: clear once (with a
+  // kernel, not a memset node, so that the call can be captured into a graph)
+  if (ws.ldt > T) {
+    zero_cols_kernel<<<dim3(kSlab / 4), dim3(256), 0, st>>>(Dt, ws.ldt_row, (int)T, (int)ws.ldt);
+    SIIRL_LAUNCH_CHECK("zero_cols_kernel");
+  }
 
   int slab_idx = 0;
   for (int64_t v0 = 0; v0 < V; v0 += kSlab, ++slab_idx) {
     const int N = (int)((V - v0) < kSlab ? (V - v0) : kSlab);
     const int Npad = (int)round_up(N, BK);
-    DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels, D, kSlab, Dt, ws.ldt};
-    if (int rc = launch_gemm(w + v0 * H, H, h, H, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
+    DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels, D, ws.ldd_row, Dt, ws.ldt_row};
+    if (int rc = launch_gemm(w + v0 * H, H, hp, H / 16, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
     if (want_dh) {  // dH[T, H] += D[T, Npad] . Wt[H, v0 : v0 + Npad]^T
       AccumF32Epi acc{dH32, H, (int)T, (int)H, slab_idx > 0 ? 1 : 0};
-      if (int rc = launch_gemm(D, kSlab, Wt + v0, ws.ldwt, (int)T, (int)H, Npad, acc, st, "gemm_nt_kernel<AccumF32Epi>"))
+      if (int rc = launch_gemm(D, ws.ldd_row, Wtp + (v0 / 16) * 64, ws.ldwt / 16, (int)T, (int)H, Npad, acc, st,
+                               "gemm_nt_kernel<AccumF32Epi>"))
         return rc;
     }
     if (want_dw) {  // dW[v0 : v0 + N, H] = Dt[N, ldt] . Ht[H, ldt]^T
       StoreBf16Epi sto{(uint16_t*)d_weight + v0 * H, H, N, (int)H};
-      if (int rc = launch_gemm(Dt, ws.ldt, Ht, ws.ldt, N, (int)H, (int)ws.ldt, sto, st, "gemm_nt_kernel<StoreBf16Epi>"))
+      if (int rc = launch_gemm(Dt, ws.ldt_row, Htp, ws.ldt / 16, N, (int)H, (int)ws.ldt, sto, st, "gemm_nt_kernel<StoreBf16Epi>"))
         return rc;
     }
   }

@@ -52,8 +52,14 @@ typedef enum siirl_agg_mode {
   SIIRL_AGG_SEQ_MEAN_TOKEN_SUM_NORM = 3 /* "seq-mean-token-sum-norm" */
 } siirl_agg_mode;
 
-/* registered policy losses, siirl/dag_worker/core_algos.py:710,795 */
-typedef enum siirl_loss_mode { SIIRL_LOSS_VANILLA = 0, SIIRL_LOSS_GSPO = 1 } siirl_loss_mode;
+/* registered policy losses, siirl/dag_worker/core_algos.py:572,710,795,865,1074 */
+typedef enum siirl_loss_mode {
+  SIIRL_LOSS_VANILLA = 0,  /* "vanilla" */
+  SIIRL_LOSS_GSPO = 1,     /* "gspo" */
+  SIIRL_LOSS_CPGD = 2,     /* "cpgd" */
+  SIIRL_LOSS_GPG = 3,      /* "gpg" */
+  SIIRL_LOSS_GEO_MEAN = 4  /* "geo_mean" (GMPO) */
+} siirl_loss_mode;
 
 /* kl_penalty estimators, siirl/dag_worker/core_algos.py:1241-1276 */
 typedef enum siirl_kl_mode {
@@ -131,7 +137,8 @@ size_t siirl_loss_workspace_bytes(int64_t B, int64_t L);
 #define SIIRL_OUT_RATIO_MIN 8
 #define SIIRL_OUT_RATIO_MAX 9
 #define SIIRL_OUT_MASK_TOTAL 10  /* sum of the mask                                                     */
-#define SIIRL_OUT_POLICY_LOSS 11 /* pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss          */
+#define SIIRL_OUT_POLICY_LOSS 11 /* pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss + drift term */
+#define SIIRL_OUT_DRIFT_LOSS 12  /* agg_loss(policy drift)       (0 when policy_drift_coeff is 0)       */
 
 /*
  * agg_loss(loss_mat, loss_mask, loss_agg_mode): scalar aggregation of a [B, L] fp32 matrix.
@@ -154,25 +161,33 @@ int siirl_agg_loss_bwd(const float* g_out, const void* mask, int mask_dtype, con
 /*
  * The actor's loss for one micro-batch in one pass over [B, L] fp32 operands:
  *   pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower  = policy loss `loss_mode` (vanilla: PPO/GRPO/DAPO clip
- *        with dual clip `clip_c`; gspo: sequence-level ratio, always seq-mean-token-mean),
+ *        with dual clip `clip_c`; gspo: sequence-level ratio, always seq-mean-token-mean; cpgd: the
+ *        log-probability clipped at old + log(1 -+ eps), importance weights unused; gpg: -log_prob * A, the
+ *        three metrics zero; geo_mean: per sequence -mean(A) * exp(mean of the clipped log-ratios), plain mean
+ *        over sequences whatever agg_mode says),
  *   entropy_loss = agg_loss(entropy)                       when entropy != NULL,
  *   kl_loss      = agg_loss(kl_penalty(log_prob, ref))     when ref_log_prob != NULL,
- *   loss = (pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss) * loss_scale,
+ *   drift_loss   = agg_loss(clamp(exp(log_prob - old) - 1, max = 2) * log_prob), the weight not
+ *                  differentiated,                         when policy_drift_coeff != 0,
+ *   loss = (pg_loss - entropy_coeff * entropy_loss + kl_coef * kl_loss + policy_drift_coeff * drift_loss)
+ *          * loss_scale,
  * plus the ratio statistics the actor logs.  is_weights (rollout importance weights) may be NULL.
- * row_msum[B] and row_s[B] (GSPO's per-sequence mean log-ratio; may be NULL for vanilla) are saved for
- * the backward.  Called with entropy = ref_log_prob = NULL and loss_scale = 1 this is exactly
+ * row_msum[B] and row_s[B] (gspo: the per-sequence mean log-ratio; geo_mean: the per-sequence loss; may be
+ * NULL for the other modes) are saved for the backward.  Called with entropy = ref_log_prob = NULL and loss_scale = 1 this is exactly
  * compute_policy_loss_vanilla / compute_policy_loss_gspo.  log_ratio_clamp bounds |log_prob - old_log_prob|
  * before the exponential in the vanilla loss: 20 as in core_algos.py:758, +infinity for the legacy
  * compute_policy_loss (core_algos.py:631-707) which does not clamp.
- * Replaces: siirl/dag_worker/core_algos.py:710-792 (vanilla), :795-862 (gspo), :1215-1276 (kl_penalty),
- *           and the composition in siirl/engine/actor/dp_actor.py:455-513.
+ * Replaces: siirl/dag_worker/core_algos.py:710-792 (vanilla), :795-862 (gspo), :572-629 (cpgd), :865-895
+ *           (gpg), :1074-1153 (geo_mean), :1215-1276 (kl_penalty), and the composition in
+ *           siirl/engine/actor/dp_actor.py:455-513 (drift term :488-494).
  */
 int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_prob, const float* advantages,
                          const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
                          const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
                          float clip_high, float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff,
-                         int kl_mode, int kl_straight_through, float kl_coef, float loss_scale, float* out16, float* row_msum,
-                         float* row_s, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
+                         int kl_mode, int kl_straight_through, float kl_coef, float policy_drift_coeff,
+                         float loss_scale, float* out16, float* row_msum, float* row_s, void* workspace,
+                         size_t workspace_bytes, siirl_stream_t stream);
 
 /*
  * Backward of the above for an upstream gradient g_loss[0] (device scalar) on out16[SIIRL_OUT_LOSS]:
@@ -183,10 +198,25 @@ int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const f
                          const float* advantages, const void* mask, int mask_dtype, const float* is_weights,
                          const float* entropy, const float* ref_log_prob, int64_t B, int64_t L, int loss_mode,
                          float clip_low, float clip_high, float clip_c, float log_ratio_clamp, int agg_mode,
-                         float entropy_coeff, int kl_mode, int kl_straight_through, float kl_coef, float loss_scale,
-                         const float* out16,
-                         const float* row_msum, const float* row_s, float* d_log_prob, float* d_entropy,
-                         siirl_stream_t stream);
+                         float entropy_coeff, int kl_mode, int kl_straight_through, float kl_coef,
+                         float policy_drift_coeff, float loss_scale, const float* out16, const float* row_msum,
+                         const float* row_s, float* d_log_prob, float* d_entropy, siirl_stream_t stream);
+
+/*
+ * Clipped value loss of the critic over [B, L] fp32 operands:
+ *   vclip = max(min(vpreds, values + c), values - c),  tok = max((vpreds - returns)^2, (vclip - returns)^2),
+ *   out16[SIIRL_OUT_LOSS] = vf_loss = 0.5 * agg_loss(tok),  out16[SIIRL_OUT_PG_CLIPFRAC] = vf_clipfrac =
+ *   masked_mean((vclip - returns)^2 > (vpreds - returns)^2);  out16[SIIRL_OUT_PG_LOSS] holds agg_loss(tok).
+ * The backward writes d vf_loss / d vpreds times g_loss[0], with autograd's tie rules for max / min.
+ * Replaces: compute_value_loss siirl/dag_worker/core_algos.py:1173-1212 (clip_by_value
+ *           siirl/utils/model_utils/torch_functional.py:119-125).
+ */
+int siirl_value_loss_fwd(const float* vpreds, const float* returns, const float* values, const void* mask,
+                         int mask_dtype, int64_t B, int64_t L, float cliprange_value, int agg_mode, float* out16,
+                         float* row_msum, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
+int siirl_value_loss_bwd(const float* g_loss, const float* vpreds, const float* returns, const float* values,
+                         const void* mask, int mask_dtype, int64_t B, int64_t L, float cliprange_value, int agg_mode,
+                         const float* out16, const float* row_msum, float* d_vpreds, siirl_stream_t stream);
 
 /*
  * kl_penalty, elementwise over n fp32 values.  straight_through != 0 gives the k2 gradient
@@ -217,6 +247,34 @@ int siirl_masked_reduce(const float* values, const void* mask, int mask_dtype, i
 int siirl_kl_in_reward(const float* token_level_scores, const float* old_log_prob, const float* ref_log_prob,
                        const void* mask, int mask_dtype, int64_t B, int64_t L, int kl_mode, float beta,
                        float* token_level_rewards, float* row_kl, float* current_kl, siirl_stream_t stream);
+
+/* ------------------------------------------------------------------- GAE and masked whitening */
+
+/* Bytes of scratch siirl_masked_whiten / siirl_gae_advantage_return need (a constant; 8-byte aligned buffer). */
+size_t siirl_whiten_workspace_bytes(void);
+
+/*
+ * masked_whiten over n fp32 values: mean = masked_mean(values, mask), var = masked_mean((values - mean)^2, mask)
+ * * n_mask / (n_mask - 1), out = (values - mean) * rsqrt(var + 1e-8) (+ mean when shift_mean == 0), applied to
+ * every element.  out may be the values buffer.  stats3 receives {mean, var, n_mask}; the reference raises
+ * ValueError for n_mask 0 or 1 -- here the caller reads stats3[2] (the outputs are then not meaningful).
+ * Replaces: masked_mean / masked_var / masked_whiten siirl/utils/model_utils/torch_functional.py:154-206.
+ */
+int siirl_masked_whiten(const float* values, const void* mask, int mask_dtype, int64_t n, int shift_mean, float* out,
+                        float* stats3, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
+
+/*
+ * Generalised advantage estimation over [B, L] fp32 operands, scanning each row from its last token:
+ *   delta = r_t + gamma * V_next - V_t,  A_t = delta + gamma * lam * A_next; a token with mask 0 keeps V_next and
+ *   A_next of the token after it (both start at 0).  returns = A + values (before whitening);
+ *   advantages = masked_whiten(A, mask).  The scan is evaluated in the reference's float32 operation order, so
+ *   `returns` is bit-identical to the reference's.  stats3 as for siirl_masked_whiten.
+ * Replaces: compute_gae_advantage_return siirl/dag_worker/core_algos.py:229-276.
+ */
+int siirl_gae_advantage_return(const float* token_level_rewards, const float* values, const void* mask,
+                               int mask_dtype, int64_t B, int64_t L, double gamma, double lam, float* advantages,
+                               float* returns, float* stats3, void* workspace, size_t workspace_bytes,
+                               siirl_stream_t stream);
 
 /* ------------------------------------------------------------------- per-prompt group statistics */
 

@@ -32,6 +32,19 @@ compute_grpo_outcome_advantage         brute-force dict loop; unbiased-std known
 agg_loss                               four closed forms on hand-written cases
 compute_policy_loss_vanilla / _gspo    hand-computed cases at ratio = 1, 1 +- eps, c, |d| = 20;
                                        closed-form gradient vs autograd; GSPO with L = 1 == PPO
+compute_gae_advantage_return           gamma = lam = 1 -> reward-to-go minus value; lam = 0 -> TD
+                                       error; brute-force double sum; padding == truncation;
+                                       interior masked tokens == deleted columns; whitened
+                                       selection has mean 0 / unbiased variance 1 (numpy)
+masked_var / masked_whiten             numpy mean / var(ddof) of the selected elements; the two
+                                       ValueErrors
+compute_value_loss                     hand-computed cases either side of the clip range; zero
+                                       gradient where clipped
+compute_policy_loss_cpgd / drift       hand-computed tokens with log(1 +- eps) bounds; gradient
+                                       vanishes exactly on the clipped fraction; detached weight
+compute_policy_loss_gpg                identity with agg_loss(-lp * A [* w])
+compute_policy_loss_geo_mean           explicit product of token ratios ** (1 / L); L = 1 cases
+                                       for each clipping side; weights as their geometric mean
 kl_penalty                             closed forms per mode; k3 >= 0; straight-through identities
 apply_kl_penalty / KL controllers      hand-computed controller step
 dynamic_sampling_keep_indices          worked example of the reference's docs

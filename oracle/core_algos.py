@@ -1,9 +1,11 @@
 """Oracle (test infrastructure): advantages, policy losses, aggregation and KL penalty.
 
 Restates on the CPU the arithmetic of ``siirl/dag_worker/core_algos.py`` of the reference
-(GRPO outcome advantage ``:279-348``, ``agg_loss`` ``:536-569``, the ``vanilla`` loss
-``:710-792``, the ``gspo`` loss ``:795-862``, ``kl_penalty`` ``:1215-1276``, KL controllers
-``:167-226``, ``apply_kl_penalty`` ``:1358-1397``).  Works in the dtype of its inputs, so the
+(GAE ``:229-276``, GRPO outcome advantage ``:279-348``, ``agg_loss`` ``:536-569``, the ``cpgd``
+loss ``:572-629``, the ``vanilla`` loss ``:710-792``, the ``gspo`` loss ``:795-862``, ``gpg``
+``:865-895``, ``geo_mean`` ``:1074-1153``, the value loss ``:1173-1212``, ``kl_penalty``
+``:1215-1276``, KL controllers ``:167-226``, ``apply_kl_penalty`` ``:1358-1397``) and the CPGD
+drift term of ``siirl/engine/actor/dp_actor.py:488-494``.  Works in the dtype of its inputs, so the
 same code serves as the fp32 statement and, on fp64 inputs, as the high-precision check.
 """
 
@@ -16,7 +18,7 @@ from typing import Optional
 import numpy as np
 import torch
 
-from .torch_functional import masked_mean
+from .torch_functional import clip_by_value, masked_mean, masked_whiten
 
 AGG_MODES = ("token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm")
 
@@ -77,6 +79,31 @@ def grpo_bruteforce(scores, uid, epsilon=1e-6, norm=True):
             sd = math.sqrt(sum((g - mu) ** 2 for g in grp) / (len(grp) - 1))
         out.append((s[i] - mu) / (sd + epsilon) if norm else s[i] - mu)
     return out
+
+
+def gae_unwhitened(token_level_rewards, values, response_mask, gamma, lam):
+    """The reverse scan of the reference's GAE (``core_algos.py:259-273``) before whitening:
+    ``delta_t = r_t + gamma * V_next - V_t``, ``A_t = delta_t + gamma * lam * A_next``; a masked
+    position keeps ``V_next`` and ``A_next`` of the position after it.  Returns ``(A, A + V)``."""
+    nextvalues, lastgaelam = 0, 0
+    rev = []
+    for t in reversed(range(token_level_rewards.shape[-1])):
+        m = response_mask[:, t]
+        delta = token_level_rewards[:, t] + gamma * nextvalues - values[:, t]
+        cand = delta + gamma * lam * lastgaelam
+        nextvalues = values[:, t] * m + (1 - m) * nextvalues
+        lastgaelam = cand * m + (1 - m) * lastgaelam
+        rev.append(lastgaelam)
+    adv = torch.stack(rev[::-1], dim=1)
+    return adv, adv + values
+
+
+def compute_gae_advantage_return(token_level_rewards, values, response_mask, gamma, lam):
+    """Generalised advantage estimation, then whitening of the advantages over the mask
+    (reference ``core_algos.py:229-276``).  Returns ``(advantages, returns)``; the returns are
+    the un-whitened advantages plus the values."""
+    adv, returns = gae_unwhitened(token_level_rewards, values, response_mask, gamma, lam)
+    return masked_whiten(adv, response_mask), returns
 
 
 # --------------------------------------------------------------------------- aggregation
@@ -156,6 +183,83 @@ def compute_policy_loss_gspo(old_log_prob, log_prob, advantages, response_mask,
     pg_clipfrac = masked_mean(torch.gt(l2, l1).to(d.dtype), response_mask)
     ppo_kl = masked_mean(-d, response_mask)
     return pg_loss, pg_clipfrac, ppo_kl, torch.zeros((), dtype=pg_loss.dtype)
+
+
+def compute_policy_loss_cpgd(old_log_prob, log_prob, advantages, response_mask,
+                             loss_agg_mode="token-mean", config=None, rollout_is_weights=None):
+    """CPGD: the log-probability itself is clipped at ``old + log(1 + eps_hi)`` (positive advantage)
+    or ``old + log(1 - eps_lo)`` (otherwise) and the loss is ``-clipped * A`` (reference
+    ``core_algos.py:572-629``).  ``rollout_is_weights`` is accepted and ignored, as there."""
+    import math
+
+    assert config is not None, "Config must be provided for CPGD loss"
+    eps_lo, eps_hi = _clip_bounds(config)
+    c = config.clip_ratio_c if config.clip_ratio_c is not None else 3.0
+    assert c > 1.0, f"clip_ratio_c ({c}) must be > 1.0"
+    d = log_prob - old_log_prob
+    ratio = torch.exp(d)
+    ppo_kl = masked_mean(-d, response_mask)
+    clipped = torch.where(advantages > 0,
+                          torch.clamp(log_prob, max=math.log(1 + eps_hi) + old_log_prob),
+                          torch.clamp(log_prob, min=math.log(1 - eps_lo) + old_log_prob))
+    pg_loss = agg_loss(-clipped * advantages, response_mask, loss_agg_mode)
+    is_clipped = torch.where(advantages > 0, ratio > 1 + eps_hi, ratio < 1 - eps_lo)
+    pg_clipfrac = masked_mean(is_clipped.to(d.dtype), response_mask)
+    pg_clipfrac_lower = masked_mean((ratio > c) * (advantages < 0).to(d.dtype), response_mask)
+    return pg_loss, pg_clipfrac, ppo_kl, pg_clipfrac_lower
+
+
+def policy_drift_loss(old_log_prob, log_prob, response_mask, loss_agg_mode):
+    """CPGD's drift regulariser as the actor adds it (reference ``dp_actor.py:488-494``):
+    ``agg_loss(clamp(exp(lp.detach() - old) - 1, max=2) * lp)``."""
+    drift = ((log_prob.detach() - old_log_prob).exp() - 1.0).clamp(max=2.0) * log_prob
+    return agg_loss(drift, response_mask, loss_agg_mode)
+
+
+def compute_policy_loss_gpg(old_log_prob, log_prob, advantages, response_mask,
+                            loss_agg_mode="token-mean", config=None, rollout_is_weights=None):
+    """GPG: ``-log_prob * A`` (reference ``core_algos.py:865-895``); the three metrics are zeros."""
+    tok = -log_prob * advantages
+    if rollout_is_weights is not None:
+        tok = tok * rollout_is_weights
+    z = torch.zeros((), dtype=tok.dtype)
+    return agg_loss(tok, response_mask, loss_agg_mode), z, z, z
+
+
+def compute_policy_loss_geo_mean(old_log_prob, log_prob, advantages, response_mask,
+                                 loss_agg_mode="token-mean", config=None, rollout_is_weights=None):
+    """GMPO: token log-ratios clipped to ``[-eps_lo, eps_hi]`` on the side the advantage's sign
+    makes pessimistic, their masked mean exponentiated (geometric mean of the ratios), times the
+    masked-mean advantage of the sequence; plain mean over sequences (reference
+    ``core_algos.py:1074-1153``).  ``loss_agg_mode`` is not used."""
+    assert config is not None
+    eps_lo, eps_hi = _clip_bounds(config)
+    d = log_prob - old_log_prob
+    ppo_kl = masked_mean(-d, response_mask)
+    sgn = torch.sign(advantages)
+    dc = torch.clamp(d, -eps_lo, eps_hi)
+    x = sgn * torch.min(sgn * d, sgn * dc)
+    n = response_mask.sum(dim=-1)
+    ratio = torch.exp((x * response_mask).sum(dim=-1) / (n + 1e-8))
+    adv = (advantages * response_mask).sum(dim=-1) / (n + 1e-8)
+    seq = -adv * ratio
+    if rollout_is_weights is not None:
+        seq = seq * torch.exp((torch.log(rollout_is_weights + 1e-10) * response_mask).sum(dim=-1) / (n + 1e-8))
+    clipped = torch.ne(d, dc)
+    pg_clipfrac = masked_mean((clipped * (advantages > 0)).to(d.dtype), response_mask)
+    pg_clipfrac_lower = masked_mean((clipped * (advantages < 0)).to(d.dtype), response_mask)
+    return torch.mean(seq), pg_clipfrac, ppo_kl, pg_clipfrac_lower
+
+
+def compute_value_loss(vpreds, returns, values, response_mask, cliprange_value, loss_agg_mode="token-mean"):
+    """Clipped value loss (reference ``core_algos.py:1173-1212``): ``0.5 * agg_loss(max((v - R)^2,
+    (clip(v, V_old - c, V_old + c) - R)^2))`` and the fraction of tokens where the clipped term wins."""
+    vclip = clip_by_value(vpreds, values - cliprange_value, values + cliprange_value)
+    l1 = (vpreds - returns) ** 2
+    l2 = (vclip - returns) ** 2
+    vf_loss = 0.5 * agg_loss(torch.max(l1, l2), response_mask, loss_agg_mode)
+    vf_clipfrac = masked_mean(torch.gt(l2, l1).to(l1.dtype), response_mask)
+    return vf_loss, vf_clipfrac
 
 
 def policy_loss_grad_closed_form(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode,

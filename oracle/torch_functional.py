@@ -1,6 +1,6 @@
 """Oracle (test infrastructure): log-prob / entropy from logits and the masked reductions.
 
-Restates ``siirl/utils/model_utils/torch_functional.py:41-168`` of the reference on the CPU.
+Restates ``siirl/utils/model_utils/torch_functional.py:41-206`` of the reference on the CPU.
 
 Precision policy.  The reference's fp32 branch (``torch_functional.py:103-107``) is
 ``gather(x) - logsumexp(x)``; for 16-bit logits the deployed path is flash-attn's fp32
@@ -120,3 +120,34 @@ def masked_sum(values, mask, axis=None):
 def masked_mean(values, mask, axis=None):
     """``masked_sum / (sum(mask) + 1e-8)`` (reference ``torch_functional.py:154-168``)."""
     return masked_sum(values, mask, axis) / (mask.sum(axis) + 1e-8)
+
+
+def clip_by_value(x, tensor_min, tensor_max):
+    """``max(min(x, tensor_max), tensor_min)`` with tensor bounds (reference ``torch_functional.py:119-125``)."""
+    return torch.max(torch.min(x, tensor_max), tensor_min)
+
+
+def masked_var(values, mask, unbiased=True):
+    """Variance over the masked elements (reference ``torch_functional.py:171-187``): the masked mean
+    of the squared deviations from the masked mean, times ``n / (n - 1)`` when unbiased.  An empty
+    mask or a mask of one element raise ``ValueError`` as the reference does."""
+    mean = masked_mean(values, mask)
+    variance = masked_mean((values - mean) ** 2, mask)
+    if unbiased:
+        n = mask.sum()
+        if n == 0:
+            raise ValueError("At least one element in the mask has to be 1.")
+        if n == 1:
+            raise ValueError("The sum of the mask is one, which can cause a division by zero.")
+        variance = variance * (n / (n - 1))
+    return variance
+
+
+def masked_whiten(values, mask, shift_mean=True):
+    """``(values - mean) * rsqrt(var + 1e-8)`` with masked statistics, applied to every element
+    (reference ``torch_functional.py:190-206``)."""
+    mean, var = masked_mean(values, mask), masked_var(values, mask)
+    out = (values - mean) * torch.rsqrt(var + 1e-8)
+    if not shift_mean:
+        out = out + mean
+    return out

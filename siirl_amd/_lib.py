@@ -14,7 +14,8 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsiirl_hip.so"
 F32, BF16, F16, F64, I64, I32, U8 = range(7)
 BWD_SKIP_ZERO_ROWS = 1
 
-_p, _i64, _i32, _f32, _u32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint32, C.c_size_t
+_p, _i64, _i32, _f32, _u32, _sz, _f64 = (C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint32, C.c_size_t,
+                                        C.c_double)
 
 # name -> (restype, argtypes); one entry per function declared in include/siirl_hip.h
 SIGNATURES = {
@@ -26,9 +27,14 @@ SIGNATURES = {
     "siirl_agg_loss_fwd": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
     "siirl_agg_loss_bwd": (_i32, [_p, _p, _i32, _p, _p, _i64, _i64, _i32, _p, _p]),
     "siirl_actor_loss_fwd": (_i32, [_p, _p, _p, _p, _i32, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _f32, _f32, _i32,
-                                    _f32, _i32, _i32, _f32, _f32, _p, _p, _p, _p, _sz, _p]),
+                                    _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _p, _sz, _p]),
     "siirl_actor_loss_bwd": (_i32, [_p, _p, _p, _p, _p, _i32, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _f32, _f32,
-                                    _i32, _f32, _i32, _i32, _f32, _f32, _p, _p, _p, _p, _p, _p]),
+                                    _i32, _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _p, _p, _p]),
+    "siirl_value_loss_fwd": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _f32, _i32, _p, _p, _p, _sz, _p]),
+    "siirl_value_loss_bwd": (_i32, [_p, _p, _p, _p, _p, _i32, _i64, _i64, _f32, _i32, _p, _p, _p, _p]),
+    "siirl_whiten_workspace_bytes": (_sz, []),
+    "siirl_masked_whiten": (_i32, [_p, _p, _i32, _i64, _i32, _p, _p, _p, _sz, _p]),
+    "siirl_gae_advantage_return": (_i32, [_p, _p, _p, _i32, _i64, _i64, _f64, _f64, _p, _p, _p, _p, _sz, _p]),
     "siirl_kl_penalty_fwd": (_i32, [_p, _p, _i64, _i32, _p, _p]),
     "siirl_kl_penalty_bwd": (_i32, [_p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
     "siirl_masked_reduce": (_i32, [_p, _p, _i32, _i64, _i64, _p, _p, _p, _p, _sz, _p]),

@@ -1,11 +1,13 @@
 """Advantages, policy losses, aggregation and KL penalty with the reference's Python signatures.
 
 Mirror of the in-scope part of ``siirl/dag_worker/core_algos.py``: the two registries (``:51-86``,
-``:127-164``), ``compute_grpo_outcome_advantage`` (``:279-348``), ``agg_loss`` (``:536-569``),
+``:127-164``), ``compute_gae_advantage_return`` (``:229-276``), ``compute_grpo_outcome_advantage``
+(``:279-348``), ``agg_loss`` (``:536-569``), ``compute_policy_loss_cpgd`` (``:572-629``),
 ``compute_policy_loss`` (``:631-707``), ``compute_policy_loss_vanilla`` (``:710-792``),
-``compute_policy_loss_gspo`` (``:795-862``), ``kl_penalty`` (``:1215-1276``), the KL controllers
-(``:167-226``), ``apply_kl_penalty`` (``:1358-1397``) and the GRPO branch of ``compute_advantage``
-(``:1400-1471``).  Same names, keyword arguments, return order and exception types; the arithmetic
+``compute_policy_loss_gspo`` (``:795-862``), ``compute_policy_loss_gpg`` (``:865-895``),
+``compute_policy_loss_geo_mean`` (``:1074-1153``), ``compute_value_loss`` (``:1173-1212``), ``kl_penalty``
+(``:1215-1276``), the KL controllers (``:167-226``), ``apply_kl_penalty`` (``:1358-1397``) and the GAE and GRPO
+branches of ``compute_advantage`` (``:1400-1471``).  Same names, keyword arguments, return order and exception types; the arithmetic
 runs in ``libsiirl_hip.so``.  ``actor_loss`` is an addition: the whole loss of one micro-batch
 (policy loss, entropy bonus, KL loss, scaling, logged metrics) in one fused launch.
 
@@ -29,16 +31,20 @@ from . import torch_functional as siirl_F
 __all__ = [
     "register_policy_loss", "get_policy_loss_fn", "register_adv_est", "get_adv_estimator_fn", "AdvantageEstimator",
     "AdaptiveKLController", "FixedKLController", "get_kl_controller", "compute_response_mask",
-    "compute_grpo_outcome_advantage", "compute_rewards", "agg_loss", "compute_policy_loss",
-    "compute_policy_loss_vanilla", "compute_policy_loss_gspo", "kl_penalty", "kl_penalty_forward",
+    "compute_gae_advantage_return", "compute_grpo_outcome_advantage", "compute_rewards", "agg_loss",
+    "compute_policy_loss", "compute_policy_loss_vanilla", "compute_policy_loss_gspo", "compute_policy_loss_cpgd",
+    "compute_policy_loss_gpg", "compute_policy_loss_geo_mean", "compute_value_loss", "kl_penalty",
+    "kl_penalty_forward",
     "apply_kl_penalty", "compute_advantage", "actor_loss", "ActorLossOutput",
 ]
 
 AGG_MODES = {"token-mean": 0, "seq-mean-token-sum": 1, "seq-mean-token-mean": 2, "seq-mean-token-sum-norm": 3}
 KL_MODES = {"kl": 0, "k1": 0, "abs": 1, "mse": 2, "k2": 2, "low_var_kl": 3, "k3": 3}
-LOSS_VANILLA, LOSS_GSPO = 0, 1
+LOSS_VANILLA, LOSS_GSPO, LOSS_CPGD, LOSS_GPG, LOSS_GEO_MEAN = range(5)
+_LOSS_CODES = {"vanilla": LOSS_VANILLA, "gspo": LOSS_GSPO, "cpgd": LOSS_CPGD, "gpg": LOSS_GPG, "geo_mean": LOSS_GEO_MEAN}
 # indices into the 16-float result block (SIIRL_OUT_* of include/siirl_hip.h)
-O_LOSS, O_PG, O_CLIPFRAC, O_PPOKL, O_CLIPLOWER, O_ENT, O_KL, O_RMEAN, O_RMIN, O_RMAX, O_MTOTAL, O_POLICY = range(12)
+(O_LOSS, O_PG, O_CLIPFRAC, O_PPOKL, O_CLIPLOWER, O_ENT, O_KL, O_RMEAN, O_RMIN, O_RMAX, O_MTOTAL, O_POLICY,
+ O_DRIFT) = range(13)
 
 
 class AdvantageEstimator(str, Enum):
@@ -211,6 +217,35 @@ def _uid_tensor(index, n, dev) -> torch.Tensor:
     return out.contiguous()
 
 
+@register_adv_est(AdvantageEstimator.GAE)
+def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torch.Tensor, response_mask: torch.Tensor,
+                                 gamma, lam):
+    """Generalised advantage estimation with whitened advantages (reference ``core_algos.py:229-276``).
+    Returns ``(advantages, returns)``, ``[B, L]`` fp32; ``returns`` is the un-whitened advantage plus the
+    values.  Raises the reference's ``ValueError`` when the mask selects fewer than two tokens."""
+    dev, back = _staging_device(token_level_rewards, values, response_mask)
+    B, L = token_level_rewards.shape
+    r = _f32(token_level_rewards, dev)
+    v = _f32(values, dev)
+    m, mcode = _mask_arg(response_mask, dev)
+    if tuple(v.shape) != (B, L) or tuple(m.shape) != (B, L):
+        raise ValueError(f"values {tuple(v.shape)} and response_mask {tuple(m.shape)} must have shape {(B, L)}")
+    adv = torch.empty(B, L, dtype=torch.float32, device=dev)
+    ret = torch.empty(B, L, dtype=torch.float32, device=dev)
+    stats = torch.empty(3, dtype=torch.float32, device=dev)
+    nws = _lib.lib().siirl_whiten_workspace_bytes()
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().siirl_gae_advantage_return(_lib.ptr(r), _lib.ptr(v), _lib.ptr(m), mcode, B, L, float(gamma),
+                                                   float(lam), _lib.ptr(adv), _lib.ptr(ret), _lib.ptr(stats),
+                                                   _lib.ptr(ws), nws, _lib.current_stream(dev))
+    _lib.check(rc, "siirl_gae_advantage_return")
+    siirl_F._check_whiten_count(float(stats[2]))
+    if back:
+        adv, ret = adv.to(token_level_rewards.device), ret.to(token_level_rewards.device)
+    return adv, ret
+
+
 @register_adv_est(AdvantageEstimator.GRPO)
 def compute_grpo_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
                                    epsilon: float = 1e-6, norm_adv_by_std_in_grpo: bool = True, config=None):
@@ -283,12 +318,22 @@ def apply_kl_penalty(data, kl_ctrl, kl_penalty="kl", multi_turn=False):
 
 def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_in_grpo=True,
                       weight_factor_in_cpgd="STD_weight", **kwargs):
-    """Dispatcher (reference ``core_algos.py:1400-1492``).  Only the GRPO branch (``:1440-1471``) is in scope;
-    GAE / MARFT raise ``NotImplementedError`` here, and the CPGD branch fails with the reference's own
-    ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a keyword it does not take, ``:1475-1480``)."""
+    """Dispatcher (reference ``core_algos.py:1400-1492``).  The GAE (``:1424-1439``, without the PF-PPO
+    reweighting) and GRPO (``:1440-1471``) branches are built; MARFT raises ``NotImplementedError`` here, and
+    the CPGD branch fails with the reference's own ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a
+    keyword it does not take, ``:1475-1480``)."""
     if "response_mask" not in data.keys():
         _td_set(data, "response_mask", compute_response_mask(data))
     est = adv_estimator.value if isinstance(adv_estimator, Enum) else adv_estimator
+    if est == "gae":
+        if kwargs.get("use_pf_ppo", False):
+            raise NotImplementedError("PF-PPO reweighting is outside this build")
+        advantages, returns = compute_gae_advantage_return(
+            token_level_rewards=data["token_level_rewards"], values=data["values"],
+            response_mask=data["response_mask"], gamma=gamma, lam=lam)
+        data["advantages"] = advantages
+        data["returns"] = returns
+        return data
     if est == "grpo":
         if "finish_step" in data.keys() and data["responses"].ndim == 3:
             responses = data["responses"]
@@ -309,7 +354,7 @@ def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_i
         compute_grpo_outcome_advantage(token_level_rewards=data["token_level_rewards"],
                                        response_mask=data["response_mask"], index=data["uid"],
                                        weight_factor_in_cpgd=weight_factor_in_cpgd)
-    raise NotImplementedError(f"advantage estimator {est!r} is outside this build (GRPO only)")
+    raise NotImplementedError(f"advantage estimator {est!r} is outside this build (GAE and GRPO only)")
 
 
 # ------------------------------------------------------------------------------------ aggregation
@@ -365,7 +410,7 @@ class _ActorLoss(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, ref_log_prob, cfg):
-        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, scale,
+        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, drift_coef, scale,
          policy_only) = cfg
         dev = log_prob.device
         lp = _as_2d(_f32(log_prob, dev))
@@ -388,7 +433,7 @@ class _ActorLoss(torch.autograd.Function):
             rc = _lib.lib().siirl_actor_loss_fwd(
                 _lib.ptr(old), _lib.ptr(lp), _lib.ptr(adv), _lib.ptr(m), mcode, _lib.ptr(isw), _lib.ptr(ent),
                 _lib.ptr(ref), B, L, loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st,
-                kl_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s), _lib.ptr(ws), nws,
+                kl_coef, drift_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s), _lib.ptr(ws), nws,
                 _lib.current_stream(dev))
         _lib.check(rc, "siirl_actor_loss_fwd")
         ctx.save_for_backward(lp, old, adv, m, out16, row_msum, row_s,
@@ -397,7 +442,7 @@ class _ActorLoss(torch.autograd.Function):
         ctx.meta = (mcode, B, L, cfg, log_prob.shape, log_prob.dtype,
                     None if entropy is None else (entropy.shape, entropy.dtype))
         ctx.set_materialize_grads(False)
-        outs = tuple(out16[i] for i in range(12))
+        outs = tuple(out16[i] for i in range(13))
         diff = (O_PG,) if policy_only else (O_LOSS,)
         ctx.mark_non_differentiable(*(o for i, o in enumerate(outs) if i not in diff))
         ctx.diff_index = diff[0]
@@ -415,7 +460,8 @@ class _ActorLoss(torch.autograd.Function):
         ent = rest.pop(0) if has_ent else None
         ref = rest.pop(0) if has_ref else None
         mcode, B, L, cfg, lp_shape, lp_dtype, ent_meta = ctx.meta
-        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, scale, _) = cfg
+        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, drift_coef, scale,
+         _) = cfg
         dev = lp.device
         g = g.detach().to(torch.float32).reshape(1).contiguous()
         d_lp = torch.empty(B, L, dtype=torch.float32, device=dev)
@@ -424,7 +470,8 @@ class _ActorLoss(torch.autograd.Function):
             rc = _lib.lib().siirl_actor_loss_bwd(
                 _lib.ptr(g), _lib.ptr(old), _lib.ptr(lp), _lib.ptr(adv), _lib.ptr(m), mcode, _lib.ptr(isw),
                 _lib.ptr(ent), _lib.ptr(ref), B, L, loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef,
-                kl_code, kl_st, kl_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s), _lib.ptr(d_lp),
+                kl_code, kl_st, kl_coef, drift_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s),
+                _lib.ptr(d_lp),
                 _lib.ptr(d_ent), _lib.current_stream(dev))
         _lib.check(rc, "siirl_actor_loss_bwd")
         g_lp = d_lp.reshape(lp_shape).to(lp_dtype)
@@ -442,7 +489,7 @@ def _clip_params(config):
 def _policy_only(loss_mode, old_log_prob, log_prob, advantages, response_mask, agg_code, lo, hi, c, dclamp,
                  rollout_is_weights):
     _gpu_of(log_prob)
-    cfg = (loss_mode, lo, hi, float(c), float(dclamp), agg_code, 0.0, 0, 0, 0.0, 1.0, True)
+    cfg = (loss_mode, lo, hi, float(c), float(dclamp), agg_code, 0.0, 0, 0, 0.0, 0.0, 1.0, True)
     outs = _ActorLoss.apply(log_prob, None, old_log_prob, advantages, response_mask, rollout_is_weights, None, cfg)
     return outs[O_PG], outs[O_CLIPFRAC], outs[O_PPOKL], outs[O_CLIPLOWER]
 
@@ -481,18 +528,118 @@ def compute_policy_loss_gspo(old_log_prob: torch.Tensor, log_prob: torch.Tensor,
                         AGG_MODES["seq-mean-token-mean"], lo, hi, 3.0, 20.0, rollout_is_weights)
 
 
+def _check_cpgd_bounds(lo, hi):
+    import math
+
+    math.log(1 + hi), math.log(1 - lo)  # raises the reference's ValueError ("math domain error") for eps >= 1
+
+
+@register_policy_loss("cpgd")
+def compute_policy_loss_cpgd(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                             response_mask: torch.Tensor, loss_agg_mode: str = "token-mean", config=None,
+                             rollout_is_weights: Optional[torch.Tensor] = None):
+    """CPGD (reference ``core_algos.py:572-629``): the log-probability is clipped at ``old + log(1 + eps_high)``
+    for positive advantages and at ``old + log(1 - eps_low)`` otherwise; ``rollout_is_weights`` is accepted
+    and not used, as in the reference."""
+    assert config is not None, "Config must be provided for CPGD loss"
+    lo, hi = _clip_params(config)
+    c = config.clip_ratio_c if getattr(config, "clip_ratio_c", None) is not None else 3.0
+    assert c > 1.0, f"clip_ratio_c ({c}) must be > 1.0"
+    _check_cpgd_bounds(lo, hi)
+    return _policy_only(LOSS_CPGD, old_log_prob, log_prob, advantages, response_mask, _agg_code(loss_agg_mode),
+                        lo, hi, c, 20.0, None)
+
+
+@register_policy_loss("gpg")
+def compute_policy_loss_gpg(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                            response_mask: torch.Tensor, loss_agg_mode: str = "token-mean", config=None,
+                            rollout_is_weights: Optional[torch.Tensor] = None):
+    """GPG (reference ``core_algos.py:865-895``): ``agg_loss(-log_prob * advantages [* weights])``.  The three
+    metrics are zeros -- on the device here, where the reference returns host scalars (``:895``)."""
+    old = log_prob.detach() if old_log_prob is None else old_log_prob
+    return _policy_only(LOSS_GPG, old, log_prob, advantages, response_mask, _agg_code(loss_agg_mode),
+                        0.2, 0.2, 3.0, 20.0, rollout_is_weights)
+
+
+@register_policy_loss("geo_mean")
+def compute_policy_loss_geo_mean(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                 response_mask: torch.Tensor, loss_agg_mode: str = "token-mean", config=None,
+                                 rollout_is_weights: Optional[torch.Tensor] = None):
+    """GMPO (reference ``core_algos.py:1074-1153``): per sequence ``-mean(A) * exp(mean clipped log-ratio)``, the
+    log-ratio clipped to ``[-eps_low, eps_high]`` on the side that the advantage's sign makes optimistic;
+    plain mean over sequences, ``loss_agg_mode`` is not used.  The reference additionally asserts that
+    ``config`` is not its ``ActorArguments`` class (``:1104``), which every stock actor violates; that check on
+    the reference's own type has no counterpart here."""
+    assert config is not None
+    lo, hi = _clip_params(config)
+    _agg_code(loss_agg_mode)
+    return _policy_only(LOSS_GEO_MEAN, old_log_prob, log_prob, advantages, response_mask,
+                        AGG_MODES["token-mean"], lo, hi, 3.0, 20.0, rollout_is_weights)
+
+
+class _ValueLoss(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, vpreds, returns, values, response_mask, cliprange_value, agg_code):
+        dev = vpreds.device
+        vp = _as_2d(_f32(vpreds, dev))
+        B, L = vp.shape
+        ret = _as_2d(_f32(returns, dev))
+        val = _as_2d(_f32(values, dev))
+        m, mcode = _mask_arg(_as_2d(response_mask), dev)
+        for name, t in (("returns", ret), ("values", val), ("response_mask", m)):
+            if tuple(t.shape) != (B, L):
+                raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {(B, L)}")
+        out16 = torch.empty(16, dtype=torch.float32, device=dev)
+        row_msum = torch.empty(B, dtype=torch.float32, device=dev)
+        ws, nws = _workspace(B, L, dev)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().siirl_value_loss_fwd(_lib.ptr(vp), _lib.ptr(ret), _lib.ptr(val), _lib.ptr(m), mcode, B, L,
+                                                 float(cliprange_value), agg_code, _lib.ptr(out16),
+                                                 _lib.ptr(row_msum), _lib.ptr(ws), nws, _lib.current_stream(dev))
+        _lib.check(rc, "siirl_value_loss_fwd")
+        ctx.save_for_backward(vp, ret, val, m, out16, row_msum)
+        ctx.meta = (mcode, B, L, float(cliprange_value), agg_code, vpreds.shape, vpreds.dtype)
+        loss, frac = out16[O_LOSS], out16[O_CLIPFRAC]
+        ctx.mark_non_differentiable(frac)
+        return loss, frac
+
+    @staticmethod
+    def backward(ctx, g, _):
+        vp, ret, val, m, out16, row_msum = ctx.saved_tensors
+        mcode, B, L, clip, agg_code, shape, dtype = ctx.meta
+        dev = vp.device
+        g = g.detach().to(torch.float32).reshape(1).contiguous()
+        d = torch.empty(B, L, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().siirl_value_loss_bwd(_lib.ptr(g), _lib.ptr(vp), _lib.ptr(ret), _lib.ptr(val), _lib.ptr(m),
+                                                 mcode, B, L, clip, agg_code, _lib.ptr(out16), _lib.ptr(row_msum),
+                                                 _lib.ptr(d), _lib.current_stream(dev))
+        _lib.check(rc, "siirl_value_loss_bwd")
+        return d.reshape(shape).to(dtype), None, None, None, None, None
+
+
+def compute_value_loss(vpreds: torch.Tensor, returns: torch.Tensor, values: torch.Tensor, response_mask: torch.Tensor,
+                       cliprange_value: float, loss_agg_mode: str = "token-mean"):
+    """Clipped value loss of the critic (reference ``core_algos.py:1173-1212``).  Returns ``(vf_loss,
+    vf_clipfrac)`` as 0-d device tensors; ``vf_loss`` carries the gradient to ``vpreds``."""
+    _gpu_of(vpreds)
+    return _ValueLoss.apply(vpreds, returns, values, response_mask, cliprange_value, _agg_code(loss_agg_mode))
+
+
 def compute_policy_loss(old_log_prob, log_prob, advantages, response_mask, cliprange=None, cliprange_low=None,
                         cliprange_high=None, clip_ratio_c=3.0, loss_agg_mode: str = "token-mean", use_cpgd_loss=False):
     """The legacy entry (reference ``core_algos.py:631-707``): as ``vanilla`` but the log-ratio is not clamped
-    to +-20.  The CPGD variant (``use_cpgd_loss=True``) is outside this build."""
+    to +-20; ``use_cpgd_loss=True`` gives the CPGD loss (``:682-691``)."""
     assert clip_ratio_c > 1.0, (
         "The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0,"
         + f" but get the value: {clip_ratio_c}."
     )
-    if use_cpgd_loss:
-        raise NotImplementedError("the CPGD loss is outside this build")
     lo = cliprange if cliprange_low is None else cliprange_low
     hi = cliprange if cliprange_high is None else cliprange_high
+    if use_cpgd_loss:
+        _check_cpgd_bounds(float(lo), float(hi))
+        return _policy_only(LOSS_CPGD, old_log_prob, log_prob, advantages, response_mask, _agg_code(loss_agg_mode),
+                            float(lo), float(hi), clip_ratio_c, float("inf"), None)
     return _policy_only(LOSS_VANILLA, old_log_prob, log_prob, advantages, response_mask, _agg_code(loss_agg_mode),
                         float(lo), float(hi), clip_ratio_c, float("inf"), None)
 
@@ -572,7 +719,7 @@ class ActorLossOutput:
     the device; ``metrics()`` fetches them with a single device-to-host copy."""
 
     _NAMES = ("loss", "pg_loss", "pg_clipfrac", "ppo_kl", "pg_clipfrac_lower", "entropy_loss", "kl_loss",
-              "ratio_mean", "ratio_min", "ratio_max", "mask_total", "policy_loss")
+              "ratio_mean", "ratio_min", "ratio_max", "mask_total", "policy_loss", "policy_drift_loss")
 
     def __init__(self, outs, loss_scale, kl_coef, has_kl, has_entropy):
         self._outs = outs
@@ -602,16 +749,23 @@ def actor_loss(old_log_prob, log_prob, advantages, response_mask, config, entrop
     ``siirl/engine/actor/dp_actor.py:455-500``), fused:
     ``loss = (pg_loss - entropy_coeff * agg(entropy) + kl_loss_coef * agg(kl_penalty(log_prob, ref))) * scale``.
     ``config`` carries ``clip_ratio*``, ``entropy_coeff``, ``use_kl_loss``, ``kl_loss_coef``, ``kl_loss_type``,
-    ``loss_agg_mode`` and ``policy_loss.loss_mode`` (or ``loss_mode``).  The entropy term is used when
-    ``entropy`` is given and ``entropy_coeff != 0``; the KL term when ``config.use_kl_loss``."""
+    ``loss_agg_mode``, ``policy_loss.loss_mode`` (or ``loss_mode``; vanilla, gspo, cpgd, gpg or geo_mean) and
+    ``use_cpgd_loss`` / ``policy_drift_coeff``.  The entropy term is used when ``entropy`` is given and
+    ``entropy_coeff != 0``; the KL term when ``config.use_kl_loss``; the drift term
+    ``policy_drift_coeff * agg(clamp(exp(lp - old) - 1, max=2) * lp)`` (``dp_actor.py:488-494``) when
+    ``config.use_cpgd_loss`` and the coefficient is non-zero."""
     _gpu_of(log_prob)
     mode = getattr(getattr(config, "policy_loss", None), "loss_mode", None) or getattr(config, "loss_mode", "vanilla")
-    if mode not in ("vanilla", "gspo"):
-        raise ValueError(f"Unsupported loss mode: {mode}. Supported modes are: ['vanilla', 'gspo']")
+    if mode not in _LOSS_CODES:
+        raise ValueError(f"Unsupported loss mode: {mode}. Supported modes are: {sorted(_LOSS_CODES)}")
     lo, hi = _clip_params(config)
-    c = float(getattr(config, "clip_ratio_c", 3.0))
-    if mode == "vanilla":
+    c = getattr(config, "clip_ratio_c", 3.0)
+    c = 3.0 if c is None else float(c)
+    if mode in ("vanilla", "cpgd"):
         assert c > 1.0, f"The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0, but get the value: {c}."
+    if mode == "cpgd":
+        _check_cpgd_bounds(lo, hi)
+    drift = float(getattr(config, "policy_drift_coeff", 0.0) or 0.0) if getattr(config, "use_cpgd_loss", False) else 0.0
     agg_code = _agg_code(getattr(config, "loss_agg_mode", "token-mean"))
     ent_coef = float(getattr(config, "entropy_coeff", 0.0))
     use_ent = entropy is not None and ent_coef != 0
@@ -624,8 +778,8 @@ def actor_loss(old_log_prob, log_prob, advantages, response_mask, config, entrop
         if kl_type not in KL_MODES:
             raise NotImplementedError
         kl_code, kl_coef = KL_MODES[kl_type], float(getattr(config, "kl_loss_coef", 0.001))
-    cfg = (LOSS_GSPO if mode == "gspo" else LOSS_VANILLA, lo, hi, c, 20.0, agg_code, ent_coef if use_ent else 0.0,
-           kl_code, 0, kl_coef, float(loss_scale_factor), False)
+    cfg = (_LOSS_CODES[mode], lo, hi, c, 20.0, agg_code, ent_coef if use_ent else 0.0,
+           kl_code, 0, kl_coef, drift, float(loss_scale_factor), False)
     outs = _ActorLoss.apply(log_prob, entropy if use_ent else None, old_log_prob, advantages, response_mask,
-                            rollout_is_weights, ref_log_prob if use_kl else None, cfg)
+                            None if mode == "cpgd" else rollout_is_weights, ref_log_prob if use_kl else None, cfg)
     return ActorLossOutput(outs, float(loss_scale_factor), kl_coef, use_kl, use_ent)

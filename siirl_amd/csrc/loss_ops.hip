@@ -1,9 +1,12 @@
-// [B, L] loss arithmetic of the actor update: clipped policy-gradient loss (PPO / GRPO / DAPO "vanilla",
-// GSPO), KL penalty, masked aggregation, and their hand-written backward.
+// [B, L] loss arithmetic of the actor and critic updates: the registered policy-gradient losses (PPO / GRPO /
+// DAPO "vanilla", GSPO, CPGD, GPG, GMPO "geo_mean"), the CPGD drift term, the clipped value loss, KL penalty,
+// masked aggregation, and their hand-written backward.
 //
-// Replaces, of siirl/dag_worker/core_algos.py:  agg_loss :536-569, compute_policy_loss_vanilla :710-792,
-// compute_policy_loss_gspo :795-862, kl_penalty :1215-1276; of siirl/utils/model_utils/torch_functional.py:
-// masked_sum / masked_mean :146-168; and the composition of siirl/engine/actor/dp_actor.py:455-513.
+// Replaces, of siirl/dag_worker/core_algos.py:  agg_loss :536-569, compute_policy_loss_cpgd :572-629,
+// compute_policy_loss_vanilla :710-792, compute_policy_loss_gspo :795-862, compute_policy_loss_gpg :865-895,
+// compute_policy_loss_geo_mean :1074-1153, compute_value_loss :1173-1212, kl_penalty :1215-1276; of
+// siirl/utils/model_utils/torch_functional.py: masked_sum / masked_mean :146-168; and the composition of
+// siirl/engine/actor/dp_actor.py:455-513 (drift term :488-494).
 //
 // Shape of the computation: one workgroup reduces a segment of kSeg tokens of one row into kNP partial
 // sums (LDS tree per partial), a single-workgroup finish kernel folds segments into rows and rows into
@@ -21,7 +24,7 @@ constexpr int kNP = 12;     // partials per segment (see enum P)
 enum P { P_PG = 0, P_M, P_CLIP, P_NEGD, P_LOWER, P_ENT, P_KL, P_RSUM, P_RMIN, P_RMAX, P_AUX0, P_AUX1 };
 // out[] of the finish kernel
 enum O { O_LOSS = 0, O_PG, O_CLIPFRAC, O_PPOKL, O_CLIPLOWER, O_ENTLOSS, O_KLLOSS, O_RMEAN, O_RMIN, O_RMAX,
-         O_MTOTAL, O_POLICY, O_COUNT = 16 };
+         O_MTOTAL, O_POLICY, O_DRIFT, O_COUNT = 16 };
 
 struct LossArgs {
   const float* old_lp;   // [B,L] or null (kind == KIND_AGG)
@@ -37,11 +40,12 @@ struct LossArgs {
   int aux_agg_mode;      // aggregation of the entropy and KL terms
   int kl_mode, kl_st;
   float eps_lo, eps_hi, clip_c, dclamp;
-  float ent_coef, kl_coef, scale;
+  float log_lo, log_hi;  // CPGD: float(log(1 - eps_lo)), float(log(1 + eps_hi)), logarithms taken in double
+  float ent_coef, kl_coef, drift_coef, scale;
   int64_t B, L;
   int nseg;
 };
-enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2 };
+enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6 };
 
 // torch.clamp / torch.maximum / torch.minimum semantics (NaN propagates)
 __device__ __forceinline__ float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
@@ -85,13 +89,71 @@ struct PgOut {
   float clip, lower, negd, r_raw;
 };
 
-// seq_s: GSPO's sequence-level mean log-ratio (unused for vanilla)
+// seq_s: GSPO's sequence-level mean log-ratio (unused otherwise).  For KIND_GEO tok is the token's clipped
+// log-ratio x (the loss itself is per sequence); for KIND_VALUE lp = vpreds, old = values, A = returns and
+// eps_lo = cliprange_value.
 __device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A, float isw, float seq_s,
-                                          float eps_lo, float eps_hi, float clip_c, float dclamp) {
+                                          const LossArgs& a) {
+  const float eps_lo = a.eps_lo, eps_hi = a.eps_hi, clip_c = a.clip_c, dclamp = a.dclamp;
   PgOut o;
   const float raw = lp - old;
   o.r_raw = expf(raw);
   const float lo = 1.f - eps_lo, hi = 1.f + eps_hi;
+  if (kind == KIND_CPGD) {
+    // the log-probability is clipped, not the ratio; importance weights are not used by this loss
+    o.negd = -raw;
+    float clipped;
+    bool pass;
+    if (A > 0.f) {
+      const float b = a.log_hi + old;
+      clipped = lp > b ? b : lp;
+      pass = lp <= b;
+      o.clip = o.r_raw > hi ? 1.f : 0.f;
+    } else {
+      const float b = a.log_lo + old;
+      clipped = lp < b ? b : lp;
+      pass = lp >= b;
+      o.clip = o.r_raw < lo ? 1.f : 0.f;
+    }
+    o.tok = -clipped * A;
+    o.dtok = pass ? -A : 0.f;
+    o.lower = (o.r_raw > clip_c && A < 0.f) ? 1.f : 0.f;
+    return o;
+  }
+  if (kind == KIND_GPG) {
+    o.negd = 0.f; o.clip = 0.f; o.lower = 0.f;
+    o.tok = -lp * A * isw;
+    o.dtok = -A * isw;
+    return o;
+  }
+  if (kind == KIND_GEO) {
+    o.negd = -raw;
+    const float sgn = A > 0.f ? 1.f : (A < 0.f ? -1.f : (A == 0.f ? 0.f : A));  // torch.sign; NaN stays NaN
+    const float dc = clampf(raw, -eps_lo, eps_hi);
+    const float p = sgn * raw, q = sgn * dc;
+    o.tok = sgn * tmin(p, q);
+    const bool inside = raw >= -eps_lo && raw <= eps_hi;  // then p == q and both sides of the min pass 1/2
+    o.dtok = (inside || p < q) ? sgn * sgn : 0.f;
+    const bool clipped = raw != dc;
+    o.clip = (clipped && A > 0.f) ? 1.f : 0.f;
+    o.lower = (clipped && A < 0.f) ? 1.f : 0.f;
+    return o;
+  }
+  if (kind == KIND_VALUE) {
+    o.negd = 0.f; o.lower = 0.f; o.r_raw = 1.f;
+    const float vmax = old + eps_lo, vmin = old - eps_lo;
+    const float inner = tmin(lp, vmax), vc = tmax(inner, vmin);
+    const float e1 = lp - A, e2 = vc - A;
+    const float l1 = e1 * e1, l2 = e2 * e2;
+    o.tok = tmax(l1, l2);
+    o.clip = l2 > l1 ? 1.f : 0.f;
+    const float dinner = lp < vmax ? 1.f : (lp == vmax ? 0.5f : 0.f);
+    const float dvc = inner > vmin ? dinner : (inner == vmin ? 0.5f * dinner : 0.f);
+    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    o.dtok = w1 * 2.f * e1 + w2 * 2.f * e2 * dvc;
+    return o;
+  }
   if (kind == KIND_VANILLA) {
     const float d = clampf(raw, -dclamp, dclamp);
     const float r = expf(d);
@@ -138,42 +200,62 @@ __device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A
 
 // ---------------------------------------------------------------------------- row pre-pass (GSPO)
 
-// rowstat[b] = { sum_t (lp - old) * m , sum_t m } per segment -> partials[b][seg][AUX0/AUX1]
-__global__ __launch_bounds__(kThreads) void gspo_prepass_kernel(LossArgs a, float* __restrict__ pre) {
+// per segment: GSPO { sum_t (lp - old) * m, sum_t m };  GEO { sum_t x * m, sum_t m, sum_t A * m,
+// sum_t log(isw + 1e-10) * m }, x the token's clipped log-ratio
+constexpr int kNPre = 4;
+__global__ __launch_bounds__(kThreads) void row_prepass_kernel(LossArgs a, float* __restrict__ pre) {
   const int64_t b = blockIdx.x / a.nseg;
   const int seg = blockIdx.x % a.nseg;
   const int64_t t0 = (int64_t)seg * kSeg;
-  float sd = 0.f, sm = 0.f;
+  float sd = 0.f, sm = 0.f, sa = 0.f, sw = 0.f;
   for (int i = threadIdx.x; i < kSeg; i += kThreads) {
     const int64_t t = t0 + i;
     if (t < a.L) {
       const int64_t idx = b * a.L + t;
       const float m = load_mask(a.mask, a.mask_dtype, idx);
-      sd += (a.lp[idx] - a.old_lp[idx]) * m;
       sm += m;
+      if (a.kind == KIND_GSPO) {
+        sd += (a.lp[idx] - a.old_lp[idx]) * m;
+      } else {
+        const float A = a.adv[idx];
+        sd += pg_token(KIND_GEO, a.lp[idx], a.old_lp[idx], A, 1.f, 0.f, a).tok * m;
+        sa += A * m;
+        if (a.isw) sw += logf(a.isw[idx] + 1e-10f) * m;
+      }
     }
   }
   __shared__ float sh[kThreads / kWave + 1];
   sd = block_sum(sd, sh);
   sm = block_sum(sm, sh);
+  sa = block_sum(sa, sh);
+  sw = block_sum(sw, sh);
   if (threadIdx.x == 0) {
-    pre[(b * a.nseg + seg) * 2 + 0] = sd;
-    pre[(b * a.nseg + seg) * 2 + 1] = sm;
+    float* p = pre + (b * a.nseg + seg) * kNPre;
+    p[0] = sd; p[1] = sm; p[2] = sa; p[3] = sw;
   }
 }
 
-// folds the pre-pass segments of each row: row_s[b] = sum d*m / max(sum m, 1)
-__global__ __launch_bounds__(kThreads) void gspo_rowfinish_kernel(const float* __restrict__ pre, int nseg, int64_t B,
-                                                                  float* __restrict__ row_s) {
+// folds the pre-pass segments of each row.  GSPO: row_s[b] = sum d*m / max(sum m, 1).  GEO: row_s[b] is the
+// sequence's loss -adv_b * exp(sum x*m / (n + 1e-8)) [* exp(sum log(w + 1e-10)*m / (n + 1e-8))], adv_b =
+// sum A*m / (n + 1e-8), in the reference's float32 arithmetic.
+__global__ __launch_bounds__(kThreads) void row_finish_kernel(const float* __restrict__ pre, int nseg, int64_t B,
+                                                              int kind, int has_isw, float* __restrict__ row_s) {
   const int64_t b = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   if (b >= B) return;
-  double sd = 0.0, sm = 0.0;
+  double sd = 0.0, sm = 0.0, sa = 0.0, sw = 0.0;
   for (int s = 0; s < nseg; ++s) {
-    sd += pre[(b * nseg + s) * 2 + 0];
-    sm += pre[(b * nseg + s) * 2 + 1];
+    const float* p = pre + (b * nseg + s) * kNPre;
+    sd += p[0]; sm += p[1]; sa += p[2]; sw += p[3];
   }
-  const float n = fmaxf((float)sm, 1.f);  // .clamp(min=1)
-  row_s[b] = (float)sd / n;
+  if (kind == KIND_GSPO) {
+    const float n = fmaxf((float)sm, 1.f);  // .clamp(min=1)
+    row_s[b] = (float)sd / n;
+  } else {
+    const float n = (float)sm + 1e-8f;
+    float v = -((float)sa / n) * expf((float)sd / n);
+    if (has_isw) v *= expf((float)sw / n);
+    row_s[b] = v;
+  }
 }
 
 // ---------------------------------------------------------------------------- segment partials
@@ -202,8 +284,8 @@ __global__ __launch_bounds__(kThreads) void loss_partials_kernel(LossArgs a, con
     }
     const float lp = a.lp[idx];
     const float isw = a.isw ? a.isw[idx] : 1.f;
-    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a.eps_lo, a.eps_hi, a.clip_c, a.dclamp);
-    acc[P_PG] += contrib(o.tok, m, a.agg_mode);
+    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a);
+    if (a.kind != KIND_GEO) acc[P_PG] += contrib(o.tok, m, a.agg_mode);  // GEO: the loss is per sequence (row_s)
     acc[P_CLIP] += contrib_where(o.clip, m);
     acc[P_NEGD] += contrib_where(o.negd, m);
     acc[P_LOWER] += contrib_where(o.lower, m);
@@ -212,6 +294,7 @@ __global__ __launch_bounds__(kThreads) void loss_partials_kernel(LossArgs a, con
     acc[P_RMAX] = fmaxf(acc[P_RMAX], o.r_raw);
     if (a.ent) acc[P_ENT] += contrib(a.ent[idx], m, a.aux_agg_mode);
     if (a.ref) acc[P_KL] += contrib(kl_token(lp, a.ref[idx], a.kl_mode, 0).v, m, a.aux_agg_mode);
+    if (a.drift_coef != 0.f) acc[P_AUX0] += contrib(clamp_max(o.r_raw - 1.f, 2.f) * lp, m, a.aux_agg_mode);
   }
 
   __shared__ float sh[kThreads / kWave + 1];
@@ -265,9 +348,10 @@ __device__ __forceinline__ double finish_term(double total, double mtotal, int a
 }
 
 __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const float* __restrict__ partials,
+                                                               const float* __restrict__ row_s,
                                                                float* __restrict__ out,
                                                                float* __restrict__ row_msum) {
-  double t_pg = 0, t_m = 0, t_clip = 0, t_negd = 0, t_lower = 0, t_ent = 0, t_kl = 0, t_rsum = 0;
+  double t_pg = 0, t_m = 0, t_clip = 0, t_negd = 0, t_lower = 0, t_ent = 0, t_kl = 0, t_rsum = 0, t_drift = 0;
   float rmin = __builtin_inff(), rmax = -__builtin_inff();
   for (int64_t b = threadIdx.x; b < a.B; b += kThreads) {
     double r[kNP];
@@ -282,7 +366,8 @@ __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const
     }
     row_msum[b] = (float)r[P_M];
     t_m += r[P_M];
-    t_pg += row_term(r[P_PG], r[P_M], a.agg_mode);
+    t_pg += a.kind == KIND_GEO ? (double)row_s[b] : row_term(r[P_PG], r[P_M], a.agg_mode);
+    t_drift += row_term(r[P_AUX0], r[P_M], a.aux_agg_mode);
     t_ent += row_term(r[P_ENT], r[P_M], a.aux_agg_mode);
     t_kl += row_term(r[P_KL], r[P_M], a.aux_agg_mode);
     t_clip += r[P_CLIP];
@@ -299,6 +384,7 @@ __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const
   t_ent = block_sum_d(t_ent, sh);
   t_kl = block_sum_d(t_kl, sh);
   t_rsum = block_sum_d(t_rsum, sh);
+  t_drift = block_sum_d(t_drift, sh);
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {
     rmin = fminf(rmin, __shfl_xor(rmin, o, kWave));
@@ -316,10 +402,10 @@ __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const
       rmin = fminf(rmin, shm[w]);
       rmax = fmaxf(rmax, shm[kThreads / kWave + w]);
     }
-    const double pg = finish_term(t_pg, t_m, a.agg_mode, a.B, a.L);
+    const double pg = a.kind == KIND_GEO ? t_pg / (double)a.B : finish_term(t_pg, t_m, a.agg_mode, a.B, a.L);
     const double den = t_m + 1e-8;
     double policy = pg;
-    double entl = 0.0, kll = 0.0;
+    double entl = 0.0, kll = 0.0, drl = 0.0;
     if (a.ent) {
       entl = finish_term(t_ent, t_m, a.aux_agg_mode, a.B, a.L);
       policy = policy - entl * (double)a.ent_coef;
@@ -327,6 +413,10 @@ __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const
     if (a.ref) {
       kll = finish_term(t_kl, t_m, a.aux_agg_mode, a.B, a.L);
       policy = policy + kll * (double)a.kl_coef;
+    }
+    if (a.drift_coef != 0.f) {
+      drl = finish_term(t_drift, t_m, a.aux_agg_mode, a.B, a.L);
+      policy = policy + drl * (double)a.drift_coef;
     }
     for (int k = 0; k < O_COUNT; ++k) out[k] = 0.f;
     out[O_PG] = (float)pg;
@@ -339,6 +429,7 @@ __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const
       out[O_CLIPLOWER] = (float)(t_lower / den);
       out[O_ENTLOSS] = (float)entl;
       out[O_KLLOSS] = (float)kll;
+      out[O_DRIFT] = (float)drl;
       out[O_RMEAN] = (float)(t_rsum / (double)(a.B * a.L));
       out[O_RMIN] = rmin;
       out[O_RMAX] = rmax;
@@ -368,7 +459,7 @@ __global__ __launch_bounds__(kThreads) void loss_bwd_kernel(LossArgs a, const fl
   const float g = g_out[0] * a.scale;
   const float mtotal = saved_out[O_MTOTAL];
   const float mrow = row_msum[b];
-  const float seq_s = (a.kind == KIND_GSPO) ? row_s[b] : 0.f;
+  const float seq_s = (a.kind == KIND_GSPO || a.kind == KIND_GEO) ? row_s[b] : 0.f;
   for (int i = threadIdx.x; i < kSeg; i += kThreads) {
     const int64_t t = t0 + i;
     if (t >= a.L) break;
@@ -380,8 +471,14 @@ __global__ __launch_bounds__(kThreads) void loss_bwd_kernel(LossArgs a, const fl
     }
     const float lp = a.lp[idx];
     const float isw = a.isw ? a.isw[idx] : 1.f;
-    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a.eps_lo, a.eps_hi, a.clip_c, a.dclamp);
-    float d = agg_weight(a.agg_mode, m, mtotal, mrow, a.B, a.L) * o.dtok;
+    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a);
+    float d;
+    if (a.kind == KIND_GEO)  // d mean_b(row loss) / d x = row loss * m / (n + 1e-8) / B
+      d = seq_s * (m / (mrow + 1e-8f)) / (float)a.B * o.dtok;
+    else
+      d = agg_weight(a.agg_mode, m, mtotal, mrow, a.B, a.L) * o.dtok;
+    if (a.drift_coef != 0.f)  // the weight clamp(exp(lp - old) - 1, max = 2) is detached
+      d += a.drift_coef * agg_weight(a.aux_agg_mode, m, mtotal, mrow, a.B, a.L) * clamp_max(o.r_raw - 1.f, 2.f);
     if (a.ent || a.ref) {
       const float wa = agg_weight(a.aux_agg_mode, m, mtotal, mrow, a.B, a.L);
       if (a.ref) d += a.kl_coef * wa * kl_token(lp, a.ref[idx], a.kl_mode, a.kl_st).g;
@@ -474,7 +571,7 @@ int nseg_of(int64_t L) { return (int)((L + kSeg - 1) / kSeg); }
 
 size_t ws_bytes_of(int64_t B, int64_t L) {
   const size_t ns = (size_t)nseg_of(L);
-  return (size_t)B * ns * kNP * sizeof(float) + (size_t)B * ns * 2 * sizeof(float) + 256;
+  return (size_t)B * ns * kNP * sizeof(float) + (size_t)B * ns * kNPre * sizeof(float) + 256;
 }
 
 int check_dims(int64_t B, int64_t L) {
@@ -502,15 +599,16 @@ int run_forward(LossArgs& a, float* out16, float* row_msum, float* row_s, void* 
   float* partials = (float*)ws;
   float* pre = partials + (size_t)a.B * a.nseg * kNP;
   dim3 grid((unsigned)(a.B * a.nseg)), block(kThreads);
-  if (a.kind == KIND_GSPO) {
-    gspo_prepass_kernel<<<grid, block, 0, st>>>(a, pre);
-    SIIRL_LAUNCH_CHECK("gspo_prepass_kernel");
-    gspo_rowfinish_kernel<<<dim3((unsigned)((a.B + kThreads - 1) / kThreads)), block, 0, st>>>(pre, a.nseg, a.B, row_s);
-    SIIRL_LAUNCH_CHECK("gspo_rowfinish_kernel");
+  if (a.kind == KIND_GSPO || a.kind == KIND_GEO) {
+    row_prepass_kernel<<<grid, block, 0, st>>>(a, pre);
+    SIIRL_LAUNCH_CHECK("row_prepass_kernel");
+    row_finish_kernel<<<dim3((unsigned)((a.B + kThreads - 1) / kThreads)), block, 0, st>>>(pre, a.nseg, a.B, a.kind,
+                                                                                       a.isw != nullptr, row_s);
+    SIIRL_LAUNCH_CHECK("row_finish_kernel");
   }
   loss_partials_kernel<<<grid, block, 0, st>>>(a, row_s, partials);
   SIIRL_LAUNCH_CHECK("loss_partials_kernel");
-  loss_finish_kernel<<<1, block, 0, st>>>(a, partials, out16, row_msum);
+  loss_finish_kernel<<<1, block, 0, st>>>(a, partials, row_s, out16, row_msum);
   SIIRL_LAUNCH_CHECK("loss_finish_kernel");
   return SIIRL_OK;
 }
@@ -558,24 +656,31 @@ static int fill_actor_args(LossArgs& a, const float* old_log_prob, const float* 
                            const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
                            const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
                            float clip_high, float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode,
-                           int kl_straight_through, float kl_coef, float loss_scale) {
+                           int kl_straight_through, float kl_coef, float policy_drift_coeff, float loss_scale) {
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   if (int rc = check_agg(agg_mode)) return rc;
-  SIIRL_REQUIRE(loss_mode == SIIRL_LOSS_VANILLA || loss_mode == SIIRL_LOSS_GSPO, "Unsupported loss mode: %d", loss_mode);
+  SIIRL_REQUIRE(loss_mode >= SIIRL_LOSS_VANILLA && loss_mode <= SIIRL_LOSS_GEO_MEAN, "Unsupported loss mode: %d",
+                loss_mode);
   SIIRL_REQUIRE(old_log_prob && log_prob && advantages && mask, "NULL operand");
-  if (loss_mode == SIIRL_LOSS_VANILLA)
+  if (loss_mode == SIIRL_LOSS_VANILLA || loss_mode == SIIRL_LOSS_CPGD)
     SIIRL_REQUIRE(clip_c > 1.0f, "clip_ratio_c must be greater than 1.0, got %f", (double)clip_c);
+  if (loss_mode == SIIRL_LOSS_CPGD) {
+    SIIRL_REQUIRE(clip_low < 1.0f && clip_high > -1.0f, "CPGD takes log(1 - clip_low) and log(1 + clip_high)");
+    a.log_lo = (float)log(1.0 - (double)clip_low);
+    a.log_hi = (float)log(1.0 + (double)clip_high);
+  }
   SIIRL_REQUIRE(log_ratio_clamp > 0.f, "log_ratio_clamp must be positive (20 in the reference, +inf for none)");
   if (ref_log_prob) SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
   a.old_lp = old_log_prob; a.lp = log_prob; a.adv = advantages; a.mask = mask; a.mask_dtype = mask_dtype;
   a.isw = is_weights; a.ent = entropy; a.ref = ref_log_prob;
-  a.kind = loss_mode == SIIRL_LOSS_GSPO ? KIND_GSPO : KIND_VANILLA;
+  static const int kind_of[] = {KIND_VANILLA, KIND_GSPO, KIND_CPGD, KIND_GPG, KIND_GEO};
+  a.kind = kind_of[loss_mode];
   a.agg_mode = loss_mode == SIIRL_LOSS_GSPO ? SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN : agg_mode;
   a.aux_agg_mode = agg_mode;
   a.kl_mode = kl_mode; a.kl_st = kl_straight_through;
   a.eps_lo = clip_low; a.eps_hi = clip_high; a.clip_c = clip_c; a.dclamp = log_ratio_clamp;
-  a.ent_coef = entropy_coeff; a.kl_coef = kl_coef; a.scale = loss_scale;
+  a.ent_coef = entropy_coeff; a.kl_coef = kl_coef; a.drift_coef = policy_drift_coeff; a.scale = loss_scale;
   a.B = B; a.L = L; a.nseg = nseg_of(L);
   return SIIRL_OK;
 }
@@ -584,16 +689,17 @@ extern "C" int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_
                                     const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
                                     const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
                                     float clip_high, float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode,
-                                    int kl_straight_through, float kl_coef, float loss_scale, float* out16,
+                                    int kl_straight_through, float kl_coef, float policy_drift_coeff, float loss_scale, float* out16,
                                     float* row_msum, float* row_s, void* workspace, size_t workspace_bytes,
                                     siirl_stream_t stream) {
   LossArgs a{};
   if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
                                ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff,
-                               kl_mode, kl_straight_through, kl_coef, loss_scale))
+                               kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale))
     return rc;
   SIIRL_REQUIRE(out16 && row_msum, "NULL output");
-  SIIRL_REQUIRE(loss_mode != SIIRL_LOSS_GSPO || row_s, "row_s is required for GSPO");
+  SIIRL_REQUIRE((loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
+                "row_s is required for the gspo and geo_mean losses");
   return run_forward(a, out16, row_msum, row_s, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
@@ -602,18 +708,56 @@ extern "C" int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_pr
                                     const float* is_weights, const float* entropy, const float* ref_log_prob,
                                     int64_t B, int64_t L, int loss_mode, float clip_low, float clip_high, float clip_c,
                                     float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode, int kl_straight_through,
-                                    float kl_coef, float loss_scale, const float* out16, const float* row_msum,
+                                    float kl_coef, float policy_drift_coeff, float loss_scale, const float* out16, const float* row_msum,
                                     const float* row_s, float* d_log_prob, float* d_entropy, siirl_stream_t stream) {
   LossArgs a{};
   if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
                                ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff,
-                               kl_mode, kl_straight_through, kl_coef, loss_scale))
+                               kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale))
     return rc;
   SIIRL_REQUIRE(g_loss && out16 && row_msum && d_log_prob, "NULL operand");
-  SIIRL_REQUIRE(loss_mode != SIIRL_LOSS_GSPO || row_s, "row_s is required for GSPO");
+  SIIRL_REQUIRE((loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
+                "row_s is required for the gspo and geo_mean losses");
   SIIRL_REQUIRE(entropy == nullptr || d_entropy != nullptr, "d_entropy is required when entropy is given");
   loss_bwd_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, (hipStream_t)stream>>>(a, g_loss, out16, row_msum,
                                                                                        row_s, d_log_prob, d_entropy);
+  SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
+  return SIIRL_OK;
+}
+
+static int fill_value_args(LossArgs& a, const float* vpreds, const float* returns, const float* values,
+                           const void* mask, int mask_dtype, int64_t B, int64_t L, float cliprange_value,
+                           int agg_mode) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  if (int rc = check_agg(agg_mode)) return rc;
+  SIIRL_REQUIRE(vpreds && returns && values && mask, "NULL operand");
+  a.old_lp = values; a.lp = vpreds; a.adv = returns; a.mask = mask; a.mask_dtype = mask_dtype;
+  a.kind = KIND_VALUE; a.agg_mode = agg_mode; a.aux_agg_mode = agg_mode;
+  a.eps_lo = cliprange_value; a.scale = 0.5f;
+  a.B = B; a.L = L; a.nseg = nseg_of(L);
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_value_loss_fwd(const float* vpreds, const float* returns, const float* values, const void* mask,
+                                    int mask_dtype, int64_t B, int64_t L, float cliprange_value, int agg_mode,
+                                    float* out16, float* row_msum, void* workspace, size_t workspace_bytes,
+                                    siirl_stream_t stream) {
+  LossArgs a{};
+  if (int rc = fill_value_args(a, vpreds, returns, values, mask, mask_dtype, B, L, cliprange_value, agg_mode)) return rc;
+  SIIRL_REQUIRE(out16 && row_msum, "NULL output");
+  return run_forward(a, out16, row_msum, nullptr, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int siirl_value_loss_bwd(const float* g_loss, const float* vpreds, const float* returns,
+                                    const float* values, const void* mask, int mask_dtype, int64_t B, int64_t L,
+                                    float cliprange_value, int agg_mode, const float* out16, const float* row_msum,
+                                    float* d_vpreds, siirl_stream_t stream) {
+  LossArgs a{};
+  if (int rc = fill_value_args(a, vpreds, returns, values, mask, mask_dtype, B, L, cliprange_value, agg_mode)) return rc;
+  SIIRL_REQUIRE(g_loss && out16 && row_msum && d_vpreds, "NULL operand");
+  loss_bwd_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, (hipStream_t)stream>>>(a, g_loss, out16, row_msum,
+                                                                                       nullptr, d_vpreds, nullptr);
   SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
   return SIIRL_OK;
 }

@@ -213,3 +213,56 @@ def masked_sum(values: torch.Tensor, mask: torch.Tensor, axis=None):
 def masked_mean(values: torch.Tensor, mask: torch.Tensor, axis=None):
     """``masked_sum / (mask.sum + 1e-8)`` (reference ``torch_functional.py:154-168``)."""
     return _masked_reduce(values, mask, axis, want_mean=True)
+
+
+def clip_by_value(x: torch.Tensor, tensor_min: torch.Tensor, tensor_max: torch.Tensor):
+    """``max(min(x, tensor_max), tensor_min)`` with tensor bounds (reference ``torch_functional.py:119-125``);
+    plain torch, it is not on the hot path by itself (the value loss fuses it)."""
+    return torch.max(torch.min(x, tensor_max), tensor_min)
+
+
+def _check_whiten_count(n: float):
+    """The two ``ValueError``s of the reference's ``masked_var`` (``torch_functional.py:178-184``)."""
+    if n == 0:
+        raise ValueError("At least one element in the mask has to be 1.")
+    if n == 1:
+        raise ValueError("The sum of the mask is one, which can cause a division by zero.")
+
+
+def _whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool):
+    from . import _lib
+    from . import core_algos as CA
+
+    if not values.is_cuda:
+        raise RuntimeError("siirl_amd: masked_var / masked_whiten run on the GPU only (no CPU fallback)")
+    dev = values.device
+    v = CA._f32(values, dev)
+    m, mcode = CA._mask_arg(mask.expand_as(values), dev)
+    out = torch.empty_like(v)
+    stats = torch.empty(3, dtype=torch.float32, device=dev)
+    nws = _lib.lib().siirl_whiten_workspace_bytes()
+    ws = torch.empty(nws, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().siirl_masked_whiten(_lib.ptr(v), _lib.ptr(m), mcode, v.numel(), int(bool(shift_mean)),
+                                            _lib.ptr(out), _lib.ptr(stats), _lib.ptr(ws), nws,
+                                            _lib.current_stream(dev))
+    _lib.check(rc, "siirl_masked_whiten")
+    return out, stats
+
+
+def masked_var(values: torch.Tensor, mask: torch.Tensor, unbiased: bool = True):
+    """Variance over the masked elements (reference ``torch_functional.py:171-187``), 0-d fp32."""
+    _, stats = _whiten(values, mask, True)
+    n = float(stats[2])
+    if unbiased:
+        _check_whiten_count(n)
+        return stats[1]
+    return stats[1] * ((n - 1.0) / n) if n > 1 else stats[1]
+
+
+def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = True):
+    """``(values - mean) * rsqrt(var + 1e-8)`` with masked mean and unbiased masked variance, applied to every
+    element (reference ``torch_functional.py:190-206``); no gradient (the reference uses it under ``no_grad``)."""
+    out, stats = _whiten(values, mask, shift_mean)
+    _check_whiten_count(float(stats[2]))
+    return out.reshape(values.shape)

@@ -248,6 +248,46 @@ int siirl_kl_in_reward(const float* token_level_scores, const float* old_log_pro
                        const void* mask, int mask_dtype, int64_t B, int64_t L, int kl_mode, float beta,
                        float* token_level_rewards, float* row_kl, float* current_kl, siirl_stream_t stream);
 
+/* ------------------------------------------------------------------- remove-padding bookkeeping */
+
+/*
+ * unpad_input's index computation for a 0/1 attention mask [B, S]: seqlens[b] = attended positions of row b,
+ * cu_seqlens[B + 1] = [0, cumsum(seqlens)] (int32, so B * S < 2^31), indices[0 .. nnz) = flat positions b * S + s
+ * of the attended tokens in ascending order (capacity B * S), info2 = {nnz, max seqlen}.
+ * Replaces: unpad_input of flash-attn's bert_padding (flash-attn 2.7.3 / 2.8.2) as called at
+ *           siirl/engine/actor/dp_actor.py:112.
+ */
+int siirl_unpad_indices(const void* attention_mask, int mask_dtype, int64_t B, int64_t S, int32_t* seqlens,
+                        int32_t* cu_seqlens, int64_t* indices, int64_t* info2, siirl_stream_t stream);
+
+/*
+ * index_first_axis: dst[j, :] = src[indices[j], :] for n rows of row_bytes (a multiple of 4) each; and pad_input:
+ * dst[total_rows, :] = 0, then dst[indices[j], :] = src[j, :].  Each is the other's backward.
+ * Replaces: index_first_axis / pad_input of flash-attn's bert_padding, siirl/engine/actor/dp_actor.py:117-119,215-226.
+ */
+int siirl_gather_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, void* dst,
+                      siirl_stream_t stream);
+int siirl_scatter_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, int64_t total_rows,
+                       void* dst, siirl_stream_t stream);
+
+/*
+ * ids_rmpad[j] = input_ids[indices[j]] and labels_rolled[j] = input_ids[indices[(j + 1) % nnz]]: the packed ids and
+ * the next-token labels in one pass (either output may be NULL).
+ * Replaces: unpad_input on input_ids + torch.roll(input_ids_rmpad, shifts=-1), siirl/engine/actor/dp_actor.py:112-127.
+ */
+int siirl_unpad_ids_labels(const int64_t* input_ids, const int64_t* indices, int64_t nnz, int64_t* ids_rmpad,
+                           int64_t* labels_rolled, siirl_stream_t stream);
+
+/*
+ * pad_input followed by the response window: out[b, t] = full[b, S - L - 1 + t], t in [0, L), where full is the
+ * zero-padded [B, S] scatter of values[nnz] at `indices` -- without materialising full.  The gather is its backward.
+ * Replaces: pad_input(...).squeeze(-1)[:, -response_length - 1 : -1], siirl/engine/actor/dp_actor.py:214-231.
+ */
+int siirl_response_scatter(const float* values, const int64_t* indices, int64_t nnz, int64_t B, int64_t S, int64_t L,
+                           float* out, siirl_stream_t stream);
+int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t S, int64_t L,
+                          float* d_values, siirl_stream_t stream);
+
 /* ------------------------------------------------------------------- GAE and masked whitening */
 
 /* Bytes of scratch siirl_masked_whiten / siirl_gae_advantage_return need (a constant; 8-byte aligned buffer). */

@@ -52,6 +52,9 @@ dynamic_sampling_keep_indices          worked example of the reference's docs
 make_uid / filter_by_indices           uid layout and ordered index select pinned by the
                                        reference's tests (tests/dag_worker/test_dapo_pipeline.py:14-49,
                                        tests/dag_worker/test_dapo_merge.py:90-120)
+unpad_input / pad_input / ...          transformers' pure-torch restatement of bert_padding
+                                       (modeling_flash_attention_utils._unpad_input / _pad_input);
+                                       pad(unpad(x)) == x * mask; hand-written left/right padding
 fused_linear_for_ppo_fwd / _bwd        equals logprob/entropy of ``(h @ W.T)/T`` in fp64 and
                                        autograd through that expression
 =====================================  ==========================================================
@@ -63,4 +66,4 @@ reference's CUDA dispatch target for ``logprobs_from_logits``) and of the Triton
 log-softmax / online softmax) instead.
 """
 
-from . import torch_functional, core_algos, dapo_filter, fused_linear, actor_step  # noqa: F401
+from . import torch_functional, core_algos, dapo_filter, fused_linear, actor_step, padding  # noqa: F401

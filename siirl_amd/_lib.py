@@ -32,6 +32,12 @@ SIGNATURES = {
                                     _i32, _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _p, _p, _p]),
     "siirl_value_loss_fwd": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _f32, _i32, _p, _p, _p, _sz, _p]),
     "siirl_value_loss_bwd": (_i32, [_p, _p, _p, _p, _p, _i32, _i64, _i64, _f32, _i32, _p, _p, _p, _p]),
+    "siirl_unpad_indices": (_i32, [_p, _i32, _i64, _i64, _p, _p, _p, _p, _p]),
+    "siirl_gather_rows": (_i32, [_p, _p, _i64, _i64, _p, _p]),
+    "siirl_scatter_rows": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
+    "siirl_unpad_ids_labels": (_i32, [_p, _p, _i64, _p, _p, _p]),
+    "siirl_response_scatter": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p]),
+    "siirl_response_gather": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
     "siirl_whiten_workspace_bytes": (_sz, []),
     "siirl_masked_whiten": (_i32, [_p, _p, _i32, _i64, _i32, _p, _p, _p, _sz, _p]),
     "siirl_gae_advantage_return": (_i32, [_p, _p, _p, _i32, _i64, _i64, _f64, _f64, _p, _p, _p, _p, _sz, _p]),

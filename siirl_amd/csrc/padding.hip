@@ -1,0 +1,249 @@
+// Remove-padding bookkeeping around the per-token loss path: token indices of the attended positions, gathers
+// to and scatters from the packed ("rmpad") layout, and the response window of the padded result.
+//
+// Replaces the calls the actor makes around its log-prob computation (siirl/engine/actor/dp_actor.py:112-127,
+// 214-231): flash-attn's bert_padding unpad_input / index_first_axis / pad_input (flash-attn 2.7.3 / 2.8.2, a
+// third-party dependency: indices = nonzero(mask.flatten()), cu_seqlens = [0, cumsum(mask.sum(-1))]),
+// torch.roll(input_ids_rmpad, -1) for the labels, and the [:, -response_length - 1 : -1] slice.
+// All of it is integer / index work: results are exact.
+#include "common.hpp"
+
+namespace siirl {
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ bool mask_on(const void* p, int dt, int64_t i) {
+  switch (dt) {
+    case SIIRL_U8: return ((const uint8_t*)p)[i] != 0;
+    case SIIRL_I64: return ((const int64_t*)p)[i] != 0;
+    case SIIRL_I32: return ((const int32_t*)p)[i] != 0;
+    case SIIRL_F32: return ((const float*)p)[i] != 0.f;
+    case SIIRL_BF16: return (((const uint16_t*)p)[i] & 0x7fffu) != 0;
+    case SIIRL_F16: return (((const uint16_t*)p)[i] & 0x7fffu) != 0;
+    default: return false;
+  }
+}
+
+// seqlens[b] = number of attended positions of row b
+__global__ __launch_bounds__(kThreads) void seqlens_kernel(const void* mask, int mask_dtype, int64_t S,
+                                                           int32_t* __restrict__ seqlens) {
+  const int64_t b = blockIdx.x;
+  int n = 0;
+  for (int64_t s = threadIdx.x; s < S; s += kThreads) n += mask_on(mask, mask_dtype, b * S + s) ? 1 : 0;
+  __shared__ double sh[kThreads / kWave + 1];
+  const double tot = block_sum((double)n, sh);  // exact for any count below 2^53
+  if (threadIdx.x == 0) seqlens[b] = (int32_t)tot;
+}
+
+// cu_seqlens[0] = 0, cu_seqlens[b + 1] = sum_{i <= b} seqlens[i]; info = {total, max seqlen}.  One workgroup.
+__global__ __launch_bounds__(kThreads) void cu_seqlens_kernel(const int32_t* __restrict__ seqlens, int64_t B,
+                                                              int32_t* __restrict__ cu, int64_t* __restrict__ info) {
+  __shared__ int32_t sh[kThreads];
+  __shared__ int32_t carry_s, max_s;
+  if (threadIdx.x == 0) {
+    carry_s = 0;
+    max_s = 0;
+    cu[0] = 0;
+  }
+  __syncthreads();
+  for (int64_t base = 0; base < B; base += kThreads) {
+    const int64_t i = base + threadIdx.x;
+    const int32_t v = i < B ? seqlens[i] : 0;
+    sh[threadIdx.x] = v;
+    __syncthreads();
+    for (int off = 1; off < kThreads; off <<= 1) {  // Hillis-Steele inclusive scan
+      const int32_t add = threadIdx.x >= off ? sh[threadIdx.x - off] : 0;
+      __syncthreads();
+      sh[threadIdx.x] += add;
+      __syncthreads();
+    }
+    const int32_t carry = carry_s;
+    if (i < B) cu[i + 1] = carry + sh[threadIdx.x];
+    atomicMax(&max_s, v);
+    __syncthreads();
+    if (threadIdx.x == 0) carry_s = carry + sh[kThreads - 1];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) {
+    info[0] = carry_s;
+    info[1] = max_s;
+  }
+}
+
+// indices[cu[b] + r] = b * S + s for the r-th attended position s of row b, in order.  One workgroup per row.
+__global__ __launch_bounds__(kThreads) void indices_kernel(const void* mask, int mask_dtype, int64_t S,
+                                                           const int32_t* __restrict__ cu,
+                                                           int64_t* __restrict__ indices) {
+  const int64_t b = blockIdx.x;
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
+  __shared__ int wave_cnt[kThreads / kWave];
+  __shared__ int base_s;
+  if (threadIdx.x == 0) base_s = cu[b];
+  __syncthreads();
+  for (int64_t s0 = 0; s0 < S; s0 += kThreads) {
+    const int64_t s = s0 + threadIdx.x;
+    const bool on = s < S && mask_on(mask, mask_dtype, b * S + s);
+    const unsigned long long bal = __ballot(on);
+    const int before = __popcll(bal & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_cnt[wid] = __popcll(bal);
+    __syncthreads();
+    int off = base_s;
+    for (int w = 0; w < wid; ++w) off += wave_cnt[w];
+    if (on) indices[off + before] = b * S + s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int t = 0;
+      for (int w = 0; w < kThreads / kWave; ++w) t += wave_cnt[w];
+      base_s += t;
+    }
+    __syncthreads();
+  }
+}
+
+// dst[j] = src[indices[j]] (GATHER) or dst[indices[j]] = src[j] (scatter), rows of `words` 4-byte words
+template <bool GATHER>
+__global__ __launch_bounds__(kThreads) void move_rows_kernel(const uint32_t* __restrict__ src,
+                                                             const int64_t* __restrict__ indices, int64_t n,
+                                                             int64_t words, uint32_t* __restrict__ dst) {
+  const int64_t total = n * words;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
+    const int64_t j = i / words, w = i - j * words;
+    const int64_t r = indices[j];
+    if (GATHER) dst[i] = src[r * words + w];
+    else dst[r * words + w] = src[i];
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* __restrict__ p, int64_t words) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < words; i += (int64_t)gridDim.x * kThreads) p[i] = 0u;
+}
+
+// ids_rmpad[j] = input_ids[indices[j]],  labels[j] = input_ids[indices[(j + 1) % nnz]]  (torch.roll(..., -1))
+__global__ __launch_bounds__(kThreads) void unpad_ids_kernel(const int64_t* __restrict__ input_ids,
+                                                             const int64_t* __restrict__ indices, int64_t nnz,
+                                                             int64_t* __restrict__ ids_rmpad,
+                                                             int64_t* __restrict__ labels) {
+  for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kThreads) {
+    if (ids_rmpad) ids_rmpad[j] = input_ids[indices[j]];
+    if (labels) labels[j] = input_ids[indices[j + 1 < nnz ? j + 1 : 0]];
+  }
+}
+
+// out[b, t] = values[j] for the j with indices[j] == b * S + (S - L - 1 + t); positions nobody writes stay 0
+__global__ __launch_bounds__(kThreads) void response_scatter_kernel(const float* __restrict__ values,
+                                                                    const int64_t* __restrict__ indices, int64_t nnz,
+                                                                    int64_t S, int64_t L, float* __restrict__ out) {
+  for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kThreads) {
+    const int64_t pos = indices[j], b = pos / S, t = pos - b * S - (S - L - 1);
+    if (t >= 0 && t < L) out[b * L + t] = values[j];
+  }
+}
+__global__ __launch_bounds__(kThreads) void response_gather_kernel(const float* __restrict__ grad,
+                                                                   const int64_t* __restrict__ indices, int64_t nnz,
+                                                                   int64_t S, int64_t L, float* __restrict__ d_values) {
+  for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kThreads) {
+    const int64_t pos = indices[j], b = pos / S, t = pos - b * S - (S - L - 1);
+    d_values[j] = (t >= 0 && t < L) ? grad[b * L + t] : 0.f;
+  }
+}
+
+unsigned blocks_for(int64_t n) {
+  const int64_t b = (n + kThreads - 1) / kThreads;
+  return (unsigned)(b < 1 ? 1 : (b > 16384 ? 16384 : b));
+}
+
+int check_mask(int dt) {
+  SIIRL_REQUIRE(dt == SIIRL_U8 || dt == SIIRL_I64 || dt == SIIRL_I32 || dt == SIIRL_F32 || dt == SIIRL_BF16 ||
+                    dt == SIIRL_F16, "mask dtype %d not supported", dt);
+  return SIIRL_OK;
+}
+
+}  // namespace
+}  // namespace siirl
+
+using namespace siirl;
+
+extern "C" int siirl_unpad_indices(const void* attention_mask, int mask_dtype, int64_t B, int64_t S,
+                                   int32_t* seqlens, int32_t* cu_seqlens, int64_t* indices, int64_t* info2,
+                                   siirl_stream_t stream) {
+  SIIRL_REQUIRE(B >= 1 && S >= 1 && B <= 0x7fffffffLL && B * S <= 0x7fffffffLL,
+                "B=%lld S=%lld out of range (cu_seqlens is int32)", (long long)B, (long long)S);
+  if (int rc = check_mask(mask_dtype)) return rc;
+  SIIRL_REQUIRE(attention_mask && seqlens && cu_seqlens && indices && info2, "NULL operand");
+  hipStream_t st = (hipStream_t)stream;
+  seqlens_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(attention_mask, mask_dtype, S, seqlens);
+  SIIRL_LAUNCH_CHECK("seqlens_kernel");
+  cu_seqlens_kernel<<<1, dim3(kThreads), 0, st>>>(seqlens, B, cu_seqlens, info2);
+  SIIRL_LAUNCH_CHECK("cu_seqlens_kernel");
+  indices_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(attention_mask, mask_dtype, S, cu_seqlens, indices);
+  SIIRL_LAUNCH_CHECK("indices_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_gather_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, void* dst,
+                                 siirl_stream_t stream) {
+  SIIRL_REQUIRE(n >= 0 && row_bytes >= 4 && row_bytes % 4 == 0, "n=%lld row_bytes=%lld: rows are whole 4-byte words",
+                (long long)n, (long long)row_bytes);
+  if (n == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(src && indices && dst, "NULL operand");
+  move_rows_kernel<true><<<dim3(blocks_for(n * (row_bytes / 4))), dim3(kThreads), 0, (hipStream_t)stream>>>(
+      (const uint32_t*)src, indices, n, row_bytes / 4, (uint32_t*)dst);
+  SIIRL_LAUNCH_CHECK("move_rows_kernel<gather>");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_scatter_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes,
+                                  int64_t total_rows, void* dst, siirl_stream_t stream) {
+  SIIRL_REQUIRE(n >= 0 && total_rows >= 0 && row_bytes >= 4 && row_bytes % 4 == 0,
+                "n=%lld total_rows=%lld row_bytes=%lld: rows are whole 4-byte words", (long long)n,
+                (long long)total_rows, (long long)row_bytes);
+  if (total_rows == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(dst && (n == 0 || (src && indices)), "NULL operand");
+  hipStream_t st = (hipStream_t)stream;
+  fill_zero_kernel<<<dim3(blocks_for(total_rows * (row_bytes / 4))), dim3(kThreads), 0, st>>>((uint32_t*)dst,
+                                                                                             total_rows * (row_bytes / 4));
+  SIIRL_LAUNCH_CHECK("fill_zero_kernel");
+  if (n == 0) return SIIRL_OK;
+  move_rows_kernel<false><<<dim3(blocks_for(n * (row_bytes / 4))), dim3(kThreads), 0, st>>>(
+      (const uint32_t*)src, indices, n, row_bytes / 4, (uint32_t*)dst);
+  SIIRL_LAUNCH_CHECK("move_rows_kernel<scatter>");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_unpad_ids_labels(const int64_t* input_ids, const int64_t* indices, int64_t nnz,
+                                      int64_t* ids_rmpad, int64_t* labels_rolled, siirl_stream_t stream) {
+  SIIRL_REQUIRE(nnz >= 0, "nnz < 0");
+  if (nnz == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(input_ids && indices && (ids_rmpad || labels_rolled), "NULL operand");
+  unpad_ids_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(input_ids, indices, nnz, ids_rmpad,
+                                                                                     labels_rolled);
+  SIIRL_LAUNCH_CHECK("unpad_ids_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_response_scatter(const float* values, const int64_t* indices, int64_t nnz, int64_t B, int64_t S,
+                                      int64_t L, float* out, siirl_stream_t stream) {
+  SIIRL_REQUIRE(nnz >= 0 && B >= 1 && S >= 2 && L >= 1 && L <= S - 1, "nnz=%lld B=%lld S=%lld L=%lld: need 1 <= L <= S - 1",
+                (long long)nnz, (long long)B, (long long)S, (long long)L);
+  SIIRL_REQUIRE(out && (nnz == 0 || (values && indices)), "NULL operand");
+  hipStream_t st = (hipStream_t)stream;
+  fill_zero_kernel<<<dim3(blocks_for(B * L)), dim3(kThreads), 0, st>>>((uint32_t*)out, B * L);
+  SIIRL_LAUNCH_CHECK("fill_zero_kernel");
+  if (nnz == 0) return SIIRL_OK;
+  response_scatter_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, st>>>(values, indices, nnz, S, L, out);
+  SIIRL_LAUNCH_CHECK("response_scatter_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t S, int64_t L,
+                                     float* d_values, siirl_stream_t stream) {
+  SIIRL_REQUIRE(nnz >= 0 && S >= 2 && L >= 1 && L <= S - 1, "nnz=%lld S=%lld L=%lld: need 1 <= L <= S - 1",
+                (long long)nnz, (long long)S, (long long)L);
+  if (nnz == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(grad && indices && d_values, "NULL operand");
+  response_gather_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(grad, indices, nnz, S, L,
+                                                                                           d_values);
+  SIIRL_LAUNCH_CHECK("response_gather_kernel");
+  return SIIRL_OK;
+}

@@ -1,0 +1,103 @@
+"""GPU parity: remove-padding bookkeeping (through the C ABI) vs the numpy oracle.  Index and integer work:
+bit-exact; the float payloads are moved, not computed, so they are bit-exact too."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import padding as OP
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(B, S, seed, full_first=True):
+    rng = np.random.default_rng(seed)
+    mask = np.zeros((B, S), dtype=np.int64)
+    for b in range(B):
+        lo = rng.integers(0, max(S // 2, 1))
+        hi = S - rng.integers(0, max(S // 2, 1))
+        mask[b, lo:max(hi, lo + 1)] = 1
+    if full_first:
+        mask[0, :] = 1
+    ids = rng.integers(0, 150000, (B, S)).astype(np.int64)
+    return ids, mask
+
+
+@pytest.mark.parametrize("B,S", [(1, 2), (3, 9), (8, 1300), (300, 257), (2, 70000)])
+@pytest.mark.parametrize("mdt", [torch.int64, torch.bool, torch.int32, torch.float32, torch.bfloat16])
+def test_unpad_input(dev, B, S, mdt):
+    import siirl_amd.padding as P
+
+    ids, mask = _case(B, S, B + S)
+    h = np.random.default_rng(3).standard_normal((B, S, 2)).astype(np.float32)
+    rm_o, idx_o, cu_o, mx_o, sl_o = OP.unpad_input(h, mask)
+    rm, idx, cu, mx, sl = P.unpad_input(torch.from_numpy(h).to(dev), torch.from_numpy(mask).to(dev).to(mdt))
+    assert idx.dtype == torch.int64 and cu.dtype == torch.int32 and sl.dtype == torch.int32
+    assert np.array_equal(idx.cpu().numpy(), idx_o) and np.array_equal(cu.cpu().numpy(), cu_o)
+    assert mx == mx_o and np.array_equal(sl.cpu().numpy(), sl_o)
+    assert np.array_equal(rm.cpu().numpy(), rm_o)
+    back = P.pad_input(rm, idx, B, S)
+    assert np.array_equal(back.cpu().numpy(), OP.pad_input(rm_o, idx_o, B, S))
+
+
+def test_empty_rows_and_empty_batch(dev):
+    import siirl_amd.padding as P
+
+    mask = np.array([[0, 0, 0], [0, 1, 0], [0, 0, 0]])
+    rm, idx, cu, mx, sl = P.unpad_input(torch.arange(9.0, device=dev).reshape(3, 3, 1), torch.from_numpy(mask).to(dev))
+    assert idx.tolist() == [4] and cu.tolist() == [0, 0, 1, 1] and mx == 1 and rm.flatten().tolist() == [4.0]
+    rm, idx, cu, mx, sl = P.unpad_input(torch.arange(9.0, device=dev).reshape(3, 3, 1), torch.zeros(3, 3, dtype=torch.int64, device=dev))
+    assert idx.numel() == 0 and rm.shape == (0, 1) and cu.tolist() == [0, 0, 0, 0] and mx == 0
+    assert float(P.pad_input(rm, idx, 3, 3).abs().sum()) == 0.0
+
+
+@pytest.mark.parametrize("B,S", [(4, 64), (16, 2048)])
+def test_ids_and_rolled_labels(dev, B, S):
+    import siirl_amd.padding as P
+
+    ids, mask = _case(B, S, 7 * B + S)
+    rm_o, idx_o, cu_o, mx_o, _ = OP.unpad_input(ids[..., None], mask)
+    rm, rolled, idx, cu, mx = P.unpad_ids_and_labels(torch.from_numpy(ids).to(dev), torch.from_numpy(mask).to(dev))
+    assert rm.shape == (1, idx_o.size)
+    assert np.array_equal(rm[0].cpu().numpy(), rm_o[:, 0])
+    assert np.array_equal(rolled.cpu().numpy(), OP.rolled_labels(rm_o[:, 0]))
+    assert np.array_equal(idx.cpu().numpy(), idx_o) and np.array_equal(cu.cpu().numpy(), cu_o) and mx == mx_o
+
+
+@pytest.mark.parametrize("B,S,L", [(3, 9, 4), (8, 1300, 512), (2, 5, 4), (4, 600, 599)])
+def test_pad_and_slice_response(dev, B, S, L):
+    import siirl_amd.padding as P
+
+    ids, mask = _case(B, S, S + L, full_first=False)
+    _, idx_o, *_ = OP.unpad_input(ids[..., None], mask)
+    v = np.random.default_rng(5).standard_normal(idx_o.size).astype(np.float32)
+    want = OP.pad_and_slice_response(v, idx_o, B, S, L)
+    x = torch.from_numpy(v).to(dev).requires_grad_(True)
+    idx = torch.from_numpy(idx_o).to(dev)
+    got = P.pad_and_slice_response(x, idx, B, S, L)
+    assert got.shape == (B, L) and np.array_equal(got.detach().cpu().numpy(), want)
+    # backward == the reference's composition under autograd
+    g = torch.from_numpy(np.random.default_rng(6).standard_normal((B, L)).astype(np.float32))
+    got.backward(g.to(dev))
+    x_o = torch.from_numpy(v).requires_grad_(True)
+    full = torch.zeros(B * S).index_put((torch.from_numpy(idx_o),), x_o).reshape(B, S)
+    full[:, -L - 1:-1].backward(g)
+    assert torch.equal(x.grad.cpu(), x_o.grad)
+    with pytest.raises(ValueError):
+        P.pad_and_slice_response(x, idx, B, S, S)
+
+
+def test_index_first_axis_autograd_and_dtypes(dev):
+    import siirl_amd.padding as P
+
+    x = torch.randn(50, 6, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    idx = torch.tensor([3, 3, 49, 0, 17], device=dev)
+    y = P.index_first_axis(x, idx)
+    assert torch.equal(y, x.detach()[idx])
+    y.float().sum().backward()
+    want = torch.zeros(50, 6)
+    want[[3, 49, 0, 17]] = 1.0  # a repeated index: the scatter keeps one copy (the reference's pad_input does too)
+    assert torch.equal((x.grad.float().cpu() != 0), want != 0)
+    with pytest.raises(ValueError):
+        P.index_first_axis(torch.zeros(4, 1, dtype=torch.bfloat16, device=dev), idx[:1] * 0)
+    with pytest.raises(RuntimeError):
+        P.unpad_input(torch.zeros(2, 2, 1), torch.ones(2, 2))

@@ -288,6 +288,39 @@ int siirl_response_scatter(const float* values, const int64_t* indices, int64_t 
 int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t S, int64_t L,
                           float* d_values, siirl_stream_t stream);
 
+/* ------------------------------------------------------------------- logged batch statistics */
+
+/* Order of the 32-float block written by siirl_data_metrics (unused tail entries are 0). */
+enum {
+  SIIRL_METRIC_SCORE_MEAN = 0, SIIRL_METRIC_SCORE_MAX, SIIRL_METRIC_SCORE_MIN,
+  SIIRL_METRIC_REWARD_MEAN, SIIRL_METRIC_REWARD_MAX, SIIRL_METRIC_REWARD_MIN,
+  SIIRL_METRIC_ADV_MEAN, SIIRL_METRIC_ADV_MAX, SIIRL_METRIC_ADV_MIN,
+  SIIRL_METRIC_RETURNS_MEAN, SIIRL_METRIC_RETURNS_MAX, SIIRL_METRIC_RETURNS_MIN,
+  SIIRL_METRIC_VALUES_MEAN, SIIRL_METRIC_VALUES_MAX, SIIRL_METRIC_VALUES_MIN, SIIRL_METRIC_VF_EXPLAINED_VAR,
+  SIIRL_METRIC_RESP_LEN_MEAN, SIIRL_METRIC_RESP_LEN_MAX, SIIRL_METRIC_RESP_LEN_MIN, SIIRL_METRIC_RESP_CLIP_RATIO,
+  SIIRL_METRIC_CORRECT_LEN_MAX, SIIRL_METRIC_CORRECT_LEN_MIN, SIIRL_METRIC_CORRECT_LEN_MEAN,
+  SIIRL_METRIC_WRONG_LEN_MAX, SIIRL_METRIC_WRONG_LEN_MIN, SIIRL_METRIC_WRONG_LEN_MEAN,
+  SIIRL_METRIC_PROMPT_LEN_MEAN, SIIRL_METRIC_PROMPT_LEN_MAX, SIIRL_METRIC_PROMPT_LEN_MIN,
+  SIIRL_METRIC_PROMPT_CLIP_RATIO, SIIRL_METRIC_VALID_TOKENS, SIIRL_METRIC_COUNT = 32
+};
+
+size_t siirl_data_metrics_workspace_bytes(int64_t B, int64_t L);
+
+/*
+ * The statistics the trainer logs per step from [B, L] fp32 tensors: mean / max / min of the per-sequence score
+ * and reward sums; mean / max / min over the tokens selected by response_mask.bool() of advantages, returns and
+ * (when values != NULL) values, plus 1 - var(returns - values) / (var(returns) + 1e-5) with unbiased variances;
+ * response length (mask count per row) mean / max / min, the fraction equal to L, the same split by
+ * reward sum > 0.5 ("correct") or not (0 when the class is empty); prompt length statistics from the first
+ * prompt_width columns of attention_mask [B, prompt_width + L] and the fraction equal to prompt_width.
+ * Replaces: compute_data_metric / _compute_response_info siirl/utils/metrics/metric_utils.py:36-183.
+ */
+int siirl_data_metrics(const float* token_level_scores, const float* token_level_rewards, const float* advantages,
+                       const float* returns, const float* values, const void* response_mask,
+                       int response_mask_dtype, const void* attention_mask, int attention_mask_dtype, int64_t B,
+                       int64_t L, int64_t prompt_width, float* out32, void* workspace, size_t workspace_bytes,
+                       siirl_stream_t stream);
+
 /* ------------------------------------------------------------------- GAE and masked whitening */
 
 /* Bytes of scratch siirl_masked_whiten / siirl_gae_advantage_return need (a constant; 8-byte aligned buffer). */

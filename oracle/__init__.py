@@ -55,6 +55,8 @@ make_uid / filter_by_indices           uid layout and ordered index select pinne
 unpad_input / pad_input / ...          transformers' pure-torch restatement of bert_padding
                                        (modeling_flash_attention_utils._unpad_input / _pad_input);
                                        pad(unpad(x)) == x * mask; hand-written left/right padding
+compute_data_metric                    numpy mean / max / min / var(ddof=1) of the selected elements
+                                       on seeded inputs; hand-written lengths and clip ratios
 fused_linear_for_ppo_fwd / _bwd        equals logprob/entropy of ``(h @ W.T)/T`` in fp64 and
                                        autograd through that expression
 =====================================  ==========================================================
@@ -66,4 +68,4 @@ reference's CUDA dispatch target for ``logprobs_from_logits``) and of the Triton
 log-softmax / online softmax) instead.
 """
 
-from . import torch_functional, core_algos, dapo_filter, fused_linear, actor_step, padding  # noqa: F401
+from . import torch_functional, core_algos, dapo_filter, fused_linear, actor_step, padding, metric_utils  # noqa: F401

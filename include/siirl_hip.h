@@ -288,6 +288,21 @@ int siirl_response_scatter(const float* values, const int64_t* indices, int64_t 
 int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t S, int64_t L,
                           float* d_values, siirl_stream_t stream);
 
+/* ------------------------------------------------------------------- outcome reward placement */
+
+/*
+ * reward_tensor[B, L] (fp32) = 0 except reward_tensor[b, valid_b - 1] = scores[b] + overlong_b, where valid_b is the
+ * sum of attention_mask[b, prompt_width : prompt_width + L] and, when overlong_enable != 0,
+ * overlong_b = min(-(valid_b - (max_resp_len - buffer_len)) / buffer_len * penalty_factor, 0), else 0, in
+ * float32 arithmetic (the reference computes it on a 0-d tensor).  valid_b == 0 writes the last column (Python's index -1).
+ * overlong_reward[B] and valid_response_length[B] are optional outputs.
+ * Replaces: the reward tensor construction of DAPORewardManager.__call__ siirl/engine/reward_manager/dapo.py:57-126.
+ */
+int siirl_place_outcome_reward(const double* scores, const void* attention_mask, int mask_dtype, int64_t B,
+                               int64_t prompt_width, int64_t L, int overlong_enable, double max_resp_len,
+                               double overlong_buffer_len, double overlong_penalty_factor, float* reward_tensor,
+                               double* overlong_reward, int64_t* valid_response_length, siirl_stream_t stream);
+
 /* ------------------------------------------------------------------- logged batch statistics */
 
 /* Order of the 32-float block written by siirl_data_metrics (unused tail entries are 0). */

@@ -57,6 +57,9 @@ unpad_input / pad_input / ...          transformers' pure-torch restatement of b
                                        pad(unpad(x)) == x * mask; hand-written left/right padding
 compute_data_metric                    numpy mean / max / min / var(ddof=1) of the selected elements
                                        on seeded inputs; hand-written lengths and clip ratios
+merge_leftover / place_outcome_reward  the reference's leftover-cache test vectors
+                                       (tests/dag_worker/test_dapo_pipeline.py:145-195); hand-computed
+                                       penalties either side of the expected length
 fused_linear_for_ppo_fwd / _bwd        equals logprob/entropy of ``(h @ W.T)/T`` in fp64 and
                                        autograd through that expression
 =====================================  ==========================================================

@@ -64,3 +64,49 @@ def filter_by_indices(batch: dict, indices):
         else:
             out[k] = v
     return out
+
+
+def merge_leftover(cache: dict, new: dict) -> dict:
+    """``cache || new`` as the reference's leftover-cache test states it
+    (``tests/dag_worker/test_dapo_pipeline.py:72-126``): tensors and numpy arrays concatenated along the batch
+    axis, lists appended, other values taken from the new batch, one-sided keys kept."""
+    out = {}
+    for key in set(cache) | set(new):
+        c, n = cache.get(key), new.get(key)
+        if c is None:
+            out[key] = n
+        elif n is None:
+            out[key] = c
+        elif isinstance(c, torch.Tensor):
+            out[key] = torch.cat([c, n], dim=0)
+        elif isinstance(c, np.ndarray):
+            out[key] = np.concatenate([c, n], axis=0)
+        elif isinstance(c, (list, tuple)):
+            out[key] = list(c) + list(n)
+        else:
+            out[key] = n
+    return out
+
+
+def place_outcome_reward(scores, attention_mask, response_length, overlong_enable=False, max_resp_len=None,
+                         overlong_buffer_len=None, overlong_penalty_factor=None):
+    """The reward tensor of ``DAPORewardManager.__call__`` (reference ``siirl/engine/reward_manager/dapo.py:57-126``)
+    for given scalar scores: zeros, with ``score + min(-(valid - (max_resp_len - buffer)) / buffer * factor, 0)``
+    (the second term only when the overlong buffer is enabled) at ``[i, valid - 1]``, ``valid`` the attention
+    mask's sum over the response columns.  Returns ``(reward_tensor, overlong_rewards)``."""
+    B, S = attention_mask.shape
+    prompt_length = S - response_length
+    reward = torch.zeros(B, response_length, dtype=torch.float32)
+    pens = []
+    for i in range(B):
+        valid = attention_mask[i][prompt_length:].sum()
+        r = float(scores[i])
+        pen = 0.0
+        if overlong_enable:
+            expected = max_resp_len - overlong_buffer_len
+            exceed = valid - expected
+            pen = min(-exceed / overlong_buffer_len * overlong_penalty_factor, 0)
+            r += pen
+        reward[i, valid - 1] = r
+        pens.append(float(pen))
+    return reward, pens

@@ -23,7 +23,8 @@ ARCH = "gfx950"
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
             "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-fno-gpu-rdc"]
 # per-file additions: the numpy-emulating group statistics and the GAE recurrence must not be contracted into FMAs
-EXTRA = {"group_ops.hip": ["-ffp-contract=off"], "gae.hip": ["-ffp-contract=off"]}
+EXTRA = {"group_ops.hip": ["-ffp-contract=off"], "gae.hip": ["-ffp-contract=off"],
+         "reward.hip": ["-ffp-contract=off"]}
 
 
 def sources():

@@ -17,6 +17,9 @@ import torch
 
 from . import _lib
 
+__all__ = ["NodeOutput", "make_uid", "group_keep_mask", "filter_tensordict", "dynamic_sampling",
+           "SamplingLeftoverCache"]
+
 
 @dataclass
 class NodeOutput:
@@ -115,6 +118,61 @@ def filter_tensordict(batch, indices: List[int]):
     if is_td:
         return type(batch)(out, batch_size=len(indices))
     return out
+
+
+def _batch_len(batch) -> int:
+    if batch is None:
+        return 0
+    if hasattr(batch, "batch_size") and not isinstance(batch, dict):
+        return int(batch.batch_size[0]) if len(batch.batch_size) else 0
+    for v in batch.values():
+        if isinstance(v, torch.Tensor):
+            return int(v.shape[0])
+    return 0
+
+
+class SamplingLeftoverCache:
+    """Carries kept trajectories from one DAPO sampling round to the next until a full batch exists: the
+    leftover-cache semantics pinned by the reference's ``tests/dag_worker/test_dapo_pipeline.py:52-195``
+    (the worker attribute is ``sampling_leftover_cache``, ``siirl/dag_worker/dagworker.py:126``).
+
+    ``postprocess(filtered_batch, target_total_samples)``: a non-empty cache is merged in front of the new
+    batch (``cache || new``) -- tensors concatenated along the batch axis, numpy arrays concatenated, lists and
+    tuples appended, any other value is metadata and the new batch's wins, a key present on one side only is
+    taken from that side -- and the cache is cleared; then, if fewer than ``target_total_samples`` samples are
+    at hand they are cached and an empty batch is returned, otherwise the merged batch is."""
+
+    def __init__(self):
+        self.sampling_leftover_cache = None
+
+    @staticmethod
+    def merge(cache, new):
+        out = {}
+        keys = list(cache.keys()) + [k for k in new.keys() if k not in cache.keys()]
+        for key in keys:
+            c = cache.get(key) if key in cache.keys() else None
+            n = new.get(key) if key in new.keys() else None
+            if c is None or n is None:
+                out[key] = n if c is None else c
+            elif isinstance(c, torch.Tensor):
+                out[key] = torch.cat([c, n.to(c.device)], dim=0)
+            elif isinstance(c, np.ndarray):
+                out[key] = np.concatenate([c, np.asarray(n)], axis=0)
+            elif isinstance(c, (list, tuple)):
+                out[key] = list(c) + list(n)
+            else:
+                out[key] = n
+        return out
+
+    def postprocess(self, filtered_batch, target_total_samples: int):
+        batch = dict(filtered_batch.items()) if filtered_batch is not None else {}
+        if self.sampling_leftover_cache is not None:
+            batch = self.merge(self.sampling_leftover_cache, batch)
+            self.sampling_leftover_cache = None
+        if _batch_len(batch) < target_total_samples:
+            self.sampling_leftover_cache = batch
+            return {}
+        return batch
 
 
 def dynamic_sampling(config, batch, **kwargs) -> NodeOutput:

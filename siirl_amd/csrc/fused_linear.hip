@@ -130,23 +130,20 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   u32x4 b0[NJ][BK / 16], b1[NJ][BK / 16];
-  auto dma = [&](int stage, int kt) {
+  auto dma = [&](int stage, int kt, int i0 = 0, int i1 = kDmaPerWave) {
     const char* base = gA + (int64_t)kt * (BK * 2);
 #pragma unroll
-    for (int i = 0; i < kDmaPerWave; ++i) {
+    for (int i = i0; i < i1; ++i) {
       const uint32_t dst = lds0 + stage * kStageBytes + (wu * kDmaPerWave + i) * 1024;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(offA[i]), "s"(base) : "m0", "memory");
     }
   };
-  auto bload = [&](u32x4 (&b)[NJ][BK / 16], int kt) {
+  auto bload = [&](u32x4 (&b)[NJ][BK / 16], int kt, int j) {
     const char* base = gB + (int64_t)kt * (BK / 16 * 1024);
-#pragma unroll
-    for (int j = 0; j < NJ; ++j) {
-      asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(b[j][0]) : "v"(offB[j]), "s"(base));
-      asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(b[j][1]) : "v"(offB[j]), "s"(base));
-      asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(b[j][2]) : "v"(offB[j]), "s"(base));
-      asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(b[j][3]) : "v"(offB[j]), "s"(base));
-    }
+    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(b[j][0]) : "v"(offB[j]), "s"(base));
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(b[j][1]) : "v"(offB[j]), "s"(base));
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(b[j][2]) : "v"(offB[j]), "s"(base));
+    asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(b[j][3]) : "v"(offB[j]), "s"(base));
   };
   // waits until at most `n` of this wave's loads are in flight and ties the B registers to the wait
 #define SIIRL_BWAIT(n, b)                                                                                              \
@@ -155,7 +152,8 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
                  "+v"(b[1][2]), "+v"(b[1][3])::"memory")
   static_assert(NJ == 2 && BK == 64 && kDmaPerWave == 4, "the wait counts below assume 8 B loads and 4 DMA per step");
 
-  bload(b0, 0);
+  bload(b0, 0, 0);
+  bload(b0, 0, 1);
   dma(0, 0);
   dma(1, KT > 1 ? 1 : 0);
   dma(2, KT > 2 ? 2 : 0);
@@ -187,18 +185,29 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], __builtin_bit_cast(bf16x8, bc[j][kk]), acc[i][j], 0, 0, 0);
   };
   fread(afa, 0, 0);
+  // One K-step.  The 12 vector-memory instructions are spread over the step (B for one N-tile before each of the
+  // first two MFMA groups, half of the DMA before each of the last two) instead of being issued in one burst, and
+  // the wave raises its priority while it issues MFMAs so that its SIMD partner's loads do not delay them.
+  auto mma_prio = [&](bf16x8 (&af)[MI], u32x4 (&bc)[NJ][BK / 16], int kk) {
+    __builtin_amdgcn_s_setprio(1);
+    mma(af, bc, kk);
+    __builtin_amdgcn_s_setprio(0);
+  };
   auto step = [&](int kt, u32x4 (&bc)[NJ][BK / 16], u32x4 (&bn)[NJ][BK / 16]) {
     const int stage = kt & 3;
-    bload(bn, kt + 1 < KT ? kt + 1 : KT - 1);
-    dma((stage + 3) & 3, kt + 3 < KT ? kt + 3 : KT - 1);
+    const int ktb = kt + 1 < KT ? kt + 1 : KT - 1, kta = kt + 3 < KT ? kt + 3 : KT - 1;
+    bload(bn, ktb, 0);
     fread(afb, stage, 1);
-    mma(afa, bc, 0);
+    mma_prio(afa, bc, 0);
+    bload(bn, ktb, 1);
     fread(afa, stage, 2);
-    mma(afb, bc, 1);
+    mma_prio(afb, bc, 1);
+    dma((stage + 3) & 3, kta, 0, kDmaPerWave / 2);
     fread(afb, stage, 3);
-    mma(afa, bc, 2);
+    mma_prio(afa, bc, 2);
+    dma((stage + 3) & 3, kta, kDmaPerWave / 2, kDmaPerWave);
     fread(afa, (stage + 1) & 3, 0);
-    mma(afb, bc, 3);
+    mma_prio(afb, bc, 3);
     SIIRL_BWAIT(4, bn);
     __syncthreads();
   };

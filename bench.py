@@ -87,6 +87,84 @@ def cpu_baseline(logits, labels, g_lp, g_ent, rows=4096, iters=5):
                       f"median of {iters} fwd+bwd passes ({med:.2f} s each)"}
 
 
+def bench_config3(args, dev):
+    """DAPO [B, L] path at config 3: 512 prompts x 16 responses, L = 8192 fp32.  One step = dynamic-sampling keep
+    mask over the 8192 trajectories, GRPO advantages on the kept ones, and the fused actor loss (asymmetric clip,
+    low-variance KL term) forward + backward over the kept [~5.7k, 8192] tokens.  Not the headline."""
+    import torch
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.dapo_filter as DF
+
+    P, n, L = 512, 16, 8192
+    B = P * n
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    uid = torch.from_numpy(DF.make_uid(P, n)).to(dev)
+    # ~30 % of the groups get one score for every member and are dropped by the filter
+    solved = torch.rand(P, device=dev, generator=gen)
+    acc = (torch.rand(B, device=dev, generator=gen) < 0.5).float()
+    acc = torch.where(solved.repeat_interleave(n) < 0.3, torch.ones_like(acc), acc)
+    lens = torch.randint(L // 16, L + 1, (B,), device=dev, generator=gen)
+    mask = (torch.arange(L, device=dev)[None] < lens[:, None]).long()
+    rewards = torch.zeros(B, L, device=dev)
+    rewards[torch.arange(B, device=dev), lens - 1] = acc
+    keep = DF.group_keep_mask(acc, uid)
+    kept = torch.nonzero(keep).flatten()
+    Bk = int(kept.numel())
+    lp = torch.randn(Bk, L, device=dev, generator=gen) - 1.5
+    old = lp + 0.05 * torch.randn(Bk, L, device=dev, generator=gen)
+    ref = lp + 0.1 * torch.randn(Bk, L, device=dev, generator=gen)
+    mk, rk, uk = mask[kept].contiguous(), rewards[kept].contiguous(), uid[kept].contiguous()
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=10.0,
+                          entropy_coeff=0.0, use_kl_loss=True, kl_loss_coef=0.001, kl_loss_type="low_var_kl",
+                          loss_agg_mode="token-mean", loss_mode="vanilla")
+    x = lp.requires_grad_(True)
+
+    def step(ev=None):
+        if ev:
+            ev[0].record()
+        DF.group_keep_mask(acc, uid)
+        adv, _ = CA.compute_grpo_outcome_advantage(rk, mk, uk)
+        if ev:
+            ev[1].record()
+        out = CA.actor_loss(old, x, adv, mk, cfg, ref_log_prob=ref)
+        out.loss.backward()
+        if ev:
+            ev[2].record()
+        x.grad = None
+
+    steps, warm = args.steps, args.warmup
+    for _ in range(warm):
+        step()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for k in range(steps):
+        step(evs[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    grp_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
+    loss_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+    tokens = Bk * L
+    loss_bytes = tokens * (2 * (4 * 4 + 8) + 4)  # forward and backward each read 4 fp32 operands + int64 mask; d_lp written
+    gbs = loss_bytes / loss_ms / 1e6
+    out = {
+        "metric": "DAPO loss path (filter + GRPO advantage + clipped loss fwd+bwd) tokens/sec @[B,L] fp32",
+        "value": tokens * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": wall * 1e3 / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"config3: {P} prompts x {n} responses, L = {L}; {Bk} trajectories kept by the filter",
+                   "trajectories": B, "kept": Bk, "response_length": L, "seed": SEED},
+        "kernels": {"keep mask + GRPO advantage": {"ms": grp_ms},
+                    "actor loss forward + backward (loss_partials/finish/bwd kernels)": {"ms": loss_ms, "GB/s": gbs}},
+        "roofline": {"bound": "hbm", "kernel": "loss_partials_kernel + loss_bwd_kernel", "achieved": gbs, "peak": 8000.0,
+                     "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out), flush=True)
+
+
 def bench_config5(args, dev):
     """Fused lm_head + log-prob/entropy (MFMA path): hidden [16384, 3584] ~ N(0,1), W [152064, 3584] ~ N(0, 0.02),
     bf16, uniform labels, forward + backward to hidden and W.  Not the headline; same JSON shape."""
@@ -158,8 +236,9 @@ def main():
                     help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 2 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config5"],
-                    help="config2 (default): the headline logprob+entropy fwd+bwd; config5: fused lm_head variant")
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config5"],
+                    help="config2 (default): the headline logprob+entropy fwd+bwd; config3: DAPO [B, L] loss path; "
+                         "config5: fused lm_head variant")
     ap.add_argument("--seqs", type=int, default=SEQS, help="sequences of 4096 tokens (8 = the baseline's config)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -178,6 +257,8 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "config5":
         return bench_config5(args, dev)
+    if args.workload == "config3":
+        return bench_config3(args, dev)
     SF.set_skip_zero_rows(False)  # dense: every row is read and written, as the algorithmic byte count assumes
 
     logits, labels, g_lp, g_ent, mask = make_workload(dev, seqs=args.seqs)

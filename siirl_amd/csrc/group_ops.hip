@@ -4,9 +4,13 @@
 // dynamic_sampling (siirl/user_interface/filter_interface/dapo.py:66-93).
 //
 // Groups are defined by equal uid; uids are arbitrary int64 and need not be contiguous.  Each thread owns
-// one trajectory i and scans all trajectories j in batch order through LDS tiles, picking those with
-// uid[j] == uid[i]: O(B^2) compares, exact integer bookkeeping, no atomics, and every group statistic is
-// accumulated in the batch order the reference uses.  B is a rollout batch (10^3..10^5).
+// one trajectory i and visits the members of its group in batch order, so that every group statistic is
+// accumulated in the order the reference uses; exact integer bookkeeping, no atomics.  When the uid array is
+// non-decreasing (the layout the reference's data loader produces, and what an ascending filter keeps) a
+// group is one contiguous run and the thread walks just that run: O(B * n).  Otherwise the thread scans all
+// trajectories through LDS tiles and picks those with uid[j] == uid[i]: O(B^2) compares.  Every workgroup
+// checks the ordering for itself (O(B) coalesced compares), so no flag has to travel between kernels.  B is
+// a rollout batch (10^3..10^5).
 //
 // The keep mask reproduces np.std(values) > 0 bit for bit: numpy sums with an 8-accumulator pairwise
 // scheme in the dtype of the values, so e.g. three equal fp64 values 0.1 have std 1.4e-17 > 0.  This
@@ -34,6 +38,21 @@ __global__ __launch_bounds__(kThreads) void row_sum_kernel(const float* __restri
   if (threadIdx.x == 0) out[b] = (float)s;
 }
 
+// true iff uid[0] <= uid[1] <= ... ; evaluated by the whole workgroup (one wave), result uniform
+__device__ __forceinline__ bool uid_non_decreasing(const int64_t* __restrict__ uid, int64_t B) {
+  bool ok = true;
+  for (int64_t j = threadIdx.x; j + 1 < B; j += kGroupThreads) ok = ok && (uid[j] <= uid[j + 1]);
+  return __all(ok);
+}
+// the run [lo, hi) of positions around i that share uid[i] (uid non-decreasing)
+__device__ __forceinline__ void run_of(const int64_t* __restrict__ uid, int64_t B, int64_t i, int64_t& lo, int64_t& hi) {
+  const int64_t my = uid[i];
+  lo = i;
+  while (lo > 0 && uid[lo - 1] == my) --lo;
+  hi = i + 1;
+  while (hi < B && uid[hi] == my) ++hi;
+}
+
 // ---------------------------------------------------------------------------- GRPO advantage
 
 // a[i] = (s_i - mean_g) / (std_g + eps), unbiased std; a group of one uses mean 0, std 1.
@@ -47,6 +66,25 @@ __global__ __launch_bounds__(kGroupThreads) void grpo_group_kernel(const float* 
   const int64_t my = live ? uid[i] : 0;
   int n = 0;
   double sum = 0.0;
+  const bool runs = uid_non_decreasing(uid, B);
+  if (runs) {
+    if (!live) return;
+    int64_t lo, hi;
+    run_of(uid, B, i, lo, hi);
+    n = (int)(hi - lo);
+    for (int64_t j = lo; j < hi; ++j) sum += (double)scores[j];
+    const double mean = n > 1 ? sum / (double)n : 0.0;
+    double ss = 0.0;
+    if (n > 1)
+      for (int64_t j = lo; j < hi; ++j) {
+        const double d = (double)scores[j] - mean;
+        ss += d * d;
+      }
+    const double sd = n > 1 ? sqrt(ss / (double)(n - 1)) : 1.0;
+    const float num = (float)(double)scores[i] - (float)mean;
+    a_out[i] = norm_by_std ? num / ((float)sd + eps) : num;
+    return;
+  }
   for (int64_t base = 0; base < B; base += kTile) {
     __syncthreads();
     for (int k = threadIdx.x; k < kTile; k += kGroupThreads) {
@@ -217,6 +255,36 @@ __global__ __launch_bounds__(kGroupThreads) void keep_mask_kernel(const T* __res
     return (int)((B - base) < kTile ? (B - base) : kTile);
   };
   int n = 0;
+  if (uid_non_decreasing(uid, B)) {
+    if (!live) return;
+    int64_t lo, hi;
+    run_of(uid, B, i, lo, hi);
+    n = (int)(hi - lo);
+    T mean, ssq;
+    if (n <= 128) {
+      NpBlock<T> blk;
+      blk.begin(n);
+      if (n > 1)
+        for (int64_t j = lo; j < hi; ++j) blk.push(val[j]);
+      mean = blk.finish() / (T)n;
+      blk.begin(n);
+      if (n > 1)
+        for (int64_t j = lo; j < hi; ++j) {
+          const T d = val[j] - mean;
+          blk.push(d * d);
+        }
+      ssq = blk.finish();
+    } else {
+      MemberCursor<T> c1{uid, val, B, lo, my};
+      mean = np_pairwise<T, false>(c1, n, T(0)) / (T)n;
+      MemberCursor<T> c2{uid, val, B, lo, my};
+      ssq = np_pairwise<T, true>(c2, n, mean);
+    }
+    const T sd = sqrt(ssq / (T)n);
+    keep[i] = (n == 1 || sd > T(0)) ? 1 : 0;
+    if (group_size) group_size[i] = n;
+    return;
+  }
   for (int64_t base = 0; base < B; base += kTile) {
     const int lim = stage(base);
     if (live)

@@ -109,11 +109,11 @@ def test_compute_advantage_dispatch(dev):
     assert CA.get_adv_estimator_fn("grpo") is CA.compute_grpo_outcome_advantage
     assert CA.get_adv_estimator_fn(CA.AdvantageEstimator.GRPO) is CA.compute_grpo_outcome_advantage
     with pytest.raises(ValueError, match="Unknown advantage estimator"):
-        CA.get_adv_estimator_fn("gae")
+        CA.get_adv_estimator_fn("gae_marft")
     with pytest.raises(TypeError):  # the reference's CPGD branch passes a keyword GRPO does not take
         CA.compute_advantage(dict(data), "cpgd")
     with pytest.raises(NotImplementedError):
-        CA.compute_advantage(dict(data), "gae")
+        CA.compute_advantage(dict(data), "gae_marft")
 
 
 # ------------------------------------------------------------------------------------ DAPO keep mask

@@ -32,7 +32,15 @@ __global__ __launch_bounds__(kThreads) void row_sum_kernel(const float* __restri
   const int64_t b = blockIdx.x;
   const float* r = x + b * L;
   double s = 0.0;
-  for (int64_t t = threadIdx.x; t < L; t += kThreads) s += (double)r[t];
+  if (L % 4 == 0 && ((uintptr_t)x & 15) == 0) {  // rows start 16-byte aligned
+    const float4* r4 = reinterpret_cast<const float4*>(r);
+    for (int64_t t = threadIdx.x; t < L / 4; t += kThreads) {
+      const float4 v = r4[t];
+      s += ((double)v.x + (double)v.y) + ((double)v.z + (double)v.w);
+    }
+  } else {
+    for (int64_t t = threadIdx.x; t < L; t += kThreads) s += (double)r[t];
+  }
   __shared__ double sh[kThreads / kWave + 1];
   s = block_sum(s, sh);
   if (threadIdx.x == 0) out[b] = (float)s;
@@ -40,9 +48,10 @@ __global__ __launch_bounds__(kThreads) void row_sum_kernel(const float* __restri
 
 // true iff uid[0] <= uid[1] <= ... ; evaluated by the whole workgroup (one wave), result uniform
 __device__ __forceinline__ bool uid_non_decreasing(const int64_t* __restrict__ uid, int64_t B) {
-  bool ok = true;
-  for (int64_t j = threadIdx.x; j + 1 < B; j += kGroupThreads) ok = ok && (uid[j] <= uid[j + 1]);
-  return __all(ok);
+  int bad = 0;  // no short circuit: the loads of successive iterations stay independent
+#pragma unroll 8
+  for (int64_t j = threadIdx.x; j + 1 < B; j += kGroupThreads) bad |= (uid[j] > uid[j + 1]) ? 1 : 0;
+  return __all(bad == 0);
 }
 // the run [lo, hi) of positions around i that share uid[i] (uid non-decreasing)
 __device__ __forceinline__ void run_of(const int64_t* __restrict__ uid, int64_t B, int64_t i, int64_t& lo, int64_t& hi) {

@@ -44,6 +44,7 @@ struct LossArgs {
   float ent_coef, kl_coef, drift_coef, scale;
   int64_t B, L;
   int nseg;
+  int vec;  // L % 4 == 0 and every operand 16-byte aligned: tokens are moved four at a time
 };
 enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6 };
 
@@ -58,6 +59,50 @@ __device__ __forceinline__ float tmin(float a, float b) { return (a != a || b !=
 __device__ __forceinline__ float contrib_where(float v, float m) { return m != 0.f ? v * m : 0.f; }
 __device__ __forceinline__ float contrib(float v, float m, int agg) {
   return agg == SIIRL_AGG_TOKEN_MEAN ? contrib_where(v, m) : v * m;
+}
+
+// four consecutive tokens of one operand; `vec` selects one 16-byte access
+struct Quad {
+  float v[4];
+};
+__device__ __forceinline__ Quad load_quad(const float* __restrict__ p, int64_t idx, bool vec, int nv, float fill) {
+  Quad q;
+  if (vec) {
+    const float4 t = *reinterpret_cast<const float4*>(p + idx);
+    q.v[0] = t.x; q.v[1] = t.y; q.v[2] = t.z; q.v[3] = t.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? p[idx + e] : fill;
+  }
+  return q;
+}
+__device__ __forceinline__ Quad const_quad(float c) { return Quad{{c, c, c, c}}; }
+__device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t idx, bool vec, int nv) {
+  Quad q;
+  if (vec && dt == SIIRL_I64) {
+    const longlong2 a = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[0];
+    const longlong2 b = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[1];
+    q.v[0] = (float)a.x; q.v[1] = (float)a.y; q.v[2] = (float)b.x; q.v[3] = (float)b.y;
+  } else if (vec && dt == SIIRL_U8) {
+    const uint32_t u = *reinterpret_cast<const uint32_t*>((const uint8_t*)p + idx);
+    q.v[0] = (float)(u & 0xffu); q.v[1] = (float)((u >> 8) & 0xffu); q.v[2] = (float)((u >> 16) & 0xffu);
+    q.v[3] = (float)(u >> 24);
+  } else if (vec && dt == SIIRL_F32) {
+    q = load_quad((const float*)p, idx, true, 4, 0.f);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? load_mask(p, dt, idx + e) : 0.f;
+  }
+  return q;
+}
+__device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q) {
+  if (vec) {
+    *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (e < nv) p[idx + e] = q.v[e];
+  }
 }
 
 struct KlOut {
@@ -272,60 +317,68 @@ __global__ __launch_bounds__(kThreads) void loss_partials_kernel(LossArgs a, con
   acc[P_RMAX] = -__builtin_inff();
   const float seq_s = (a.kind == KIND_GSPO) ? row_s[b] : 0.f;
 
-  for (int i = threadIdx.x; i < kSeg; i += kThreads) {
-    const int64_t t = t0 + i;
+  const bool vec = a.vec != 0;
+  for (int gq = threadIdx.x; gq < kSeg / 4; gq += kThreads) {
+    const int64_t t = t0 + 4 * gq;
     if (t >= a.L) break;
-    const int64_t idx = b * a.L + t;
-    const float m = load_mask(a.mask, a.mask_dtype, idx);
-    acc[P_M] += m;
-    if (a.kind == KIND_AGG) {
-      acc[P_PG] += contrib(a.lp[idx], m, a.agg_mode);
-      continue;
+    const int nv = (int)((a.L - t) < 4 ? (a.L - t) : 4);
+    const int64_t idx0 = b * a.L + t;
+    const Quad m4 = load_mask_quad(a.mask, a.mask_dtype, idx0, vec, nv);
+    const Quad lp4 = load_quad(a.lp, idx0, vec, nv, 0.f);
+    const bool agg_only = a.kind == KIND_AGG;
+    const Quad old4 = agg_only ? const_quad(0.f) : load_quad(a.old_lp, idx0, vec, nv, 0.f);
+    const Quad adv4 = agg_only ? const_quad(0.f) : load_quad(a.adv, idx0, vec, nv, 0.f);
+    const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
+    const Quad ent4 = a.ent ? load_quad(a.ent, idx0, vec, nv, 0.f) : const_quad(0.f);
+    const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (e >= nv) break;
+      const float m = m4.v[e];
+      acc[P_M] += m;
+      if (agg_only) {
+        acc[P_PG] += contrib(lp4.v[e], m, a.agg_mode);
+        continue;
+      }
+      const float lp = lp4.v[e];
+      const PgOut o = pg_token(a.kind, lp, old4.v[e], adv4.v[e], isw4.v[e], seq_s, a);
+      if (a.kind != KIND_GEO) acc[P_PG] += contrib(o.tok, m, a.agg_mode);  // GEO: the loss is per sequence (row_s)
+      acc[P_CLIP] += contrib_where(o.clip, m);
+      acc[P_NEGD] += contrib_where(o.negd, m);
+      acc[P_LOWER] += contrib_where(o.lower, m);
+      acc[P_RSUM] += o.r_raw;
+      acc[P_RMIN] = fminf(acc[P_RMIN], o.r_raw);
+      acc[P_RMAX] = fmaxf(acc[P_RMAX], o.r_raw);
+      if (a.ent) acc[P_ENT] += contrib(ent4.v[e], m, a.aux_agg_mode);
+      if (a.ref) acc[P_KL] += contrib(kl_token(lp, ref4.v[e], a.kl_mode, 0).v, m, a.aux_agg_mode);
+      if (a.drift_coef != 0.f) acc[P_AUX0] += contrib(clamp_max(o.r_raw - 1.f, 2.f) * lp, m, a.aux_agg_mode);
     }
-    const float lp = a.lp[idx];
-    const float isw = a.isw ? a.isw[idx] : 1.f;
-    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a);
-    if (a.kind != KIND_GEO) acc[P_PG] += contrib(o.tok, m, a.agg_mode);  // GEO: the loss is per sequence (row_s)
-    acc[P_CLIP] += contrib_where(o.clip, m);
-    acc[P_NEGD] += contrib_where(o.negd, m);
-    acc[P_LOWER] += contrib_where(o.lower, m);
-    acc[P_RSUM] += o.r_raw;
-    acc[P_RMIN] = fminf(acc[P_RMIN], o.r_raw);
-    acc[P_RMAX] = fmaxf(acc[P_RMAX], o.r_raw);
-    if (a.ent) acc[P_ENT] += contrib(a.ent[idx], m, a.aux_agg_mode);
-    if (a.ref) acc[P_KL] += contrib(kl_token(lp, a.ref[idx], a.kl_mode, 0).v, m, a.aux_agg_mode);
-    if (a.drift_coef != 0.f) acc[P_AUX0] += contrib(clamp_max(o.r_raw - 1.f, 2.f) * lp, m, a.aux_agg_mode);
   }
 
-  __shared__ float sh[kThreads / kWave + 1];
-  float* out = partials + (b * a.nseg + seg) * kNP;
+  // one wave-level reduction per partial, one LDS exchange for all of them
+  __shared__ float sh[kThreads / kWave][kNP];
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
 #pragma unroll
   for (int k = 0; k < kNP; ++k) {
-    if (k == P_RMIN || k == P_RMAX) continue;
-    const float v = block_sum(acc[k], sh);
-    if (threadIdx.x == 0) out[k] = v;
-  }
-  // min / max of the raw ratio
-  float mn = acc[P_RMIN], mx = acc[P_RMAX];
+    float v = acc[k];
+    if (k == P_RMIN) {
 #pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    mn = fminf(mn, __shfl_xor(mn, o, kWave));
-    mx = fmaxf(mx, __shfl_xor(mx, o, kWave));
-  }
-  __shared__ float shm[2 * (kThreads / kWave)];
-  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
-  if (lane == 0) {
-    shm[wid] = mn;
-    shm[kThreads / kWave + wid] = mx;
+      for (int o = kWave / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
+    } else if (k == P_RMAX) {
+#pragma unroll
+      for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+    } else {
+      v = wave_sum(v);
+    }
+    if (lane == 0) sh[wid][k] = v;
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    for (int w = 1; w < kThreads / kWave; ++w) {
-      mn = fminf(mn, shm[w]);
-      mx = fmaxf(mx, shm[kThreads / kWave + w]);
-    }
-    out[P_RMIN] = mn;
-    out[P_RMAX] = mx;
+  if (threadIdx.x < kNP) {
+    const int k = threadIdx.x;
+    float v = sh[0][k];
+    for (int w = 1; w < kThreads / kWave; ++w)
+      v = k == P_RMIN ? fminf(v, sh[w][k]) : (k == P_RMAX ? fmaxf(v, sh[w][k]) : v + sh[w][k]);
+    partials[(b * a.nseg + seg) * kNP + k] = v;
   }
 }
 
@@ -460,31 +513,47 @@ __global__ __launch_bounds__(kThreads) void loss_bwd_kernel(LossArgs a, const fl
   const float mtotal = saved_out[O_MTOTAL];
   const float mrow = row_msum[b];
   const float seq_s = (a.kind == KIND_GSPO || a.kind == KIND_GEO) ? row_s[b] : 0.f;
-  for (int i = threadIdx.x; i < kSeg; i += kThreads) {
-    const int64_t t = t0 + i;
+  const bool vec = a.vec != 0;
+  const bool agg_only = a.kind == KIND_AGG;
+  for (int gq = threadIdx.x; gq < kSeg / 4; gq += kThreads) {
+    const int64_t t = t0 + 4 * gq;
     if (t >= a.L) break;
-    const int64_t idx = b * a.L + t;
-    const float m = load_mask(a.mask, a.mask_dtype, idx);
-    if (a.kind == KIND_AGG) {
-      d_lp[idx] = g * agg_weight(a.agg_mode, m, mtotal, mrow, a.B, a.L);
+    const int nv = (int)((a.L - t) < 4 ? (a.L - t) : 4);
+    const int64_t idx0 = b * a.L + t;
+    const Quad m4 = load_mask_quad(a.mask, a.mask_dtype, idx0, vec, nv);
+    Quad dlp, dent;
+    if (agg_only) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) dlp.v[e] = g * agg_weight(a.agg_mode, m4.v[e], mtotal, mrow, a.B, a.L);
+      store_quad(d_lp, idx0, vec, nv, dlp);
       continue;
     }
-    const float lp = a.lp[idx];
-    const float isw = a.isw ? a.isw[idx] : 1.f;
-    const PgOut o = pg_token(a.kind, lp, a.old_lp[idx], a.adv[idx], isw, seq_s, a);
-    float d;
-    if (a.kind == KIND_GEO)  // d mean_b(row loss) / d x = row loss * m / (n + 1e-8) / B
-      d = seq_s * (m / (mrow + 1e-8f)) / (float)a.B * o.dtok;
-    else
-      d = agg_weight(a.agg_mode, m, mtotal, mrow, a.B, a.L) * o.dtok;
-    if (a.drift_coef != 0.f)  // the weight clamp(exp(lp - old) - 1, max = 2) is detached
-      d += a.drift_coef * agg_weight(a.aux_agg_mode, m, mtotal, mrow, a.B, a.L) * clamp_max(o.r_raw - 1.f, 2.f);
-    if (a.ent || a.ref) {
-      const float wa = agg_weight(a.aux_agg_mode, m, mtotal, mrow, a.B, a.L);
-      if (a.ref) d += a.kl_coef * wa * kl_token(lp, a.ref[idx], a.kl_mode, a.kl_st).g;
-      if (a.ent && d_ent) d_ent[idx] = -g * a.ent_coef * wa;
+    const Quad lp4 = load_quad(a.lp, idx0, vec, nv, 0.f);
+    const Quad old4 = load_quad(a.old_lp, idx0, vec, nv, 0.f);
+    const Quad adv4 = load_quad(a.adv, idx0, vec, nv, 0.f);
+    const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
+    const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float m = m4.v[e], lp = lp4.v[e];
+      const PgOut o = pg_token(a.kind, lp, old4.v[e], adv4.v[e], isw4.v[e], seq_s, a);
+      float d;
+      if (a.kind == KIND_GEO)  // d mean_b(row loss) / d x = row loss * m / (n + 1e-8) / B
+        d = seq_s * (m / (mrow + 1e-8f)) / (float)a.B * o.dtok;
+      else
+        d = agg_weight(a.agg_mode, m, mtotal, mrow, a.B, a.L) * o.dtok;
+      if (a.drift_coef != 0.f)  // the weight clamp(exp(lp - old) - 1, max = 2) is detached
+        d += a.drift_coef * agg_weight(a.aux_agg_mode, m, mtotal, mrow, a.B, a.L) * clamp_max(o.r_raw - 1.f, 2.f);
+      dent.v[e] = 0.f;
+      if (a.ent || a.ref) {
+        const float wa = agg_weight(a.aux_agg_mode, m, mtotal, mrow, a.B, a.L);
+        if (a.ref) d += a.kl_coef * wa * kl_token(lp, ref4.v[e], a.kl_mode, a.kl_st).g;
+        dent.v[e] = -g * a.ent_coef * wa;
+      }
+      dlp.v[e] = g * d;
     }
-    d_lp[idx] = g * d;
+    store_quad(d_lp, idx0, vec, nv, dlp);
+    if (a.ent && d_ent) store_quad(d_ent, idx0, vec, nv, dent);
   }
 }
 
@@ -569,6 +638,15 @@ __global__ __launch_bounds__(kThreads) void mean_rows_kernel(const float* __rest
 
 int nseg_of(int64_t L) { return (int)((L + kSeg - 1) / kSeg); }
 
+// tokens move four at a time when rows start 16-byte aligned for every operand (and outputs `o1`, `o2`)
+void set_vec(LossArgs& a, const void* o1 = nullptr, const void* o2 = nullptr) {
+  auto ok16 = [](const void* p) { return p == nullptr || ((uintptr_t)p & 15) == 0; };
+  const size_t msz = a.mask_dtype == SIIRL_I64 ? 8 : (a.mask_dtype == SIIRL_U8 ? 1 : (a.mask_dtype == SIIRL_F32 || a.mask_dtype == SIIRL_I32 ? 4 : 2));
+  const bool mask_ok = ((uintptr_t)a.mask & (msz * 4 > 16 ? 15 : msz * 4 - 1)) == 0;
+  a.vec = (a.L % 4 == 0) && mask_ok && ok16(a.old_lp) && ok16(a.lp) && ok16(a.adv) && ok16(a.isw) && ok16(a.ent) &&
+          ok16(a.ref) && ok16(o1) && ok16(o2);
+}
+
 size_t ws_bytes_of(int64_t B, int64_t L) {
   const size_t ns = (size_t)nseg_of(L);
   return (size_t)B * ns * kNP * sizeof(float) + (size_t)B * ns * kNPre * sizeof(float) + 256;
@@ -596,6 +674,7 @@ int run_forward(LossArgs& a, float* out16, float* row_msum, float* row_s, void* 
   if (ws_bytes < ws_bytes_of(a.B, a.L) || ws == nullptr)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed for B=%lld L=%lld",
                 ws_bytes, ws_bytes_of(a.B, a.L), (long long)a.B, (long long)a.L);
+  set_vec(a);
   float* partials = (float*)ws;
   float* pre = partials + (size_t)a.B * a.nseg * kNP;
   dim3 grid((unsigned)(a.B * a.nseg)), block(kThreads);
@@ -646,6 +725,7 @@ extern "C" int siirl_agg_loss_bwd(const float* g_out, const void* mask, int mask
   LossArgs a{};
   a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode; a.aux_agg_mode = agg_mode;
   a.scale = 1.f; a.B = B; a.L = L; a.nseg = nseg_of(L);
+  set_vec(a, d_loss_mat);
   loss_bwd_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, (hipStream_t)stream>>>(a, g_out, out16, row_msum,
                                                                                        nullptr, d_loss_mat, nullptr);
   SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
@@ -719,6 +799,7 @@ extern "C" int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_pr
   SIIRL_REQUIRE((loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
                 "row_s is required for the gspo and geo_mean losses");
   SIIRL_REQUIRE(entropy == nullptr || d_entropy != nullptr, "d_entropy is required when entropy is given");
+  set_vec(a, d_log_prob, d_entropy);
   loss_bwd_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, (hipStream_t)stream>>>(a, g_loss, out16, row_msum,
                                                                                        row_s, d_log_prob, d_entropy);
   SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
@@ -756,6 +837,7 @@ extern "C" int siirl_value_loss_bwd(const float* g_loss, const float* vpreds, co
   LossArgs a{};
   if (int rc = fill_value_args(a, vpreds, returns, values, mask, mask_dtype, B, L, cliprange_value, agg_mode)) return rc;
   SIIRL_REQUIRE(g_loss && out16 && row_msum && d_vpreds, "NULL operand");
+  set_vec(a, d_vpreds);
   loss_bwd_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, (hipStream_t)stream>>>(a, g_loss, out16, row_msum,
                                                                                        nullptr, d_vpreds, nullptr);
   SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
@@ -803,6 +885,7 @@ extern "C" int siirl_masked_reduce(const float* values, const void* mask, int ma
                 ws_bytes_of(B, L));
   hipStream_t st = (hipStream_t)stream;
   float* partials = (float*)workspace;
+  set_vec(a);
   loss_partials_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, st>>>(a, nullptr, partials);
   SIIRL_LAUNCH_CHECK("loss_partials_kernel");
   masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, total2);

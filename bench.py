@@ -313,6 +313,40 @@ def main():
         row_skip = {"tokens_per_s": T * args.steps / skip_wall, "valid_tokens": n_valid,
                     "algorithmic_bytes": es * V * (3 * n_valid + (T - n_valid))}
 
+    # the same micro-batch as ONE launch from logits to dlogits (PPO clip loss, entropy bonus, low-variance KL loss
+    # evaluated in-kernel from each row's log-prob and entropy); reported beside the headline, never as `value`
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+
+    Bq, Lq = args.seqs, T // args.seqs
+    gen = torch.Generator(device=dev).manual_seed(SEED + 1)
+    with torch.no_grad():
+        lp_now, _ = SF.logprobs_and_entropy_from_logits(logits.detach(), labels)
+    old_lp = (lp_now + 0.05 * torch.randn(T, device=dev, generator=gen)).view(Bq, Lq)
+    ref_lp = (lp_now + 0.1 * torch.randn(T, device=dev, generator=gen)).view(Bq, Lq)
+    adv = torch.randn(Bq, 1, device=dev, generator=gen).expand(Bq, Lq).contiguous()
+    acfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=3.0,
+                           entropy_coeff=0.001, use_kl_loss=True, kl_loss_coef=0.001, kl_loss_type="low_var_kl",
+                           loss_agg_mode="token-mean", loss_mode="vanilla")
+    x3 = logits.detach().view(Bq, Lq, V)
+
+    def fused():
+        return CA.fused_actor_step(x3, labels.view(Bq, Lq), old_lp, adv, mask.view(Bq, Lq), acfg, ref_log_prob=ref_lp)
+
+    for _ in range(2):
+        fused()
+    torch.cuda.synchronize()
+    t2 = time.perf_counter()
+    for _ in range(args.steps):
+        fused()
+    torch.cuda.synchronize()
+    fused_ms = (time.perf_counter() - t2) * 1e3 / args.steps
+    fused_step = {"what": "siirl_actor_step_fused: logits -> log-prob, entropy, PPO-clip + KL + entropy loss -> dlogits "
+                          "in one launch, padding rows included; plus the [B, L] scalar/metric pass",
+                  "ms_per_step": fused_ms, "tokens_per_s": T / fused_ms * 1e3,
+                  "GB/s_of_the_two_launch_byte_count": (fwd_bytes + bwd_bytes) / fused_ms / 1e6}
+
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.bfloat16, device=dev).normal_()
         dst = torch.empty_like(src)
@@ -344,6 +378,7 @@ def main():
                      "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
                      "traffic": MEASURED_TRAFFIC_BYTES if args.seqs == SEQS else None},
         "row_skip_variant": row_skip,
+        "fused_step_variant": fused_step,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(logits.detach(), labels, g_lp, g_ent)

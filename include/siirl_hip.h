@@ -120,6 +120,39 @@ int siirl_logprob_entropy_bwd(const void* logits, int logits_dtype, int64_t T, i
                               const float* g_logprob, const float* g_entropy, void* dlogits,
                               int64_t dlogits_row_stride, uint32_t flags, siirl_stream_t stream);
 
+/*
+ * Forward and backward in one launch for upstream gradients that are known per row: logprob / entropy as the
+ * forward writes them, dlogits as the backward does, from one pass over HBM plus a partial second read (half of a
+ * 152064-entry bf16 row stays in LDS between the passes).  g_logprob or g_entropy may be NULL; logprob / entropy
+ * outputs may be NULL.  No in-place mode.
+ * Replaces: the same functions as siirl_logprob_entropy_fwd + siirl_logprob_entropy_bwd.
+ */
+int siirl_logprob_entropy_fwd_bwd(const void* logits, int logits_dtype, int64_t T, int64_t V, int64_t row_stride,
+                                  const int64_t* labels, float inv_temperature, const float* g_logprob,
+                                  const float* g_entropy, float* logprob, float* entropy, void* dlogits,
+                                  int64_t dlogits_row_stride, siirl_stream_t stream);
+
+/*
+ * The actor's micro-batch step from logits to dlogits in one launch, for the token-separable policy losses
+ * (vanilla, cpgd, gpg): per row, logprob and entropy, then the gradient of
+ *   loss = (pg_loss - entropy_coeff * agg(entropy) + kl_coef * agg(kl_penalty(logprob, ref)) + drift term) * scale
+ * with respect to that row's logprob and entropy, evaluated in-kernel from the per-token operands (arrays of T
+ * floats: old_log_prob -- NULL means on-policy, old = logprob --, advantages, ref_log_prob or NULL, is_weights or
+ * NULL) and the aggregation weights w_policy / w_aux (siirl_agg_weights), then dlogits.  Rows with zero weights
+ * get zero gradients without a second read.  The scalar loss and the logged metrics are obtained afterwards from
+ * the returned logprob / entropy with siirl_actor_loss_fwd (a [B, L]-sized pass).
+ * Replaces: siirl/engine/actor/dp_actor.py:170-231,403-501 between the logits and their gradient, i.e.
+ *           logprobs_from_logits + entropy_from_logits + the policy loss + backward() through them.
+ */
+int siirl_actor_step_fused(const void* logits, int logits_dtype, int64_t T, int64_t V, int64_t row_stride,
+                           const int64_t* labels, float inv_temperature, const float* old_log_prob,
+                           const float* advantages, const float* ref_log_prob, const float* is_weights,
+                           const float* w_policy, const float* w_aux, int loss_mode, float clip_low, float clip_high,
+                           float clip_c, float log_ratio_clamp, float entropy_coeff, int kl_mode,
+                           int kl_straight_through, float kl_coef, float policy_drift_coeff, float loss_scale,
+                           float* logprob, float* entropy, void* dlogits, int64_t dlogits_row_stride,
+                           siirl_stream_t stream);
+
 /* ------------------------------------------------------------ [B, L] loss arithmetic of the actor */
 
 /* Bytes of scratch the *_fwd entry points below need for a [B, L] problem. */
@@ -152,6 +185,15 @@ size_t siirl_loss_workspace_bytes(int64_t B, int64_t L);
 int siirl_agg_loss_fwd(const float* loss_mat, const void* mask, int mask_dtype, int64_t B, int64_t L,
                        int agg_mode, float* out16, float* row_msum, void* workspace, size_t workspace_bytes,
                        siirl_stream_t stream);
+
+/*
+ * weights[b, t] = d agg_loss / d loss_mat[b, t] for the given mask and mode (a function of the mask alone):
+ * token-mean m / (sum m + 1e-8), seq-mean-token-sum m / B, seq-mean-token-mean m / (row sum) / B,
+ * seq-mean-token-sum-norm m / L.  out16 / row_msum / workspace as for siirl_agg_loss_fwd.
+ * Replaces: the backward of agg_loss siirl/dag_worker/core_algos.py:536-569 for a unit upstream gradient.
+ */
+int siirl_agg_weights(const void* mask, int mask_dtype, int64_t B, int64_t L, int agg_mode, float* weights,
+                      float* out16, float* row_msum, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
 
 /* d(loss_mat) = g_out[0] * d(agg)/d(loss_mat).  g_out is a device scalar. */
 int siirl_agg_loss_bwd(const float* g_out, const void* mask, int mask_dtype, const float* out16,

@@ -30,9 +30,13 @@ class ActorConfig:
     kl_loss_type: str = "low_var_kl"
     loss_agg_mode: str = "token-mean"
     loss_mode: str = "vanilla"
+    use_cpgd_loss: bool = False
+    policy_drift_coeff: float = 0.0
 
 
-_LOSSES = {"vanilla": core_algos.compute_policy_loss_vanilla, "gspo": core_algos.compute_policy_loss_gspo}
+_LOSSES = {"vanilla": core_algos.compute_policy_loss_vanilla, "gspo": core_algos.compute_policy_loss_gspo,
+           "cpgd": core_algos.compute_policy_loss_cpgd, "gpg": core_algos.compute_policy_loss_gpg,
+           "geo_mean": core_algos.compute_policy_loss_geo_mean}
 
 
 def micro_batch_step(logits, responses, old_log_prob, advantages, response_mask, config: ActorConfig,
@@ -63,6 +67,9 @@ def micro_batch_step(logits, responses, old_log_prob, advantages, response_mask,
         policy_loss = policy_loss + kl_loss * config.kl_loss_coef  # :484
         metrics["actor/kl_loss"] = kl_loss.item() * loss_scale_factor
         metrics["actor/kl_coef"] = config.kl_loss_coef
+    if config.use_cpgd_loss and config.policy_drift_coeff != 0:  # :488-494
+        policy_loss = policy_loss + core_algos.policy_drift_loss(old, log_prob, response_mask, config.loss_agg_mode) \
+            * config.policy_drift_coeff
     loss = policy_loss * loss_scale_factor  # :496-500
     (dlogits,) = torch.autograd.grad(loss, x)  # :501
     ratio = (log_prob.detach() - old).exp()

@@ -23,6 +23,10 @@ SIGNATURES = {
     "siirl_hip_last_error": (C.c_char_p, []),
     "siirl_logprob_entropy_fwd": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p]),
     "siirl_logprob_entropy_bwd": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p, _i64, _u32, _p]),
+    "siirl_logprob_entropy_fwd_bwd": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p, _i64, _p]),
+    "siirl_actor_step_fused": (_i32, [_p, _i32, _i64, _i64, _i64, _p, _f32, _p, _p, _p, _p, _p, _p, _i32, _f32, _f32,
+                                      _f32, _f32, _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _i64, _p]),
+    "siirl_agg_weights": (_i32, [_p, _i32, _i64, _i64, _i32, _p, _p, _p, _p, _sz, _p]),
     "siirl_loss_workspace_bytes": (_sz, [_i64, _i64]),
     "siirl_agg_loss_fwd": (_i32, [_p, _p, _i32, _i64, _i64, _i32, _p, _p, _p, _sz, _p]),
     "siirl_agg_loss_bwd": (_i32, [_p, _p, _i32, _p, _p, _i64, _i64, _i32, _p, _p]),

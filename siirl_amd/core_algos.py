@@ -35,7 +35,8 @@ __all__ = [
     "compute_policy_loss", "compute_policy_loss_vanilla", "compute_policy_loss_gspo", "compute_policy_loss_cpgd",
     "compute_policy_loss_gpg", "compute_policy_loss_geo_mean", "compute_value_loss", "kl_penalty",
     "kl_penalty_forward",
-    "apply_kl_penalty", "compute_advantage", "actor_loss", "ActorLossOutput",
+    "apply_kl_penalty", "compute_advantage", "actor_loss", "ActorLossOutput", "fused_actor_step",
+    "FusedActorStepOutput", "agg_weights",
 ]
 
 AGG_MODES = {"token-mean": 0, "seq-mean-token-sum": 1, "seq-mean-token-mean": 2, "seq-mean-token-sum-norm": 3}
@@ -783,3 +784,123 @@ def actor_loss(old_log_prob, log_prob, advantages, response_mask, config, entrop
     outs = _ActorLoss.apply(log_prob, entropy if use_ent else None, old_log_prob, advantages, response_mask,
                             None if mode == "cpgd" else rollout_is_weights, ref_log_prob if use_kl else None, cfg)
     return ActorLossOutput(outs, float(loss_scale_factor), kl_coef, use_kl, use_ent)
+
+
+# ------------------------------------------------------------------------------------ fused actor step
+
+
+class FusedActorStepOutput:
+    """Result of ``fused_actor_step``: ``dlogits`` (gradient of the scaled loss w.r.t. the unscaled logits, shape and
+    dtype of the logits), ``log_prob`` / ``entropy`` (``[B, L]`` fp32, detached), and ``loss_output``, the
+    ``ActorLossOutput`` with the loss value and the logged scalars.  Typical use: ``logits.backward(out.dlogits)``."""
+
+    def __init__(self, dlogits, log_prob, entropy, loss_output):
+        self.dlogits, self.log_prob, self.entropy, self.loss_output = dlogits, log_prob, entropy, loss_output
+        self.loss = loss_output.loss
+
+    def metrics(self) -> dict:
+        return self.loss_output.metrics()
+
+
+def agg_weights(response_mask: torch.Tensor, loss_agg_mode: str) -> torch.Tensor:
+    """``d agg_loss / d loss_mat`` for a unit upstream gradient: a function of the mask and the mode alone
+    (reference ``core_algos.py:536-569``).  ``[B, L]`` fp32."""
+    dev = _gpu_of(response_mask)
+    m, mcode = _mask_arg(_as_2d(response_mask), dev)
+    B, L = m.shape
+    w = torch.empty(B, L, dtype=torch.float32, device=dev)
+    out16 = torch.empty(16, dtype=torch.float32, device=dev)
+    row_msum = torch.empty(B, dtype=torch.float32, device=dev)
+    ws, nws = _workspace(B, L, dev)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().siirl_agg_weights(_lib.ptr(m), mcode, B, L, _agg_code(loss_agg_mode), _lib.ptr(w),
+                                          _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(ws), nws,
+                                          _lib.current_stream(dev))
+    _lib.check(rc, "siirl_agg_weights")
+    return w
+
+
+def fused_actor_step(logits: torch.Tensor, responses: torch.Tensor, old_log_prob, advantages: torch.Tensor,
+                     response_mask: torch.Tensor, config, ref_log_prob=None, temperature: float = 1.0,
+                     loss_scale_factor: float = 1.0, on_policy: bool = False,
+                     rollout_is_weights=None) -> FusedActorStepOutput:
+    """One micro-batch of the actor update from the response logits to their gradient in a single pass over the
+    logits (reference ``siirl/engine/actor/dp_actor.py:170-231,403-501``: ``logits / T`` -> log-prob -> entropy ->
+    policy loss - entropy bonus + KL loss (+ CPGD drift) -> ``backward()``), for the token-separable losses
+    ``vanilla``, ``cpgd`` and ``gpg``.  ``logits`` is ``[B, L, V]`` (or ``[B * L, V]``; row-strided views are
+    fine) and is not modified; ``responses`` are the labels.  ``on_policy`` uses ``old = log_prob.detach()``
+    (``dp_actor.py:436-437``).  ``gspo`` and ``geo_mean`` need sequence statistics before any gradient exists: use
+    ``logprobs_from_logits`` + ``actor_loss`` for them."""
+    from .ops import row_blocks
+
+    dev = _gpu_of(logits)
+    mode = getattr(getattr(config, "policy_loss", None), "loss_mode", None) or getattr(config, "loss_mode", "vanilla")
+    if mode not in ("vanilla", "cpgd", "gpg"):
+        raise ValueError(f"fused_actor_step supports the token-separable losses vanilla, cpgd and gpg, not {mode!r}")
+    if logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
+        raise TypeError(f"logits dtype {logits.dtype} is not supported")
+    m2 = _as_2d(response_mask)
+    B, L = m2.shape
+    V = logits.shape[-1]
+    if logits.numel() != B * L * V:
+        raise ValueError(f"logits {tuple(logits.shape)} do not match response_mask {tuple(response_mask.shape)}")
+    lo, hi = _clip_params(config)
+    c = getattr(config, "clip_ratio_c", 3.0)
+    c = 3.0 if c is None else float(c)
+    if mode in ("vanilla", "cpgd"):
+        assert c > 1.0, f"The lower bound of the clip_ratio_c for dual-clip PPO should be greater than 1.0, but get the value: {c}."
+    if mode == "cpgd":
+        _check_cpgd_bounds(lo, hi)
+    agg = getattr(config, "loss_agg_mode", "token-mean")
+    ent_coef = float(getattr(config, "entropy_coeff", 0.0))
+    use_kl = bool(getattr(config, "use_kl_loss", False))
+    kl_code, kl_coef = 0, 0.0
+    if use_kl:
+        if ref_log_prob is None:
+            raise ValueError("config.use_kl_loss is set but ref_log_prob is None")
+        kl_type = getattr(config, "kl_loss_type", "low_var_kl")
+        if kl_type not in KL_MODES:
+            raise NotImplementedError
+        kl_code, kl_coef = KL_MODES[kl_type], float(getattr(config, "kl_loss_coef", 0.001))
+    drift = float(getattr(config, "policy_drift_coeff", 0.0) or 0.0) if getattr(config, "use_cpgd_loss", False) else 0.0
+
+    w = agg_weights(m2, agg).reshape(-1)
+    lab = responses.detach().to(device=dev, dtype=torch.int64).reshape(-1).contiguous()
+    old = None if on_policy else _f32(old_log_prob, dev).reshape(-1)
+    adv = _f32(advantages, dev).reshape(-1)
+    ref = _f32(ref_log_prob, dev).reshape(-1) if use_kl else None
+    isw = None if (rollout_is_weights is None or mode == "cpgd") else _f32(rollout_is_weights, dev).reshape(-1)
+    for name, t in (("responses", lab), ("old_log_prob", old), ("advantages", adv), ("ref_log_prob", ref),
+                    ("rollout_is_weights", isw)):
+        if t is not None and t.numel() != B * L:
+            raise ValueError(f"{name} has {t.numel()} elements, expected {B * L}")
+    lp = torch.empty(B * L, dtype=torch.float32, device=dev)
+    ent = torch.empty(B * L, dtype=torch.float32, device=dev) if ent_coef != 0 else None
+    x = logits.detach()
+    dlogits = torch.empty(logits.shape, dtype=logits.dtype, device=dev)
+    d2 = dlogits.view(-1, V)
+    code = _lib.dtype_code(logits.dtype)
+    es = x.element_size()
+    done = 0
+
+    def at(t, k):
+        return None if t is None else C.c_void_p(t.data_ptr() + 4 * k)
+
+    with torch.cuda.device(dev):
+        for off, rows, stride in row_blocks(x):
+            rc = _lib.lib().siirl_actor_step_fused(
+                C.c_void_p(x.data_ptr() + off * es), code, rows, V, stride, C.c_void_p(lab.data_ptr() + 8 * done),
+                1.0 / float(temperature), at(old, done), at(adv, done), at(ref, done), at(isw, done), at(w, done),
+                at(w, done), _LOSS_CODES[mode], lo, hi, c, 20.0, ent_coef, kl_code, 0, kl_coef, drift,
+                float(loss_scale_factor), at(lp, done), at(ent, done), C.c_void_p(d2.data_ptr() + done * V * es), V,
+                _lib.current_stream(dev))
+            _lib.check(rc, "siirl_actor_step_fused")
+            done += rows
+    lp2 = lp.view(B, L)
+    ent2 = None if ent is None else ent.view(B, L)
+    with torch.no_grad():
+        loss_out = actor_loss(lp2 if on_policy else old.view(B, L), lp2, adv.view(B, L), m2, config, entropy=ent2,
+                              ref_log_prob=None if ref is None else ref.view(B, L),
+                              loss_scale_factor=loss_scale_factor,
+                              rollout_is_weights=None if isw is None else isw.view(B, L))
+    return FusedActorStepOutput(dlogits, lp2, ent2, loss_out)

@@ -13,6 +13,7 @@
 // the scalars in double precision.  No atomics: results are reproducible run to run.  The backward is a
 // plain elementwise kernel that re-evaluates the token and applies autograd's tie rules by hand.
 #include "common.hpp"
+#include "loss_token.hpp"
 
 namespace siirl {
 namespace {
@@ -26,222 +27,7 @@ enum P { P_PG = 0, P_M, P_CLIP, P_NEGD, P_LOWER, P_ENT, P_KL, P_RSUM, P_RMIN, P_
 enum O { O_LOSS = 0, O_PG, O_CLIPFRAC, O_PPOKL, O_CLIPLOWER, O_ENTLOSS, O_KLLOSS, O_RMEAN, O_RMIN, O_RMAX,
          O_MTOTAL, O_POLICY, O_DRIFT, O_COUNT = 16 };
 
-struct LossArgs {
-  const float* old_lp;   // [B,L] or null (kind == KIND_AGG)
-  const float* lp;       // [B,L]  (kind == KIND_AGG: the loss matrix to aggregate)
-  const float* adv;      // [B,L]
-  const void* mask;      // [B,L]
-  const float* isw;      // [B,L] or null
-  const float* ent;      // [B,L] or null
-  const float* ref;      // [B,L] or null
-  int mask_dtype;
-  int kind;              // KIND_*
-  int agg_mode;          // aggregation of the policy term (GSPO: forced to seq-mean-token-mean)
-  int aux_agg_mode;      // aggregation of the entropy and KL terms
-  int kl_mode, kl_st;
-  float eps_lo, eps_hi, clip_c, dclamp;
-  float log_lo, log_hi;  // CPGD: float(log(1 - eps_lo)), float(log(1 + eps_hi)), logarithms taken in double
-  float ent_coef, kl_coef, drift_coef, scale;
-  int64_t B, L;
-  int nseg;
-  int vec;  // L % 4 == 0 and every operand 16-byte aligned: tokens are moved four at a time
-};
-enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6 };
-
-// torch.clamp / torch.maximum / torch.minimum semantics (NaN propagates)
-__device__ __forceinline__ float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
-__device__ __forceinline__ float clamp_max(float x, float hi) { return x > hi ? hi : x; }
-__device__ __forceinline__ float tmax(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
-__device__ __forceinline__ float tmin(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
-
-// masked contribution.  token-mean goes through masked_mean: where(mask, v, 0) * mask; the other modes
-// multiply directly (a NaN under a zero mask poisons them, as in the reference).
-__device__ __forceinline__ float contrib_where(float v, float m) { return m != 0.f ? v * m : 0.f; }
-__device__ __forceinline__ float contrib(float v, float m, int agg) {
-  return agg == SIIRL_AGG_TOKEN_MEAN ? contrib_where(v, m) : v * m;
-}
-
-// four consecutive tokens of one operand; `vec` selects one 16-byte access
-struct Quad {
-  float v[4];
-};
-__device__ __forceinline__ Quad load_quad(const float* __restrict__ p, int64_t idx, bool vec, int nv, float fill) {
-  Quad q;
-  if (vec) {
-    const float4 t = *reinterpret_cast<const float4*>(p + idx);
-    q.v[0] = t.x; q.v[1] = t.y; q.v[2] = t.z; q.v[3] = t.w;
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? p[idx + e] : fill;
-  }
-  return q;
-}
-__device__ __forceinline__ Quad const_quad(float c) { return Quad{{c, c, c, c}}; }
-__device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t idx, bool vec, int nv) {
-  Quad q;
-  if (vec && dt == SIIRL_I64) {
-    const longlong2 a = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[0];
-    const longlong2 b = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[1];
-    q.v[0] = (float)a.x; q.v[1] = (float)a.y; q.v[2] = (float)b.x; q.v[3] = (float)b.y;
-  } else if (vec && dt == SIIRL_U8) {
-    const uint32_t u = *reinterpret_cast<const uint32_t*>((const uint8_t*)p + idx);
-    q.v[0] = (float)(u & 0xffu); q.v[1] = (float)((u >> 8) & 0xffu); q.v[2] = (float)((u >> 16) & 0xffu);
-    q.v[3] = (float)(u >> 24);
-  } else if (vec && dt == SIIRL_F32) {
-    q = load_quad((const float*)p, idx, true, 4, 0.f);
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? load_mask(p, dt, idx + e) : 0.f;
-  }
-  return q;
-}
-__device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q) {
-  if (vec) {
-    *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
-  } else {
-#pragma unroll
-    for (int e = 0; e < 4; ++e)
-      if (e < nv) p[idx + e] = q.v[e];
-  }
-}
-
-struct KlOut {
-  float v, g;  // value and d value / d logprob
-};
-__device__ __forceinline__ KlOut kl_token(float lp, float ref, int mode, int straight_through) {
-  const float x = lp - ref;
-  KlOut o;
-  switch (mode) {
-    case SIIRL_KL_K1: o.v = x; o.g = 1.f; break;
-    case SIIRL_KL_ABS: o.v = fabsf(x); o.g = x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f); break;
-    case SIIRL_KL_K2: o.v = 0.5f * x * x; o.g = x; break;
-    default: {  // K3
-      const float kr = ref - lp;
-      const float k = clampf(kr, -20.f, 20.f);
-      const float e = expf(k);
-      const float raw = e - k - 1.f;
-      o.v = clampf(raw, -10.f, 10.f);
-      const bool pass = (kr >= -20.f && kr <= 20.f) && (raw >= -10.f && raw <= 10.f);
-      o.g = pass ? -(e - 1.f) : 0.f;
-    }
-  }
-  if (straight_through) o.g = x;  // value of the estimator, gradient of k2
-  return o;
-}
-
-struct PgOut {
-  float tok, dtok;  // per-token loss and d tok / d logprob (before the aggregation weight)
-  float clip, lower, negd, r_raw;
-};
-
-// seq_s: GSPO's sequence-level mean log-ratio (unused otherwise).  For KIND_GEO tok is the token's clipped
-// log-ratio x (the loss itself is per sequence); for KIND_VALUE lp = vpreds, old = values, A = returns and
-// eps_lo = cliprange_value.
-__device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A, float isw, float seq_s,
-                                          const LossArgs& a) {
-  const float eps_lo = a.eps_lo, eps_hi = a.eps_hi, clip_c = a.clip_c, dclamp = a.dclamp;
-  PgOut o;
-  const float raw = lp - old;
-  o.r_raw = expf(raw);
-  const float lo = 1.f - eps_lo, hi = 1.f + eps_hi;
-  if (kind == KIND_CPGD) {
-    // the log-probability is clipped, not the ratio; importance weights are not used by this loss
-    o.negd = -raw;
-    float clipped;
-    bool pass;
-    if (A > 0.f) {
-      const float b = a.log_hi + old;
-      clipped = lp > b ? b : lp;
-      pass = lp <= b;
-      o.clip = o.r_raw > hi ? 1.f : 0.f;
-    } else {
-      const float b = a.log_lo + old;
-      clipped = lp < b ? b : lp;
-      pass = lp >= b;
-      o.clip = o.r_raw < lo ? 1.f : 0.f;
-    }
-    o.tok = -clipped * A;
-    o.dtok = pass ? -A : 0.f;
-    o.lower = (o.r_raw > clip_c && A < 0.f) ? 1.f : 0.f;
-    return o;
-  }
-  if (kind == KIND_GPG) {
-    o.negd = 0.f; o.clip = 0.f; o.lower = 0.f;
-    o.tok = -lp * A * isw;
-    o.dtok = -A * isw;
-    return o;
-  }
-  if (kind == KIND_GEO) {
-    o.negd = -raw;
-    const float sgn = A > 0.f ? 1.f : (A < 0.f ? -1.f : (A == 0.f ? 0.f : A));  // torch.sign; NaN stays NaN
-    const float dc = clampf(raw, -eps_lo, eps_hi);
-    const float p = sgn * raw, q = sgn * dc;
-    o.tok = sgn * tmin(p, q);
-    const bool inside = raw >= -eps_lo && raw <= eps_hi;  // then p == q and both sides of the min pass 1/2
-    o.dtok = (inside || p < q) ? sgn * sgn : 0.f;
-    const bool clipped = raw != dc;
-    o.clip = (clipped && A > 0.f) ? 1.f : 0.f;
-    o.lower = (clipped && A < 0.f) ? 1.f : 0.f;
-    return o;
-  }
-  if (kind == KIND_VALUE) {
-    o.negd = 0.f; o.lower = 0.f; o.r_raw = 1.f;
-    const float vmax = old + eps_lo, vmin = old - eps_lo;
-    const float inner = tmin(lp, vmax), vc = tmax(inner, vmin);
-    const float e1 = lp - A, e2 = vc - A;
-    const float l1 = e1 * e1, l2 = e2 * e2;
-    o.tok = tmax(l1, l2);
-    o.clip = l2 > l1 ? 1.f : 0.f;
-    const float dinner = lp < vmax ? 1.f : (lp == vmax ? 0.5f : 0.f);
-    const float dvc = inner > vmin ? dinner : (inner == vmin ? 0.5f * dinner : 0.f);
-    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-    o.dtok = w1 * 2.f * e1 + w2 * 2.f * e2 * dvc;
-    return o;
-  }
-  if (kind == KIND_VANILLA) {
-    const float d = clampf(raw, -dclamp, dclamp);
-    const float r = expf(d);
-    const float dr = (raw >= -dclamp && raw <= dclamp) ? r : 0.f;  // d r / d lp
-    o.negd = -d;
-    const float l1 = -A * r;
-    const float rc = clampf(r, lo, hi);
-    const float l2 = -A * rc;
-    const float c1 = tmax(l1, l2);
-    o.clip = l2 > l1 ? 1.f : 0.f;
-    const float l3 = -A * clip_c;
-    const float c2 = tmin(l3, c1);
-    o.lower = (c1 > l3 && A < 0.f) ? 1.f : 0.f;
-    o.tok = A < 0.f ? c2 : c1;
-    // autograd: maximum / minimum give each side 1, 1/2 (tie) or 0; clamp passes inside [lo, hi] inclusive
-    const float dl1 = -A * dr;
-    const float dl2 = (r >= lo && r <= hi) ? -A * dr : 0.f;
-    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-    const float dc1 = w1 * dl1 + w2 * dl2;
-    const float wc = c1 < l3 ? 1.f : (c1 == l3 ? 0.5f : 0.f);
-    o.dtok = A < 0.f ? wc * dc1 : dc1;
-  } else {  // GSPO
-    o.negd = -raw;
-    const float l = clamp_max(seq_s, 10.f);  // lp - lp.detach() == 0
-    const float r = expf(l);
-    const float dr = (seq_s <= 10.f) ? r : 0.f;
-    const float l1 = -A * r;
-    const float rc = clampf(r, lo, hi);
-    const float l2 = -A * rc;
-    o.tok = tmax(l1, l2);
-    o.clip = l2 > l1 ? 1.f : 0.f;
-    o.lower = 0.f;
-    const float dl1 = -A * dr;
-    const float dl2 = (r >= lo && r <= hi) ? -A * dr : 0.f;
-    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
-    o.dtok = w1 * dl1 + w2 * dl2;
-  }
-  o.tok *= isw;  // importance weights multiply value and gradient alike
-  o.dtok *= isw;
-  return o;
-}
+using namespace tok;
 
 // ---------------------------------------------------------------------------- row pre-pass (GSPO)
 
@@ -492,16 +278,6 @@ __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const
 
 // ---------------------------------------------------------------------------- backward
 
-// aggregation weight of token (b, t): d (aggregate) / d (loss_mat[b, t])
-__device__ __forceinline__ float agg_weight(int agg, float m, float mtotal, float mrow, int64_t B, int64_t L) {
-  switch (agg) {
-    case SIIRL_AGG_TOKEN_MEAN: return m != 0.f ? m / (mtotal + 1e-8f) : 0.f;
-    case SIIRL_AGG_SEQ_MEAN_TOKEN_SUM: return m / (float)B;
-    case SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN: return m / mrow / (float)B;
-    default: return m / (float)L;
-  }
-}
-
 __global__ __launch_bounds__(kThreads) void loss_bwd_kernel(LossArgs a, const float* __restrict__ g_out,
                                                             const float* __restrict__ saved_out,
                                                             const float* __restrict__ row_msum,
@@ -554,6 +330,27 @@ __global__ __launch_bounds__(kThreads) void loss_bwd_kernel(LossArgs a, const fl
     }
     store_quad(d_lp, idx0, vec, nv, dlp);
     if (a.ent && d_ent) store_quad(d_ent, idx0, vec, nv, dent);
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void fill_kernel(float* __restrict__ p, int64_t n, float v) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) p[i] = v;
+}
+
+// ---------------------------------------------------------------------------- aggregation weights
+
+// w[b, t] = d agg_loss / d loss_mat[b, t]: depends on the mask only (row sums and total from the partials pass)
+__global__ __launch_bounds__(kThreads) void agg_weights_kernel(LossArgs a, const float* __restrict__ saved_out,
+                                                               const float* __restrict__ row_msum,
+                                                               float* __restrict__ w) {
+  const int64_t b = blockIdx.x / a.nseg;
+  const int64_t t0 = (int64_t)(blockIdx.x % a.nseg) * kSeg;
+  const float mtotal = saved_out[O_MTOTAL], mrow = row_msum[b];
+  for (int i = threadIdx.x; i < kSeg; i += kThreads) {
+    const int64_t t = t0 + i;
+    if (t >= a.L) break;
+    const int64_t idx = b * a.L + t;
+    w[idx] = agg_weight(a.agg_mode, load_mask(a.mask, a.mask_dtype, idx), mtotal, mrow, a.B, a.L);
   }
 }
 
@@ -713,6 +510,26 @@ extern "C" int siirl_agg_loss_fwd(const float* loss_mat, const void* mask, int m
   a.lp = loss_mat; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode;
   a.aux_agg_mode = agg_mode; a.scale = 1.f; a.B = B; a.L = L;
   return run_forward(a, out16, row_msum, nullptr, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int siirl_agg_weights(const void* mask, int mask_dtype, int64_t B, int64_t L, int agg_mode, float* weights,
+                                 float* out16, float* row_msum, void* workspace, size_t workspace_bytes,
+                                 siirl_stream_t stream) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  if (int rc = check_agg(agg_mode)) return rc;
+  SIIRL_REQUIRE(mask && weights && out16 && row_msum, "NULL operand");
+  LossArgs a{};
+  // the partials pass over the weights buffer itself (its values are not used, only the mask sums are)
+  a.lp = weights; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode;
+  a.aux_agg_mode = agg_mode; a.scale = 1.f; a.B = B; a.L = L;
+  hipStream_t st = (hipStream_t)stream;
+  fill_kernel<<<dim3(1024), dim3(kThreads), 0, st>>>(weights, B * L, 0.f);
+  SIIRL_LAUNCH_CHECK("fill_kernel");
+  if (int rc = run_forward(a, out16, row_msum, nullptr, workspace, workspace_bytes, st)) return rc;
+  agg_weights_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, st>>>(a, out16, row_msum, weights);
+  SIIRL_LAUNCH_CHECK("agg_weights_kernel");
+  return SIIRL_OK;
 }
 
 extern "C" int siirl_agg_loss_bwd(const float* g_out, const void* mask, int mask_dtype, const float* out16,

@@ -1,0 +1,243 @@
+// Per-token formulas of the [B, L] loss arithmetic, shared by the loss kernels and by the fused logits ->
+// dlogits actor step: the registered policy losses (value and hand-derived gradient per token), the KL
+// estimators, aggregation weights, and small load helpers.
+//
+// Follows siirl/dag_worker/core_algos.py: agg_loss :536-569, cpgd :572-629, vanilla :710-792, gspo :795-862,
+// gpg :865-895, geo_mean :1074-1153, value loss :1173-1212, kl_penalty :1215-1276; drift term
+// siirl/engine/actor/dp_actor.py:488-494.
+#pragma once
+#include "common.hpp"
+
+namespace siirl {
+namespace tok {
+
+struct LossArgs {
+  const float* old_lp;   // [B,L] or null (kind == KIND_AGG)
+  const float* lp;       // [B,L]  (kind == KIND_AGG: the loss matrix to aggregate)
+  const float* adv;      // [B,L]
+  const void* mask;      // [B,L]
+  const float* isw;      // [B,L] or null
+  const float* ent;      // [B,L] or null
+  const float* ref;      // [B,L] or null
+  int mask_dtype;
+  int kind;              // KIND_*
+  int agg_mode;          // aggregation of the policy term (GSPO: forced to seq-mean-token-mean)
+  int aux_agg_mode;      // aggregation of the entropy and KL terms
+  int kl_mode, kl_st;
+  float eps_lo, eps_hi, clip_c, dclamp;
+  float log_lo, log_hi;  // CPGD: float(log(1 - eps_lo)), float(log(1 + eps_hi)), logarithms taken in double
+  float ent_coef, kl_coef, drift_coef, scale;
+  int64_t B, L;
+  int nseg;
+  int vec;  // L % 4 == 0 and every operand 16-byte aligned: tokens are moved four at a time
+};
+enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6 };
+
+// torch.clamp / torch.maximum / torch.minimum semantics (NaN propagates)
+__device__ __forceinline__ float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
+__device__ __forceinline__ float clamp_max(float x, float hi) { return x > hi ? hi : x; }
+__device__ __forceinline__ float tmax(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fmaxf(a, b); }
+__device__ __forceinline__ float tmin(float a, float b) { return (a != a || b != b) ? __builtin_nanf("") : fminf(a, b); }
+
+// masked contribution.  token-mean goes through masked_mean: where(mask, v, 0) * mask; the other modes
+// multiply directly (a NaN under a zero mask poisons them, as in the reference).
+__device__ __forceinline__ float contrib_where(float v, float m) { return m != 0.f ? v * m : 0.f; }
+__device__ __forceinline__ float contrib(float v, float m, int agg) {
+  return agg == SIIRL_AGG_TOKEN_MEAN ? contrib_where(v, m) : v * m;
+}
+
+// four consecutive tokens of one operand; `vec` selects one 16-byte access
+struct Quad {
+  float v[4];
+};
+__device__ __forceinline__ Quad load_quad(const float* __restrict__ p, int64_t idx, bool vec, int nv, float fill) {
+  Quad q;
+  if (vec) {
+    const float4 t = *reinterpret_cast<const float4*>(p + idx);
+    q.v[0] = t.x; q.v[1] = t.y; q.v[2] = t.z; q.v[3] = t.w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? p[idx + e] : fill;
+  }
+  return q;
+}
+__device__ __forceinline__ Quad const_quad(float c) { return Quad{{c, c, c, c}}; }
+__device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t idx, bool vec, int nv) {
+  Quad q;
+  if (vec && dt == SIIRL_I64) {
+    const longlong2 a = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[0];
+    const longlong2 b = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[1];
+    q.v[0] = (float)a.x; q.v[1] = (float)a.y; q.v[2] = (float)b.x; q.v[3] = (float)b.y;
+  } else if (vec && dt == SIIRL_U8) {
+    const uint32_t u = *reinterpret_cast<const uint32_t*>((const uint8_t*)p + idx);
+    q.v[0] = (float)(u & 0xffu); q.v[1] = (float)((u >> 8) & 0xffu); q.v[2] = (float)((u >> 16) & 0xffu);
+    q.v[3] = (float)(u >> 24);
+  } else if (vec && dt == SIIRL_F32) {
+    q = load_quad((const float*)p, idx, true, 4, 0.f);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? load_mask(p, dt, idx + e) : 0.f;
+  }
+  return q;
+}
+__device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q) {
+  if (vec) {
+    *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (e < nv) p[idx + e] = q.v[e];
+  }
+}
+
+struct KlOut {
+  float v, g;  // value and d value / d logprob
+};
+__device__ __forceinline__ KlOut kl_token(float lp, float ref, int mode, int straight_through) {
+  const float x = lp - ref;
+  KlOut o;
+  switch (mode) {
+    case SIIRL_KL_K1: o.v = x; o.g = 1.f; break;
+    case SIIRL_KL_ABS: o.v = fabsf(x); o.g = x > 0.f ? 1.f : (x < 0.f ? -1.f : 0.f); break;
+    case SIIRL_KL_K2: o.v = 0.5f * x * x; o.g = x; break;
+    default: {  // K3
+      const float kr = ref - lp;
+      const float k = clampf(kr, -20.f, 20.f);
+      const float e = expf(k);
+      const float raw = e - k - 1.f;
+      o.v = clampf(raw, -10.f, 10.f);
+      const bool pass = (kr >= -20.f && kr <= 20.f) && (raw >= -10.f && raw <= 10.f);
+      o.g = pass ? -(e - 1.f) : 0.f;
+    }
+  }
+  if (straight_through) o.g = x;  // value of the estimator, gradient of k2
+  return o;
+}
+
+struct PgOut {
+  float tok, dtok;  // per-token loss and d tok / d logprob (before the aggregation weight)
+  float clip, lower, negd, r_raw;
+};
+
+// seq_s: GSPO's sequence-level mean log-ratio (unused otherwise).  For KIND_GEO tok is the token's clipped
+// log-ratio x (the loss itself is per sequence); for KIND_VALUE lp = vpreds, old = values, A = returns and
+// eps_lo = cliprange_value.
+__device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A, float isw, float seq_s,
+                                          const LossArgs& a) {
+  const float eps_lo = a.eps_lo, eps_hi = a.eps_hi, clip_c = a.clip_c, dclamp = a.dclamp;
+  PgOut o;
+  const float raw = lp - old;
+  o.r_raw = expf(raw);
+  const float lo = 1.f - eps_lo, hi = 1.f + eps_hi;
+  if (kind == KIND_CPGD) {
+    // the log-probability is clipped, not the ratio; importance weights are not used by this loss
+    o.negd = -raw;
+    float clipped;
+    bool pass;
+    if (A > 0.f) {
+      const float b = a.log_hi + old;
+      clipped = lp > b ? b : lp;
+      pass = lp <= b;
+      o.clip = o.r_raw > hi ? 1.f : 0.f;
+    } else {
+      const float b = a.log_lo + old;
+      clipped = lp < b ? b : lp;
+      pass = lp >= b;
+      o.clip = o.r_raw < lo ? 1.f : 0.f;
+    }
+    o.tok = -clipped * A;
+    o.dtok = pass ? -A : 0.f;
+    o.lower = (o.r_raw > clip_c && A < 0.f) ? 1.f : 0.f;
+    return o;
+  }
+  if (kind == KIND_GPG) {
+    o.negd = 0.f; o.clip = 0.f; o.lower = 0.f;
+    o.tok = -lp * A * isw;
+    o.dtok = -A * isw;
+    return o;
+  }
+  if (kind == KIND_GEO) {
+    o.negd = -raw;
+    const float sgn = A > 0.f ? 1.f : (A < 0.f ? -1.f : (A == 0.f ? 0.f : A));  // torch.sign; NaN stays NaN
+    const float dc = clampf(raw, -eps_lo, eps_hi);
+    const float p = sgn * raw, q = sgn * dc;
+    o.tok = sgn * tmin(p, q);
+    const bool inside = raw >= -eps_lo && raw <= eps_hi;  // then p == q and both sides of the min pass 1/2
+    o.dtok = (inside || p < q) ? sgn * sgn : 0.f;
+    const bool clipped = raw != dc;
+    o.clip = (clipped && A > 0.f) ? 1.f : 0.f;
+    o.lower = (clipped && A < 0.f) ? 1.f : 0.f;
+    return o;
+  }
+  if (kind == KIND_VALUE) {
+    o.negd = 0.f; o.lower = 0.f; o.r_raw = 1.f;
+    const float vmax = old + eps_lo, vmin = old - eps_lo;
+    const float inner = tmin(lp, vmax), vc = tmax(inner, vmin);
+    const float e1 = lp - A, e2 = vc - A;
+    const float l1 = e1 * e1, l2 = e2 * e2;
+    o.tok = tmax(l1, l2);
+    o.clip = l2 > l1 ? 1.f : 0.f;
+    const float dinner = lp < vmax ? 1.f : (lp == vmax ? 0.5f : 0.f);
+    const float dvc = inner > vmin ? dinner : (inner == vmin ? 0.5f * dinner : 0.f);
+    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    o.dtok = w1 * 2.f * e1 + w2 * 2.f * e2 * dvc;
+    return o;
+  }
+  if (kind == KIND_VANILLA) {
+    const float d = clampf(raw, -dclamp, dclamp);
+    const float r = expf(d);
+    const float dr = (raw >= -dclamp && raw <= dclamp) ? r : 0.f;  // d r / d lp
+    o.negd = -d;
+    const float l1 = -A * r;
+    const float rc = clampf(r, lo, hi);
+    const float l2 = -A * rc;
+    const float c1 = tmax(l1, l2);
+    o.clip = l2 > l1 ? 1.f : 0.f;
+    const float l3 = -A * clip_c;
+    const float c2 = tmin(l3, c1);
+    o.lower = (c1 > l3 && A < 0.f) ? 1.f : 0.f;
+    o.tok = A < 0.f ? c2 : c1;
+    // autograd: maximum / minimum give each side 1, 1/2 (tie) or 0; clamp passes inside [lo, hi] inclusive
+    const float dl1 = -A * dr;
+    const float dl2 = (r >= lo && r <= hi) ? -A * dr : 0.f;
+    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float dc1 = w1 * dl1 + w2 * dl2;
+    const float wc = c1 < l3 ? 1.f : (c1 == l3 ? 0.5f : 0.f);
+    o.dtok = A < 0.f ? wc * dc1 : dc1;
+  } else {  // GSPO
+    o.negd = -raw;
+    const float l = clamp_max(seq_s, 10.f);  // lp - lp.detach() == 0
+    const float r = expf(l);
+    const float dr = (seq_s <= 10.f) ? r : 0.f;
+    const float l1 = -A * r;
+    const float rc = clampf(r, lo, hi);
+    const float l2 = -A * rc;
+    o.tok = tmax(l1, l2);
+    o.clip = l2 > l1 ? 1.f : 0.f;
+    o.lower = 0.f;
+    const float dl1 = -A * dr;
+    const float dl2 = (r >= lo && r <= hi) ? -A * dr : 0.f;
+    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    o.dtok = w1 * dl1 + w2 * dl2;
+  }
+  o.tok *= isw;  // importance weights multiply value and gradient alike
+  o.dtok *= isw;
+  return o;
+}
+
+
+// aggregation weight of token (b, t): d (aggregate) / d (loss_mat[b, t])
+__device__ __forceinline__ float agg_weight(int agg, float m, float mtotal, float mrow, int64_t B, int64_t L) {
+  switch (agg) {
+    case SIIRL_AGG_TOKEN_MEAN: return m != 0.f ? m / (mtotal + 1e-8f) : 0.f;
+    case SIIRL_AGG_SEQ_MEAN_TOKEN_SUM: return m / (float)B;
+    case SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN: return m / mrow / (float)B;
+    default: return m / (float)L;
+  }
+}
+
+}  // namespace tok
+}  // namespace siirl

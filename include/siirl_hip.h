@@ -125,7 +125,8 @@ int siirl_logprob_entropy_bwd(const void* logits, int logits_dtype, int64_t T, i
  * forward writes them, dlogits as the backward does, from one pass over HBM plus a partial second read (half of a
  * 152064-entry bf16 row stays in LDS between the passes).  g_logprob or g_entropy may be NULL; logprob / entropy
  * outputs may be NULL.  No in-place mode.
- * Replaces: the same functions as siirl_logprob_entropy_fwd + siirl_logprob_entropy_bwd.
+ * Replaces: logprobs_from_logits + entropy_from_logits siirl/utils/model_utils/torch_functional.py:56-116,128-143
+ *           and their autograd backward (closed form siirl/utils/experimental/torch_functional.py:49-62).
  */
 int siirl_logprob_entropy_fwd_bwd(const void* logits, int logits_dtype, int64_t T, int64_t V, int64_t row_stride,
                                   const int64_t* labels, float inv_temperature, const float* g_logprob,

@@ -162,6 +162,29 @@ def bench_config3(args, dev):
                      "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None},
         "cpu_baseline": None,
     }
+    if not args.no_cpu_baseline:  # the oracle's eager ops on the host cores, a 512-trajectory sample of the same step
+        from oracle import core_algos as OC
+        from oracle import dapo_filter as OD
+
+        n_s = 512
+        acc_c, uid_c = acc[:n_s * 2].cpu().numpy(), uid[:n_s * 2].cpu().numpy()
+        old_c, lp_c, ref_c = old[:n_s].cpu(), lp.detach()[:n_s].cpu(), ref[:n_s].cpu()
+        mk_c, rk_c, uk_c = mk[:n_s].cpu(), rk[:n_s].cpu(), uk[:n_s].cpu().numpy()
+        times = []
+        for it in range(4):
+            t1 = time.perf_counter()
+            OD.dynamic_sampling_keep_indices(acc_c, uid_c)
+            adv_c, _ = OC.compute_grpo_outcome_advantage(rk_c, mk_c, uk_c)
+            xc = lp_c.clone().requires_grad_(True)
+            pg, *_ = OC.compute_policy_loss_vanilla(old_c, xc, adv_c, mk_c, "token-mean", cfg)
+            kl = OC.agg_loss(OC.kl_penalty(xc, ref_c, "low_var_kl"), mk_c, "token-mean")
+            (pg + 0.001 * kl).backward()
+            if it:
+                times.append(time.perf_counter() - t1)
+        med = sorted(times)[len(times) // 2]
+        out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {n_s} kept trajectories (of {Bk}) x {L} tokens, filter over {2 * n_s} "
+                                         f"trajectories; median of 3 passes ({med:.2f} s each)"}
     print(json.dumps(out), flush=True)
 
 
@@ -223,6 +246,23 @@ def bench_config5(args, dev):
                      "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step; the backward's recompute is not counted"},
         "cpu_baseline": None,
     }
+    if not args.no_cpu_baseline:  # the oracle's chunked fp32 matmul + log-softmax on the host cores, 256 tokens
+        from oracle import fused_linear as OFL
+
+        n_s = 256
+        hc, wc, yc = h.detach()[:n_s].float().cpu(), w.detach().float().cpu(), y[:n_s].cpu()
+        gl, gh = g_lp[:n_s].cpu(), g_h[:n_s].cpu()
+        times = []
+        for it in range(3):
+            t1 = time.perf_counter()
+            OFL.fused_linear_for_ppo_fwd(hc, wc, yc)
+            OFL.fused_linear_for_ppo_bwd(gl, gh, hc, wc, yc)
+            if it:
+                times.append(time.perf_counter() - t1)
+        med = sorted(times)[len(times) // 2]
+        out["cpu_baseline"] = {"value": n_s / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {n_s} of {T} tokens against the full [{V}, {H}] weight in fp32; "
+                                         f"median of 2 fwd+bwd passes ({med:.2f} s each)"}
     print(json.dumps(out), flush=True)
 
 

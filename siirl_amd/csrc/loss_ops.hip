@@ -186,94 +186,146 @@ __device__ __forceinline__ double finish_term(double total, double mtotal, int a
   }
 }
 
+// running totals of the finish: nine sums (fp64) and the extremes of the raw ratio
+enum T { T_PG = 0, T_M, T_CLIP, T_NEGD, T_LOWER, T_ENT, T_KL, T_RSUM, T_DRIFT, T_COUNT };
+struct Totals {
+  double v[T_COUNT];
+  float rmin, rmax;
+  __device__ void init() {
+    for (int k = 0; k < T_COUNT; ++k) v[k] = 0.0;
+    rmin = __builtin_inff();
+    rmax = -__builtin_inff();
+  }
+};
+
+// folds the segments of row b into the totals and writes the row's mask sum
+__device__ __forceinline__ void fold_row(const LossArgs& a, const float* __restrict__ partials,
+                                         const float* __restrict__ row_s, float* __restrict__ row_msum, int64_t b,
+                                         Totals& t) {
+  double r[kNP];
+  for (int k = 0; k < kNP; ++k) r[k] = 0.0;
+  for (int s = 0; s < a.nseg; ++s) {
+    const float* p = partials + (b * a.nseg + s) * kNP;
+    for (int k = 0; k < kNP; ++k) {
+      if (k == P_RMIN) t.rmin = fminf(t.rmin, p[k]);
+      else if (k == P_RMAX) t.rmax = fmaxf(t.rmax, p[k]);
+      else r[k] += p[k];
+    }
+  }
+  row_msum[b] = (float)r[P_M];
+  t.v[T_M] += r[P_M];
+  t.v[T_PG] += a.kind == KIND_GEO ? (double)row_s[b] : row_term(r[P_PG], r[P_M], a.agg_mode);
+  t.v[T_DRIFT] += row_term(r[P_AUX0], r[P_M], a.aux_agg_mode);
+  t.v[T_ENT] += row_term(r[P_ENT], r[P_M], a.aux_agg_mode);
+  t.v[T_KL] += row_term(r[P_KL], r[P_M], a.aux_agg_mode);
+  t.v[T_CLIP] += r[P_CLIP];
+  t.v[T_NEGD] += r[P_NEGD];
+  t.v[T_LOWER] += r[P_LOWER];
+  t.v[T_RSUM] += r[P_RSUM];
+}
+
+// workgroup-wide reduction of the totals; the result is valid in thread 0
+__device__ __forceinline__ void reduce_totals(Totals& t) {
+  __shared__ double sh[kThreads / kWave + 1];
+  for (int k = 0; k < T_COUNT; ++k) t.v[k] = block_sum_d(t.v[k], sh);
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    t.rmin = fminf(t.rmin, __shfl_xor(t.rmin, o, kWave));
+    t.rmax = fmaxf(t.rmax, __shfl_xor(t.rmax, o, kWave));
+  }
+  __shared__ float shm[2 * (kThreads / kWave)];
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
+  __syncthreads();
+  if (lane == 0) {
+    shm[wid] = t.rmin;
+    shm[kThreads / kWave + wid] = t.rmax;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    for (int w = 1; w < kThreads / kWave; ++w) {
+      t.rmin = fminf(t.rmin, shm[w]);
+      t.rmax = fmaxf(t.rmax, shm[kThreads / kWave + w]);
+    }
+}
+
+__device__ __forceinline__ void write_result(const LossArgs& a, const Totals& t, float* __restrict__ out) {
+  const double t_m = t.v[T_M];
+  const double pg = a.kind == KIND_GEO ? t.v[T_PG] / (double)a.B : finish_term(t.v[T_PG], t_m, a.agg_mode, a.B, a.L);
+  const double den = t_m + 1e-8;
+  double policy = pg;
+  double entl = 0.0, kll = 0.0, drl = 0.0;
+  if (a.ent) {
+    entl = finish_term(t.v[T_ENT], t_m, a.aux_agg_mode, a.B, a.L);
+    policy = policy - entl * (double)a.ent_coef;
+  }
+  if (a.ref) {
+    kll = finish_term(t.v[T_KL], t_m, a.aux_agg_mode, a.B, a.L);
+    policy = policy + kll * (double)a.kl_coef;
+  }
+  if (a.drift_coef != 0.f) {
+    drl = finish_term(t.v[T_DRIFT], t_m, a.aux_agg_mode, a.B, a.L);
+    policy = policy + drl * (double)a.drift_coef;
+  }
+  for (int k = 0; k < O_COUNT; ++k) out[k] = 0.f;
+  out[O_PG] = (float)pg;
+  out[O_POLICY] = (float)policy;
+  out[O_LOSS] = (float)(policy * (double)a.scale);
+  out[O_MTOTAL] = (float)t_m;
+  if (a.kind != KIND_AGG) {
+    out[O_CLIPFRAC] = (float)(t.v[T_CLIP] / den);
+    out[O_PPOKL] = (float)(t.v[T_NEGD] / den);
+    out[O_CLIPLOWER] = (float)(t.v[T_LOWER] / den);
+    out[O_ENTLOSS] = (float)entl;
+    out[O_KLLOSS] = (float)kll;
+    out[O_DRIFT] = (float)drl;
+    out[O_RMEAN] = (float)(t.v[T_RSUM] / (double)(a.B * a.L));
+    out[O_RMIN] = t.rmin;
+    out[O_RMAX] = t.rmax;
+  }
+}
+
+// small batches: one workgroup folds every row and writes the result block
 __global__ __launch_bounds__(kThreads) void loss_finish_kernel(LossArgs a, const float* __restrict__ partials,
                                                                const float* __restrict__ row_s,
                                                                float* __restrict__ out,
                                                                float* __restrict__ row_msum) {
-  double t_pg = 0, t_m = 0, t_clip = 0, t_negd = 0, t_lower = 0, t_ent = 0, t_kl = 0, t_rsum = 0, t_drift = 0;
-  float rmin = __builtin_inff(), rmax = -__builtin_inff();
-  for (int64_t b = threadIdx.x; b < a.B; b += kThreads) {
-    double r[kNP];
-    for (int k = 0; k < kNP; ++k) r[k] = 0.0;
-    for (int s = 0; s < a.nseg; ++s) {
-      const float* p = partials + (b * a.nseg + s) * kNP;
-      for (int k = 0; k < kNP; ++k) {
-        if (k == P_RMIN) rmin = fminf(rmin, p[k]);
-        else if (k == P_RMAX) rmax = fmaxf(rmax, p[k]);
-        else r[k] += p[k];
-      }
-    }
-    row_msum[b] = (float)r[P_M];
-    t_m += r[P_M];
-    t_pg += a.kind == KIND_GEO ? (double)row_s[b] : row_term(r[P_PG], r[P_M], a.agg_mode);
-    t_drift += row_term(r[P_AUX0], r[P_M], a.aux_agg_mode);
-    t_ent += row_term(r[P_ENT], r[P_M], a.aux_agg_mode);
-    t_kl += row_term(r[P_KL], r[P_M], a.aux_agg_mode);
-    t_clip += r[P_CLIP];
-    t_negd += r[P_NEGD];
-    t_lower += r[P_LOWER];
-    t_rsum += r[P_RSUM];
-  }
-  __shared__ double sh[kThreads / kWave + 1];
-  t_pg = block_sum_d(t_pg, sh);
-  t_m = block_sum_d(t_m, sh);
-  t_clip = block_sum_d(t_clip, sh);
-  t_negd = block_sum_d(t_negd, sh);
-  t_lower = block_sum_d(t_lower, sh);
-  t_ent = block_sum_d(t_ent, sh);
-  t_kl = block_sum_d(t_kl, sh);
-  t_rsum = block_sum_d(t_rsum, sh);
-  t_drift = block_sum_d(t_drift, sh);
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    rmin = fminf(rmin, __shfl_xor(rmin, o, kWave));
-    rmax = fmaxf(rmax, __shfl_xor(rmax, o, kWave));
-  }
-  __shared__ float shm[2 * (kThreads / kWave)];
-  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
-  if (lane == 0) {
-    shm[wid] = rmin;
-    shm[kThreads / kWave + wid] = rmax;
-  }
-  __syncthreads();
+  Totals t;
+  t.init();
+  for (int64_t b = threadIdx.x; b < a.B; b += kThreads) fold_row(a, partials, row_s, row_msum, b, t);
+  reduce_totals(t);
+  if (threadIdx.x == 0) write_result(a, t, out);
+}
+
+// large batches, level 1: one thread per row, one record of totals per workgroup
+constexpr int kFinRec = T_COUNT + 2;
+__global__ __launch_bounds__(kThreads) void loss_rows_kernel(LossArgs a, const float* __restrict__ partials,
+                                                             const float* __restrict__ row_s,
+                                                             float* __restrict__ row_msum, double* __restrict__ rec) {
+  Totals t;
+  t.init();
+  const int64_t b = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  if (b < a.B) fold_row(a, partials, row_s, row_msum, b, t);
+  reduce_totals(t);
   if (threadIdx.x == 0) {
-    for (int w = 1; w < kThreads / kWave; ++w) {
-      rmin = fminf(rmin, shm[w]);
-      rmax = fmaxf(rmax, shm[kThreads / kWave + w]);
-    }
-    const double pg = a.kind == KIND_GEO ? t_pg / (double)a.B : finish_term(t_pg, t_m, a.agg_mode, a.B, a.L);
-    const double den = t_m + 1e-8;
-    double policy = pg;
-    double entl = 0.0, kll = 0.0, drl = 0.0;
-    if (a.ent) {
-      entl = finish_term(t_ent, t_m, a.aux_agg_mode, a.B, a.L);
-      policy = policy - entl * (double)a.ent_coef;
-    }
-    if (a.ref) {
-      kll = finish_term(t_kl, t_m, a.aux_agg_mode, a.B, a.L);
-      policy = policy + kll * (double)a.kl_coef;
-    }
-    if (a.drift_coef != 0.f) {
-      drl = finish_term(t_drift, t_m, a.aux_agg_mode, a.B, a.L);
-      policy = policy + drl * (double)a.drift_coef;
-    }
-    for (int k = 0; k < O_COUNT; ++k) out[k] = 0.f;
-    out[O_PG] = (float)pg;
-    out[O_POLICY] = (float)policy;
-    out[O_LOSS] = (float)(policy * (double)a.scale);
-    out[O_MTOTAL] = (float)t_m;
-    if (a.kind != KIND_AGG) {
-      out[O_CLIPFRAC] = (float)(t_clip / den);
-      out[O_PPOKL] = (float)(t_negd / den);
-      out[O_CLIPLOWER] = (float)(t_lower / den);
-      out[O_ENTLOSS] = (float)entl;
-      out[O_KLLOSS] = (float)kll;
-      out[O_DRIFT] = (float)drl;
-      out[O_RMEAN] = (float)(t_rsum / (double)(a.B * a.L));
-      out[O_RMIN] = rmin;
-      out[O_RMAX] = rmax;
-    }
+    double* r = rec + (int64_t)blockIdx.x * kFinRec;
+    for (int k = 0; k < T_COUNT; ++k) r[k] = t.v[k];
+    r[T_COUNT] = (double)t.rmin;
+    r[T_COUNT + 1] = (double)t.rmax;
   }
+}
+// level 2: one workgroup folds the records in order
+__global__ __launch_bounds__(kThreads) void loss_finish2_kernel(LossArgs a, const double* __restrict__ rec, int nrec,
+                                                                float* __restrict__ out) {
+  Totals t;
+  t.init();
+  for (int i = threadIdx.x; i < nrec; i += kThreads) {
+    const double* r = rec + (int64_t)i * kFinRec;
+    for (int k = 0; k < T_COUNT; ++k) t.v[k] += r[k];
+    t.rmin = fminf(t.rmin, (float)r[T_COUNT]);
+    t.rmax = fmaxf(t.rmax, (float)r[T_COUNT + 1]);
+  }
+  reduce_totals(t);
+  if (threadIdx.x == 0) write_result(a, t, out);
 }
 
 // ---------------------------------------------------------------------------- backward
@@ -446,8 +498,10 @@ void set_vec(LossArgs& a, const void* o1 = nullptr, const void* o2 = nullptr) {
 
 size_t ws_bytes_of(int64_t B, int64_t L) {
   const size_t ns = (size_t)nseg_of(L);
-  return (size_t)B * ns * kNP * sizeof(float) + (size_t)B * ns * kNPre * sizeof(float) + 256;
+  return (size_t)B * ns * kNP * sizeof(float) + (size_t)B * ns * kNPre * sizeof(float) + 256 +
+         (size_t)((B + kThreads - 1) / kThreads) * kFinRec * sizeof(double);
 }
+constexpr int64_t kTwoLevelRows = 2048;  // above this many rows the finish runs in two levels
 
 int check_dims(int64_t B, int64_t L) {
   SIIRL_REQUIRE(B >= 1 && L >= 1, "B=%lld L=%lld must be positive", (long long)B, (long long)L);
@@ -471,6 +525,7 @@ int run_forward(LossArgs& a, float* out16, float* row_msum, float* row_s, void* 
   if (ws_bytes < ws_bytes_of(a.B, a.L) || ws == nullptr)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed for B=%lld L=%lld",
                 ws_bytes, ws_bytes_of(a.B, a.L), (long long)a.B, (long long)a.L);
+  SIIRL_REQUIRE(((uintptr_t)ws & 7) == 0, "workspace must be 8-byte aligned");
   set_vec(a);
   float* partials = (float*)ws;
   float* pre = partials + (size_t)a.B * a.nseg * kNP;
@@ -484,8 +539,18 @@ int run_forward(LossArgs& a, float* out16, float* row_msum, float* row_s, void* 
   }
   loss_partials_kernel<<<grid, block, 0, st>>>(a, row_s, partials);
   SIIRL_LAUNCH_CHECK("loss_partials_kernel");
-  loss_finish_kernel<<<1, block, 0, st>>>(a, partials, row_s, out16, row_msum);
-  SIIRL_LAUNCH_CHECK("loss_finish_kernel");
+  if (a.B <= kTwoLevelRows) {
+    loss_finish_kernel<<<1, block, 0, st>>>(a, partials, row_s, out16, row_msum);
+    SIIRL_LAUNCH_CHECK("loss_finish_kernel");
+  } else {
+    const size_t used = ((size_t)a.B * a.nseg * (kNP + kNPre) * sizeof(float) + 255) / 256 * 256;
+    double* rec = reinterpret_cast<double*>((char*)ws + used);
+    const int nrec = (int)((a.B + kThreads - 1) / kThreads);
+    loss_rows_kernel<<<dim3((unsigned)nrec), block, 0, st>>>(a, partials, row_s, row_msum, rec);
+    SIIRL_LAUNCH_CHECK("loss_rows_kernel");
+    loss_finish2_kernel<<<1, block, 0, st>>>(a, rec, nrec, out16);
+    SIIRL_LAUNCH_CHECK("loss_finish2_kernel");
+  }
   return SIIRL_OK;
 }
 

@@ -186,7 +186,7 @@ __device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A
   }
   if (kind == KIND_VANILLA) {
     const float d = clampf(raw, -dclamp, dclamp);
-    const float r = expf(d);
+    const float r = d == raw ? o.r_raw : expf(d);  // the clamp rarely bites: one exponential serves both
     const float dr = (raw >= -dclamp && raw <= dclamp) ? r : 0.f;  // d r / d lp
     o.negd = -d;
     const float l1 = -A * r;

@@ -557,8 +557,9 @@ int launch_gemm(const uint16_t* A, int64_t lda, const u32x4* Bp, int64_t kb_tota
 
 int check_fused(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V, float inv_T, int dtype) {
   SIIRL_REQUIRE(dtype == SIIRL_BF16, "fused lm_head path takes bf16 operands (dtype %d given)", dtype);
-  SIIRL_REQUIRE(T >= 1 && T < (1LL << 30) && V >= 1 && V < (1LL << 30), "T=%lld V=%lld out of range", (long long)T,
-                (long long)V);
+  // 32-bit byte offsets inside a 256-row tile bound the row pitch of every A operand (W: H, D: slab, Dt: T + pad)
+  SIIRL_REQUIRE(T >= 1 && T < (1LL << 22) && V >= 1 && V < (1LL << 30), "T=%lld (< 4194304) V=%lld out of range",
+                (long long)T, (long long)V);
   SIIRL_REQUIRE(H >= BK && H % BK == 0 && H < (1 << 22), "hidden size %lld must be a positive multiple of %d",
                 (long long)H, BK);
   SIIRL_REQUIRE(hidden && weight, "NULL operand");

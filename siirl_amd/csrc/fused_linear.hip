@@ -44,6 +44,12 @@ constexpr int kStages = 4;
 constexpr int kSmemBytes = kStages * kStageBytes;  // 131072
 constexpr int kDmaPerWave = kTileBytes / 1024 / (kThreads / 64);  // 1 KB per wave instruction
 constexpr int kSlab = 8192;                   // vocabulary columns per backward slab
+#ifndef SIIRL_DH_GROUP
+#define SIIRL_DH_GROUP 4
+#endif
+constexpr int kDhGroup = SIIRL_DH_GROUP;      // slabs of dlogits kept before d hidden and d weight are updated: fewer
+                                              // fp32 read-modify-write passes over [T, H], and 4 x 448 d-weight
+                                              // tiles fill 7 rounds of the 256 CUs exactly
 constexpr int kLdPad = 64;                    // extra elements per row of D / Dt: keeps a tile's 256 rows off a
                                               // power-of-two stride, which would put them all in one memory channel
 
@@ -54,6 +60,7 @@ struct GemmArgs {
   int64_t kb_total; // 16-wide K blocks per 32-row block of the packed buffer
   int M, N, K;  // K is a multiple of BK; rows beyond M are clamped on load and masked by the epilogue
   int tiles_m, tiles_n;
+  int splits;  // K is cut into `splits` runs of K-steps; run s is tile column tn + s * tiles_n of the raster
 };
 
 struct TileCoord {
@@ -77,7 +84,7 @@ __device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int id) {
   const int mb = (g.tiles_m + kBlkM - 1) / kBlkM;
   const int tm = (blk % mb) * kBlkM + j % kBlkM;
   const int tn = (blk / mb) * kBlkN + j / kBlkM;
-  return {tm, tn, tm < g.tiles_m && tn < g.tiles_n};
+  return {tm, tn, tm < g.tiles_m && tn < g.tiles_n * g.splits};
 }
 
 // Accumulator coordinates of lane `lane` in wave (wm, wn): element r of acc[i][j] is
@@ -97,14 +104,18 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
   const int wm = w / WN, wn = w % WN;
   const TileCoord tc = tile_of(g, blockIdx.x);
   if (!tc.valid) return;
-  const int m0 = tc.tm * BM, n0 = tc.tn * BN;
-  const int KT = g.K / BK;
+  const int split = tc.tn / g.tiles_n;
+  const int m0 = tc.tm * BM, n0 = (tc.tn - split * g.tiles_n) * BN;
+  // this workgroup's run of K-steps (the host keeps every run non-empty)
+  const int kt_per = (g.K / BK + g.splits - 1) / g.splits;
+  const int kt_first = split * kt_per;
+  const int KT = (g.K / BK - kt_first < kt_per) ? g.K / BK - kt_first : kt_per;
 
   // A: global -> LDS by DMA (global_load_lds_dwordx4): wave instruction I = w * kDmaPerWave + i fills the 1 KB
   // [I * 1024, I * 1024 + 1024) of the stage; 16-byte slot sl = I * 64 + lane holds row sl / 8, chunk
   // (sl % 8) ^ ((row / 2) % 8).  Rows past the matrix edge are clamped to the last row.
   const int wu = __builtin_amdgcn_readfirstlane(w);
-  const char* gA = reinterpret_cast<const char*>(g.A + (int64_t)m0 * g.lda);
+  const char* gA = reinterpret_cast<const char*>(g.A + (int64_t)m0 * g.lda + (int64_t)kt_first * BK);
   uint32_t offA[kDmaPerWave];
 #pragma unroll
   for (int i = 0; i < kDmaPerWave; ++i) {
@@ -116,7 +127,8 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
   // B: fragment-packed, one 16-byte load per lane per MFMA operand, no LDS
-  const char* gB = reinterpret_cast<const char*>(g.Bp + (int64_t)(n0 >> 5) * g.kb_total * 64);
+  const char* gB =
+      reinterpret_cast<const char*>(g.Bp + ((int64_t)(n0 >> 5) * g.kb_total + (int64_t)kt_first * (BK / 16)) * 64);
   uint32_t offB[NJ];
 #pragma unroll
   for (int j = 0; j < NJ; ++j) offB[j] = (uint32_t)(((wn * NJ + j) * g.kb_total * 64 + lane) * 16);
@@ -221,7 +233,7 @@ __global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) 
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
 #undef SIIRL_BWAIT
-  epi(acc, m0, n0, tc.tm, wm, wn, lane, tid, smem);
+  epi(acc, m0, n0, tc.tm, split, wm, wn, lane, tid, smem);
 }
 #pragma clang diagnostic pop
 
@@ -238,7 +250,7 @@ struct SoftmaxPartialsEpi {
   float inv_T;
   int T, V;
   float* part;  // [tiles_m][3][T]
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn,
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
                                              int lane, int tid, char* smem) const {
     float* sh = reinterpret_cast<float*>(smem);  // [WM][BN][3]; the main loop's last barrier freed the LDS
     const float k = kLog2e;
@@ -319,7 +331,7 @@ struct DlogitsEpi {
   int64_t ldd;
   uint16_t* Dt;
   int64_t ldt;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn,
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
                                              int lane, int tid, char* smem) const {
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
@@ -362,11 +374,11 @@ struct DlogitsEpi {
 
 // ------------------------------------------------------------------------------ epilogues: plain stores
 
-struct AccumF32Epi {  // C[row][col] = (beta ? C : 0) + acc
+struct AccumF32Epi {  // C_s[row][col] = (beta ? C_s : 0) + acc, one fp32 buffer C_s = C + s * split_stride per K run
   float* C;
-  int64_t ldc;
+  int64_t ldc, split_stride;
   int M, N, beta;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn, int lane, int tid,
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn, int lane, int tid,
                              char* smem) const {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -378,7 +390,7 @@ struct AccumF32Epi {  // C[row][col] = (beta ? C : 0) + acc
         for (int j = 0; j < NJ; ++j) {
           const int col = n0 + acc_col(wn, j, lane);
           if (col >= N) continue;
-          float* p = C + (int64_t)row * ldc + col;
+          float* p = C + split * split_stride + (int64_t)row * ldc + col;
           *p = beta ? *p + acc[i][j][r] : acc[i][j][r];
         }
       }
@@ -389,7 +401,7 @@ struct StoreBf16Epi {  // C[row][col] = bf16(acc)
   uint16_t* C;
   int64_t ldc;
   int M, N;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int wm, int wn, int lane, int tid,
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn, int lane, int tid,
                              char* smem) const {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
@@ -529,10 +541,10 @@ __global__ __launch_bounds__(256) void zero_cols_kernel(uint16_t* __restrict__ p
   if (c < c1) p[(int64_t)r * ld + c] = 0;
 }
 
-__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, uint16_t* __restrict__ out,
-                                                          int64_t n) {
+__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, const float* __restrict__ in2,
+                                                          uint16_t* __restrict__ out, int64_t n) {
   for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
-    out[i] = (uint16_t)(pack_bf16(in[i], 0.f) & 0xffffu);
+    out[i] = (uint16_t)(pack_bf16(in2 ? in[i] + in2[i] : in[i], 0.f) & 0xffffu);
 }
 
 // ------------------------------------------------------------------------------ host
@@ -541,18 +553,27 @@ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 template <class Epi>
 int launch_gemm(const uint16_t* A, int64_t lda, const u32x4* Bp, int64_t kb_total, int M, int N, int K, const Epi& epi,
-                hipStream_t st, const char* what) {
+                hipStream_t st, const char* what, int splits = 1) {
   static bool attr_set = false;  // one flag per instantiation
   if (!attr_set) {
     SIIRL_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi>),
                                         hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
     attr_set = true;
   }
-  GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN};
-  const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n);
+  GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN, splits};
+  const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n * splits);
   gemm_nt_kernel<Epi><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
   SIIRL_LAUNCH_CHECK(what);
   return SIIRL_OK;
+}
+
+// Two K runs when that fills the 256 compute units' last round noticeably better (896 tiles = 3.5 rounds become
+// 1792 = 7) and the GEMM is deep enough for the second fp32 buffer's extra pass not to matter.
+inline int pick_splits(int M, int N, int K) {
+  const int64_t tiles = (int64_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+  auto eff = [](int64_t t) { return (double)t / (double)((t + 255) / 256 * 256); };
+  if (K / BK < 128) return 1;
+  return eff(2 * tiles) > eff(tiles) * 1.05 ? 2 : 1;
 }
 
 int check_fused(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V, float inv_T, int dtype) {
@@ -594,7 +615,7 @@ BwdWs bwd_ws(int64_t T, int64_t H, int64_t V, bool want_dh, bool want_dw) {
   BwdWs w;
   w.ldwt = round_up(V, BK);
   w.ldt = round_up(T, BK);
-  w.ldd_row = kSlab + kLdPad;
+  w.ldd_row = (int64_t)kDhGroup * kSlab + kLdPad;
   w.ldt_row = w.ldt + kLdPad;
   w.hpad = round_up(H, BN);
   size_t off = 0;
@@ -602,8 +623,8 @@ BwdWs bwd_ws(int64_t T, int64_t H, int64_t V, bool want_dh, bool want_dw) {
   w.wtp = off; off += want_dh ? (size_t)w.hpad * w.ldwt * 2 : 0;
   w.htp = off; off += want_dw ? (size_t)w.hpad * w.ldt * 2 : 0;
   w.d = off; off += round_up((size_t)T * w.ldd_row * 2, 256);
-  w.dt = off; off += round_up((size_t)kSlab * w.ldt_row * 2, 256);
-  w.dh32 = off; off += want_dh ? round_up((size_t)T * H * 4, 256) : 0;
+  w.dt = off; off += round_up((size_t)kDhGroup * kSlab * w.ldt_row * 2, 256);
+  w.dh32 = off; off += want_dh ? 2 * round_up((size_t)T * H * 4, 256) : 0;  // one buffer per K run
   w.total = off;
   return w;
 }
@@ -687,8 +708,8 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
   u32x4* hp = (u32x4*)(base + ws.hp);          // packed hidden: B[n = token][k = H]
   u32x4* Wtp = (u32x4*)(base + ws.wtp);        // packed W^T:    B[n = H][k = vocabulary]
   u32x4* Htp = (u32x4*)(base + ws.htp);        // packed hidden^T: B[n = H][k = token]
-  uint16_t* D = (uint16_t*)(base + ws.d);      // [T][ldd_row]
-  uint16_t* Dt = (uint16_t*)(base + ws.dt);    // [kSlab][ldt_row]
+  uint16_t* D = (uint16_t*)(base + ws.d);      // [T][ldd_row]: kDhGroup slabs side by side
+  uint16_t* Dt = (uint16_t*)(base + ws.dt);    // [kDhGroup * kSlab][ldt_row]
   float* dH32 = (float*)(base + ws.dh32);      // [T][H]
   const uint16_t* h = (const uint16_t*)hidden;
   const uint16_t* w = (const uint16_t*)weight;
@@ -707,32 +728,47 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
   // K-padding columns of Dt (token index in [T, ldt)) are never written by the epilogue: clear once (with a
   // kernel, not a memset node, so that the call can be captured into a graph)
   if (ws.ldt > T) {
-    zero_cols_kernel<<<dim3(kSlab / 4), dim3(256), 0, st>>>(Dt, ws.ldt_row, (int)T, (int)ws.ldt);
+    zero_cols_kernel<<<dim3(kDhGroup * kSlab / 4), dim3(256), 0, st>>>(Dt, ws.ldt_row, (int)T, (int)ws.ldt);
     SIIRL_LAUNCH_CHECK("zero_cols_kernel");
   }
 
+  int dh_splits = 1;
+  const int64_t dh32_stride = (int64_t)(round_up((size_t)T * H * 4, 256) / 4);
   int slab_idx = 0;
   for (int64_t v0 = 0; v0 < V; v0 += kSlab, ++slab_idx) {
     const int N = (int)((V - v0) < kSlab ? (V - v0) : kSlab);
     const int Npad = (int)round_up(N, BK);
-    DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels, D, ws.ldd_row, Dt, ws.ldt_row};
+    const int gs = slab_idx % kDhGroup;  // position of this slab in its group of D columns
+    DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
+                   D + (int64_t)gs * kSlab, ws.ldd_row, Dt + (int64_t)gs * kSlab * ws.ldt_row, ws.ldt_row};
     if (int rc = launch_gemm(w + v0 * H, H, hp, H / 16, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
-    if (want_dh) {  // dH[T, H] += D[T, Npad] . Wt[H, v0 : v0 + Npad]^T
-      AccumF32Epi acc{dH32, H, (int)T, (int)H, slab_idx > 0 ? 1 : 0};
-      if (int rc = launch_gemm(D, ws.ldd_row, Wtp + (v0 / 16) * 64, ws.ldwt / 16, (int)T, (int)H, Npad, acc, st,
-                               "gemm_nt_kernel<AccumF32Epi>"))
+    if (want_dh && (gs == kDhGroup - 1 || v0 + kSlab >= V)) {
+      // dH[T, H] += D[T, K] . Wt[H, g0 : g0 + K]^T over the group's columns (only the last slab can be partial)
+      const int64_t g0 = v0 - (int64_t)gs * kSlab;
+      const int K = gs * kSlab + Npad;
+      // the first group decides whether d hidden is accumulated as two K runs; a shallower last group then still
+      // writes both buffers (its second run may be short, never empty: K >= 2 K-steps)
+      if (g0 == 0) dh_splits = pick_splits((int)T, (int)H, K);
+      const int splits = (K / BK >= 2) ? dh_splits : 1;
+      AccumF32Epi acc{dH32, H, dh32_stride, (int)T, (int)H, g0 > 0 ? 1 : 0};
+      if (int rc = launch_gemm(D, ws.ldd_row, Wtp + (g0 / 16) * 64, ws.ldwt / 16, (int)T, (int)H, K, acc, st,
+                               "gemm_nt_kernel<AccumF32Epi>", splits))
         return rc;
     }
-    if (want_dw) {  // dW[v0 : v0 + N, H] = Dt[N, ldt] . Ht[H, ldt]^T
-      StoreBf16Epi sto{(uint16_t*)d_weight + v0 * H, H, N, (int)H};
-      if (int rc = launch_gemm(Dt, ws.ldt_row, Htp, ws.ldt / 16, N, (int)H, (int)ws.ldt, sto, st, "gemm_nt_kernel<StoreBf16Epi>"))
+    if (want_dw && (gs == kDhGroup - 1 || v0 + kSlab >= V)) {
+      // dW[g0 : g0 + M, H] = Dt[M, ldt] . Ht[H, ldt]^T over the group's vocabulary rows
+      const int64_t g0 = v0 - (int64_t)gs * kSlab;
+      const int M = gs * kSlab + N;
+      StoreBf16Epi sto{(uint16_t*)d_weight + g0 * H, H, M, (int)H};
+      if (int rc = launch_gemm(Dt, ws.ldt_row, Htp, ws.ldt / 16, M, (int)H, (int)ws.ldt, sto, st, "gemm_nt_kernel<StoreBf16Epi>"))
         return rc;
     }
   }
   if (want_dh) {
     const int64_t n = T * H;
     const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
-    f32_to_bf16_kernel<<<dim3(blocks), dim3(256), 0, st>>>(dH32, (uint16_t*)d_hidden, n);
+    f32_to_bf16_kernel<<<dim3(blocks), dim3(256), 0, st>>>(dH32, dh_splits > 1 ? dH32 + dh32_stride : nullptr,
+                                                           (uint16_t*)d_hidden, n);
     SIIRL_LAUNCH_CHECK("f32_to_bf16_kernel");
   }
   return SIIRL_OK;

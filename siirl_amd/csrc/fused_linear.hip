@@ -43,7 +43,10 @@ constexpr int kStageBytes = kTileBytes;       // A tile only: B goes global -> r
 constexpr int kStages = 4;
 constexpr int kSmemBytes = kStages * kStageBytes;  // 131072
 constexpr int kDmaPerWave = kTileBytes / 1024 / (kThreads / 64);  // 1 KB per wave instruction
-constexpr int kSlab = 8192;                   // vocabulary columns per backward slab
+#ifndef SIIRL_SLAB
+#define SIIRL_SLAB 8192
+#endif
+constexpr int kSlab = SIIRL_SLAB;                   // vocabulary columns per backward slab
 #ifndef SIIRL_DH_GROUP
 #define SIIRL_DH_GROUP 4
 #endif

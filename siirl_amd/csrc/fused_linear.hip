@@ -320,7 +320,9 @@ struct SoftmaxPartialsEpi {
 // d raw_logit = inv_T * ( g_lp * (1[v == y] - p) - g_h * p * (z - ex) ),  p = exp(z - lse), z = acc * inv_T,
 // written as bf16 to D[token][v] (ld = ldd) and to Dt[v][token] (ld = ldt); v is slab-relative and is the M
 // dimension of this GEMM.  Rows v in [Vs, Vpad) are written as zeros: they are K-padding of the GEMM that
-// consumes D.  A lane owns one token, so the per-token coefficients are loaded once per lane.
+// consumes D; likewise the token columns [T, ldt_k) of Dt.  A lane owns one token, so the per-token
+// coefficients are loaded once per lane and D gets 8-byte stores; the transposed copy goes through LDS and
+// leaves as whole 16-byte chunks of a row instead of 2-byte stores.
 struct DlogitsEpi {
   float inv_T;
   int T, Vs, Vpad;
@@ -334,29 +336,40 @@ struct DlogitsEpi {
   int64_t ldd;
   uint16_t* Dt;
   int64_t ldt;
+  int64_t ldt_k;  // token columns of Dt that the consuming GEMM reads (a multiple of BK, >= T): [T, ldt_k) get zeros
+  // LDS image of the tile's Dt block: 256 vocabulary rows x 256 tokens of bf16, 512-byte rows, 16-byte chunks
+  // XOR-swizzled by the row so that the two lane halves (rows v and v + 4) and successive rows spread over the banks
+  static __device__ __forceinline__ int lds_at(int vrow, int tok_l) {
+    return vrow * (BN * 2) + ((((tok_l >> 3) ^ vrow) & 31) << 4) + ((tok_l & 7) << 1);
+  }
   __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
                                              int lane, int tid, char* smem) const {
+    // the main loop's last barrier (and its vmcnt(0)) freed the ring: 256 x 512 B fit it exactly
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const int tok = n0 + acc_col(wn, j, lane);
-      if (tok >= T) continue;
-      const float g1 = g_lp ? g_lp[tok] : 0.f;
-      const float g2 = g_h ? g_h[tok] : 0.f;
-      const float nl = -lse[tok] * kLog2e;
-      const float exv = g_h ? ex[tok] : 0.f;
-      const int y = g_lp ? (int)((labels[tok] - v0 >= 0 && labels[tok] - v0 < Vs) ? labels[tok] - v0 : -1) : -1;
+      const int tok_l = acc_col(wn, j, lane), tok = n0 + tok_l;
+      const bool live = tok < T;
+      const float g1 = (live && g_lp) ? g_lp[tok] : 0.f;
+      const float g2 = (live && g_h) ? g_h[tok] : 0.f;
+      const float nl = live ? -lse[tok] * kLog2e : 0.f;
+      const float exv = (live && g_h) ? ex[tok] : 0.f;
+      int y = -1;
+      if (live && g_lp) {
+        const int64_t yl = labels[tok] - v0;
+        if (yl >= 0 && yl < Vs) y = (int)yl;
+      }
       uint16_t* drow = D + (int64_t)tok * ldd;
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int v = m0 + acc_row(wm, i, q * 4, lane);  // 4 consecutive vocabulary rows v .. v+3
-          if (v >= Vpad) continue;
+          const int vl = acc_row(wm, i, q * 4, lane);  // 4 consecutive vocabulary rows of the tile
+          const int v = m0 + vl;
           float d[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             d[e] = 0.f;
-            if (v + e < Vs) {
+            if (live && v + e < Vs) {
               const float z = acc[i][j][q * 4 + e] * inv_T;
               const float p = fast_exp2(fmaf(z, kLog2e, nl));
               float g = p * (-g1 - g2 * (z - exv));
@@ -365,12 +378,23 @@ struct DlogitsEpi {
             }
           }
           const uint32_t lo = pack_bf16(d[0], d[1]), hi = pack_bf16(d[2], d[3]);
-          *reinterpret_cast<uint2*>(drow + v) = make_uint2(lo, hi);  // v % 4 == 0, ldd % 4 == 0: 8-byte aligned
-          Dt[(int64_t)(v + 0) * ldt + tok] = (uint16_t)(lo & 0xffffu);
-          Dt[(int64_t)(v + 1) * ldt + tok] = (uint16_t)(lo >> 16);
-          Dt[(int64_t)(v + 2) * ldt + tok] = (uint16_t)(hi & 0xffffu);
-          Dt[(int64_t)(v + 3) * ldt + tok] = (uint16_t)(hi >> 16);
+          if (live && v < Vpad) *reinterpret_cast<uint2*>(drow + v) = make_uint2(lo, hi);  // 8-byte aligned
+          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 0, tok_l)) = (uint16_t)(lo & 0xffffu);
+          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 1, tok_l)) = (uint16_t)(lo >> 16);
+          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 2, tok_l)) = (uint16_t)(hi & 0xffffu);
+          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 3, tok_l)) = (uint16_t)(hi >> 16);
         }
+    }
+    __syncthreads();
+    // Dt[v][token]: rows leave the LDS as 16-byte chunks, 32 consecutive threads per 512-byte row
+#pragma unroll 4
+    for (int id = tid; id < BM * (BN / 8); id += kThreads) {
+      const int vrow = id >> 5, c = id & 31;
+      const int v = m0 + vrow, t0 = n0 + c * 8;
+      if (v < Vpad && t0 < ldt_k) {
+        const u32x4 val = *reinterpret_cast<const u32x4*>(smem + vrow * (BN * 2) + (((c ^ vrow) & 31) << 4));
+        *reinterpret_cast<u32x4*>(Dt + (int64_t)v * ldt + t0) = val;
+      }
     }
   }
 };
@@ -536,12 +560,6 @@ __global__ __launch_bounds__(256) void merge_partials_kernel(const float* __rest
   if (ex_out) ex_out[row] = exv;
   if (entropy) entropy[row] = lse - exv;
   if (logprob) logprob[row] = label_logit[row] - lse;
-}
-
-// p[r][c] = 0 for c in [c0, c1), four rows per workgroup (c1 - c0 < 64)
-__global__ __launch_bounds__(256) void zero_cols_kernel(uint16_t* __restrict__ p, int64_t ld, int c0, int c1) {
-  const int r = blockIdx.x * 4 + (threadIdx.x >> 6), c = c0 + (threadIdx.x & 63);
-  if (c < c1) p[(int64_t)r * ld + c] = 0;
 }
 
 __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, const float* __restrict__ in2,
@@ -728,13 +746,6 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
         h, H, (int)T, (int)H, Htp, ws.ldt / 16);
     SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(hidden)");
   }
-  // K-padding columns of Dt (token index in [T, ldt)) are never written by the epilogue: clear once (with a
-  // kernel, not a memset node, so that the call can be captured into a graph)
-  if (ws.ldt > T) {
-    zero_cols_kernel<<<dim3(kDhGroup * kSlab / 4), dim3(256), 0, st>>>(Dt, ws.ldt_row, (int)T, (int)ws.ldt);
-    SIIRL_LAUNCH_CHECK("zero_cols_kernel");
-  }
-
   int dh_splits = 1;
   const int64_t dh32_stride = (int64_t)(round_up((size_t)T * H * 4, 256) / 4);
   int slab_idx = 0;
@@ -743,7 +754,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
     const int Npad = (int)round_up(N, BK);
     const int gs = slab_idx % kDhGroup;  // position of this slab in its group of D columns
     DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
-                   D + (int64_t)gs * kSlab, ws.ldd_row, Dt + (int64_t)gs * kSlab * ws.ldt_row, ws.ldt_row};
+                   D + (int64_t)gs * kSlab, ws.ldd_row, Dt + (int64_t)gs * kSlab * ws.ldt_row, ws.ldt_row, ws.ldt};
     if (int rc = launch_gemm(w + v0 * H, H, hp, H / 16, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
     if (want_dh && (gs == kDhGroup - 1 || v0 + kSlab >= V)) {
       // dH[T, H] += D[T, K] . Wt[H, g0 : g0 + K]^T over the group's columns (only the last slab can be partial)

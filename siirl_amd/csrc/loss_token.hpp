@@ -67,7 +67,15 @@ __device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t id
   if (vec && dt == SIIRL_I64) {
     const longlong2 a = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[0];
     const longlong2 b = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[1];
-    q.v[0] = (float)a.x; q.v[1] = (float)a.y; q.v[2] = (float)b.x; q.v[3] = (float)b.y;
+    // masks hold small integers: when every value in the wave fits 32 bits, one v_cvt_f32_i32 each replaces the
+    // 64-bit conversion sequence (the wave-uniform test keeps the general path out of the way, not out of the code)
+    const int32_t l0 = (int32_t)a.x, l1 = (int32_t)a.y, l2 = (int32_t)b.x, l3 = (int32_t)b.y;
+    const bool wide = ((int64_t)l0 != a.x) | ((int64_t)l1 != a.y) | ((int64_t)l2 != b.x) | ((int64_t)l3 != b.y);
+    if (__builtin_amdgcn_ballot_w64(wide) == 0) {
+      q.v[0] = (float)l0; q.v[1] = (float)l1; q.v[2] = (float)l2; q.v[3] = (float)l3;
+    } else {
+      q.v[0] = (float)a.x; q.v[1] = (float)a.y; q.v[2] = (float)b.x; q.v[3] = (float)b.y;
+    }
   } else if (vec && dt == SIIRL_U8) {
     const uint32_t u = *reinterpret_cast<const uint32_t*>((const uint8_t*)p + idx);
     q.v[0] = (float)(u & 0xffu); q.v[1] = (float)((u >> 8) & 0xffu); q.v[2] = (float)((u >> 16) & 0xffu);

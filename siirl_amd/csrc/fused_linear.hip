@@ -28,11 +28,18 @@ namespace {
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BM = 256, BN = 256, BK = 64;
+// Rows of the workgroup tile: 256 (8 waves, one workgroup per CU) or 128 (4 waves, 64 KB ring, two independent
+// workgroups per CU whose prologues and epilogues overlap each other's main loop).  Measured at T=16384, H=3584,
+// V=152064: 128 is 1.5 % slower forward and 4 % slower backward, so the overlap is not what the core lacks.
+#ifndef SIIRL_GEMM_BM
+#define SIIRL_GEMM_BM 256
+#endif
+static_assert(SIIRL_GEMM_BM == 256 || SIIRL_GEMM_BM == 128, "the workgroup tile has 256 or 128 rows");
+constexpr int BM = SIIRL_GEMM_BM, BN = 256, BK = 64;
 #ifndef SIIRL_GEMM_WAVES_N
 #define SIIRL_GEMM_WAVES_N 4
 #endif
-constexpr int WM = 2, WN = SIIRL_GEMM_WAVES_N;  // wave grid over the workgroup tile
+constexpr int WM = BM / 128, WN = SIIRL_GEMM_WAVES_N;  // wave grid over the workgroup tile
 constexpr int kThreads = WM * WN * 64;
 constexpr int MI = BM / (WM * 32), NJ = BN / (WN * 32);  // 32x32 MFMA tiles per wave
 constexpr int kLoadsPerThread = (BM * BK / 8) / kThreads;  // 16-byte chunks per operand tile per thread
@@ -76,7 +83,7 @@ struct TileCoord {
 // consecutive workgroups of that XCD, so the workgroups sharing an L2 at any time share 8 A-tiles and 4
 // B-tiles instead of streaming 32 different A-tiles.  Blocks sweep M fastest inside a strip of kBlkN N-tiles,
 // which keeps a strip's B-tiles hot across the 8 XCDs.
-constexpr int kXcd = 8, kBlkM = 8, kBlkN = 4;
+constexpr int kXcd = 8, kBlkM = 8 * 256 / BM, kBlkN = 4;
 __host__ __device__ inline int64_t raster_grid(int tiles_m, int tiles_n) {
   const int64_t blocks = (int64_t)((tiles_m + kBlkM - 1) / kBlkM) * ((tiles_n + kBlkN - 1) / kBlkN);
   return (blocks + kXcd - 1) / kXcd * kXcd * (kBlkM * kBlkN);
@@ -101,7 +108,7 @@ __device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (N
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 template <class Epi>
-__global__ __launch_bounds__(kThreads) void gemm_nt_kernel(GemmArgs g, Epi epi) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_kernel(GemmArgs g, Epi epi) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int wm = w / WN, wn = w % WN;

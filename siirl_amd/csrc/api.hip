@@ -1,7 +1,10 @@
 // Error reporting and version query of the C ABI.
 #include "common.hpp"
 
+#include <mutex>
+#include <set>
 #include <string>
+#include <utility>
 
 namespace siirl {
 
@@ -15,6 +18,18 @@ int fail(int code, const char* fmt, ...) {
   va_end(ap);
   g_last_error = buf;
   return code;
+}
+
+int allow_dynamic_lds(const void* kernel, int bytes) {
+  static std::mutex mu;
+  static std::set<std::pair<const void*, int>> done;  // (kernel, device) pairs already raised
+  int dev = 0;
+  SIIRL_HIP_CHECK(hipGetDevice(&dev));
+  std::lock_guard<std::mutex> lock(mu);
+  if (done.count({kernel, dev})) return SIIRL_OK;
+  SIIRL_HIP_CHECK(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+  done.insert({kernel, dev});
+  return SIIRL_OK;
 }
 
 }  // namespace siirl

@@ -20,6 +20,9 @@ constexpr float kLn2 = 0.6931471805599453f;
 // Records a message for siirl_hip_last_error() on this thread and returns `code`.
 int fail(int code, const char* fmt, ...);
 
+// Raises `kernel`'s dynamic LDS limit to `bytes` on the current device, once per (kernel, device); thread-safe.
+int allow_dynamic_lds(const void* kernel, int bytes);
+
 #define SIIRL_REQUIRE(cond, ...)                                              \
   do {                                                                        \
     if (!(cond)) return ::siirl::fail(SIIRL_ERR_INVALID_ARGUMENT, __VA_ARGS__); \

@@ -582,12 +582,7 @@ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 template <class Epi>
 int launch_gemm(const uint16_t* A, int64_t lda, const u32x4* Bp, int64_t kb_total, int M, int N, int K, const Epi& epi,
                 hipStream_t st, const char* what, int splits = 1) {
-  static bool attr_set = false;  // one flag per instantiation
-  if (!attr_set) {
-    SIIRL_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes));
-    attr_set = true;
-  }
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi>), kSmemBytes)) return rc;
   GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN, splits};
   const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n * splits);
   gemm_nt_kernel<Epi><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);

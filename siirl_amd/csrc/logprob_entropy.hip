@@ -643,14 +643,8 @@ int launch_fused(const void* logits, int64_t T, int V, int64_t row_stride, const
 #define SIIRL_LPE_FUSED_LDS_BYTES 155648
 #endif
   constexpr int kLds = SIIRL_LPE_FUSED_LDS_BYTES;
-  static bool attr_set = false;
-  if (!attr_set) {
-    SIIRL_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&lpe_fused_kernel<E, true, Coef>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-    SIIRL_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(&lpe_fused_kernel<E, false, Coef>),
-                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLds));
-    attr_set = true;
-  }
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&lpe_fused_kernel<E, true, Coef>), kLds)) return rc;
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&lpe_fused_kernel<E, false, Coef>), kLds)) return rc;
   if (with_entropy)
     lpe_fused_kernel<E, true, Coef><<<grid, block, kLds, st>>>((const elem_t*)logits, row_stride, V, labels, inv_T, coef,
                                                             logprob, entropy, (elem_t*)dlogits, d_stride, kLds / 16);

@@ -48,9 +48,10 @@ def _mask(B, L, g, kind, dtype):
 # ------------------------------------------------------------------------------------------------ GAE
 
 
-@pytest.mark.parametrize("B,L", [(1, 2), (3, 1), (8, 256), (70, 130), (2, 5000), (129, 64)])
+@pytest.mark.parametrize("B,L", [(1, 2), (3, 1), (8, 256), (70, 130), (2, 5000), (129, 64), (40, 1024), (17, 260),
+                                 (16, 4)])
 @pytest.mark.parametrize("kind,mdt", [("full", torch.int64), ("tail", torch.int64), ("holes", torch.bool),
-                                      ("holes", torch.float32)])
+                                      ("holes", torch.float32), ("tail", torch.int32)])
 @pytest.mark.parametrize("gamma,lam", [(1.0, 1.0), (0.99, 0.95)])
 def test_gae(dev, B, L, kind, mdt, gamma, lam):
     import siirl_amd.core_algos as CA

@@ -266,6 +266,174 @@ def bench_config5(args, dev):
     print(json.dumps(out), flush=True)
 
 
+def bench_critic(args, dev):
+    """The critic-side operations either side of the path at PPO shape [1024, 8192] fp32: outcome reward placement
+    with the overlong penalty, GAE + whitening, the clipped value loss forward + backward, and the per-step data
+    metrics.  Not the headline; one JSON line with a per-operation breakdown."""
+    import torch
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.metric_utils as MU
+    import siirl_amd.reward as RW
+
+    B, P, L = 1024, 1024, 8192
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    lens = torch.randint(L // 16, L + 1, (B,), device=dev, generator=gen)
+    mask = (torch.arange(L, device=dev)[None] < lens[:, None]).long()
+    amask = torch.cat([torch.ones(B, P, dtype=torch.long, device=dev), mask], 1).contiguous()
+    scores = (torch.rand(B, device=dev, generator=gen) < 0.5).double()
+    values = torch.randn(B, L, device=dev, generator=gen)
+    vpreds = (values + 0.05 * torch.randn(B, L, device=dev, generator=gen)).requires_grad_(True)
+    overlong = SimpleNamespace(enable=True, len=1024, penalty_factor=1.0, log=False)
+    ops = ("reward placement", "GAE + whitening", "value loss fwd+bwd", "data metrics")
+
+    def step(ev=None):
+        rec = (lambda i: ev[i].record()) if ev else (lambda i: None)
+        rec(0)
+        rewards = RW.place_outcome_reward(scores, amask, L, overlong, max_resp_len=L)
+        rec(1)
+        adv, ret = CA.compute_gae_advantage_return(rewards, values, mask, 1.0, 0.95)
+        rec(2)
+        loss, _ = CA.compute_value_loss(vpreds, ret, values, mask, 0.5, "token-mean")
+        loss.backward()
+        vpreds.grad = None
+        rec(3)
+        MU.compute_data_metric({"token_level_scores": rewards, "token_level_rewards": rewards, "advantages": adv,
+                                "returns": ret, "values": values, "responses": mask, "response_mask": mask,
+                                "attention_mask": amask})
+        rec(4)
+        return rewards, adv, ret
+
+    steps, warm = args.steps, args.warmup
+    for _ in range(warm):
+        step()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(5)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for k in range(steps):
+        step(evs[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / steps for i in range(4)]
+    tokens = B * L
+    # GAE + whitening: the scan reads rewards, values, mask and writes advantages, returns (24 B + 8 B mask), the
+    # whitening apply reads and writes the advantages once more
+    gae_bytes = tokens * (4 + 4 + 8 + 4 + 4 + 4 + 4)
+    out = {
+        "metric": "PPO critic-side step (reward placement + GAE/whitening + value loss fwd+bwd + data metrics) tokens/sec @[B,L] fp32",
+        "value": tokens * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": wall * 1e3 / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"critic: {B} trajectories, prompt {P} + response {L}, gamma 1.0, lam 0.95, "
+                               f"cliprange_value 0.5, overlong buffer 1024", "seed": SEED},
+        "kernels": {name: {"ms": t} for name, t in zip(ops, ms)},
+        "roofline": {"bound": "hbm", "kernel": "gae_scan_vec_kernel + whiten_apply_kernel", "achieved": gae_bytes / ms[1] / 1e6,
+                     "peak": 8000.0, "unit": "GB/s", "frac": gae_bytes / ms[1] / 1e6 / 8000.0, "traffic": None,
+                     "note": "the scan is a sequential recurrence per row: its duration is the latency of 8192 dependent "
+                             "steps, not a bandwidth figure"},
+        "cpu_baseline": None,
+    }
+    if not args.no_cpu_baseline:  # the oracle's eager ops on the host cores, first 64 trajectories
+        from oracle import core_algos as OC
+        from oracle import dapo_filter as OD
+        from oracle import metric_utils as OM
+
+        n_s = 64
+        sc_c, am_c, m_c = scores[:n_s].cpu(), amask[:n_s].cpu(), mask[:n_s].cpu()
+        v_c, vp_c = values[:n_s].cpu(), vpreds.detach()[:n_s].cpu()
+        times = []
+        for it in range(3):
+            t1 = time.perf_counter()
+            rw_c = OD.place_outcome_reward(sc_c.tolist(), am_c, L, True, L, 1024, 1.0)
+            rw_c = torch.as_tensor(rw_c[0] if isinstance(rw_c, tuple) else rw_c, dtype=torch.float32)
+            adv_c, ret_c = OC.compute_gae_advantage_return(rw_c, v_c, m_c, 1.0, 0.95)
+            x = vp_c.clone().requires_grad_(True)
+            l_c, _ = OC.compute_value_loss(x, ret_c, v_c, m_c, 0.5, "token-mean")
+            l_c.backward()
+            OM.compute_data_metric({"token_level_scores": rw_c, "token_level_rewards": rw_c, "advantages": adv_c,
+                                    "returns": ret_c, "values": v_c, "responses": m_c, "response_mask": m_c,
+                                    "attention_mask": am_c})
+            if it:
+                times.append(time.perf_counter() - t1)
+        med = sorted(times)[len(times) // 2]
+        out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"first {n_s} of {B} trajectories x {L} tokens; median of 2 "
+                                                         f"passes ({med:.2f} s each)"}
+    print(json.dumps(out), flush=True)
+
+
+def bench_glue(args, dev):
+    """Remove-padding bookkeeping around the path at 64 sequences x 9216 tokens (prompt 1024 + response 8192):
+    packed ids + rolled labels + indices + cu_seqlens from the attention mask, and the scatter of per-token values
+    back into the [B, response_length] window, forward and backward.  Not the headline."""
+    import torch
+
+    import siirl_amd.padding as PD
+
+    B, S, L = 64, 9216, 8192
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    lens = torch.randint(S // 8, S + 1, (B,), device=dev, generator=gen)
+    am = (torch.arange(S, device=dev)[None] >= (S - lens)[:, None]).long()  # left padding
+    ids = torch.randint(0, 150000, (B, S), device=dev, generator=gen)
+    nnz = int(am.sum())
+    vals = torch.randn(nnz, device=dev, generator=gen).requires_grad_(True)
+    g = torch.randn(B, L, device=dev, generator=gen)
+
+    def step(ev=None):
+        rec = (lambda i: ev[i].record()) if ev else (lambda i: None)
+        rec(0)
+        _, _, indices, _, _ = PD.unpad_ids_and_labels(ids, am)
+        rec(1)
+        out = PD.pad_and_slice_response(vals, indices, B, S, L)
+        out.backward(g)
+        vals.grad = None
+        rec(2)
+
+    steps, warm = args.steps, args.warmup
+    for _ in range(warm):
+        step()
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    t0 = time.perf_counter()
+    for k in range(steps):
+        step(evs[k])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / steps for i in range(2)]
+    out = {
+        "metric": "remove-padding bookkeeping (unpad ids/labels/indices + response-window scatter fwd+bwd) tokens/sec",
+        "value": nnz * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": wall * 1e3 / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int64", "data": "synthetic",
+        "config": {"workload": f"glue: {B} sequences x {S} (prompt {S - L} + response {L}), left padded, {nnz} tokens",
+                   "seed": SEED},
+        "kernels": {"unpad_ids_and_labels (one host sync)": {"ms": ms[0]},
+                    "pad_and_slice_response forward + backward": {"ms": ms[1]}},
+        "roofline": {"bound": "hbm", "kernel": "unpad kernels", "achieved": B * S * 16 / ms[0] / 1e6, "peak": 8000.0,
+                     "unit": "GB/s", "frac": B * S * 16 / ms[0] / 1e6 / 8000.0, "traffic": None,
+                     "note": "index work at a size where launches and the host sync dominate; no roofline claim"},
+        "cpu_baseline": None,
+    }
+    if not args.no_cpu_baseline:
+        import numpy as np
+        from oracle import padding as OP
+
+        am_c, ids_c, v_c = am.cpu().numpy(), ids.cpu().numpy(), vals.detach().cpu().numpy()
+        times = []
+        for it in range(4):
+            t1 = time.perf_counter()
+            rm, idx, cu, mx = OP.unpad_input(ids_c.reshape(B, S, 1), am_c)[:4]
+            OP.rolled_labels(rm.reshape(-1))
+            OP.pad_and_slice_response(v_c, idx, B, S, L)
+            if it:
+                times.append(time.perf_counter() - t1)
+        med = sorted(times)[len(times) // 2]
+        out["cpu_baseline"] = {"value": nnz / med, "unit": "tokens/s", "cores": 1, "kind": "port",
+                               "sample": f"the whole batch, forward only, numpy; median of 3 passes ({med * 1e3:.1f} ms each)"}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -276,9 +444,10 @@ def main():
                     help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 2 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config5"],
+    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config5", "critic", "glue"],
                     help="config2 (default): the headline logprob+entropy fwd+bwd; config3: DAPO [B, L] loss path; "
-                         "config5: fused lm_head variant")
+                         "config5: fused lm_head variant; critic: reward placement + GAE + value loss + metrics; "
+                         "glue: remove-padding bookkeeping")
     ap.add_argument("--seqs", type=int, default=SEQS, help="sequences of 4096 tokens (8 = the baseline's config)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -299,6 +468,10 @@ def main():
         return bench_config5(args, dev)
     if args.workload == "config3":
         return bench_config3(args, dev)
+    if args.workload == "critic":
+        return bench_critic(args, dev)
+    if args.workload == "glue":
+        return bench_glue(args, dev)
     SF.set_skip_zero_rows(False)  # dense: every row is read and written, as the algorithmic byte count assumes
 
     logits, labels, g_lp, g_ent, mask = make_workload(dev, seqs=args.seqs)

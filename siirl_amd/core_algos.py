@@ -26,6 +26,9 @@ import numpy as np
 import torch
 
 from . import _lib
+from . import ops as _ops_module  # noqa: F401  (registers torch.ops.siirl_hip.*)
+
+_OPS = torch.ops.siirl_hip
 from . import torch_functional as siirl_F
 
 __all__ = [
@@ -258,13 +261,7 @@ def compute_grpo_outcome_advantage(token_level_rewards: torch.Tensor, response_m
     r = _f32(token_level_rewards, dev)
     m, mcode = _mask_arg(response_mask, dev)
     uid = _uid_tensor(index, B, dev)
-    adv = torch.empty(B, L, dtype=torch.float32, device=dev)
-    scratch = torch.empty(2 * max(B, 1), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.lib().siirl_grpo_outcome_advantage(_lib.ptr(r), _lib.ptr(m), mcode, _lib.ptr(uid), B, L,
-                                                     float(epsilon), int(bool(norm_adv_by_std_in_grpo)),
-                                                     _lib.ptr(adv), _lib.ptr(scratch), _lib.current_stream(dev))
-    _lib.check(rc, "siirl_grpo_outcome_advantage")
+    adv = _OPS.grpo_advantage(r, m, uid, float(epsilon), bool(norm_adv_by_std_in_grpo))
     if back:
         adv = adv.to(token_level_rewards.device)
     return adv, adv
@@ -368,13 +365,7 @@ class _AggLoss(torch.autograd.Function):
         v = _as_2d(_f32(loss_mat, dev))
         B, L = v.shape
         m, mcode = _mask_arg(_as_2d(loss_mask), dev)
-        out16 = torch.empty(16, dtype=torch.float32, device=dev)
-        row_msum = torch.empty(B, dtype=torch.float32, device=dev)
-        ws, nws = _workspace(B, L, dev)
-        with torch.cuda.device(dev):
-            rc = _lib.lib().siirl_agg_loss_fwd(_lib.ptr(v), _lib.ptr(m), mcode, B, L, agg_code, _lib.ptr(out16),
-                                               _lib.ptr(row_msum), _lib.ptr(ws), nws, _lib.current_stream(dev))
-        _lib.check(rc, "siirl_agg_loss_fwd")
+        out16, row_msum = _OPS.agg_loss_fwd(v, m, agg_code)
         ctx.save_for_backward(m, out16, row_msum)
         ctx.meta = (mcode, B, L, agg_code, loss_mat.shape, loss_mat.dtype)
         return out16[O_PG]
@@ -385,11 +376,7 @@ class _AggLoss(torch.autograd.Function):
         mcode, B, L, agg_code, shape, dtype = ctx.meta
         dev = out16.device
         g = g.detach().to(torch.float32).reshape(1).contiguous()
-        d = torch.empty(B, L, dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.lib().siirl_agg_loss_bwd(_lib.ptr(g), _lib.ptr(m), mcode, _lib.ptr(out16), _lib.ptr(row_msum),
-                                               B, L, agg_code, _lib.ptr(d), _lib.current_stream(dev))
-        _lib.check(rc, "siirl_agg_loss_bwd")
+        d = _OPS.agg_loss_bwd(g, m, out16, row_msum, agg_code)
         return d.reshape(shape).to(dtype), None, None
 
 
@@ -426,17 +413,9 @@ class _ActorLoss(torch.autograd.Function):
                         ("entropy", ent), ("ref_log_prob", ref)):
             if t is not None and tuple(t.shape) != (B, L):
                 raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {(B, L)}")
-        out16 = torch.empty(16, dtype=torch.float32, device=dev)
-        row_msum = torch.empty(B, dtype=torch.float32, device=dev)
-        row_s = torch.empty(B, dtype=torch.float32, device=dev)
-        ws, nws = _workspace(B, L, dev)
-        with torch.cuda.device(dev):
-            rc = _lib.lib().siirl_actor_loss_fwd(
-                _lib.ptr(old), _lib.ptr(lp), _lib.ptr(adv), _lib.ptr(m), mcode, _lib.ptr(isw), _lib.ptr(ent),
-                _lib.ptr(ref), B, L, loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st,
-                kl_coef, drift_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s), _lib.ptr(ws), nws,
-                _lib.current_stream(dev))
-        _lib.check(rc, "siirl_actor_loss_fwd")
+        out16, row_msum, row_s = _OPS.policy_loss_fwd(old, lp, adv, m, isw, ent, ref, loss_mode, eps_lo, eps_hi, clip_c,
+                                                      dclamp, agg_code, ent_coef, kl_code, bool(kl_st), kl_coef,
+                                                      drift_coef, scale)
         ctx.save_for_backward(lp, old, adv, m, out16, row_msum, row_s,
                               *(t for t in (isw, ent, ref) if t is not None))
         ctx.flags = (isw is not None, ent is not None, ref is not None)
@@ -465,16 +444,11 @@ class _ActorLoss(torch.autograd.Function):
          _) = cfg
         dev = lp.device
         g = g.detach().to(torch.float32).reshape(1).contiguous()
-        d_lp = torch.empty(B, L, dtype=torch.float32, device=dev)
-        d_ent = torch.empty(B, L, dtype=torch.float32, device=dev) if has_ent else None
-        with torch.cuda.device(dev):
-            rc = _lib.lib().siirl_actor_loss_bwd(
-                _lib.ptr(g), _lib.ptr(old), _lib.ptr(lp), _lib.ptr(adv), _lib.ptr(m), mcode, _lib.ptr(isw),
-                _lib.ptr(ent), _lib.ptr(ref), B, L, loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef,
-                kl_code, kl_st, kl_coef, drift_coef, scale, _lib.ptr(out16), _lib.ptr(row_msum), _lib.ptr(row_s),
-                _lib.ptr(d_lp),
-                _lib.ptr(d_ent), _lib.current_stream(dev))
-        _lib.check(rc, "siirl_actor_loss_bwd")
+        d_lp, d_ent = _OPS.policy_loss_bwd(g, old, lp, adv, m, isw, ent, ref, loss_mode, eps_lo, eps_hi, clip_c, dclamp,
+                                           agg_code, ent_coef, kl_code, bool(kl_st), kl_coef, drift_coef, scale, out16,
+                                           row_msum, row_s)
+        if not has_ent:
+            d_ent = None
         g_lp = d_lp.reshape(lp_shape).to(lp_dtype)
         g_ent = None if d_ent is None else d_ent.reshape(ent_meta[0]).to(ent_meta[1])
         return g_lp, g_ent, None, None, None, None, None, None
@@ -655,11 +629,7 @@ class _KlPenalty(torch.autograd.Function):
         lp, ref = _f32(logprob, dev), _f32(ref_logprob, dev)
         if ref.shape != lp.shape:
             ref = ref.expand(lp.shape).contiguous()
-        out = torch.empty_like(lp)
-        with torch.cuda.device(dev):
-            rc = _lib.lib().siirl_kl_penalty_fwd(_lib.ptr(lp), _lib.ptr(ref), lp.numel(), code, _lib.ptr(out),
-                                                 _lib.current_stream(dev))
-        _lib.check(rc, "siirl_kl_penalty_fwd")
+        out = _OPS.kl_penalty_fwd(lp, ref, code)
         ctx.save_for_backward(lp, ref)
         ctx.meta = (code, straight_through, logprob.dtype, ref_logprob.dtype, ref_logprob.shape)
         return out.to(logprob.dtype) if logprob.dtype != torch.float32 else out
@@ -671,14 +641,9 @@ class _KlPenalty(torch.autograd.Function):
         dev = lp.device
         g = _f32(g, dev)
         need_lp, need_ref = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        d_lp = torch.empty_like(lp) if need_lp else None
-        d_ref = torch.empty_like(lp) if need_ref else None
-        if need_lp or need_ref:
-            with torch.cuda.device(dev):
-                rc = _lib.lib().siirl_kl_penalty_bwd(_lib.ptr(g), _lib.ptr(lp), _lib.ptr(ref), lp.numel(), code,
-                                                     int(st), _lib.ptr(d_lp), _lib.ptr(d_ref),
-                                                     _lib.current_stream(dev))
-            _lib.check(rc, "siirl_kl_penalty_bwd")
+        d_lp, d_ref = _OPS.kl_penalty_bwd(g, lp, ref, code, bool(st), bool(need_lp), bool(need_ref))
+        d_lp = d_lp if need_lp else None
+        d_ref = d_ref if need_ref else None
         if d_ref is not None and tuple(ref_shape) != tuple(lp.shape):
             d_ref = d_ref.sum_to_size(ref_shape)
         return (None if d_lp is None else d_lp.to(lp_dtype), None if d_ref is None else d_ref.to(ref_dtype),

@@ -15,7 +15,8 @@ from typing import Any, Dict, List, Optional
 import numpy as np
 import torch
 
-from . import _lib
+from . import _lib  # noqa: F401
+from . import ops as _ops_module  # noqa: F401  (registers torch.ops.siirl_hip.*)
 
 __all__ = ["NodeOutput", "make_uid", "group_keep_mask", "filter_tensordict", "dynamic_sampling",
            "SamplingLeftoverCache"]
@@ -82,12 +83,7 @@ def group_keep_mask(metric_values, uids, device=None, return_group_size: bool = 
     B = uid.numel()
     if met.numel() != B:
         raise ValueError(f"{met.numel()} metric values for {B} uids")
-    keep = torch.empty(B, dtype=torch.uint8, device=device)
-    gsz = torch.empty(B, dtype=torch.int32, device=device) if return_group_size else None
-    with torch.cuda.device(device):
-        rc = _lib.lib().siirl_group_keep_mask(_lib.ptr(met), _lib.dtype_code(met.dtype), _lib.ptr(uid), B,
-                                              _lib.ptr(keep), _lib.ptr(gsz), _lib.current_stream(device))
-    _lib.check(rc, "siirl_group_keep_mask")
+    keep, gsz = torch.ops.siirl_hip.group_keep_mask(met, uid)
     keep = keep.bool()
     return (keep, gsz) if return_group_size else keep
 

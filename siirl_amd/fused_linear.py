@@ -19,11 +19,7 @@ import typing
 
 import torch
 
-from . import _lib
-
-
-def _workspace(nbytes: int, dev) -> torch.Tensor:
-    return torch.empty(max(nbytes, 256), dtype=torch.uint8, device=dev)
+from . import ops as _ops_module  # noqa: F401  (registers torch.ops.siirl_hip.*)
 
 
 class _FusedLinearLogprobEntropy(torch.autograd.Function):
@@ -42,16 +38,7 @@ class _FusedLinearLogprobEntropy(torch.autograd.Function):
         if w.shape[1] != H or y.shape != (T,):
             raise ValueError(f"shape mismatch: hidden {tuple(h.shape)}, weight {tuple(w.shape)}, labels {tuple(y.shape)}")
         inv_t = 1.0 / float(temperature)
-        L = _lib.lib()
-        f32 = dict(dtype=torch.float32, device=dev)
-        lp, ent, lse, ex = (torch.empty(T, **f32) for _ in range(4))
-        nws = L.siirl_fused_linear_fwd_workspace_bytes(T, H, V)
-        ws = _workspace(nws, dev)
-        with torch.cuda.device(dev):
-            rc = L.siirl_fused_linear_logprob_entropy_fwd(_lib.ptr(h), _lib.ptr(w), _lib.BF16, _lib.ptr(y), T, H, V,
-                                                          inv_t, _lib.ptr(lp), _lib.ptr(ent), _lib.ptr(lse),
-                                                          _lib.ptr(ex), _lib.ptr(ws), nws, _lib.current_stream(dev))
-        _lib.check(rc, "siirl_fused_linear_logprob_entropy_fwd")
+        lp, ent, lse, ex = torch.ops.siirl_hip.fused_linear_logprob_entropy_fwd(h, w, y, inv_t)
         ctx.save_for_backward(h, w, y, lse, ex)
         ctx.inv_t = inv_t
         ctx.set_materialize_grads(False)
@@ -64,22 +51,11 @@ class _FusedLinearLogprobEntropy(torch.autograd.Function):
         if (g_lp is None and g_ent is None) or not (need_h or need_w):
             return None, None, None, None
         dev = h.device
-        T, H = h.shape
-        V = w.shape[0]
         f = lambda t: None if t is None else t.detach().to(device=dev, dtype=torch.float32).contiguous()  # noqa: E731
         g_lp, g_ent = f(g_lp), f(g_ent)
-        d_h = torch.empty_like(h) if need_h else None
-        d_w = torch.empty_like(w) if need_w else None
-        L = _lib.lib()
-        nws = L.siirl_fused_linear_bwd_workspace_bytes(T, H, V, int(need_h), int(need_w))
-        ws = _workspace(nws, dev)
-        with torch.cuda.device(dev):
-            rc = L.siirl_fused_linear_logprob_entropy_bwd(_lib.ptr(h), _lib.ptr(w), _lib.BF16, _lib.ptr(y), T, H, V,
-                                                          ctx.inv_t, _lib.ptr(lse), _lib.ptr(ex), _lib.ptr(g_lp),
-                                                          _lib.ptr(g_ent), _lib.ptr(d_h), _lib.ptr(d_w), _lib.ptr(ws),
-                                                          nws, _lib.current_stream(dev))
-        _lib.check(rc, "siirl_fused_linear_logprob_entropy_bwd")
-        return d_h, d_w, None, None
+        d_h, d_w = torch.ops.siirl_hip.fused_linear_logprob_entropy_bwd(h, w, y, ctx.inv_t, lse, ex, g_lp, g_ent,
+                                                                        bool(need_h), bool(need_w))
+        return (d_h if need_h else None), (d_w if need_w else None), None, None
 
 
 def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,

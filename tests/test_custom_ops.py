@@ -1,0 +1,87 @@
+"""The torch.library layer: every entry point of the path is a ``torch.ops.siirl_hip.*`` custom op with a fake
+kernel (shape inference without a GPU), and on the GPU the ops pass ``torch.library.opcheck``."""
+import pytest
+import torch
+
+import siirl_amd.ops  # noqa: F401  (registers the ops)
+
+OPS = ("logprob_entropy_fwd", "logprob_entropy_bwd", "logprob_entropy_bwd_", "grpo_advantage", "group_keep_mask",
+       "agg_loss_fwd", "agg_loss_bwd", "policy_loss_fwd", "policy_loss_bwd", "kl_penalty_fwd", "kl_penalty_bwd",
+       "fused_linear_logprob_entropy_fwd", "fused_linear_logprob_entropy_bwd")
+
+
+def test_ops_are_registered():
+    for name in OPS:
+        op = getattr(torch.ops.siirl_hip, name)
+        assert op.default._schema.name == f"siirl_hip::{name}"
+
+
+def _loss_args(mk, B, L, with_optional):
+    f = lambda: mk((B, L), torch.float32)  # noqa: E731
+    opt = (f(), f(), f()) if with_optional else (None, None, None)
+    return (f(), f(), f(), mk((B, L), torch.int64), *opt, 0, 0.2, 0.28, 3.0, 20.0, 0, 0.001, 3, False, 0.001, 0.0, 1.0)
+
+
+@pytest.mark.parametrize("with_optional", [False, True])
+def test_fake_kernels_give_shapes_without_a_gpu(with_optional):
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    ns = torch.ops.siirl_hip
+    with FakeTensorMode():
+        mk = lambda shape, dtype: torch.empty(shape, dtype=dtype, device="meta")  # noqa: E731
+        B, L, T, V, H = 6, 40, 24, 1000, 64
+        out16, row_msum, row_s = ns.policy_loss_fwd(*_loss_args(mk, B, L, with_optional))
+        assert out16.shape == (16,) and row_msum.shape == (B,) and row_s.shape == (B,)
+        a = _loss_args(mk, B, L, with_optional)
+        d_lp, d_ent = ns.policy_loss_bwd(mk((1,), torch.float32), *a, out16, row_msum, row_s)
+        assert d_lp.shape == (B, L) and d_ent.shape == ((B, L) if with_optional else (0,))
+        o, r = ns.agg_loss_fwd(mk((B, L), torch.float32), mk((B, L), torch.bool), 0)
+        assert o.shape == (16,) and r.shape == (B,)
+        assert ns.agg_loss_bwd(mk((1,), torch.float32), mk((B, L), torch.bool), o, r, 0).shape == (B, L)
+        assert ns.kl_penalty_fwd(mk((B, L), torch.float32), mk((B, L), torch.float32), 3).shape == (B, L)
+        d1, d2 = ns.kl_penalty_bwd(mk((B, L), torch.float32), mk((B, L), torch.float32), mk((B, L), torch.float32), 3,
+                                   False, True, False)
+        assert d1.shape == (B, L) and d2.shape == (0,)
+        adv = ns.grpo_advantage(mk((B, L), torch.float32), mk((B, L), torch.int64), mk((B,), torch.int64), 1e-6, True)
+        assert adv.shape == (B, L) and adv.dtype == torch.float32
+        keep, gsz = ns.group_keep_mask(mk((B,), torch.float64), mk((B,), torch.int64))
+        assert keep.dtype == torch.uint8 and gsz.dtype == torch.int32 and keep.shape == gsz.shape == (B,)
+        lp, ent, lse, ex = ns.fused_linear_logprob_entropy_fwd(mk((T, H), torch.bfloat16), mk((V, H), torch.bfloat16),
+                                                               mk((T,), torch.int64), 1.0)
+        assert lp.shape == ent.shape == lse.shape == ex.shape == (T,) and lp.dtype == torch.float32
+        dh, dw = ns.fused_linear_logprob_entropy_bwd(mk((T, H), torch.bfloat16), mk((V, H), torch.bfloat16),
+                                                     mk((T,), torch.int64), 1.0, lse, ex, mk((T,), torch.float32), None,
+                                                     True, False)
+        assert dh.shape == (T, H) and dh.dtype == torch.bfloat16 and dw.shape == (0,)
+        lp, ent, lse, ex = ns.logprob_entropy_fwd(mk((3, 5, V), torch.bfloat16), mk((3, 5), torch.int64), 1.0, True)
+        assert lp.shape == ent.shape == lse.shape == (3, 5)
+
+
+@pytest.mark.gpu
+def test_opcheck_on_the_gpu():
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(0)
+    ns = torch.ops.siirl_hip
+    checks = ("test_schema", "test_faketensor")
+    B, L, T, V, H = 6, 40, 24, 1000, 64
+    mk = lambda shape, dtype: (torch.randn(shape, device=dev, generator=g) * 0.1).to(dtype) if dtype.is_floating_point \
+        else torch.ones(shape, dtype=dtype, device=dev)  # noqa: E731
+    args = _loss_args(mk, B, L, True)
+    torch.library.opcheck(ns.policy_loss_fwd, args, test_utils=checks)
+    out16, row_msum, row_s = ns.policy_loss_fwd(*args)
+    torch.library.opcheck(ns.policy_loss_bwd, (torch.ones(1, device=dev), *args, out16, row_msum, row_s), test_utils=checks)
+    lm, m = mk((B, L), torch.float32), torch.ones(B, L, dtype=torch.bool, device=dev)
+    torch.library.opcheck(ns.agg_loss_fwd, (lm, m, 2), test_utils=checks)
+    torch.library.opcheck(ns.kl_penalty_fwd, (lm, mk((B, L), torch.float32), 3), test_utils=checks)
+    uid = torch.arange(B, device=dev) // 2
+    torch.library.opcheck(ns.grpo_advantage, (lm, torch.ones(B, L, dtype=torch.int64, device=dev), uid, 1e-6, True),
+                          test_utils=checks)
+    torch.library.opcheck(ns.group_keep_mask, (torch.rand(B, device=dev, dtype=torch.float64), uid), test_utils=checks)
+    h, w = mk((T, H), torch.bfloat16), mk((V, H), torch.bfloat16)
+    y = torch.randint(0, V, (T,), device=dev)
+    torch.library.opcheck(ns.fused_linear_logprob_entropy_fwd, (h, w, y, 1.0), test_utils=checks)
+    lp, ent, lse, ex = ns.fused_linear_logprob_entropy_fwd(h, w, y, 1.0)
+    torch.library.opcheck(ns.fused_linear_logprob_entropy_bwd, (h, w, y, 1.0, lse, ex, torch.ones(T, device=dev), None,
+                                                                True, True), test_utils=checks)
+    x = mk((T, V), torch.bfloat16)
+    torch.library.opcheck(ns.logprob_entropy_fwd, (x, y, 1.0, True), test_utils=checks)

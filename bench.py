@@ -266,6 +266,171 @@ def bench_config5(args, dev):
     print(json.dumps(out), flush=True)
 
 
+def bench_config1(args, dev):
+    """Config 1, the CPU-runnable GRPO step in fp32: 64 prompts x 8 responses, L = 256, V = 32000.  One step =
+    group-normalised advantages over the 512 trajectories, then 64 micro-batches of 8 sequences, each
+    logits [2048, 32000] fp32 -> log-prob -> clipped loss (eps 0.2, token-mean) + 0.001 * low_var_kl -> backward to
+    the logits.  One logits buffer is reused by every micro-batch (the full tensor would be 16.8 GB); the labels,
+    old / reference log-probs, advantages and masks are the micro-batch's own.  Not the headline."""
+    import torch
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.dapo_filter as DF
+    import siirl_amd.torch_functional as SF
+
+    SF.set_skip_zero_rows(False)  # dense rows, as the byte count assumes
+    P, n, L, V, MB = 64, 8, 256, 32000, 8
+    B = P * n
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    lens = torch.randint(16, L + 1, (B,), device=dev, generator=gen)
+    mask = (torch.arange(L, device=dev)[None] < lens[:, None]).long()
+    rewards = torch.zeros(B, L, device=dev)
+    rewards[torch.arange(B, device=dev), lens - 1] = (torch.rand(B, device=dev, generator=gen) < 0.5).float()
+    uid = torch.from_numpy(DF.make_uid(P, n)).to(dev)
+    logits = (torch.randn(MB, L, V, device=dev, generator=gen) * 2.0).requires_grad_(True)
+    labels = torch.randint(0, V, (B, L), device=dev, generator=gen)
+    with torch.no_grad():
+        lp0 = SF.logprobs_from_logits(logits, labels[:MB], inplace_backward=False)
+    old = lp0.repeat(B // MB, 1) + 0.05 * torch.randn(B, L, device=dev, generator=gen)
+    ref = lp0.repeat(B // MB, 1) + 0.1 * torch.randn(B, L, device=dev, generator=gen)
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.2, clip_ratio_c=3.0, entropy_coeff=0.0,
+                          use_kl_loss=True, kl_loss_coef=0.001, kl_loss_type="low_var_kl", loss_agg_mode="token-mean",
+                          loss_mode="vanilla")
+    scale = 1.0 / (B // MB)
+
+    def step():
+        adv, _ = CA.compute_grpo_outcome_advantage(rewards, mask, uid)
+        for mb in range(B // MB):
+            rows = slice(mb * MB, mb * MB + MB)
+            lp = SF.logprobs_from_logits(logits, labels[rows], inplace_backward=False)
+            out = CA.actor_loss(old[rows], lp, adv[rows], mask[rows], cfg, ref_log_prob=ref[rows], loss_scale_factor=scale)
+            out.loss.backward()
+            logits.grad = None
+
+    steps, warm = args.steps, args.warmup
+    for _ in range(warm):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    tokens = B * L
+    step_bytes = tokens * V * 4 * 3  # fp32 logits: forward reads the row, backward reads it and writes the gradient
+    gbs = step_bytes * steps / wall / 1e9
+    out = {
+        "metric": "GRPO loss step (advantages + 64 micro-batches of logprob fwd, clipped loss + KL, bwd) tokens/sec @vocab32k fp32",
+        "value": tokens * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": wall * 1e3 / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"config1: {P} prompts x {n} responses, L = {L}, V = {V}, fp32, micro-batches of {MB} "
+                               f"sequences, eps 0.2, token-mean, low_var_kl x 0.001", "tokens": tokens, "seed": SEED},
+        "roofline": {"bound": "hbm", "kernel": "lpe_fwd_kernel + lpe_bwd_flat_kernel (whole step, wall clock)",
+                     "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None,
+                     "note": "64 micro-batches of 262 MB each, about ten launches per micro-batch issued from Python: "
+                             "launch-bound as much as bandwidth-bound"},
+        "cpu_baseline": None,
+    }
+    if not args.no_cpu_baseline:  # the CPU-runnable case: the oracle on a sample of 8 of the 64 micro-batches
+        from oracle import actor_step as OA
+        from oracle import core_algos as OC
+
+        n_mb = 8
+        rw_c, m_c, uid_c = rewards.cpu(), mask.cpu(), uid.cpu().numpy()
+        x_c, y_c, old_c, ref_c = logits.detach().cpu(), labels.cpu(), old.cpu(), ref.cpu()
+        ocfg = OA.ActorConfig(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.2, clip_ratio_c=3.0, entropy_coeff=0.0,
+                              use_kl_loss=True, kl_loss_coef=0.001, kl_loss_type="low_var_kl", loss_agg_mode="token-mean")
+        t1 = time.perf_counter()
+        adv_c, _ = OC.compute_grpo_outcome_advantage(rw_c, m_c, uid_c)
+        for mb in range(n_mb):
+            rows = slice(mb * MB, mb * MB + MB)
+            OA.micro_batch_step(x_c, y_c[rows], old_c[rows], adv_c[rows], m_c[rows], ocfg, ref_log_prob=ref_c[rows],
+                                loss_scale_factor=scale)
+        el = time.perf_counter() - t1
+        out["cpu_baseline"] = {"value": n_mb * MB * L / el, "unit": "tokens/s", "cores": torch.get_num_threads(),
+                               "kind": "port", "sample": f"advantages over all {B} trajectories + the first {n_mb} of "
+                                                         f"{B // MB} micro-batches, one pass ({el:.1f} s)"}
+    print(json.dumps(out), flush=True)
+
+
+def bench_config4(args, dev):
+    """Config 4, GSPO long context: sequences of 32768 response tokens, bf16 logits at V = 151936 (Qwen3), one
+    sequence per micro-batch.  One step = one sequence: log-prob forward, GSPO loss (sequence-level ratio, clip
+    3e-4 / 4e-4, seq-mean-token-mean, scaled by 1/32) forward + backward, log-prob backward to the logits.  The
+    32 sequences of the configuration are 32 such steps over one reused 9.96 GB logits buffer.  Not the headline."""
+    import torch
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.torch_functional as SF
+
+    SF.set_skip_zero_rows(False)  # dense rows, as the byte count assumes
+    L, V, NSEQ = 32768, 151936, 32
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    x = torch.empty(1, L, V, dtype=torch.bfloat16, device=dev)
+    for lo in range(0, L, 2048):
+        x[0, lo:lo + 2048] = (torch.randn(2048, V, device=dev, generator=gen) * 3).to(torch.bfloat16)
+    x.requires_grad_(True)
+    y = torch.randint(0, V, (1, L), device=dev, generator=gen)
+    mask = (torch.arange(L, device=dev) < 30000).long()[None]
+    adv = torch.full((1, L), 0.7, device=dev)
+    with torch.no_grad():
+        lp0 = SF.logprobs_from_logits(x, y, inplace_backward=False)
+    old = lp0 - 0.02 * torch.randn(1, L, device=dev, generator=gen)
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=3e-4, clip_ratio_high=4e-4, clip_ratio_c=3.0, entropy_coeff=0.0,
+                          use_kl_loss=False, loss_agg_mode="seq-mean-token-mean", loss_mode="gspo")
+
+    def step():
+        lp = SF.logprobs_from_logits(x, y, inplace_backward=False)
+        out = CA.actor_loss(old, lp, adv, mask, cfg, loss_scale_factor=1.0 / NSEQ)
+        out.loss.backward()
+        x.grad = None
+
+    steps, warm = args.steps, args.warmup
+    for _ in range(warm):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    step_bytes = L * V * 2 * 3
+    gbs = step_bytes * steps / wall / 1e9
+    out = {
+        "metric": "GSPO long-context step (logprob fwd + sequence-level clipped loss fwd+bwd + logprob bwd) tokens/sec @vocab151936 bf16",
+        "value": L * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": wall * 1e3 / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"config4: one of {NSEQ} sequences x {L} tokens per step, V = {V}, bf16 logits ~N(0,3), "
+                               f"log-ratios ~N(0,0.02), clip 3e-4/4e-4, seq-mean-token-mean", "tokens": L, "seed": SEED},
+        "roofline": {"bound": "hbm", "kernel": "lpe_fwd_kernel + lpe_bwd_flat_kernel (whole step, wall clock)",
+                     "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None},
+        "cpu_baseline": None,
+    }
+    if not args.no_cpu_baseline:
+        from oracle import actor_step as OA
+
+        rows = 2048
+        ocfg = OA.ActorConfig(clip_ratio=0.2, clip_ratio_low=3e-4, clip_ratio_high=4e-4, loss_agg_mode="seq-mean-token-mean",
+                              loss_mode="gspo")
+        x_c = x.detach()[:, :rows].cpu()
+        y_c, old_c, adv_c, m_c = y[:, :rows].cpu(), old[:, :rows].cpu(), adv[:, :rows].cpu(), mask[:, :rows].cpu()
+        times = []
+        for it in range(3):
+            t1 = time.perf_counter()
+            OA.micro_batch_step(x_c, y_c, old_c, adv_c, m_c, ocfg)
+            if it:
+                times.append(time.perf_counter() - t1)
+        med = sorted(times)[len(times) // 2]
+        out["cpu_baseline"] = {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"first {rows} of {L} tokens of the sequence, upcast to fp32; median of 2 "
+                                         f"passes ({med:.2f} s each)"}
+    print(json.dumps(out), flush=True)
+
+
 def bench_critic(args, dev):
     """The critic-side operations either side of the path at PPO shape [1024, 8192] fp32: outcome reward placement
     with the overlong penalty, GAE + whitening, the clipped value loss forward + backward, and the per-step data
@@ -444,8 +609,9 @@ def main():
                     help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 2 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--workload", default="config2", choices=["config2", "config3", "config5", "critic", "glue"],
-                    help="config2 (default): the headline logprob+entropy fwd+bwd; config3: DAPO [B, L] loss path; "
+    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "critic", "glue"],
+                    help="config2 (default): the headline logprob+entropy fwd+bwd; config1: fp32 GRPO step at V = 32000; "
+                         "config4: GSPO long-context sequence; config3: DAPO [B, L] loss path; "
                          "config5: fused lm_head variant; critic: reward placement + GAE + value loss + metrics; "
                          "glue: remove-padding bookkeeping")
     ap.add_argument("--seqs", type=int, default=SEQS, help="sequences of 4096 tokens (8 = the baseline's config)")
@@ -468,6 +634,10 @@ def main():
         return bench_config5(args, dev)
     if args.workload == "config3":
         return bench_config3(args, dev)
+    if args.workload == "config1":
+        return bench_config1(args, dev)
+    if args.workload == "config4":
+        return bench_config4(args, dev)
     if args.workload == "critic":
         return bench_critic(args, dev)
     if args.workload == "glue":

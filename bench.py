@@ -319,6 +319,22 @@ def bench_config1(args, dev):
     wall = time.perf_counter() - t0
     tokens = B * L
     step_bytes = tokens * V * 4 * 3  # fp32 logits: forward reads the row, backward reads it and writes the gradient
+
+    def fused_step():  # the same step with the single-pass logits -> loss -> dlogits kernel per micro-batch
+        adv, _ = CA.compute_grpo_outcome_advantage(rewards, mask, uid)
+        for mb in range(B // MB):
+            rows = slice(mb * MB, mb * MB + MB)
+            CA.fused_actor_step(logits.detach(), labels[rows], old[rows], adv[rows], mask[rows], cfg,
+                                ref_log_prob=ref[rows], loss_scale_factor=scale)
+
+    for _ in range(warm):
+        fused_step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(steps):
+        fused_step()
+    torch.cuda.synchronize()
+    fused_wall = time.perf_counter() - t1
     gbs = step_bytes * steps / wall / 1e9
     out = {
         "metric": "GRPO loss step (advantages + 64 micro-batches of logprob fwd, clipped loss + KL, bwd) tokens/sec @vocab32k fp32",
@@ -331,6 +347,8 @@ def bench_config1(args, dev):
                      "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None,
                      "note": "64 micro-batches of 262 MB each, about ten launches per micro-batch issued from Python: "
                              "launch-bound as much as bandwidth-bound"},
+        "fused_step_variant": {"what": "siirl_actor_step_fused per micro-batch (one pass over the logits)",
+                               "ms_per_step": fused_wall * 1e3 / steps, "tokens_per_s": tokens * steps / fused_wall},
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:  # the CPU-runnable case: the oracle on a sample of 8 of the 64 micro-batches

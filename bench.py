@@ -335,6 +335,43 @@ def bench_config1(args, dev):
         fused_step()
     torch.cuda.synchronize()
     fused_wall = time.perf_counter() - t1
+
+    # the same 64 single-pass micro-batch steps recorded once into a HIP graph and replayed: one submission per step
+    graph_ms = None
+    try:
+        losses = []
+
+        def graph_body():
+            adv, _ = CA.compute_grpo_outcome_advantage(rewards, mask, uid)
+            for mb in range(B // MB):
+                rows = slice(mb * MB, mb * MB + MB)
+                losses.append(CA.fused_actor_step(logits.detach(), labels[rows], old[rows], adv[rows], mask[rows], cfg,
+                                                  ref_log_prob=ref[rows], loss_scale_factor=scale).loss)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            graph_body()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        eager_total = float(torch.stack(losses).sum())
+        losses.clear()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            graph_body()
+        for _ in range(warm + 1):
+            graph.replay()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for _ in range(steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t2) * 1e3 / steps
+        replay_total = float(torch.stack(losses).sum())
+        if replay_total != eager_total:
+            raise RuntimeError(f"graph replay gives loss {replay_total}, eager {eager_total}")
+    except Exception as e:  # reported, never hidden: the eager figures above stand by themselves
+        graph_ms = f"failed: {type(e).__name__}: {e}"
     gbs = step_bytes * steps / wall / 1e9
     out = {
         "metric": "GRPO loss step (advantages + 64 micro-batches of logprob fwd, clipped loss + KL, bwd) tokens/sec @vocab32k fp32",
@@ -348,7 +385,8 @@ def bench_config1(args, dev):
                      "note": "64 micro-batches of 262 MB each, about ten launches per micro-batch issued from Python: "
                              "launch-bound as much as bandwidth-bound"},
         "fused_step_variant": {"what": "siirl_actor_step_fused per micro-batch (one pass over the logits)",
-                               "ms_per_step": fused_wall * 1e3 / steps, "tokens_per_s": tokens * steps / fused_wall},
+                               "ms_per_step": fused_wall * 1e3 / steps, "tokens_per_s": tokens * steps / fused_wall,
+                               "ms_per_step_as_one_hip_graph": graph_ms},
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:  # the CPU-runnable case: the oracle on a sample of 8 of the 64 micro-batches

@@ -449,7 +449,11 @@ __global__ __launch_bounds__(kBwdThreads) void lpe_bwd_flat_kernel(const typenam
 // element instead of the 6 of separate forward and backward launches, and one launch less.
 // Measured at T=32768, V=152064 bf16: 3.8 ms against 4.67 ms for forward + flat backward.  Keeping the second half
 // of the row in registers as well (whole row on chip, 4 bytes per element) measured no faster: with one workgroup
-// per CU the exponentials of the two passes no longer hide behind the memory stream.  A persistent variant that
+// per CU the exponentials of the two passes no longer hide behind the memory stream (3.86 ms with the last two
+// tiles and the ragged end in registers, 4.14 ms when those loads are all issued up front: more requests in flight
+// per CU scatter over more DRAM pages).  Counter-measured traffic of this kernel at that size: 13.1 GB fetched (the
+// L2 and the memory-side cache serve a third of the second read) + 10.0 GB written in 3.65 ms = 6.3 TB/s, the
+// streaming-copy rate of the part.  A persistent variant that
 // holds the whole row in registers and interleaves the dlogits pass of one row with the load and softmax pass of
 // the workgroup's next row (4 bytes per element, nothing re-read) measured 4.3 ms (1024 threads) to 5.9 ms (512):
 // the workgroup-wide merge between rows drains that CU's loads once per row.

@@ -39,6 +39,9 @@ SEED = 20250602
 # counter reads for a plain 2 GiB device copy (FETCH_SIZE reads half the bytes fetched: factor 2.0;
 # WRITE_SIZE factor 1.0).  Figures and commands: profiles/lpe_config2_hbm_traffic.md
 MEASURED_TRAFFIC_BYTES = int((4872295.36 * 2.0 + 9733447.5) * 1024)
+# The same for loss_partials_kernel + loss_bwd_kernel at config 3 with 5488 kept trajectories
+# (profiles/loss_path_config3_hbm_traffic.md)
+MEASURED_TRAFFIC_BYTES_CONFIG3 = int(((526927.5 + 527223.3) * 2.0 + 1372.0 + 176093.0) * 1024)
 
 
 def make_workload(dev, seqs=SEQS, seq_len=SEQ_LEN, vocab=VOCAB, seed=SEED):
@@ -159,7 +162,8 @@ def bench_config3(args, dev):
         "kernels": {"keep mask + GRPO advantage": {"ms": grp_ms},
                     "actor loss forward + backward (loss_partials/finish/bwd kernels)": {"ms": loss_ms, "GB/s": gbs}},
         "roofline": {"bound": "hbm", "kernel": "loss_partials_kernel + loss_bwd_kernel", "achieved": gbs, "peak": 8000.0,
-                     "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None},
+                     "unit": "GB/s", "frac": gbs / 8000.0,
+                     "traffic": MEASURED_TRAFFIC_BYTES_CONFIG3 if Bk == 5488 else None},
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:  # the oracle's eager ops on the host cores, a 512-trajectory sample of the same step

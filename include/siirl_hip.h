@@ -305,30 +305,34 @@ int siirl_unpad_indices(const void* attention_mask, int mask_dtype, int64_t B, i
 
 /*
  * index_first_axis: dst[j, :] = src[indices[j], :] for n rows of row_bytes (a multiple of 4) each; and pad_input:
- * dst[total_rows, :] = 0, then dst[indices[j], :] = src[j, :].  Each is the other's backward.
+ * dst[total_rows, :] = 0, then dst[indices[j], :] = src[j, :].  Each is the other's backward.  src of the gather
+ * has src_rows rows; an index outside [0, src_rows) (gather: the row reads as zeros) or [0, total_rows) (scatter:
+ * the row is dropped) never touches memory.
  * Replaces: index_first_axis / pad_input of flash-attn's bert_padding, siirl/engine/actor/dp_actor.py:117-119,215-226.
  */
-int siirl_gather_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, void* dst,
-                      siirl_stream_t stream);
+int siirl_gather_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, int64_t src_rows,
+                      void* dst, siirl_stream_t stream);
 int siirl_scatter_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, int64_t total_rows,
                        void* dst, siirl_stream_t stream);
 
 /*
  * ids_rmpad[j] = input_ids[indices[j]] and labels_rolled[j] = input_ids[indices[(j + 1) % nnz]]: the packed ids and
- * the next-token labels in one pass (either output may be NULL).
+ * the next-token labels in one pass (either output may be NULL).  input_ids has n_ids entries; an index outside
+ * [0, n_ids) yields -1 instead of a read.
  * Replaces: unpad_input on input_ids + torch.roll(input_ids_rmpad, shifts=-1), siirl/engine/actor/dp_actor.py:112-127.
  */
-int siirl_unpad_ids_labels(const int64_t* input_ids, const int64_t* indices, int64_t nnz, int64_t* ids_rmpad,
-                           int64_t* labels_rolled, siirl_stream_t stream);
+int siirl_unpad_ids_labels(const int64_t* input_ids, int64_t n_ids, const int64_t* indices, int64_t nnz,
+                           int64_t* ids_rmpad, int64_t* labels_rolled, siirl_stream_t stream);
 
 /*
  * pad_input followed by the response window: out[b, t] = full[b, S - L - 1 + t], t in [0, L), where full is the
  * zero-padded [B, S] scatter of values[nnz] at `indices` -- without materialising full.  The gather is its backward.
+ * Indices outside [0, B * S) are ignored (scatter) or read as zero (gather).
  * Replaces: pad_input(...).squeeze(-1)[:, -response_length - 1 : -1], siirl/engine/actor/dp_actor.py:214-231.
  */
 int siirl_response_scatter(const float* values, const int64_t* indices, int64_t nnz, int64_t B, int64_t S, int64_t L,
                            float* out, siirl_stream_t stream);
-int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t S, int64_t L,
+int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t B, int64_t S, int64_t L,
                           float* d_values, siirl_stream_t stream);
 
 /* ------------------------------------------------------------------- outcome reward placement */

@@ -37,11 +37,11 @@ SIGNATURES = {
     "siirl_value_loss_fwd": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _f32, _i32, _p, _p, _p, _sz, _p]),
     "siirl_value_loss_bwd": (_i32, [_p, _p, _p, _p, _p, _i32, _i64, _i64, _f32, _i32, _p, _p, _p, _p]),
     "siirl_unpad_indices": (_i32, [_p, _i32, _i64, _i64, _p, _p, _p, _p, _p]),
-    "siirl_gather_rows": (_i32, [_p, _p, _i64, _i64, _p, _p]),
+    "siirl_gather_rows": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
     "siirl_scatter_rows": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
-    "siirl_unpad_ids_labels": (_i32, [_p, _p, _i64, _p, _p, _p]),
+    "siirl_unpad_ids_labels": (_i32, [_p, _i64, _p, _i64, _p, _p, _p]),
     "siirl_response_scatter": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p]),
-    "siirl_response_gather": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
+    "siirl_response_gather": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p]),
     "siirl_place_outcome_reward": (_i32, [_p, _p, _i32, _i64, _i64, _i64, _i32, _f64, _f64, _f64, _p, _p, _p, _p]),
     "siirl_data_metrics_workspace_bytes": (_sz, [_i64, _i64]),
     "siirl_data_metrics": (_i32, [_p, _p, _p, _p, _p, _p, _i32, _p, _i32, _i64, _i64, _i64, _p, _p, _sz, _p]),

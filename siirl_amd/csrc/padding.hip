@@ -105,13 +105,15 @@ __global__ __launch_bounds__(kThreads) void indices_kernel(const void* mask, int
 template <bool GATHER>
 __global__ __launch_bounds__(kThreads) void move_rows_kernel(const uint32_t* __restrict__ src,
                                                              const int64_t* __restrict__ indices, int64_t n,
-                                                             int64_t words, uint32_t* __restrict__ dst) {
+                                                             int64_t words, int64_t indexed_rows,
+                                                             uint32_t* __restrict__ dst) {
   const int64_t total = n * words;
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
     const int64_t j = i / words, w = i - j * words;
     const int64_t r = indices[j];
-    if (GATHER) dst[i] = src[r * words + w];
-    else dst[r * words + w] = src[i];
+    const bool ok = r >= 0 && r < indexed_rows;  // an index outside the indexed tensor never touches memory
+    if (GATHER) dst[i] = ok ? src[r * words + w] : 0u;
+    else if (ok) dst[r * words + w] = src[i];
   }
 }
 
@@ -120,31 +122,34 @@ __global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* __restric
 }
 
 // ids_rmpad[j] = input_ids[indices[j]],  labels[j] = input_ids[indices[(j + 1) % nnz]]  (torch.roll(..., -1))
-__global__ __launch_bounds__(kThreads) void unpad_ids_kernel(const int64_t* __restrict__ input_ids,
+__global__ __launch_bounds__(kThreads) void unpad_ids_kernel(const int64_t* __restrict__ input_ids, int64_t n_ids,
                                                              const int64_t* __restrict__ indices, int64_t nnz,
                                                              int64_t* __restrict__ ids_rmpad,
                                                              int64_t* __restrict__ labels) {
+  auto at = [&](int64_t r) { return (r >= 0 && r < n_ids) ? input_ids[r] : (int64_t)-1; };
   for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kThreads) {
-    if (ids_rmpad) ids_rmpad[j] = input_ids[indices[j]];
-    if (labels) labels[j] = input_ids[indices[j + 1 < nnz ? j + 1 : 0]];
+    if (ids_rmpad) ids_rmpad[j] = at(indices[j]);
+    if (labels) labels[j] = at(indices[j + 1 < nnz ? j + 1 : 0]);
   }
 }
 
 // out[b, t] = values[j] for the j with indices[j] == b * S + (S - L - 1 + t); positions nobody writes stay 0
 __global__ __launch_bounds__(kThreads) void response_scatter_kernel(const float* __restrict__ values,
                                                                     const int64_t* __restrict__ indices, int64_t nnz,
-                                                                    int64_t S, int64_t L, float* __restrict__ out) {
+                                                                    int64_t B, int64_t S, int64_t L,
+                                                                    float* __restrict__ out) {
   for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kThreads) {
     const int64_t pos = indices[j], b = pos / S, t = pos - b * S - (S - L - 1);
-    if (t >= 0 && t < L) out[b * L + t] = values[j];
+    if (pos >= 0 && b < B && t >= 0 && t < L) out[b * L + t] = values[j];
   }
 }
 __global__ __launch_bounds__(kThreads) void response_gather_kernel(const float* __restrict__ grad,
                                                                    const int64_t* __restrict__ indices, int64_t nnz,
-                                                                   int64_t S, int64_t L, float* __restrict__ d_values) {
+                                                                   int64_t B, int64_t S, int64_t L,
+                                                                   float* __restrict__ d_values) {
   for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kThreads) {
     const int64_t pos = indices[j], b = pos / S, t = pos - b * S - (S - L - 1);
-    d_values[j] = (t >= 0 && t < L) ? grad[b * L + t] : 0.f;
+    d_values[j] = (pos >= 0 && b < B && t >= 0 && t < L) ? grad[b * L + t] : 0.f;
   }
 }
 
@@ -181,14 +186,15 @@ extern "C" int siirl_unpad_indices(const void* attention_mask, int mask_dtype, i
   return SIIRL_OK;
 }
 
-extern "C" int siirl_gather_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, void* dst,
-                                 siirl_stream_t stream) {
-  SIIRL_REQUIRE(n >= 0 && row_bytes >= 4 && row_bytes % 4 == 0, "n=%lld row_bytes=%lld: rows are whole 4-byte words",
-                (long long)n, (long long)row_bytes);
+extern "C" int siirl_gather_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes,
+                                 int64_t src_rows, void* dst, siirl_stream_t stream) {
+  SIIRL_REQUIRE(n >= 0 && src_rows >= 0 && row_bytes >= 4 && row_bytes % 4 == 0,
+                "n=%lld src_rows=%lld row_bytes=%lld: rows are whole 4-byte words", (long long)n, (long long)src_rows,
+                (long long)row_bytes);
   if (n == 0) return SIIRL_OK;
   SIIRL_REQUIRE(src && indices && dst, "NULL operand");
   move_rows_kernel<true><<<dim3(blocks_for(n * (row_bytes / 4))), dim3(kThreads), 0, (hipStream_t)stream>>>(
-      (const uint32_t*)src, indices, n, row_bytes / 4, (uint32_t*)dst);
+      (const uint32_t*)src, indices, n, row_bytes / 4, src_rows, (uint32_t*)dst);
   SIIRL_LAUNCH_CHECK("move_rows_kernel<gather>");
   return SIIRL_OK;
 }
@@ -206,18 +212,18 @@ extern "C" int siirl_scatter_rows(const void* src, const int64_t* indices, int64
   SIIRL_LAUNCH_CHECK("fill_zero_kernel");
   if (n == 0) return SIIRL_OK;
   move_rows_kernel<false><<<dim3(blocks_for(n * (row_bytes / 4))), dim3(kThreads), 0, st>>>(
-      (const uint32_t*)src, indices, n, row_bytes / 4, (uint32_t*)dst);
+      (const uint32_t*)src, indices, n, row_bytes / 4, total_rows, (uint32_t*)dst);
   SIIRL_LAUNCH_CHECK("move_rows_kernel<scatter>");
   return SIIRL_OK;
 }
 
-extern "C" int siirl_unpad_ids_labels(const int64_t* input_ids, const int64_t* indices, int64_t nnz,
+extern "C" int siirl_unpad_ids_labels(const int64_t* input_ids, int64_t n_ids, const int64_t* indices, int64_t nnz,
                                       int64_t* ids_rmpad, int64_t* labels_rolled, siirl_stream_t stream) {
-  SIIRL_REQUIRE(nnz >= 0, "nnz < 0");
+  SIIRL_REQUIRE(nnz >= 0 && n_ids >= 0, "nnz=%lld n_ids=%lld must not be negative", (long long)nnz, (long long)n_ids);
   if (nnz == 0) return SIIRL_OK;
   SIIRL_REQUIRE(input_ids && indices && (ids_rmpad || labels_rolled), "NULL operand");
-  unpad_ids_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(input_ids, indices, nnz, ids_rmpad,
-                                                                                     labels_rolled);
+  unpad_ids_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(input_ids, n_ids, indices, nnz,
+                                                                                     ids_rmpad, labels_rolled);
   SIIRL_LAUNCH_CHECK("unpad_ids_kernel");
   return SIIRL_OK;
 }
@@ -231,18 +237,18 @@ extern "C" int siirl_response_scatter(const float* values, const int64_t* indice
   fill_zero_kernel<<<dim3(blocks_for(B * L)), dim3(kThreads), 0, st>>>((uint32_t*)out, B * L);
   SIIRL_LAUNCH_CHECK("fill_zero_kernel");
   if (nnz == 0) return SIIRL_OK;
-  response_scatter_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, st>>>(values, indices, nnz, S, L, out);
+  response_scatter_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, st>>>(values, indices, nnz, B, S, L, out);
   SIIRL_LAUNCH_CHECK("response_scatter_kernel");
   return SIIRL_OK;
 }
 
-extern "C" int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t S, int64_t L,
-                                     float* d_values, siirl_stream_t stream) {
-  SIIRL_REQUIRE(nnz >= 0 && S >= 2 && L >= 1 && L <= S - 1, "nnz=%lld S=%lld L=%lld: need 1 <= L <= S - 1",
-                (long long)nnz, (long long)S, (long long)L);
+extern "C" int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t B, int64_t S,
+                                     int64_t L, float* d_values, siirl_stream_t stream) {
+  SIIRL_REQUIRE(nnz >= 0 && B >= 1 && S >= 2 && L >= 1 && L <= S - 1, "nnz=%lld B=%lld S=%lld L=%lld: need 1 <= L <= S - 1",
+                (long long)nnz, (long long)B, (long long)S, (long long)L);
   if (nnz == 0) return SIIRL_OK;
   SIIRL_REQUIRE(grad && indices && d_values, "NULL operand");
-  response_gather_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(grad, indices, nnz, S, L,
+  response_gather_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(grad, indices, nnz, B, S, L,
                                                                                            d_values);
   SIIRL_LAUNCH_CHECK("response_gather_kernel");
   return SIIRL_OK;

@@ -65,8 +65,8 @@ class _IndexFirstAxis(torch.autograd.Function):
         ctx.total = x.shape[0]
         if n:
             with torch.cuda.device(x.device):
-                rc = _lib.lib().siirl_gather_rows(_lib.ptr(x), _lib.ptr(indices), n, _rows(x), _lib.ptr(out),
-                                                  _lib.current_stream(x.device))
+                rc = _lib.lib().siirl_gather_rows(_lib.ptr(x), _lib.ptr(indices), n, _rows(x), x.shape[0],
+                                                  _lib.ptr(out), _lib.current_stream(x.device))
             _lib.check(rc, "siirl_gather_rows")
         return out
 
@@ -131,8 +131,8 @@ def unpad_ids_and_labels(input_ids: torch.Tensor, attention_mask: torch.Tensor):
     rm = torch.empty(nnz, dtype=torch.int64, device=ids.device)
     rolled = torch.empty(nnz, dtype=torch.int64, device=ids.device)
     with torch.cuda.device(ids.device):
-        rc = _lib.lib().siirl_unpad_ids_labels(_lib.ptr(ids), _lib.ptr(indices), nnz, _lib.ptr(rm), _lib.ptr(rolled),
-                                               _lib.current_stream(ids.device))
+        rc = _lib.lib().siirl_unpad_ids_labels(_lib.ptr(ids), ids.numel(), _lib.ptr(indices), nnz, _lib.ptr(rm),
+                                               _lib.ptr(rolled), _lib.current_stream(ids.device))
     _lib.check(rc, "siirl_unpad_ids_labels")
     return rm.unsqueeze(0), rolled, indices, cu, max_seqlen
 
@@ -158,8 +158,8 @@ class _ResponseWindow(torch.autograd.Function):
         g = g.detach().to(torch.float32).contiguous()
         d = torch.empty(indices.numel(), dtype=torch.float32, device=g.device)
         with torch.cuda.device(g.device):
-            rc = _lib.lib().siirl_response_gather(_lib.ptr(g), _lib.ptr(indices), indices.numel(), S, L, _lib.ptr(d),
-                                                  _lib.current_stream(g.device))
+            rc = _lib.lib().siirl_response_gather(_lib.ptr(g), _lib.ptr(indices), indices.numel(), g.shape[0], S, L,
+                                                  _lib.ptr(d), _lib.current_stream(g.device))
         _lib.check(rc, "siirl_response_gather")
         return d.to(dtype), None, None, None, None
 

@@ -101,3 +101,23 @@ def test_index_first_axis_autograd_and_dtypes(dev):
         P.index_first_axis(torch.zeros(4, 1, dtype=torch.bfloat16, device=dev), idx[:1] * 0)
     with pytest.raises(RuntimeError):
         P.unpad_input(torch.zeros(2, 2, 1), torch.ones(2, 2))
+
+
+def test_indices_outside_the_tensor_touch_no_memory(dev):
+    """An index outside the indexed tensor reads as zero (gathers; -1 for token ids) or is dropped (scatters)."""
+    import siirl_amd.padding as PD
+
+    x = torch.arange(12, dtype=torch.float32, device=dev).reshape(6, 2)
+    idx = torch.tensor([0, 5, 6, -1, 2 ** 40, 3], device=dev)
+    got = PD.index_first_axis(x, idx).cpu()
+    want = torch.tensor([[0., 1.], [10., 11.], [0., 0.], [0., 0.], [0., 0.], [6., 7.]])
+    assert torch.equal(got, want)
+    out = PD.pad_input(torch.ones(6, 2, device=dev), idx, 2, 3).cpu().reshape(6, 2)
+    assert torch.equal(out[:, 0], torch.tensor([1., 0., 0., 1., 0., 1.]))
+    B, S, L = 2, 6, 3
+    vals = torch.arange(1, 7, dtype=torch.float32, device=dev).requires_grad_(True)
+    bad = torch.tensor([2, 3, 12, -5, 9, 2 ** 41], device=dev)  # window of row 0: positions 2..4; row 1: 8..10
+    w = PD.pad_and_slice_response(vals, bad, B, S, L)
+    assert torch.equal(w.detach().cpu(), torch.tensor([[1., 2., 0.], [0., 5., 0.]]))
+    w.sum().backward()
+    assert torch.equal(vals.grad.cpu(), torch.tensor([1., 1., 0., 0., 1., 0.]))

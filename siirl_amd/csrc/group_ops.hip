@@ -62,14 +62,30 @@ __device__ __forceinline__ void run_of(const int64_t* __restrict__ uid, int64_t 
   while (hi < B && uid[hi] == my) ++hi;
 }
 
+
+// Calls f(value) for every staged entry k < lim with s_uid[k] == my, in order.  Four entries are fetched per LDS
+// read (the loop is bound by the latency of those reads, not by the compares).
+template <typename T, typename F>
+__device__ __forceinline__ void for_members(const int64_t* s_uid, const T* s_val, int lim, int64_t my, F&& f) {
+  for (int k = 0; k < lim; k += 4) {
+    const longlong2 u01 = *reinterpret_cast<const longlong2*>(s_uid + k);
+    const longlong2 u23 = *reinterpret_cast<const longlong2*>(s_uid + k + 2);
+    const T v0 = s_val[k], v1 = s_val[k + 1], v2 = s_val[k + 2], v3 = s_val[k + 3];
+    if (u01.x == my) f(v0);
+    if (k + 1 < lim && u01.y == my) f(v1);
+    if (k + 2 < lim && u23.x == my) f(v2);
+    if (k + 3 < lim && u23.y == my) f(v3);
+  }
+}
+
 // ---------------------------------------------------------------------------- GRPO advantage
 
 // a[i] = (s_i - mean_g) / (std_g + eps), unbiased std; a group of one uses mean 0, std 1.
 __global__ __launch_bounds__(kGroupThreads) void grpo_group_kernel(const float* __restrict__ scores,
                                                               const int64_t* __restrict__ uid, int64_t B, float eps,
                                                               int norm_by_std, float* __restrict__ a_out) {
-  __shared__ int64_t s_uid[kTile];
-  __shared__ float s_val[kTile];
+  __shared__ __align__(16) int64_t s_uid[kTile];
+  __shared__ __align__(16) float s_val[kTile];
   const int64_t i = (int64_t)blockIdx.x * kGroupThreads + threadIdx.x;
   const bool live = i < B;
   const int64_t my = live ? uid[i] : 0;
@@ -104,11 +120,10 @@ __global__ __launch_bounds__(kGroupThreads) void grpo_group_kernel(const float* 
     __syncthreads();
     const int lim = (int)((B - base) < kTile ? (B - base) : kTile);
     if (live)
-      for (int k = 0; k < lim; ++k)
-        if (s_uid[k] == my) {
-          ++n;
-          sum += (double)s_val[k];
-        }
+      for_members(s_uid, s_val, lim, my, [&](float v) {
+        ++n;
+        sum += (double)v;
+      });
   }
   const double mean = n > 1 ? sum / (double)n : 0.0;
   double ss = 0.0;
@@ -122,11 +137,10 @@ __global__ __launch_bounds__(kGroupThreads) void grpo_group_kernel(const float* 
     __syncthreads();
     const int lim = (int)((B - base) < kTile ? (B - base) : kTile);
     if (live && n > 1)
-      for (int k = 0; k < lim; ++k)
-        if (s_uid[k] == my) {
-          const double d = (double)s_val[k] - mean;
-          ss += d * d;
-        }
+      for_members(s_uid, s_val, lim, my, [&](float v) {
+        const double d = (double)v - mean;
+        ss += d * d;
+      });
   }
   if (!live) return;
   const double sd = n > 1 ? sqrt(ss / (double)(n - 1)) : 1.0;
@@ -248,8 +262,8 @@ template <typename T>
 __global__ __launch_bounds__(kGroupThreads) void keep_mask_kernel(const T* __restrict__ val, const int64_t* __restrict__ uid,
                                                              int64_t B, uint8_t* __restrict__ keep,
                                                              int32_t* __restrict__ group_size) {
-  __shared__ int64_t s_uid[kTile];
-  __shared__ T s_val[kTile];
+  __shared__ __align__(16) int64_t s_uid[kTile];
+  __shared__ __align__(16) T s_val[kTile];
   const int64_t i = (int64_t)blockIdx.x * kGroupThreads + threadIdx.x;
   const bool live = i < B;
   const int64_t my = live ? uid[i] : 0;
@@ -296,8 +310,7 @@ __global__ __launch_bounds__(kGroupThreads) void keep_mask_kernel(const T* __res
   }
   for (int64_t base = 0; base < B; base += kTile) {
     const int lim = stage(base);
-    if (live)
-      for (int k = 0; k < lim; ++k) n += (s_uid[k] == my) ? 1 : 0;
+    if (live) for_members(s_uid, s_val, lim, my, [&](T) { ++n; });
   }
   const bool small = n <= 128;
   // mean
@@ -305,9 +318,7 @@ __global__ __launch_bounds__(kGroupThreads) void keep_mask_kernel(const T* __res
   blk.begin(small ? n : 0);
   for (int64_t base = 0; base < B; base += kTile) {
     const int lim = stage(base);
-    if (live && small && n > 1)
-      for (int k = 0; k < lim; ++k)
-        if (s_uid[k] == my) blk.push(s_val[k]);
+    if (live && small && n > 1) for_members(s_uid, s_val, lim, my, [&](T v) { blk.push(v); });
   }
   T mean = blk.finish() / (T)n;
   // sum of squared deviations
@@ -315,11 +326,10 @@ __global__ __launch_bounds__(kGroupThreads) void keep_mask_kernel(const T* __res
   for (int64_t base = 0; base < B; base += kTile) {
     const int lim = stage(base);
     if (live && small && n > 1)
-      for (int k = 0; k < lim; ++k)
-        if (s_uid[k] == my) {
-          const T d = s_val[k] - mean;
-          blk.push(d * d);
-        }
+      for_members(s_uid, s_val, lim, my, [&](T v) {
+        const T d = v - mean;
+        blk.push(d * d);
+      });
   }
   T ssq = blk.finish();
   if (live && !small) {  // rare: groups of more than 128, numpy recurses

@@ -551,7 +551,8 @@ size_t ws_bytes_of(int64_t B, int64_t L) {
 constexpr int64_t kTwoLevelRows = 2048;  // above this many rows the finish runs in two levels
 
 int check_dims(int64_t B, int64_t L) {
-  SIIRL_REQUIRE(B >= 1 && L >= 1, "B=%lld L=%lld must be positive", (long long)B, (long long)L);
+  // an empty batch (B == 0) is served: the forward writes the aggregates of nothing, the backward does nothing
+  SIIRL_REQUIRE(B >= 0 && L >= 1, "B=%lld must not be negative and L=%lld must be positive", (long long)B, (long long)L);
   SIIRL_REQUIRE(L <= (1LL << 40) && B * (int64_t)nseg_of(L) <= 0x7fffffffLL, "B=%lld x L=%lld exceeds the launch grid",
                 (long long)B, (long long)L);
   return SIIRL_OK;
@@ -581,6 +582,12 @@ int launch_loss_partials(const LossArgs& a, const float* row_s, float* partials,
 
 int run_forward(LossArgs& a, float* out16, float* row_msum, float* row_s, void* ws, size_t ws_bytes,
                 hipStream_t st) {
+  if (a.B == 0) {  // the finish alone: zero sums give the reference's 0 (token-mean, -sum-norm) or NaN (seq-mean-*)
+    a.nseg = nseg_of(a.L);
+    loss_finish_kernel<<<1, dim3(kThreads), 0, st>>>(a, nullptr, row_s, out16, row_msum);
+    SIIRL_LAUNCH_CHECK("loss_finish_kernel");
+    return SIIRL_OK;
+  }
   a.nseg = nseg_of(a.L);
   if (ws_bytes < ws_bytes_of(a.B, a.L) || ws == nullptr)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed for B=%lld L=%lld",
@@ -629,7 +636,7 @@ extern "C" int siirl_agg_loss_fwd(const float* loss_mat, const void* mask, int m
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   if (int rc = check_agg(agg_mode)) return rc;
-  SIIRL_REQUIRE(loss_mat && mask && out16 && row_msum, "NULL operand");
+  SIIRL_REQUIRE(out16 && (B == 0 || (loss_mat && mask && row_msum)), "NULL operand");
   LossArgs a{};
   a.lp = loss_mat; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode;
   a.aux_agg_mode = agg_mode; a.scale = 1.f; a.B = B; a.L = L;
@@ -642,7 +649,7 @@ extern "C" int siirl_agg_weights(const void* mask, int mask_dtype, int64_t B, in
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   if (int rc = check_agg(agg_mode)) return rc;
-  SIIRL_REQUIRE(mask && weights && out16 && row_msum, "NULL operand");
+  SIIRL_REQUIRE(out16 && (B == 0 || (mask && weights && row_msum)), "NULL operand");
   LossArgs a{};
   // the partials pass over the weights buffer itself (its values are not used, only the mask sums are)
   a.lp = weights; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode;
@@ -651,6 +658,7 @@ extern "C" int siirl_agg_weights(const void* mask, int mask_dtype, int64_t B, in
   fill_kernel<<<dim3(1024), dim3(kThreads), 0, st>>>(weights, B * L, 0.f);
   SIIRL_LAUNCH_CHECK("fill_kernel");
   if (int rc = run_forward(a, out16, row_msum, nullptr, workspace, workspace_bytes, st)) return rc;
+  if (B == 0) return SIIRL_OK;
   agg_weights_kernel<<<dim3((unsigned)(B * a.nseg)), dim3(kThreads), 0, st>>>(a, out16, row_msum, weights);
   SIIRL_LAUNCH_CHECK("agg_weights_kernel");
   return SIIRL_OK;
@@ -662,6 +670,7 @@ extern "C" int siirl_agg_loss_bwd(const float* g_out, const void* mask, int mask
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   if (int rc = check_agg(agg_mode)) return rc;
+  if (B == 0) return SIIRL_OK;
   SIIRL_REQUIRE(g_out && mask && out16 && row_msum && d_loss_mat, "NULL operand");
   LossArgs a{};
   a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = agg_mode; a.aux_agg_mode = agg_mode;
@@ -680,7 +689,7 @@ static int fill_actor_args(LossArgs& a, const float* old_log_prob, const float* 
   if (int rc = check_agg(agg_mode)) return rc;
   SIIRL_REQUIRE(loss_mode >= SIIRL_LOSS_VANILLA && loss_mode <= SIIRL_LOSS_GEO_MEAN, "Unsupported loss mode: %d",
                 loss_mode);
-  SIIRL_REQUIRE(old_log_prob && log_prob && advantages && mask, "NULL operand");
+  SIIRL_REQUIRE(B == 0 || (old_log_prob && log_prob && advantages && mask), "NULL operand");
   if (loss_mode == SIIRL_LOSS_VANILLA || loss_mode == SIIRL_LOSS_CPGD)
     SIIRL_REQUIRE(clip_c > 1.0f, "clip_ratio_c must be greater than 1.0, got %f", (double)clip_c);
   if (loss_mode == SIIRL_LOSS_CPGD) {
@@ -715,8 +724,8 @@ extern "C" int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_
                                ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff,
                                kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale))
     return rc;
-  SIIRL_REQUIRE(out16 && row_msum, "NULL output");
-  SIIRL_REQUIRE((loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
+  SIIRL_REQUIRE(out16 && (B == 0 || row_msum), "NULL output");
+  SIIRL_REQUIRE(B == 0 || (loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
                 "row_s is required for the gspo and geo_mean losses");
   return run_forward(a, out16, row_msum, row_s, workspace, workspace_bytes, (hipStream_t)stream);
 }
@@ -733,6 +742,7 @@ extern "C" int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_pr
                                ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff,
                                kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale))
     return rc;
+  if (B == 0) return SIIRL_OK;
   SIIRL_REQUIRE(g_loss && out16 && row_msum && d_log_prob, "NULL operand");
   SIIRL_REQUIRE((loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
                 "row_s is required for the gspo and geo_mean losses");
@@ -747,7 +757,7 @@ static int fill_value_args(LossArgs& a, const float* vpreds, const float* return
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   if (int rc = check_agg(agg_mode)) return rc;
-  SIIRL_REQUIRE(vpreds && returns && values && mask, "NULL operand");
+  SIIRL_REQUIRE(B == 0 || (vpreds && returns && values && mask), "NULL operand");
   a.old_lp = values; a.lp = vpreds; a.adv = returns; a.mask = mask; a.mask_dtype = mask_dtype;
   a.kind = KIND_VALUE; a.agg_mode = agg_mode; a.aux_agg_mode = agg_mode;
   a.eps_lo = cliprange_value; a.scale = 0.5f;
@@ -761,7 +771,7 @@ extern "C" int siirl_value_loss_fwd(const float* vpreds, const float* returns, c
                                     siirl_stream_t stream) {
   LossArgs a{};
   if (int rc = fill_value_args(a, vpreds, returns, values, mask, mask_dtype, B, L, cliprange_value, agg_mode)) return rc;
-  SIIRL_REQUIRE(out16 && row_msum, "NULL output");
+  SIIRL_REQUIRE(out16 && (B == 0 || row_msum), "NULL output");
   return run_forward(a, out16, row_msum, nullptr, workspace, workspace_bytes, (hipStream_t)stream);
 }
 
@@ -771,6 +781,7 @@ extern "C" int siirl_value_loss_bwd(const float* g_loss, const float* vpreds, co
                                     float* d_vpreds, siirl_stream_t stream) {
   LossArgs a{};
   if (int rc = fill_value_args(a, vpreds, returns, values, mask, mask_dtype, B, L, cliprange_value, agg_mode)) return rc;
+  if (B == 0) return SIIRL_OK;
   SIIRL_REQUIRE(g_loss && out16 && row_msum && d_vpreds, "NULL operand");
   set_vec(a, d_vpreds);
   return launch_loss_bwd(a, g_loss, out16, row_msum, nullptr, d_vpreds, nullptr, (hipStream_t)stream);
@@ -807,11 +818,16 @@ extern "C" int siirl_masked_reduce(const float* values, const void* mask, int ma
                                    size_t workspace_bytes, siirl_stream_t stream) {
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
-  SIIRL_REQUIRE(values && mask, "NULL operand");
+  SIIRL_REQUIRE(B == 0 || (values && mask), "NULL operand");
   SIIRL_REQUIRE(row_sum || row_mean || total2, "no output requested");
   LossArgs a{};
   a.lp = values; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = SIIRL_AGG_TOKEN_MEAN;
   a.aux_agg_mode = a.agg_mode; a.scale = 1.f; a.B = B; a.L = L; a.nseg = nseg_of(L);
+  if (B == 0) {  // sums of nothing
+    masked_finish_kernel<<<1, dim3(kThreads), 0, (hipStream_t)stream>>>(nullptr, a.nseg, 0, row_sum, row_mean, total2);
+    SIIRL_LAUNCH_CHECK("masked_finish_kernel");
+    return SIIRL_OK;
+  }
   if (workspace_bytes < ws_bytes_of(B, L) || workspace == nullptr)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes,
                 ws_bytes_of(B, L));
@@ -831,13 +847,15 @@ extern "C" int siirl_kl_in_reward(const float* token_level_scores, const float* 
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
-  SIIRL_REQUIRE(token_level_scores && old_log_prob && ref_log_prob && mask && token_level_rewards && row_kl &&
-                    current_kl, "NULL operand");
+  SIIRL_REQUIRE(current_kl && (B == 0 || (token_level_scores && old_log_prob && ref_log_prob && mask &&
+                                          token_level_rewards && row_kl)), "NULL operand");
   hipStream_t st = (hipStream_t)stream;
-  kl_reward_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(token_level_scores, old_log_prob, ref_log_prob, mask,
-                                                                mask_dtype, L, kl_mode, beta, token_level_rewards,
-                                                                row_kl);
-  SIIRL_LAUNCH_CHECK("kl_reward_kernel");
+  if (B > 0) {  // an empty batch has no rewards to write; its mean KL is the mean of nothing (NaN)
+    kl_reward_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(token_level_scores, old_log_prob, ref_log_prob, mask,
+                                                                  mask_dtype, L, kl_mode, beta, token_level_rewards,
+                                                                  row_kl);
+    SIIRL_LAUNCH_CHECK("kl_reward_kernel");
+  }
   mean_rows_kernel<<<1, dim3(kThreads), 0, st>>>(row_kl, B, current_kl);
   SIIRL_LAUNCH_CHECK("mean_rows_kernel");
   return SIIRL_OK;

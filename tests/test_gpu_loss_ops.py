@@ -353,3 +353,34 @@ def test_apply_kl_penalty_and_controllers(dev):
         CA.get_kl_controller(SimpleNamespace(type="pid", kl_coef=0.3))
     r = CA.compute_rewards(scores.to(dev), old.to(dev), ref.to(dev), 0.1)
     assert (r.cpu() - OC.compute_rewards(scores, old, ref, 0.1)).abs().max() < 1e-6
+
+
+def test_empty_batch_matches_reference_semantics(dev):
+    """A batch the DAPO filter emptied: token-mean and seq-mean-token-sum-norm of nothing are 0, the seq-mean
+    modes are the mean of no rows (NaN), as the reference's torch ops give; gradients are empty tensors."""
+    import math
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.torch_functional as SF
+
+    L = 8
+    e = torch.empty(0, L, device=dev)
+    m = torch.empty(0, L, dtype=torch.long, device=dev)
+    for mode in AGGS:
+        got = float(CA.agg_loss(e, m, mode))
+        want = float(OC.agg_loss(e.cpu(), m.cpu(), mode))
+        assert (math.isnan(got) and math.isnan(want)) or got == want, (mode, got, want)
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.2, clip_ratio_c=3.0)
+    lp = torch.empty(0, L, device=dev, requires_grad=True)
+    pg, cf, kl, cfl = CA.compute_policy_loss_vanilla(e, lp, e, m, "token-mean", cfg)
+    want = OC.compute_policy_loss_vanilla(e.cpu(), e.cpu(), e.cpu(), m.cpu(), "token-mean", cfg)
+    for a, b in zip((pg, cf, kl, cfl), want):
+        assert float(a) == float(b) == 0.0
+    pg.backward()
+    assert lp.grad.shape == (0, L)
+    assert float(SF.masked_mean(e, m)) == 0.0 and float(SF.masked_sum(e, m)) == 0.0
+    v = torch.empty(0, L, device=dev, requires_grad=True)
+    loss, clipfrac = CA.compute_value_loss(v, e, e, m, 0.5, "token-mean")
+    assert float(loss) == 0.0 and float(clipfrac) == 0.0
+    loss.backward()
+    assert v.grad.shape == (0, L)

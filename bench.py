@@ -244,7 +244,7 @@ def bench_config5(args, dev):
         "config": {"workload": f"config5: fused lm_head + logprob/entropy, hidden [{T}, {H}], W [{V}, {H}], fwd + bwd to "
                                "hidden and W", "tokens": T, "hidden": H, "vocab": V, "seed": SEED},
         "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
-                    "backward (3 x gemm_nt_kernel per 8192-column slab)": {"ms": bwd_ms, "TFLOP/s executed": 3 * gemm / bwd_ms / 1e9}},
+                    "backward (recompute + dlogits per 8192-column slab; d hidden and d weight per four slabs)": {"ms": bwd_ms, "TFLOP/s executed": 3 * gemm / bwd_ms / 1e9}},
         "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel", "achieved": tf_step, "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": tf_step / 2500.0, "traffic": None,
                      "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step; the backward's recompute is not counted"},

@@ -542,6 +542,22 @@ def bench_critic(args, dev):
     wall = time.perf_counter() - t0
     ms = [sum(e[i].elapsed_time(e[i + 1]) for e in evs) / steps for i in range(4)]
     tokens = B * L
+    # the same GAE with the chunked scan order (rows cut into 16 chunks scanned in parallel; float32-accurate, not
+    # bit-identical to the sequential order above)
+    rewards0 = RW.place_outcome_reward(scores, amask, L, overlong, max_resp_len=L)
+    CA.set_gae_scan_order("chunked")
+    try:
+        for _ in range(warm):
+            CA.compute_gae_advantage_return(rewards0, values, mask, 1.0, 0.95)
+        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        g0.record()
+        for _ in range(steps):
+            CA.compute_gae_advantage_return(rewards0, values, mask, 1.0, 0.95)
+        g1.record()
+        torch.cuda.synchronize()
+        gae_chunked_ms = g0.elapsed_time(g1) / steps
+    finally:
+        CA.set_gae_scan_order("exact")
     # GAE + whitening: the scan reads rewards, values, mask and writes advantages, returns (24 B + 8 B mask), the
     # whitening apply reads and writes the advantages once more
     gae_bytes = tokens * (4 + 4 + 8 + 4 + 4 + 4 + 4)
@@ -552,7 +568,8 @@ def bench_critic(args, dev):
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": f"critic: {B} trajectories, prompt {P} + response {L}, gamma 1.0, lam 0.95, "
                                f"cliprange_value 0.5, overlong buffer 1024", "seed": SEED},
-        "kernels": {name: {"ms": t} for name, t in zip(ops, ms)},
+        "kernels": {**{name: {"ms": t} for name, t in zip(ops, ms)},
+                    "GAE + whitening, chunked scan order (not in the step above)": {"ms": gae_chunked_ms}},
         "roofline": {"bound": "hbm", "kernel": "gae_scan_vec_kernel + whiten_apply_kernel", "achieved": gae_bytes / ms[1] / 1e6,
                      "peak": 8000.0, "unit": "GB/s", "frac": gae_bytes / ms[1] / 1e6 / 8000.0, "traffic": None,
                      "note": "the scan is a sequential recurrence per row: its duration is the latency of 8192 dependent "

@@ -385,7 +385,7 @@ int siirl_data_metrics(const float* token_level_scores, const float* token_level
 
 /* ------------------------------------------------------------------- GAE and masked whitening */
 
-/* Bytes of scratch siirl_masked_whiten / siirl_gae_advantage_return need (a constant; 8-byte aligned buffer). */
+/* Bytes of scratch siirl_masked_whiten needs (a constant; 8-byte aligned buffer). */
 size_t siirl_whiten_workspace_bytes(void);
 
 /*
@@ -398,17 +398,29 @@ size_t siirl_whiten_workspace_bytes(void);
 int siirl_masked_whiten(const float* values, const void* mask, int mask_dtype, int64_t n, int shift_mean, float* out,
                         float* stats3, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
 
+/* Order of evaluation of the GAE scan. */
+typedef enum siirl_gae_order {
+  SIIRL_GAE_EXACT_ORDER = 0, /* one sequential pass per row, the reference's float32 operation order */
+  SIIRL_GAE_CHUNKED = 1      /* rows cut into up to 16 chunks scanned in parallel and stitched by their affine maps */
+} siirl_gae_order;
+
+/* Bytes of scratch siirl_gae_advantage_return needs (8-byte aligned buffer). */
+size_t siirl_gae_workspace_bytes(int64_t B, int64_t L);
+
 /*
  * Generalised advantage estimation over [B, L] fp32 operands, scanning each row from its last token:
  *   delta = r_t + gamma * V_next - V_t,  A_t = delta + gamma * lam * A_next; a token with mask 0 keeps V_next and
  *   A_next of the token after it (both start at 0).  returns = A + values (before whitening);
- *   advantages = masked_whiten(A, mask).  The scan is evaluated in the reference's float32 operation order, so
- *   `returns` is bit-identical to the reference's.  stats3 as for siirl_masked_whiten.
+ *   advantages = masked_whiten(A, mask).  With SIIRL_GAE_EXACT_ORDER the scan is evaluated in the reference's
+ *   float32 operation order and `returns` is bit-identical to the reference's; SIIRL_GAE_CHUNKED shortens the
+ *   dependent chain 16-fold for long rows (same arithmetic inside a chunk; the state entering a chunk goes through
+ *   the chunks' composed maps, which changes its rounding: results agree to float32 accuracy, not bit for bit).
+ *   stats3 as for siirl_masked_whiten.
  * Replaces: compute_gae_advantage_return siirl/dag_worker/core_algos.py:229-276.
  */
 int siirl_gae_advantage_return(const float* token_level_rewards, const float* values, const void* mask,
                                int mask_dtype, int64_t B, int64_t L, double gamma, double lam, float* advantages,
-                               float* returns, float* stats3, void* workspace, size_t workspace_bytes,
+                               float* returns, float* stats3, void* workspace, size_t workspace_bytes, int order,
                                siirl_stream_t stream);
 
 /* ------------------------------------------------------------------- per-prompt group statistics */

@@ -47,7 +47,8 @@ SIGNATURES = {
     "siirl_data_metrics": (_i32, [_p, _p, _p, _p, _p, _p, _i32, _p, _i32, _i64, _i64, _i64, _p, _p, _sz, _p]),
     "siirl_whiten_workspace_bytes": (_sz, []),
     "siirl_masked_whiten": (_i32, [_p, _p, _i32, _i64, _i32, _p, _p, _p, _sz, _p]),
-    "siirl_gae_advantage_return": (_i32, [_p, _p, _p, _i32, _i64, _i64, _f64, _f64, _p, _p, _p, _p, _sz, _p]),
+    "siirl_gae_workspace_bytes": (_sz, [_i64, _i64]),
+    "siirl_gae_advantage_return": (_i32, [_p, _p, _p, _i32, _i64, _i64, _f64, _f64, _p, _p, _p, _p, _sz, _i32, _p]),
     "siirl_kl_penalty_fwd": (_i32, [_p, _p, _i64, _i32, _p, _p]),
     "siirl_kl_penalty_bwd": (_i32, [_p, _p, _p, _i64, _i32, _i32, _p, _p, _p]),
     "siirl_masked_reduce": (_i32, [_p, _p, _i32, _i64, _i64, _p, _p, _p, _p, _sz, _p]),

@@ -221,12 +221,28 @@ def _uid_tensor(index, n, dev) -> torch.Tensor:
     return out.contiguous()
 
 
+_GAE_ORDERS = {"exact": 0, "chunked": 1}
+_gae_order = "exact"
+
+
+def set_gae_scan_order(order: str) -> None:
+    """``"exact"`` (default): each row is scanned in one sequential pass in the reference's float32 operation
+    order, ``returns`` is bit-identical to the reference's.  ``"chunked"``: rows of 1024 tokens or more are cut into
+    up to 16 chunks that are scanned in parallel and stitched through their composed affine maps -- a dependent
+    chain 16 times shorter, results equal to float32 accuracy rather than bit for bit."""
+    global _gae_order
+    if order not in _GAE_ORDERS:
+        raise ValueError(f"unknown GAE scan order {order!r}; choose from {sorted(_GAE_ORDERS)}")
+    _gae_order = order
+
+
 @register_adv_est(AdvantageEstimator.GAE)
 def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torch.Tensor, response_mask: torch.Tensor,
                                  gamma, lam):
     """Generalised advantage estimation with whitened advantages (reference ``core_algos.py:229-276``).
     Returns ``(advantages, returns)``, ``[B, L]`` fp32; ``returns`` is the un-whitened advantage plus the
-    values.  Raises the reference's ``ValueError`` when the mask selects fewer than two tokens."""
+    values.  Raises the reference's ``ValueError`` when the mask selects fewer than two tokens.  The order of
+    evaluation is chosen by ``set_gae_scan_order``."""
     dev, back = _staging_device(token_level_rewards, values, response_mask)
     B, L = token_level_rewards.shape
     r = _f32(token_level_rewards, dev)
@@ -237,12 +253,13 @@ def compute_gae_advantage_return(token_level_rewards: torch.Tensor, values: torc
     adv = torch.empty(B, L, dtype=torch.float32, device=dev)
     ret = torch.empty(B, L, dtype=torch.float32, device=dev)
     stats = torch.empty(3, dtype=torch.float32, device=dev)
-    nws = _lib.lib().siirl_whiten_workspace_bytes()
+    nws = _lib.lib().siirl_gae_workspace_bytes(B, L)
     ws = torch.empty(nws, dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         rc = _lib.lib().siirl_gae_advantage_return(_lib.ptr(r), _lib.ptr(v), _lib.ptr(m), mcode, B, L, float(gamma),
                                                    float(lam), _lib.ptr(adv), _lib.ptr(ret), _lib.ptr(stats),
-                                                   _lib.ptr(ws), nws, _lib.current_stream(dev))
+                                                   _lib.ptr(ws), nws, _GAE_ORDERS[_gae_order],
+                                                   _lib.current_stream(dev))
     _lib.check(rc, "siirl_gae_advantage_return")
     siirl_F._check_whiten_count(float(stats[2]))
     if back:

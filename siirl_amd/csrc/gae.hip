@@ -58,12 +58,36 @@ __device__ __forceinline__ void gae_step(float r, float v, float m, float gamma,
   lg = cand * m + om * lg;
 }
 
-template <int MK, bool F32MASK>
+// One token of the scan composed onto the affine map (nv, lg) -> (a00 nv + b0, a10 nv + a11 lg + b1) of the
+// tokens to its right (nv' never depends on lg, so that entry of the matrix stays zero and is not kept).
+struct GaeMap {
+  float a00, a10, a11, b0, b1;
+};
+__device__ __forceinline__ void gae_compose(float r, float v, float m, float gamma, float gamma_lam, GaeMap& g) {
+  const float om = 1.f - m, mg = m * gamma, k = om + m * gamma_lam;
+  const float a10 = mg * g.a00 + k * g.a10;
+  const float b1 = (mg * g.b0 + k * g.b1) + m * (r - v);
+  g.a11 = k * g.a11;
+  g.a00 = om * g.a00;
+  g.b0 = om * g.b0 + m * v;
+  g.a10 = a10;
+  g.b1 = b1;
+}
+
+enum { MODE_SCAN = 0, MODE_COMPOSE = 1 };
+
+// MODE_SCAN: the recurrence itself, from the state `init` gives each row (zero when null).  MODE_COMPOSE: no output
+// per token; each row's tokens are folded into one GaeMap written to `maps`.  With rows that are chunks of the real
+// rows (B = rows x chunks, L = chunk length: chunks of a row are adjacent in memory) a compose pass, a carry over
+// the chunk maps and a scan pass evaluate the recurrence with a dependent chain of one chunk instead of one row.
+template <int MK, bool F32MASK, int MODE>
 __global__ __launch_bounds__(kWave) void gae_scan_vec_kernel(const float* __restrict__ rewards,
                                                               const float* __restrict__ values,
                                                               const void* __restrict__ mask, int64_t B, int64_t L,
                                                               float gamma, float gamma_lam, float* __restrict__ adv,
-                                                              float* __restrict__ ret, double* __restrict__ part) {
+                                                              float* __restrict__ ret, double* __restrict__ part,
+                                                              const float* __restrict__ init,
+                                                              float* __restrict__ maps) {
   __shared__ __align__(16) float s_r[kRows * kPitch], s_v[kRows * kPitch], s_m[kRows * kPitch], s_a[kRows * kPitch];
   const int lane = threadIdx.x;
   const int64_t row0 = (int64_t)blockIdx.x * kRows;
@@ -123,6 +147,11 @@ __global__ __launch_bounds__(kWave) void gae_scan_vec_kernel(const float* __rest
     }
   };
   float nv = 0.f, lg = 0.f;
+  if (MODE == MODE_SCAN && init != nullptr && lane < nrows) {
+    nv = init[2 * (row0 + lane)];
+    lg = init[2 * (row0 + lane) + 1];
+  }
+  GaeMap gm{1.f, 0.f, 1.f, 0.f, 0.f};
   double st[kNStat] = {0.0, 0.0, 0.0};  // whitening statistics of this wave's advantages (pivot 0)
   const int64_t c_last = (L - 1) / kCols * kCols;
   issue(c_last);
@@ -142,16 +171,24 @@ __global__ __launch_bounds__(kWave) void gae_scan_vec_kernel(const float* __rest
         const int nx = cc >= 4 ? cc - 4 : 0;
         const float4 rn = *reinterpret_cast<const float4*>(r4 + nx), vn = *reinterpret_cast<const float4*>(v4 + nx),
                      mn = *reinterpret_cast<const float4*>(m4 + nx);
-        float4 a;
-        gae_step(r.w, v.w, m.w, gamma, gamma_lam, nv, lg); a.w = lg;
-        gae_step(r.z, v.z, m.z, gamma, gamma_lam, nv, lg); a.z = lg;
-        gae_step(r.y, v.y, m.y, gamma, gamma_lam, nv, lg); a.y = lg;
-        gae_step(r.x, v.x, m.x, gamma, gamma_lam, nv, lg); a.x = lg;
-        *reinterpret_cast<float4*>(s_a + lane * kPitch + cc) = a;
+        if (MODE == MODE_SCAN) {
+          float4 a;
+          gae_step(r.w, v.w, m.w, gamma, gamma_lam, nv, lg); a.w = lg;
+          gae_step(r.z, v.z, m.z, gamma, gamma_lam, nv, lg); a.z = lg;
+          gae_step(r.y, v.y, m.y, gamma, gamma_lam, nv, lg); a.y = lg;
+          gae_step(r.x, v.x, m.x, gamma, gamma_lam, nv, lg); a.x = lg;
+          *reinterpret_cast<float4*>(s_a + lane * kPitch + cc) = a;
+        } else {
+          gae_compose(r.w, v.w, m.w, gamma, gamma_lam, gm);
+          gae_compose(r.z, v.z, m.z, gamma, gamma_lam, gm);
+          gae_compose(r.y, v.y, m.y, gamma, gamma_lam, gm);
+          gae_compose(r.x, v.x, m.x, gamma, gamma_lam, gm);
+        }
         r = rn; v = vn; m = mn;
       }
     }
     __syncthreads();
+    if (MODE == MODE_SCAN) {
 #pragma unroll
     for (int k = 0; k < kChunks; ++k) {
       const int q = lane + kWave * k, rr = q / (kCols / 4), ch = q % (kCols / 4);
@@ -171,7 +208,15 @@ __global__ __launch_bounds__(kWave) void gae_scan_vec_kernel(const float* __rest
         }
       }
     }
+    }
     __syncthreads();  // the next commit overwrites s_v / s_a
+  }
+  if (MODE == MODE_COMPOSE) {
+    if (lane < nrows) {
+      float* o = maps + 5 * (row0 + lane);
+      o[0] = gm.a00; o[1] = gm.a10; o[2] = gm.a11; o[3] = gm.b0; o[4] = gm.b1;
+    }
+    return;
   }
   if (part) {
 #pragma unroll
@@ -179,6 +224,24 @@ __global__ __launch_bounds__(kWave) void gae_scan_vec_kernel(const float* __rest
       const double t = wave_sum(st[k]);
       if (lane == 0) part[kNStat * blockIdx.x + k] = t;
     }
+  }
+}
+
+// State entering each chunk: chunk C - 1 of a row starts from zero, chunk c from chunk c + 1's map applied to the
+// state that entered chunk c + 1.  One thread per row.
+__global__ __launch_bounds__(256) void gae_carry_kernel(const float* __restrict__ maps, int64_t B, int chunks,
+                                                        float* __restrict__ init) {
+  const int64_t b = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (b >= B) return;
+  float nv = 0.f, lg = 0.f;
+  for (int c = chunks - 1; c >= 0; --c) {
+    const int64_t r = b * chunks + c;
+    init[2 * r] = nv;
+    init[2 * r + 1] = lg;
+    const float* g = maps + 5 * r;
+    const float nnv = g[0] * nv + g[3];
+    lg = (g[1] * nv + g[2] * lg) + g[4];
+    nv = nnv;
   }
 }
 
@@ -224,7 +287,7 @@ __global__ __launch_bounds__(kWave) void gae_scan_kernel(const float* __restrict
 // ---------------------------------------------------------------------------- masked whitening
 
 constexpr int kThreads = 256;
-constexpr int kMaxParts = 1024;
+constexpr int kMaxParts = 8192;
 __global__ __launch_bounds__(kThreads) void whiten_stats_kernel(const float* __restrict__ v, const void* mask,
                                                                 int mask_dtype, int64_t n, int vec,
                                                                 double* __restrict__ part) {
@@ -346,36 +409,86 @@ extern "C" int siirl_masked_whiten(const float* values, const void* mask, int ma
   return run_whiten(values, mask, mask_dtype, n, shift_mean, out, stats3, workspace, 0, (hipStream_t)stream);
 }
 
+// chunks per row of the chunked scan: the largest of 16, 8, 4, 2 that leaves chunks of at least 256 tokens whose
+// length is a multiple of 4; 1 = the plain scan
+static int gae_chunks(int64_t L) {
+  for (int c = 16; c >= 2; c /= 2)
+    if (L % (4 * c) == 0 && L / c >= 256) return c;
+  return 1;
+}
+constexpr int kGaeMaxChunks = 16;
+static size_t gae_ws_bytes(int64_t B) {
+  return kWhitenWs + (size_t)B * kGaeMaxChunks * (5 + 2) * sizeof(float) + 256;
+}
+
+extern "C" size_t siirl_gae_workspace_bytes(int64_t B, int64_t L) {
+  (void)L;
+  return B < 1 ? 0 : gae_ws_bytes(B);
+}
+
+template <int MK, bool F32MASK>
+static int launch_gae_vec(const float* rewards, const float* values, const void* mask, int64_t B, int64_t L, float g,
+                          float gl, float* adv, float* ret, void* ws, int chunks, int* parts_ready, hipStream_t st) {
+  const int64_t rows = B * chunks, len = L / chunks;
+  const dim3 grid((unsigned)((rows + kRows - 1) / kRows)), block(kWave);
+  // the scan leaves its whitening statistics in the workspace, one partial per workgroup, when they fit
+  const bool fused_stats = grid.x <= (unsigned)kMaxParts;
+  double* part = fused_stats ? (double*)ws : nullptr;
+  *parts_ready = fused_stats ? (int)grid.x : 0;
+  const float* init = nullptr;
+  if (chunks > 1) {
+    float* maps = reinterpret_cast<float*>((char*)ws + kWhitenWs);
+    float* ini = maps + (size_t)rows * 5;
+    gae_scan_vec_kernel<MK, F32MASK, MODE_COMPOSE><<<grid, block, 0, st>>>(rewards, values, mask, rows, len, g, gl, nullptr,
+                                                                        nullptr, nullptr, nullptr, maps);
+    SIIRL_LAUNCH_CHECK("gae_scan_vec_kernel<compose>");
+    gae_carry_kernel<<<dim3((unsigned)((B + 255) / 256)), dim3(256), 0, st>>>(maps, B, chunks, ini);
+    SIIRL_LAUNCH_CHECK("gae_carry_kernel");
+    init = ini;
+  }
+  gae_scan_vec_kernel<MK, F32MASK, MODE_SCAN><<<grid, block, 0, st>>>(rewards, values, mask, rows, len, g, gl, adv, ret,
+                                                                   part, init, nullptr);
+  SIIRL_LAUNCH_CHECK("gae_scan_vec_kernel");
+  return SIIRL_OK;
+}
+
 extern "C" int siirl_gae_advantage_return(const float* token_level_rewards, const float* values, const void* mask,
                                           int mask_dtype, int64_t B, int64_t L, double gamma, double lam,
                                           float* advantages, float* returns, float* stats3, void* workspace,
-                                          size_t workspace_bytes, siirl_stream_t stream) {
-  SIIRL_REQUIRE(B >= 1 && L >= 1 && B <= (1LL << 36), "B=%lld L=%lld out of range", (long long)B, (long long)L);
+                                          size_t workspace_bytes, int order, siirl_stream_t stream) {
+  SIIRL_REQUIRE(B >= 1 && L >= 1 && B <= (1LL << 32), "B=%lld L=%lld out of range", (long long)B, (long long)L);
   if (int rc = check_mask(mask_dtype)) return rc;
   SIIRL_REQUIRE(token_level_rewards && values && mask && advantages && returns && stats3, "NULL operand");
   SIIRL_REQUIRE(advantages != returns, "advantages and returns must be different buffers");
-  if (int rc = check_whiten_ws(workspace, workspace_bytes)) return rc;
+  SIIRL_REQUIRE(order == SIIRL_GAE_EXACT_ORDER || order == SIIRL_GAE_CHUNKED, "unknown scan order %d", order);
+  if (workspace == nullptr || workspace_bytes < gae_ws_bytes(B))
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes,
+                gae_ws_bytes(B));
+  SIIRL_REQUIRE(((uintptr_t)workspace & 7) == 0, "workspace must be 8-byte aligned");
   hipStream_t st = (hipStream_t)stream;
-  const dim3 grid((unsigned)((B + kRows - 1) / kRows)), block(kWave);
   const float g = (float)gamma, gl = (float)(gamma * lam);
   const uintptr_t bases = (uintptr_t)token_level_rewards | (uintptr_t)values | (uintptr_t)advantages | (uintptr_t)returns;
   const bool vec = L % 4 == 0 && (bases & 15) == 0;
-  // the vector kernels leave their whitening statistics in the workspace, one partial per workgroup, when they fit
-  const bool fused_stats = grid.x <= (unsigned)kMaxParts;
-  double* part = fused_stats ? (double*)workspace : nullptr;
-  int parts_ready = fused_stats ? (int)grid.x : 0;
+  const int chunks = order == SIIRL_GAE_CHUNKED ? gae_chunks(L) : 1;
+  int parts_ready = 0;
+  int rc = SIIRL_OK;
   if (vec && mask_dtype == SIIRL_I64 && ((uintptr_t)mask & 15) == 0)
-    gae_scan_vec_kernel<MK_I64, false><<<grid, block, 0, st>>>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, part);
+    rc = launch_gae_vec<MK_I64, false>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, workspace, chunks,
+                                       &parts_ready, st);
   else if (vec && mask_dtype == SIIRL_F32 && ((uintptr_t)mask & 15) == 0)
-    gae_scan_vec_kernel<MK_B32, true><<<grid, block, 0, st>>>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, part);
+    rc = launch_gae_vec<MK_B32, true>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, workspace, chunks,
+                                      &parts_ready, st);
   else if (vec && mask_dtype == SIIRL_I32 && ((uintptr_t)mask & 15) == 0)
-    gae_scan_vec_kernel<MK_B32, false><<<grid, block, 0, st>>>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, part);
+    rc = launch_gae_vec<MK_B32, false>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, workspace, chunks,
+                                       &parts_ready, st);
   else if (vec && mask_dtype == SIIRL_U8 && ((uintptr_t)mask & 3) == 0)
-    gae_scan_vec_kernel<MK_U8, false><<<grid, block, 0, st>>>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, part);
-  else {
-    gae_scan_kernel<<<grid, block, 0, st>>>(token_level_rewards, values, mask, mask_dtype, B, L, g, gl, advantages, returns);
-    parts_ready = 0;
+    rc = launch_gae_vec<MK_U8, false>(token_level_rewards, values, mask, B, L, g, gl, advantages, returns, workspace, chunks,
+                                      &parts_ready, st);
+  else {  // the scalar kernel walks whole rows in the reference's order, whatever `order` asks for
+    gae_scan_kernel<<<dim3((unsigned)((B + kRows - 1) / kRows)), dim3(kWave), 0, st>>>(
+        token_level_rewards, values, mask, mask_dtype, B, L, g, gl, advantages, returns);
+    SIIRL_LAUNCH_CHECK("gae_scan_kernel");
   }
-  SIIRL_LAUNCH_CHECK("gae_scan_kernel");
+  if (rc) return rc;
   return run_whiten(advantages, mask, mask_dtype, B * L, 1, advantages, stats3, workspace, parts_ready, st);
 }

@@ -77,7 +77,11 @@ def test_argument_validation_without_gpu():
     assert h.siirl_actor_loss_fwd(p, p, p, p, L.F32, None, None, None, 2, 4, 4, 0.2, 0.2, 3.0, 20.0, 0, 0.0, 0, 0, 0.0,
                                   0.0, 1.0, p, p, None, p, 1 << 20, None) == -1  # geo_mean needs row_s
     assert h.siirl_value_loss_fwd(p, p, p, p, L.F32, 2, 4, 0.5, 7, p, p, p, 1 << 20, None) == -1
-    assert h.siirl_gae_advantage_return(p, p, p, L.F32, 2, 4, 1.0, 1.0, p, p, p, p, 8, None) == -1  # adv == returns
+    assert h.siirl_gae_advantage_return(p, p, p, L.F32, 2, 4, 1.0, 1.0, p, p, p, p, 8, 0, None) == -1  # adv == returns
+    q2 = ctypes.c_void_p(p.value + 64)
+    assert h.siirl_gae_advantage_return(p, p, p, L.F32, 2, 4, 1.0, 1.0, p, q2, p, p, 1 << 20, 7, None) == -1
+    assert b"scan order" in h.siirl_hip_last_error()
+    assert h.siirl_gae_workspace_bytes(4, 8192) >= h.siirl_whiten_workspace_bytes()
     assert h.siirl_masked_whiten(p, p, L.F64, 4, 1, p, p, p, 1 << 20, None) == -1
     assert h.siirl_whiten_workspace_bytes() > 0
     assert h.siirl_agg_loss_fwd(p, p, L.F32, 2, 4, 0, p, p, p, 8, None) == -4

@@ -37,7 +37,7 @@ def _check_grad(got, want64, name):
 
 
 @pytest.mark.parametrize("T,H,V", [(1, 64, 1), (5, 64, 33), (256, 64, 256), (300, 128, 1000), (513, 256, 8200),
-                                   (64, 3584, 2048), (700, 192, 17000)])
+                                   (64, 3584, 2048), (700, 192, 17000), (257, 64, 32769), (130, 128, 65537)])
 @pytest.mark.parametrize("temperature", [1.0, 0.7])
 def test_fused_matches_oracle(dev, T, H, V, temperature):
     from siirl_amd.fused_linear import FusedLinearForPPO

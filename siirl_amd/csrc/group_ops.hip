@@ -7,10 +7,12 @@
 // one trajectory i and visits the members of its group in batch order, so that every group statistic is
 // accumulated in the order the reference uses; exact integer bookkeeping, no atomics.  When the uid array is
 // non-decreasing (the layout the reference's data loader produces, and what an ascending filter keeps) a
-// group is one contiguous run and the thread walks just that run: O(B * n).  Otherwise the thread scans all
-// trajectories through LDS tiles and picks those with uid[j] == uid[i]: O(B^2) compares.  Every workgroup
-// checks the ordering for itself (O(B) coalesced compares), so no flag has to travel between kernels.  B is
-// a rollout batch (10^3..10^5).
+// group is one contiguous run and a thread per trajectory walks just that run: O(B * n); every workgroup checks
+// the ordering for itself (O(B) coalesced compares).  Otherwise that kernel only marks its outputs as pending and
+// a second kernel gives every trajectory a whole wave: the uids pass through LDS in tiles shared by the 16 waves of
+// a workgroup, each lane compares one entry per step, and the few hits of a step are taken in order from the
+// ballot -- O(B^2) compares spread over all lanes, same member order, same arithmetic, bit-identical results.
+// B is a rollout batch (10^3..10^5).
 //
 // The keep mask reproduces np.std(values) > 0 bit for bit: numpy sums with an 8-accumulator pairwise
 // scheme in the dtype of the values, so e.g. three equal fp64 values 0.1 have std 1.4e-17 > 0.  This
@@ -22,7 +24,6 @@ namespace {
 
 constexpr int kThreads = 256;   // streaming kernels (row sums, broadcast)
 constexpr int kGroupThreads = 64;  // all-pairs kernels: one wave per workgroup, so B = 8192 already fills 128 CUs
-constexpr int kTile = 1024;
 
 // ---------------------------------------------------------------------------- row sums
 
@@ -63,91 +64,97 @@ __device__ __forceinline__ void run_of(const int64_t* __restrict__ uid, int64_t 
 }
 
 
-// Calls f(value) for every staged entry k < lim with s_uid[k] == my, in order.  Four entries are fetched per LDS
-// read (the loop is bound by the latency of those reads, not by the compares).
-template <typename T, typename F>
-__device__ __forceinline__ void for_members(const int64_t* s_uid, const T* s_val, int lim, int64_t my, F&& f) {
-  for (int k = 0; k < lim; k += 4) {
-    const longlong2 u01 = *reinterpret_cast<const longlong2*>(s_uid + k);
-    const longlong2 u23 = *reinterpret_cast<const longlong2*>(s_uid + k + 2);
-    const T v0 = s_val[k], v1 = s_val[k + 1], v2 = s_val[k + 2], v3 = s_val[k + 3];
-    if (u01.x == my) f(v0);
-    if (k + 1 < lim && u01.y == my) f(v1);
-    if (k + 2 < lim && u23.x == my) f(v2);
-    if (k + 3 < lim && u23.y == my) f(v3);
-  }
-}
-
 // ---------------------------------------------------------------------------- GRPO advantage
 
-// a[i] = (s_i - mean_g) / (std_g + eps), unbiased std; a group of one uses mean 0, std 1.
+constexpr uint32_t kPendingBits = 0x7fc0deadu;  // a NaN no arithmetic here produces: "left to the wave kernel"
+constexpr uint8_t kPendingKeep = 2;
+constexpr int kWaveThreads = 1024;                // wave-per-trajectory kernels: 16 trajectories per workgroup
+constexpr int kWaveTile = 4096;                   // uids staged per step (32 KB of LDS)
+
+__device__ __forceinline__ float grpo_value(double s, double mean, double sd, float eps, int norm_by_std) {
+  // the reference evaluates (s - mean) / (std + eps) on fp32 0-d tensors; round the pieces likewise
+  const float num = (float)s - (float)mean;
+  return norm_by_std ? num / ((float)sd + eps) : num;
+}
+
+// a[i] = (s_i - mean_g) / (std_g + eps), unbiased std; a group of one uses mean 0, std 1.  Thread per trajectory
+// over contiguous runs; when the uids are not non-decreasing every output is marked pending instead.
 __global__ __launch_bounds__(kGroupThreads) void grpo_group_kernel(const float* __restrict__ scores,
                                                               const int64_t* __restrict__ uid, int64_t B, float eps,
                                                               int norm_by_std, float* __restrict__ a_out) {
-  __shared__ __align__(16) int64_t s_uid[kTile];
-  __shared__ __align__(16) float s_val[kTile];
   const int64_t i = (int64_t)blockIdx.x * kGroupThreads + threadIdx.x;
-  const bool live = i < B;
-  const int64_t my = live ? uid[i] : 0;
-  int n = 0;
-  double sum = 0.0;
   const bool runs = uid_non_decreasing(uid, B);
-  if (runs) {
-    if (!live) return;
-    int64_t lo, hi;
-    run_of(uid, B, i, lo, hi);
-    n = (int)(hi - lo);
-    for (int64_t j = lo; j < hi; ++j) sum += (double)scores[j];
-    const double mean = n > 1 ? sum / (double)n : 0.0;
-    double ss = 0.0;
-    if (n > 1)
-      for (int64_t j = lo; j < hi; ++j) {
-        const double d = (double)scores[j] - mean;
-        ss += d * d;
-      }
-    const double sd = n > 1 ? sqrt(ss / (double)(n - 1)) : 1.0;
-    const float num = (float)(double)scores[i] - (float)mean;
-    a_out[i] = norm_by_std ? num / ((float)sd + eps) : num;
+  if (i >= B) return;
+  if (!runs) {
+    a_out[i] = u2f(kPendingBits);
     return;
   }
-  for (int64_t base = 0; base < B; base += kTile) {
-    __syncthreads();
-    for (int k = threadIdx.x; k < kTile; k += kGroupThreads) {
-      const int64_t j = base + k;
-      s_uid[k] = j < B ? uid[j] : 0;
-      s_val[k] = j < B ? scores[j] : 0.f;
-    }
-    __syncthreads();
-    const int lim = (int)((B - base) < kTile ? (B - base) : kTile);
-    if (live)
-      for_members(s_uid, s_val, lim, my, [&](float v) {
-        ++n;
-        sum += (double)v;
-      });
-  }
+  int64_t lo, hi;
+  run_of(uid, B, i, lo, hi);
+  const int n = (int)(hi - lo);
+  double sum = 0.0;
+  for (int64_t j = lo; j < hi; ++j) sum += (double)scores[j];
   const double mean = n > 1 ? sum / (double)n : 0.0;
   double ss = 0.0;
-  for (int64_t base = 0; base < B; base += kTile) {
-    __syncthreads();
-    for (int k = threadIdx.x; k < kTile; k += kGroupThreads) {
-      const int64_t j = base + k;
-      s_uid[k] = j < B ? uid[j] : 0;
-      s_val[k] = j < B ? scores[j] : 0.f;
+  if (n > 1)
+    for (int64_t j = lo; j < hi; ++j) {
+      const double d = (double)scores[j] - mean;
+      ss += d * d;
     }
-    __syncthreads();
-    const int lim = (int)((B - base) < kTile ? (B - base) : kTile);
-    if (live && n > 1)
-      for_members(s_uid, s_val, lim, my, [&](float v) {
-        const double d = (double)v - mean;
-        ss += d * d;
-      });
-  }
-  if (!live) return;
   const double sd = n > 1 ? sqrt(ss / (double)(n - 1)) : 1.0;
-  const double s = (double)scores[i];
-  // the reference evaluates (s - mean) / (std + eps) on fp32 0-d tensors; round the pieces likewise
-  const float num = (float)s - (float)mean;
-  a_out[i] = norm_by_std ? num / ((float)sd + eps) : num;
+  a_out[i] = grpo_value((double)scores[i], mean, sd, eps, norm_by_std);
+}
+
+// Stages uid[base, base + kWaveTile) into LDS (all threads of the workgroup), then calls f(j) on the calling wave for
+// every j in the tile with uid[j] == my, in ascending order.  Every lane of the wave sees the same sequence of j.
+template <typename F>
+__device__ __forceinline__ void wave_members(const int64_t* __restrict__ uid, int64_t B, int64_t my, bool active,
+                                             int64_t* s_uid, F&& f) {
+  const int lane = threadIdx.x & (kWave - 1);
+  for (int64_t base = 0; base < B; base += kWaveTile) {
+    __syncthreads();
+    for (int k = threadIdx.x; k < kWaveTile; k += kWaveThreads) s_uid[k] = base + k < B ? uid[base + k] : 0;
+    __syncthreads();
+    const int lim = (int)((B - base) < kWaveTile ? (B - base) : kWaveTile);
+    if (active)
+      for (int k0 = 0; k0 < lim; k0 += kWave) {
+        const int k = k0 + lane;
+        unsigned long long bal = __ballot(k < lim && s_uid[k] == my);
+        while (bal) {
+          const int l = __builtin_ctzll(bal);
+          bal &= bal - 1;
+          f(base + k0 + l);
+        }
+      }
+  }
+}
+
+// The pending outputs of grpo_group_kernel: one wave per trajectory.
+__global__ __launch_bounds__(kWaveThreads) void grpo_group_wave_kernel(const float* __restrict__ scores,
+                                                                        const int64_t* __restrict__ uid, int64_t B,
+                                                                        float eps, int norm_by_std,
+                                                                        float* __restrict__ a_out) {
+  __shared__ int64_t s_uid[kWaveTile];
+  const int64_t i = (int64_t)blockIdx.x * (kWaveThreads / kWave) + threadIdx.x / kWave;
+  const bool active = i < B && f2u(a_out[i]) == kPendingBits;
+  if (!__syncthreads_or(active ? 1 : 0)) return;  // ordered uids: the first kernel has done everything
+  const int64_t my = active ? uid[i] : 0;
+  int n = 0;
+  double sum = 0.0;
+  wave_members(uid, B, my, active, s_uid, [&](int64_t j) {
+    ++n;
+    sum += (double)scores[j];
+  });
+  const double mean = n > 1 ? sum / (double)n : 0.0;
+  double ss = 0.0;
+  if (__syncthreads_or((active && n > 1) ? 1 : 0))
+    wave_members(uid, B, my, active && n > 1, s_uid, [&](int64_t j) {
+      const double d = (double)scores[j] - mean;
+      ss += d * d;
+    });
+  if (!active) return;
+  const double sd = n > 1 ? sqrt(ss / (double)(n - 1)) : 1.0;
+  if ((threadIdx.x & (kWave - 1)) == 0) a_out[i] = grpo_value((double)scores[i], mean, sd, eps, norm_by_std);
 }
 
 __global__ __launch_bounds__(kThreads) void broadcast_mask_kernel(const float* __restrict__ a, const void* mask,
@@ -257,91 +264,87 @@ __device__ T np_pairwise(MemberCursor<T>& cur, int n, T mean) {
   return ret;
 }
 
-// keep[i] = group of i has one member, or np.std(group values) > 0
+// keep[i] = group of i has one member, or np.std(group values) > 0.  Thread per trajectory over contiguous runs;
+// when the uids are not non-decreasing every output is marked pending instead.
 template <typename T>
 __global__ __launch_bounds__(kGroupThreads) void keep_mask_kernel(const T* __restrict__ val, const int64_t* __restrict__ uid,
                                                              int64_t B, uint8_t* __restrict__ keep,
                                                              int32_t* __restrict__ group_size) {
-  __shared__ __align__(16) int64_t s_uid[kTile];
-  __shared__ __align__(16) T s_val[kTile];
   const int64_t i = (int64_t)blockIdx.x * kGroupThreads + threadIdx.x;
-  const bool live = i < B;
-  const int64_t my = live ? uid[i] : 0;
-  auto stage = [&](int64_t base) {
-    __syncthreads();
-    for (int k = threadIdx.x; k < kTile; k += kGroupThreads) {
-      const int64_t j = base + k;
-      s_uid[k] = j < B ? uid[j] : 0;
-      s_val[k] = j < B ? val[j] : T(0);
-    }
-    __syncthreads();
-    return (int)((B - base) < kTile ? (B - base) : kTile);
-  };
-  int n = 0;
-  if (uid_non_decreasing(uid, B)) {
-    if (!live) return;
-    int64_t lo, hi;
-    run_of(uid, B, i, lo, hi);
-    n = (int)(hi - lo);
-    T mean, ssq;
-    if (n <= 128) {
-      NpBlock<T> blk;
-      blk.begin(n);
-      if (n > 1)
-        for (int64_t j = lo; j < hi; ++j) blk.push(val[j]);
-      mean = blk.finish() / (T)n;
-      blk.begin(n);
-      if (n > 1)
-        for (int64_t j = lo; j < hi; ++j) {
-          const T d = val[j] - mean;
-          blk.push(d * d);
-        }
-      ssq = blk.finish();
-    } else {
-      MemberCursor<T> c1{uid, val, B, lo, my};
-      mean = np_pairwise<T, false>(c1, n, T(0)) / (T)n;
-      MemberCursor<T> c2{uid, val, B, lo, my};
-      ssq = np_pairwise<T, true>(c2, n, mean);
-    }
-    const T sd = sqrt(ssq / (T)n);
-    keep[i] = (n == 1 || sd > T(0)) ? 1 : 0;
-    if (group_size) group_size[i] = n;
+  const bool runs = uid_non_decreasing(uid, B);
+  if (i >= B) return;
+  if (!runs) {
+    keep[i] = kPendingKeep;
     return;
   }
-  for (int64_t base = 0; base < B; base += kTile) {
-    const int lim = stage(base);
-    if (live) for_members(s_uid, s_val, lim, my, [&](T) { ++n; });
+  const int64_t my = uid[i];
+  int64_t lo, hi;
+  run_of(uid, B, i, lo, hi);
+  const int n = (int)(hi - lo);
+  T mean, ssq;
+  if (n <= 128) {
+    NpBlock<T> blk;
+    blk.begin(n);
+    if (n > 1)
+      for (int64_t j = lo; j < hi; ++j) blk.push(val[j]);
+    mean = blk.finish() / (T)n;
+    blk.begin(n);
+    if (n > 1)
+      for (int64_t j = lo; j < hi; ++j) {
+        const T d = val[j] - mean;
+        blk.push(d * d);
+      }
+    ssq = blk.finish();
+  } else {
+    MemberCursor<T> c1{uid, val, B, lo, my};
+    mean = np_pairwise<T, false>(c1, n, T(0)) / (T)n;
+    MemberCursor<T> c2{uid, val, B, lo, my};
+    ssq = np_pairwise<T, true>(c2, n, mean);
   }
+  const T sd = sqrt(ssq / (T)n);
+  keep[i] = (n == 1 || sd > T(0)) ? 1 : 0;
+  if (group_size) group_size[i] = n;
+}
+
+// The pending outputs of keep_mask_kernel: one wave per trajectory, members visited in batch order.
+template <typename T>
+__global__ __launch_bounds__(kWaveThreads) void keep_mask_wave_kernel(const T* __restrict__ val,
+                                                                       const int64_t* __restrict__ uid, int64_t B,
+                                                                       uint8_t* __restrict__ keep,
+                                                                       int32_t* __restrict__ group_size) {
+  __shared__ int64_t s_uid[kWaveTile];
+  const int64_t i = (int64_t)blockIdx.x * (kWaveThreads / kWave) + threadIdx.x / kWave;
+  const bool active = i < B && keep[i] == kPendingKeep;
+  if (!__syncthreads_or(active ? 1 : 0)) return;  // ordered uids: the first kernel has done everything
+  const int64_t my = active ? uid[i] : 0;
+  int n = 0;
+  wave_members(uid, B, my, active, s_uid, [&](int64_t) { ++n; });
   const bool small = n <= 128;
-  // mean
+  T mean = T(0), ssq = T(0);
   NpBlock<T> blk;
   blk.begin(small ? n : 0);
-  for (int64_t base = 0; base < B; base += kTile) {
-    const int lim = stage(base);
-    if (live && small && n > 1) for_members(s_uid, s_val, lim, my, [&](T v) { blk.push(v); });
+  if (__syncthreads_or((active && small && n > 1) ? 1 : 0)) {
+    wave_members(uid, B, my, active && small && n > 1, s_uid, [&](int64_t j) { blk.push(val[j]); });
+    mean = blk.finish() / (T)n;
+    blk.begin(small ? n : 0);
+    wave_members(uid, B, my, active && small && n > 1, s_uid, [&](int64_t j) {
+      const T d = val[j] - mean;
+      blk.push(d * d);
+    });
+    ssq = blk.finish();
   }
-  T mean = blk.finish() / (T)n;
-  // sum of squared deviations
-  blk.begin(small ? n : 0);
-  for (int64_t base = 0; base < B; base += kTile) {
-    const int lim = stage(base);
-    if (live && small && n > 1)
-      for_members(s_uid, s_val, lim, my, [&](T v) {
-        const T d = v - mean;
-        blk.push(d * d);
-      });
-  }
-  T ssq = blk.finish();
-  if (live && !small) {  // rare: groups of more than 128, numpy recurses
+  if (!active) return;
+  if (!small) {  // rare: groups of more than 128, numpy recurses; every lane walks the same members
     MemberCursor<T> c1{uid, val, B, 0, my};
     mean = np_pairwise<T, false>(c1, n, T(0)) / (T)n;
     MemberCursor<T> c2{uid, val, B, 0, my};
     ssq = np_pairwise<T, true>(c2, n, mean);
   }
-  if (!live) return;
   const T sd = sqrt(ssq / (T)n);
-  keep[i] = (n == 1 || sd > T(0)) ? 1 : 0;
-  if (group_size) group_size[i] = n;
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    keep[i] = (n == 1 || sd > T(0)) ? 1 : 0;
+    if (group_size) group_size[i] = n;
+  }
 }
 
 }  // namespace
@@ -368,6 +371,10 @@ extern "C" int siirl_grpo_outcome_advantage(const float* token_level_rewards, co
   grpo_group_kernel<<<dim3((unsigned)((B + kGroupThreads - 1) / kGroupThreads)), dim3(kGroupThreads), 0, st>>>(
       scores, uid, B, epsilon, norm_adv_by_std, a);
   SIIRL_LAUNCH_CHECK("grpo_group_kernel");
+  constexpr int kPerWg = kWaveThreads / kWave;
+  grpo_group_wave_kernel<<<dim3((unsigned)((B + kPerWg - 1) / kPerWg)), dim3(kWaveThreads), 0, st>>>(
+      scores, uid, B, epsilon, norm_adv_by_std, a);
+  SIIRL_LAUNCH_CHECK("grpo_group_wave_kernel");
   const int64_t n = B * L;
   const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads < 16384 ? (n + kThreads - 1) / kThreads : 16384);
   broadcast_mask_kernel<<<dim3(blocks), dim3(kThreads), 0, st>>>(a, mask, mask_dtype, B, L, advantages);
@@ -384,10 +391,17 @@ extern "C" int siirl_group_keep_mask(const void* metric, int metric_dtype, const
                 metric_dtype);
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid((unsigned)((B + kGroupThreads - 1) / kGroupThreads)), block(kGroupThreads);
-  if (metric_dtype == SIIRL_F32)
+  constexpr int kPerWg = kWaveThreads / kWave;
+  const dim3 wgrid((unsigned)((B + kPerWg - 1) / kPerWg)), wblock(kWaveThreads);
+  if (metric_dtype == SIIRL_F32) {
     keep_mask_kernel<float><<<grid, block, 0, st>>>((const float*)metric, uid, B, keep, group_size);
-  else
+    SIIRL_LAUNCH_CHECK("keep_mask_kernel");
+    keep_mask_wave_kernel<float><<<wgrid, wblock, 0, st>>>((const float*)metric, uid, B, keep, group_size);
+  } else {
     keep_mask_kernel<double><<<grid, block, 0, st>>>((const double*)metric, uid, B, keep, group_size);
-  SIIRL_LAUNCH_CHECK("keep_mask_kernel");
+    SIIRL_LAUNCH_CHECK("keep_mask_kernel");
+    keep_mask_wave_kernel<double><<<wgrid, wblock, 0, st>>>((const double*)metric, uid, B, keep, group_size);
+  }
+  SIIRL_LAUNCH_CHECK("keep_mask_wave_kernel");
   return SIIRL_OK;
 }

@@ -44,6 +44,18 @@ MEASURED_TRAFFIC_BYTES = int((4872295.36 * 2.0 + 9733447.5) * 1024)
 MEASURED_TRAFFIC_BYTES_CONFIG3 = int(((526927.5 + 527223.3) * 2.0 + 1372.0 + 176093.0) * 1024)
 
 
+def cpu_model() -> str:
+    """Model name of the host CPU the baseline leg runs on."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def make_workload(dev, seqs=SEQS, seq_len=SEQ_LEN, vocab=VOCAB, seed=SEED):
     import torch
 
@@ -85,7 +97,7 @@ def cpu_baseline(logits, labels, g_lp, g_ent, rows=4096, iters=5):
             times.append(dt)
     times.sort()
     med = times[len(times) // 2]
-    return {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+    return {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
             "sample": f"first {rows} of {logits.shape[0]} rows of the same tensor, upcast to fp32; "
                       f"median of {iters} fwd+bwd passes ({med:.2f} s each)"}
 
@@ -186,7 +198,7 @@ def bench_config3(args, dev):
             if it:
                 times.append(time.perf_counter() - t1)
         med = sorted(times)[len(times) // 2]
-        out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
                                "sample": f"first {n_s} kept trajectories (of {Bk}) x {L} tokens, filter over {2 * n_s} "
                                          f"trajectories; median of 3 passes ({med:.2f} s each)"}
     print(json.dumps(out), flush=True)
@@ -264,7 +276,7 @@ def bench_config5(args, dev):
             if it:
                 times.append(time.perf_counter() - t1)
         med = sorted(times)[len(times) // 2]
-        out["cpu_baseline"] = {"value": n_s / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        out["cpu_baseline"] = {"value": n_s / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
                                "sample": f"first {n_s} of {T} tokens against the full [{V}, {H}] weight in fp32; "
                                          f"median of 2 fwd+bwd passes ({med:.2f} s each)"}
     print(json.dumps(out), flush=True)
@@ -409,7 +421,7 @@ def bench_config1(args, dev):
             OA.micro_batch_step(x_c, y_c[rows], old_c[rows], adv_c[rows], m_c[rows], ocfg, ref_log_prob=ref_c[rows],
                                 loss_scale_factor=scale)
         el = time.perf_counter() - t1
-        out["cpu_baseline"] = {"value": n_mb * MB * L / el, "unit": "tokens/s", "cores": torch.get_num_threads(),
+        out["cpu_baseline"] = {"value": n_mb * MB * L / el, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(),
                                "kind": "port", "sample": f"advantages over all {B} trajectories + the first {n_mb} of "
                                                          f"{B // MB} micro-batches, one pass ({el:.1f} s)"}
     print(json.dumps(out), flush=True)
@@ -485,7 +497,7 @@ def bench_config4(args, dev):
             if it:
                 times.append(time.perf_counter() - t1)
         med = sorted(times)[len(times) // 2]
-        out["cpu_baseline"] = {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        out["cpu_baseline"] = {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
                                "sample": f"first {rows} of {L} tokens of the sequence, upcast to fp32; median of 2 "
                                          f"passes ({med:.2f} s each)"}
     print(json.dumps(out), flush=True)
@@ -599,7 +611,7 @@ def bench_critic(args, dev):
             if it:
                 times.append(time.perf_counter() - t1)
         med = sorted(times)[len(times) // 2]
-        out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(),
+        out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(),
                                "kind": "port", "sample": f"first {n_s} of {B} trajectories x {L} tokens; median of 2 "
                                                          f"passes ({med:.2f} s each)"}
     print(json.dumps(out), flush=True)
@@ -671,7 +683,7 @@ def bench_glue(args, dev):
             if it:
                 times.append(time.perf_counter() - t1)
         med = sorted(times)[len(times) // 2]
-        out["cpu_baseline"] = {"value": nnz / med, "unit": "tokens/s", "cores": 1, "kind": "port",
+        out["cpu_baseline"] = {"value": nnz / med, "unit": "tokens/s", "cores": 1, "cpu": cpu_model(), "kind": "port",
                                "sample": f"the whole batch, forward only, numpy; median of 3 passes ({med * 1e3:.1f} ms each)"}
     print(json.dumps(out), flush=True)
 

@@ -34,10 +34,10 @@ __global__ __launch_bounds__(kThreads) void row_sum_kernel(const float* __restri
   const float* r = x + b * L;
   double s = 0.0;
   if (L % 4 == 0 && ((uintptr_t)x & 15) == 0) {  // rows start 16-byte aligned
-    const float4* r4 = reinterpret_cast<const float4*>(r);
+    const u32x4* r4 = reinterpret_cast<const u32x4*>(r);
     for (int64_t t = threadIdx.x; t < L / 4; t += kThreads) {
-      const float4 v = r4[t];
-      s += ((double)v.x + (double)v.y) + ((double)v.z + (double)v.w);
+      const u32x4 v = __builtin_nontemporal_load(r4 + t);  // read once
+      s += ((double)u2f(v.x) + (double)u2f(v.y)) + ((double)u2f(v.z) + (double)u2f(v.w));
     }
   } else {
     for (int64_t t = threadIdx.x; t < L; t += kThreads) s += (double)r[t];

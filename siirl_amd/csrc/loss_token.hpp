@@ -8,6 +8,15 @@
 #pragma once
 #include "common.hpp"
 
+// Cache hints of the [B, L] streaming kernels.  Measured at [5488, 8192] fp32 with an int64 mask (actor loss forward +
+// backward): non-temporal loads 0.467 -> 0.428 ms, non-temporal stores of the gradient a further 0.428 -> 0.420 ms.
+#ifndef SIIRL_LOSS_NT_STORE
+#define SIIRL_LOSS_NT_STORE 1
+#endif
+#ifndef SIIRL_LOSS_NT_LOAD
+#define SIIRL_LOSS_NT_LOAD 1
+#endif
+
 namespace siirl {
 namespace tok {
 
@@ -53,8 +62,13 @@ struct Quad {
 __device__ __forceinline__ Quad load_quad(const float* __restrict__ p, int64_t idx, bool vec, int nv, float fill) {
   Quad q;
   if (vec) {
+#if SIIRL_LOSS_NT_LOAD
+    const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + idx));
+    q.v[0] = u2f(t.x); q.v[1] = u2f(t.y); q.v[2] = u2f(t.z); q.v[3] = u2f(t.w);
+#else
     const float4 t = *reinterpret_cast<const float4*>(p + idx);
     q.v[0] = t.x; q.v[1] = t.y; q.v[2] = t.z; q.v[3] = t.w;
+#endif
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? p[idx + e] : fill;
@@ -65,8 +79,16 @@ __device__ __forceinline__ Quad const_quad(float c) { return Quad{{c, c, c, c}};
 __device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t idx, bool vec, int nv) {
   Quad q;
   if (vec && dt == SIIRL_I64) {
+#if SIIRL_LOSS_NT_LOAD
+    const u32x4 ra = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const int64_t*)p + idx));
+    const u32x4 rb = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const int64_t*)p + idx) + 1);
+    longlong2 a, b;
+    a.x = (int64_t)(((uint64_t)ra.y << 32) | ra.x); a.y = (int64_t)(((uint64_t)ra.w << 32) | ra.z);
+    b.x = (int64_t)(((uint64_t)rb.y << 32) | rb.x); b.y = (int64_t)(((uint64_t)rb.w << 32) | rb.z);
+#else
     const longlong2 a = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[0];
     const longlong2 b = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[1];
+#endif
     // masks hold small integers: when every value in the wave fits 32 bits, one v_cvt_f32_i32 each replaces the
     // 64-bit conversion sequence (the wave-uniform test keeps the general path out of the way, not out of the code)
     const int32_t l0 = (int32_t)a.x, l1 = (int32_t)a.y, l2 = (int32_t)b.x, l3 = (int32_t)b.y;
@@ -90,7 +112,11 @@ __device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t id
 }
 __device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q) {
   if (vec) {
+#if SIIRL_LOSS_NT_STORE
+    __builtin_nontemporal_store(u32x4{f2u(q.v[0]), f2u(q.v[1]), f2u(q.v[2]), f2u(q.v[3])}, reinterpret_cast<u32x4*>(p + idx));
+#else
     *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
+#endif
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e)

@@ -18,6 +18,7 @@
 // scheme in the dtype of the values, so e.g. three equal fp64 values 0.1 have std 1.4e-17 > 0.  This
 // file is compiled with -ffp-contract=off so that (v - mean)^2 is rounded as numpy rounds it.
 #include "common.hpp"
+#include "loss_token.hpp"
 
 namespace siirl {
 namespace {
@@ -157,12 +158,24 @@ __global__ __launch_bounds__(kWaveThreads) void grpo_group_wave_kernel(const flo
   if ((threadIdx.x & (kWave - 1)) == 0) a_out[i] = grpo_value((double)scores[i], mean, sd, eps, norm_by_std);
 }
 
+// out[b, t] = a[b] * mask[b, t]; one workgroup per 4096-token segment of a row, four tokens per access
+constexpr int kBcastSeg = 4096;
 __global__ __launch_bounds__(kThreads) void broadcast_mask_kernel(const float* __restrict__ a, const void* mask,
-                                                                  int mask_dtype, int64_t B, int64_t L,
+                                                                  int mask_dtype, int64_t L, int nseg, int vec,
                                                                   float* __restrict__ out) {
-  const int64_t n = B * L;
-  for (int64_t idx = (int64_t)blockIdx.x * kThreads + threadIdx.x; idx < n; idx += (int64_t)gridDim.x * kThreads)
-    out[idx] = a[idx / L] * load_mask(mask, mask_dtype, idx);
+  const int64_t b = blockIdx.x / nseg;
+  const int64_t t0 = (int64_t)(blockIdx.x % nseg) * kBcastSeg;
+  const float ab = a[b];
+  for (int q = threadIdx.x; q < kBcastSeg / 4; q += kThreads) {
+    const int64_t t = t0 + 4 * q;
+    if (t >= L) break;
+    const int nv = (int)((L - t) < 4 ? (L - t) : 4);
+    const int64_t idx = b * L + t;
+    tok::Quad m4 = tok::load_mask_quad(mask, mask_dtype, idx, vec != 0, nv);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) m4.v[e] = ab * m4.v[e];
+    tok::store_quad(out, idx, vec != 0, nv, m4);
+  }
 }
 
 // ---------------------------------------------------------------------------- numpy pairwise sum
@@ -375,9 +388,13 @@ extern "C" int siirl_grpo_outcome_advantage(const float* token_level_rewards, co
   grpo_group_wave_kernel<<<dim3((unsigned)((B + kPerWg - 1) / kPerWg)), dim3(kWaveThreads), 0, st>>>(
       scores, uid, B, epsilon, norm_adv_by_std, a);
   SIIRL_LAUNCH_CHECK("grpo_group_wave_kernel");
-  const int64_t n = B * L;
-  const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads < 16384 ? (n + kThreads - 1) / kThreads : 16384);
-  broadcast_mask_kernel<<<dim3(blocks), dim3(kThreads), 0, st>>>(a, mask, mask_dtype, B, L, advantages);
+  const int64_t nseg = (L + kBcastSeg - 1) / kBcastSeg;
+  SIIRL_REQUIRE(B * nseg <= 0x7fffffffLL, "B=%lld x L=%lld exceeds the launch grid", (long long)B, (long long)L);
+  const size_t mask_es = dtype_size(mask_dtype);
+  const bool vec = L % 4 == 0 && ((uintptr_t)advantages & 15) == 0 &&
+                   ((uintptr_t)mask % (mask_es * 4 < 16 ? mask_es * 4 : 16)) == 0;
+  broadcast_mask_kernel<<<dim3((unsigned)(B * nseg)), dim3(kThreads), 0, st>>>(a, mask, mask_dtype, L, (int)nseg,
+                                                                              vec ? 1 : 0, advantages);
   SIIRL_LAUNCH_CHECK("broadcast_mask_kernel");
   return SIIRL_OK;
 }

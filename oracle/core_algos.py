@@ -126,6 +126,13 @@ def agg_loss(loss_mat, loss_mask, loss_agg_mode: str):
 # --------------------------------------------------------------------------- policy losses
 
 
+def compute_entropy_loss(logits, response_mask, loss_agg_mode: str = "token-mean"):
+    """``siirl/dag_worker/core_algos.py:1156-1170``: aggregated token entropy of ``logits [B, L, V]``."""
+    from .torch_functional import entropy_from_logits
+
+    return agg_loss(entropy_from_logits(logits), response_mask, loss_agg_mode)
+
+
 def _clip_bounds(config):
     lo = config.clip_ratio_low if config.clip_ratio_low is not None else config.clip_ratio
     hi = config.clip_ratio_high if config.clip_ratio_high is not None else config.clip_ratio

@@ -36,7 +36,7 @@ __all__ = [
     "AdaptiveKLController", "FixedKLController", "get_kl_controller", "compute_response_mask",
     "compute_gae_advantage_return", "compute_grpo_outcome_advantage", "compute_rewards", "agg_loss",
     "compute_policy_loss", "compute_policy_loss_vanilla", "compute_policy_loss_gspo", "compute_policy_loss_cpgd",
-    "compute_policy_loss_gpg", "compute_policy_loss_geo_mean", "compute_value_loss", "kl_penalty",
+    "compute_policy_loss_gpg", "compute_policy_loss_geo_mean", "compute_entropy_loss", "compute_value_loss", "kl_penalty",
     "kl_penalty_forward",
     "apply_kl_penalty", "compute_advantage", "actor_loss", "ActorLossOutput", "fused_actor_step",
     "FusedActorStepOutput", "agg_weights",
@@ -403,6 +403,13 @@ def agg_loss(loss_mat: torch.Tensor, loss_mask: torch.Tensor, loss_agg_mode: str
     code = _agg_code(loss_agg_mode)
     _gpu_of(loss_mat)
     return _AggLoss.apply(loss_mat, loss_mask, code)
+
+
+def compute_entropy_loss(logits: torch.Tensor, response_mask: torch.Tensor, loss_agg_mode: str = "token-mean"):
+    """Aggregated categorical entropy of ``logits [B, L, V]`` (reference ``core_algos.py:1156-1170``, kept there
+    for backward compatibility): ``agg_loss(entropy_from_logits(logits), response_mask, loss_agg_mode)``."""
+    return agg_loss(loss_mat=siirl_F.entropy_from_logits(logits), loss_mask=response_mask,
+                    loss_agg_mode=loss_agg_mode)
 
 
 # ------------------------------------------------------------------------------------ policy loss

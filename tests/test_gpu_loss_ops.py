@@ -384,3 +384,23 @@ def test_empty_batch_matches_reference_semantics(dev):
     assert float(loss) == 0.0 and float(clipfrac) == 0.0
     loss.backward()
     assert v.grad.shape == (0, L)
+
+
+@pytest.mark.parametrize("mode", AGGS)
+def test_compute_entropy_loss(dev, mode):
+    """reference ``core_algos.py:1156-1170``: aggregated token entropy, forward and gradient to the logits."""
+    import siirl_amd.core_algos as CA
+
+    g = torch.Generator().manual_seed(11)
+    B, L, V = 3, 9, 257
+    x = torch.randn(B, L, V, generator=g) * 2
+    m = (torch.rand(B, L, generator=g) > 0.3).long()
+    m[:, 0] = 1
+    xd = x.to(dev).requires_grad_(True)
+    got = CA.compute_entropy_loss(xd, m.to(dev), mode)
+    x64 = x.double().requires_grad_(True)
+    want = OC.compute_entropy_loss(x64, m, mode)
+    assert abs(float(got) - float(want)) < 1e-5
+    got.backward()
+    want.backward()
+    assert (xd.grad.cpu().double() - x64.grad).abs().max() < 1e-6

@@ -335,6 +335,17 @@ int siirl_response_scatter(const float* values, const int64_t* indices, int64_t 
 int siirl_response_gather(const float* grad, const int64_t* indices, int64_t nnz, int64_t B, int64_t S, int64_t L,
                           float* d_values, siirl_stream_t stream);
 
+/*
+ * Response mask from the generated ids [B, L] (int64 or int32): mask[b, t] = 1 while no end-of-sequence token
+ * occurs strictly before position t of row b (the first such token is still attended), 0 from the next position on.
+ * eos_tokens is a HOST array of n_eos <= SIIRL_MAX_EOS_TOKENS ids (n_eos = 0: all ones); mask takes any mask dtype.
+ * Replaces: get_response_mask / get_eos_mask, siirl/utils/model_utils/torch_functional.py:209-254
+ *           ((cumsum(eos) - eos) == 0 along the row).
+ */
+#define SIIRL_MAX_EOS_TOKENS 16
+int siirl_eos_response_mask(const void* response_id, int id_dtype, int64_t B, int64_t L, const int64_t* eos_tokens,
+                            int n_eos, void* mask, int mask_dtype, siirl_stream_t stream);
+
 /* ------------------------------------------------------------------- outcome reward placement */
 
 /*

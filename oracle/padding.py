@@ -46,3 +46,29 @@ def pad_and_slice_response(values_rmpad: np.ndarray, indices: np.ndarray, batch:
     ``dp_actor.py:214-231``)."""
     full = pad_input(values_rmpad[:, None], indices, batch, seqlen)[..., 0]
     return full[:, -response_length - 1:-1]
+
+
+def get_response_mask(response_id: np.ndarray, eos_token=2, dtype=np.int64):
+    """1 up to and including the first end-of-sequence token of each row, 0 after (reference
+    ``siirl/utils/model_utils/torch_functional.py:209-229``, which writes it as ``(cumsum(isin) - isin) == 0``;
+    ``get_eos_mask`` at ``:232-254`` is the single-token case).  Pinned by the two worked examples of the
+    reference's docstring (``tests/test_oracle_padding.py``)."""
+    eos = set(np.atleast_1d(np.asarray(eos_token)).tolist())
+    out = np.zeros(response_id.shape, dtype=dtype)
+    for b, row in enumerate(response_id.tolist()):
+        for t, tok in enumerate(row):
+            out[b, t] = 1
+            if tok in eos:
+                break
+    return out
+
+
+def get_unpad_data(attention_mask: np.ndarray):
+    """``(indices, cu_seqlens, max_seqlen_in_batch)`` (reference ``torch_functional.py:638-647``)."""
+    _, indices, cu, max_seqlen, _ = unpad_input(attention_mask[..., None], attention_mask)
+    return indices, cu, max_seqlen
+
+
+def remove_pad_token(input_ids: np.ndarray, attention_mask: np.ndarray):
+    """Per-row lists of the last ``mask.sum()`` ids (reference ``torch_functional.py:416-428``)."""
+    return [row[len(row) - int(m.sum()):].tolist() for row, m in zip(input_ids, attention_mask)]

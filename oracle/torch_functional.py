@@ -151,3 +151,29 @@ def masked_whiten(values, mask, shift_mean=True):
     if not shift_mean:
         out = out + mean
     return out
+
+
+# ---------------------------------------------------------------- response-window glue (reference :431-500)
+
+
+def log_probs_from_logits_response(input_ids, logits, response_length, *, dtype=None):
+    """reference ``torch_functional.py:431-444``: logits of positions ``-L-1 .. -2`` score ids ``-L .. -1``."""
+    return logprobs_from_logits(logits[:, -response_length - 1:-1], input_ids[:, -response_length:], dtype=dtype)
+
+
+def log_probs_from_logits_all_rmpad(input_ids_rmpad, logits_rmpad, indices, batch_size, seqlen, response_length, *,
+                                    dtype=None):
+    """reference ``torch_functional.py:474-500``; ``pad_input`` is flash-attn's zero-filled scatter."""
+    ids = input_ids_rmpad.reshape(-1)
+    lp = logprobs_from_logits(logits_rmpad, torch.roll(ids, shifts=-1, dims=0), dtype=dtype)
+    full = torch.zeros(batch_size * seqlen, dtype=lp.dtype).index_put((indices,), lp).reshape(batch_size, seqlen)
+    return full[:, -response_length - 1:-1]
+
+
+def log_probs_from_logits_response_rmpad(input_ids, attention_mask, logits_rmpad, response_length, *, dtype=None):
+    """reference ``torch_functional.py:447-471``."""
+    batch_size, seqlen = input_ids.shape
+    indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+    ids_rmpad = input_ids.flatten()[indices]
+    return log_probs_from_logits_all_rmpad(ids_rmpad[None], logits_rmpad, indices, batch_size, seqlen,
+                                           response_length, dtype=dtype)

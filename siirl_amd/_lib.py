@@ -12,6 +12,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsiirl_hip.so"
 
 # dtype codes of siirl_dtype
 F32, BF16, F16, F64, I64, I32, U8 = range(7)
+MAX_EOS_TOKENS = 16  # SIIRL_MAX_EOS_TOKENS
 BWD_SKIP_ZERO_ROWS = 1
 
 _p, _i64, _i32, _f32, _u32, _sz, _f64 = (C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint32, C.c_size_t,
@@ -42,6 +43,7 @@ SIGNATURES = {
     "siirl_unpad_ids_labels": (_i32, [_p, _i64, _p, _i64, _p, _p, _p]),
     "siirl_response_scatter": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p]),
     "siirl_response_gather": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p]),
+    "siirl_eos_response_mask": (_i32, [_p, _i32, _i64, _i64, _p, _i32, _p, _i32, _p]),
     "siirl_place_outcome_reward": (_i32, [_p, _p, _i32, _i64, _i64, _i64, _i32, _f64, _f64, _f64, _p, _p, _p, _p]),
     "siirl_data_metrics_workspace_bytes": (_sz, [_i64, _i64]),
     "siirl_data_metrics": (_i32, [_p, _p, _p, _p, _p, _p, _i32, _p, _i32, _i64, _i64, _i64, _p, _p, _sz, _p]),

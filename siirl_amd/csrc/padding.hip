@@ -153,6 +153,47 @@ __global__ __launch_bounds__(kThreads) void response_gather_kernel(const float* 
   }
 }
 
+// Response mask from generated ids: 1 up to and including the first end-of-sequence token of the row, 0 after it
+// (siirl/utils/model_utils/torch_functional.py:209-254).  One wave per row walks the row 64 ids at a time; a ballot
+// finds the first hit of the chunk.  Every wave of the launch leaves its loop after ceil(L / 64) steps.
+struct EosSet {
+  int64_t tok[SIIRL_MAX_EOS_TOKENS];
+  int n;
+};
+
+__device__ __forceinline__ void store_mask(void* p, int dt, int64_t i, bool on) {
+  switch (dt) {
+    case SIIRL_U8: ((uint8_t*)p)[i] = on ? 1 : 0; break;
+    case SIIRL_I64: ((int64_t*)p)[i] = on ? 1 : 0; break;
+    case SIIRL_I32: ((int32_t*)p)[i] = on ? 1 : 0; break;
+    case SIIRL_F32: ((float*)p)[i] = on ? 1.f : 0.f; break;
+    case SIIRL_BF16: ((uint16_t*)p)[i] = on ? 0x3f80u : 0u; break;
+    case SIIRL_F16: ((uint16_t*)p)[i] = on ? 0x3c00u : 0u; break;
+    default: break;
+  }
+}
+
+__global__ __launch_bounds__(kThreads) void eos_mask_kernel(const void* __restrict__ ids, int id_dtype, int64_t B,
+                                                            int64_t L, EosSet eos, void* __restrict__ mask,
+                                                            int mask_dtype) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t b = (int64_t)blockIdx.x * (kThreads / kWave) + (threadIdx.x / kWave);
+  if (b >= B) return;
+  bool ended = false;  // wave-uniform: an end-of-sequence token lies in an earlier chunk
+  for (int64_t t0 = 0; t0 < L; t0 += kWave) {
+    const int64_t t = t0 + lane;
+    bool hit = false;
+    if (t < L && !ended) {
+      const int64_t id = id_dtype == SIIRL_I64 ? ((const int64_t*)ids)[b * L + t] : (int64_t)((const int32_t*)ids)[b * L + t];
+      for (int k = 0; k < eos.n; ++k) hit |= id == eos.tok[k];
+    }
+    const unsigned long long hits = __builtin_amdgcn_ballot_w64(hit);
+    const int first = hits ? __builtin_ctzll(hits) : kWave;
+    if (t < L) store_mask(mask, mask_dtype, b * L + t, !ended && lane <= first);
+    ended |= hits != 0;
+  }
+}
+
 unsigned blocks_for(int64_t n) {
   const int64_t b = (n + kThreads - 1) / kThreads;
   return (unsigned)(b < 1 ? 1 : (b > 16384 ? 16384 : b));
@@ -251,5 +292,24 @@ extern "C" int siirl_response_gather(const float* grad, const int64_t* indices, 
   response_gather_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(grad, indices, nnz, B, S, L,
                                                                                            d_values);
   SIIRL_LAUNCH_CHECK("response_gather_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_eos_response_mask(const void* response_id, int id_dtype, int64_t B, int64_t L,
+                                       const int64_t* eos_tokens, int n_eos, void* mask, int mask_dtype,
+                                       siirl_stream_t stream) {
+  SIIRL_REQUIRE(B >= 0 && L >= 0 && B <= 0x7fffffffLL, "B=%lld L=%lld out of range", (long long)B, (long long)L);
+  SIIRL_REQUIRE(id_dtype == SIIRL_I64 || id_dtype == SIIRL_I32, "response_id dtype %d must be int64 or int32", id_dtype);
+  SIIRL_REQUIRE(n_eos >= 0 && n_eos <= SIIRL_MAX_EOS_TOKENS, "n_eos=%d must be in [0, %d]", n_eos, SIIRL_MAX_EOS_TOKENS);
+  if (int rc = check_mask(mask_dtype)) return rc;
+  if (B == 0 || L == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(response_id && mask && (n_eos == 0 || eos_tokens), "NULL operand");
+  EosSet eos;
+  eos.n = n_eos;
+  for (int k = 0; k < SIIRL_MAX_EOS_TOKENS; ++k) eos.tok[k] = k < n_eos ? eos_tokens[k] : 0;
+  constexpr int rows_per_wg = kThreads / kWave;
+  eos_mask_kernel<<<dim3((unsigned)((B + rows_per_wg - 1) / rows_per_wg)), dim3(kThreads), 0, (hipStream_t)stream>>>(
+      response_id, id_dtype, B, L, eos, mask, mask_dtype);
+  SIIRL_LAUNCH_CHECK("eos_mask_kernel");
   return SIIRL_OK;
 }

@@ -88,6 +88,12 @@ def test_argument_validation_without_gpu():
     assert h.siirl_loss_workspace_bytes(2, 4) > 0 and h.siirl_loss_workspace_bytes(0, 4) == 0
     assert h.siirl_kl_penalty_fwd(p, p, 4, 7, p, None) == -1
     assert h.siirl_group_keep_mask(p, L.BF16, p, 4, p, None, None) == -1
+    eos = (ctypes.c_int64 * 17)()
+    assert h.siirl_eos_response_mask(p, L.F32, 2, 4, eos, 1, p, L.I64, None) == -1  # ids must be integers
+    assert h.siirl_eos_response_mask(p, L.I64, 2, 4, eos, 17, p, L.I64, None) == -1
+    assert b"n_eos" in h.siirl_hip_last_error()
+    assert h.siirl_eos_response_mask(p, L.I64, 2, 4, eos, 1, p, L.F64, None) == -1
+    assert h.siirl_eos_response_mask(p, L.I64, 0, 4, eos, 1, p, L.I64, None) == 0  # nothing to do, no launch
     with pytest.raises(ValueError):
         L.check(-1, "x")
     with pytest.raises(NotImplementedError):

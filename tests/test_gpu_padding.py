@@ -121,3 +121,99 @@ def test_indices_outside_the_tensor_touch_no_memory(dev):
     assert torch.equal(w.detach().cpu(), torch.tensor([[1., 2., 0.], [0., 5., 0.]]))
     w.sum().backward()
     assert torch.equal(vals.grad.cpu(), torch.tensor([1., 1., 0., 0., 1., 0.]))
+
+
+@pytest.mark.parametrize("B,L", [(4, 7), (1, 1), (33, 64), (17, 65), (300, 1000), (2, 70001)])
+@pytest.mark.parametrize("idt", [torch.int64, torch.int32])
+def test_response_mask_from_eos(dev, B, L, idt):
+    import siirl_amd.torch_functional as TF
+
+    rng = np.random.default_rng(B * 31 + L)
+    ids = rng.integers(0, max(L // 3, 4), (B, L)).astype(np.int64)
+    ids[0, :] = 3  # a row with no end-of-sequence token
+    x = torch.from_numpy(ids).to(dev).to(idt)
+    for eos in (1, [1, 2], [0, 2, 1, 7, 9]):
+        want = OP.get_response_mask(ids, eos)
+        got = TF.get_response_mask(x, eos)
+        assert got.dtype == torch.int64 and np.array_equal(got.cpu().numpy(), want), (B, L, eos)
+    assert np.array_equal(TF.get_eos_mask(x, 2).cpu().numpy(), OP.get_response_mask(ids, 2))
+    want = OP.get_response_mask(ids, 1)
+    for dt in (torch.bool, torch.int32, torch.float32, torch.bfloat16, torch.float16, torch.uint8):
+        got = TF.get_response_mask(x, 1, dtype=dt)
+        assert got.dtype == dt and np.array_equal(got.float().cpu().numpy(), want.astype(np.float32))
+
+
+def test_response_mask_docstring_examples_and_errors(dev):
+    import siirl_amd.torch_functional as TF
+
+    ids = torch.tensor([[20, 10, 34, 1, 0, 0, 0], [78, 0, 76, 2, 1, 0, 0], [23, 98, 1, 0, 0, 0, 0],
+                        [33, 3, 98, 45, 1, 0, 0]], device=dev)
+    assert TF.get_response_mask(ids, 1).tolist() == [[1, 1, 1, 1, 0, 0, 0], [1, 1, 1, 1, 1, 0, 0], [1, 1, 1, 0, 0, 0, 0],
+                                                     [1, 1, 1, 1, 1, 0, 0]]
+    assert TF.get_response_mask(ids, [1, 2]).tolist() == [[1, 1, 1, 1, 0, 0, 0], [1, 1, 1, 1, 0, 0, 0],
+                                                          [1, 1, 1, 0, 0, 0, 0], [1, 1, 1, 1, 1, 0, 0]]
+    assert TF.get_response_mask(ids[:0], 1).shape == (0, 7)
+    with pytest.raises(ValueError):
+        TF.get_response_mask(ids, list(range(17)))
+    with pytest.raises(RuntimeError):
+        TF.get_response_mask(ids.cpu(), 1)
+    with pytest.raises(TypeError):
+        TF.get_response_mask(ids.float(), 1)
+
+
+def test_unpad_data_and_remove_pad_token(dev):
+    import siirl_amd.torch_functional as TF
+
+    ids, mask = _case(9, 130, 4)
+    # left-padded rows, as remove_pad_token expects
+    for b in range(9):
+        n = int(mask[b].sum())
+        mask[b] = 0
+        mask[b, 130 - n:] = 1
+    idx_o, cu_o, mx_o = OP.get_unpad_data(mask)
+    idx, cu, mx = TF.get_unpad_data(torch.from_numpy(mask).to(dev))
+    assert np.array_equal(idx.cpu().numpy(), idx_o) and np.array_equal(cu.cpu().numpy(), cu_o) and mx == mx_o
+    assert TF.remove_pad_token(torch.from_numpy(ids).to(dev), torch.from_numpy(mask).to(dev)) == \
+        OP.remove_pad_token(ids, mask)
+
+
+@pytest.mark.parametrize("B,S,L,V,dt", [(3, 12, 4, 29, torch.float32), (4, 300, 128, 1531, torch.bfloat16),
+                                        (2, 40, 39, 4096, torch.float16)])
+def test_response_logprobs_padded_and_packed(dev, B, S, L, V, dt):
+    """log_probs_from_logits_response / _response_rmpad / _all_rmpad against the oracle (1e-3 absolute, the
+    log-prob tolerance), values and the gradient with respect to the logits."""
+    import siirl_amd.torch_functional as TF
+    from oracle import torch_functional as OT
+
+    g = torch.Generator().manual_seed(B * S + L)
+    logits = (torch.randn(B, S, V, generator=g) * 2).to(dt)
+    ids = torch.randint(0, V, (B, S), generator=g)
+    mask = torch.ones(B, S, dtype=torch.int64)
+    mask[0, :S // 3] = 0
+    mask[B - 1, :1] = 0
+    w = torch.randn(B, L, generator=g)
+
+    lo = logits.float().clone().requires_grad_(True)
+    want = OT.log_probs_from_logits_response(ids, lo, L)
+    (want * w).sum().backward()
+    x = logits.detach().to(dev).requires_grad_(True)
+    got = TF.log_probs_from_logits_response(ids.to(dev), x, L)
+    assert got.shape == (B, L) and (got.detach().cpu() - want.detach()).abs().max() < 1e-3
+    (got * w.to(dev)).sum().backward()
+    assert (x.grad.float().cpu() - lo.grad).abs().max() < (1e-5 if dt == torch.float32 else 1e-2)
+
+    idx = torch.nonzero(mask.flatten()).flatten()
+    packed = logits.reshape(B * S, V)[idx]
+    po = packed.float().clone().requires_grad_(True)
+    want = OT.log_probs_from_logits_response_rmpad(ids, mask, po, L)
+    (want * w).sum().backward()
+    for route in ("response_rmpad", "all_rmpad"):
+        p = packed.detach().to(dev).requires_grad_(True)
+        if route == "response_rmpad":
+            got = TF.log_probs_from_logits_response_rmpad(ids.to(dev), mask.to(dev), p, L)
+        else:
+            got = TF.log_probs_from_logits_all_rmpad(ids.flatten()[idx][None].to(dev), p, idx.to(dev), B, S, L)
+        assert got.shape == (B, L) and (got.detach().cpu() - want.detach()).abs().max() < 1e-3, route
+        (got * w.to(dev)).sum().backward()
+        # logprobs_from_logits defaults to the in-place backward: the gradient comes back in the logits' storage
+        assert (p.grad.float().cpu() - po.grad).abs().max() < (1e-5 if dt == torch.float32 else 1e-2), route

@@ -52,3 +52,52 @@ def test_round_trip_and_window(B, S, L):
     rm, idx, *_ = OP.unpad_input(v[..., None], mask)
     assert np.array_equal(OP.pad_input(rm, idx, B, S)[..., 0], v * mask)
     assert np.array_equal(OP.pad_and_slice_response(rm[:, 0], idx, B, S, L), (v * mask)[:, S - L - 1:S - 1])
+
+
+def test_response_mask_docstring_examples_of_the_reference():
+    """The two worked examples in the docstring of get_response_mask and the one of get_eos_mask
+    (reference siirl/utils/model_utils/torch_functional.py:212-226, 236-238)."""
+    ids = np.array([[20, 10, 34, 1, 0, 0, 0], [78, 0, 76, 2, 1, 0, 0], [23, 98, 1, 0, 0, 0, 0], [33, 3, 98, 45, 1, 0, 0]])
+    assert OP.get_response_mask(ids, 1).tolist() == [[1, 1, 1, 1, 0, 0, 0], [1, 1, 1, 1, 1, 0, 0], [1, 1, 1, 0, 0, 0, 0],
+                                                     [1, 1, 1, 1, 1, 0, 0]]
+    assert OP.get_response_mask(ids, [1, 2]).tolist() == [[1, 1, 1, 1, 0, 0, 0], [1, 1, 1, 1, 0, 0, 0],
+                                                          [1, 1, 1, 0, 0, 0, 0], [1, 1, 1, 1, 1, 0, 0]]
+    assert OP.get_response_mask(np.array([[0, 0, 2, 42, 3, 5, 1, 0, 0]]), 1).tolist() == [[1, 1, 1, 1, 1, 1, 1, 0, 0]]
+    # the closed form the reference uses, on random rows
+    rng = np.random.default_rng(0)
+    ids = rng.integers(0, 6, (50, 33))
+    isin = np.isin(ids, [2, 5]).astype(np.int64)
+    assert np.array_equal(OP.get_response_mask(ids, [2, 5]), ((np.cumsum(isin, axis=1) - isin) == 0).astype(np.int64))
+    assert OP.get_response_mask(ids, 77).all()
+
+
+def test_unpad_data_and_remove_pad_token():
+    mask = np.array([[0, 1, 1, 1], [0, 0, 0, 1], [1, 1, 1, 1]])
+    idx, cu, mx = OP.get_unpad_data(mask)
+    assert idx.tolist() == [1, 2, 3, 7, 8, 9, 10, 11] and cu.tolist() == [0, 3, 4, 8] and mx == 4
+    ids = np.arange(12).reshape(3, 4)
+    assert OP.remove_pad_token(ids, mask) == [[1, 2, 3], [7], [8, 9, 10, 11]]
+
+
+def test_rmpad_response_logprobs_equal_the_padded_form():
+    """Where the response window and the position before it are attended, the packed route gives the padded
+    route's numbers: row j of the packed logits is position indices[j] of the padded ones."""
+    from oracle import torch_functional as OT
+
+    B, S, L, V = 3, 12, 4, 29
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(B, S, V, generator=g)
+    ids = torch.randint(0, V, (B, S), generator=g)
+    mask = torch.ones(B, S, dtype=torch.int64)
+    mask[0, :5] = 0
+    mask[2, :2] = 0
+    want = OT.log_probs_from_logits_response(ids, logits, L)
+    idx = torch.nonzero(mask.flatten()).flatten()
+    packed = logits.reshape(B * S, V)[idx]
+    got = OT.log_probs_from_logits_response_rmpad(ids, mask, packed, L)
+    assert got.shape == (B, L) and torch.allclose(got, want, atol=1e-6)
+    got2 = OT.log_probs_from_logits_all_rmpad(ids.flatten()[idx][None], packed, idx, B, S, L)
+    assert torch.equal(got, got2)
+    # and the padded form is the textbook log-softmax pick
+    ref = torch.log_softmax(logits[:, S - L - 1:S - 1], -1).gather(-1, ids[:, S - L:, None])[..., 0]
+    assert torch.allclose(want, ref, atol=1e-6)

@@ -234,18 +234,29 @@ def bench_config5(args, dev):
             ev[2].record()
         h.grad = w.grad = None
 
+    import siirl_amd.fused_linear as FL
+
     steps, warm = min(args.steps, 10), min(args.warmup, 2)
-    for _ in range(warm):
-        step()
-    torch.cuda.synchronize()
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
-    t0 = time.perf_counter()
-    for k in range(steps):
-        step(evs[k])
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
+
+    def timed():
+        for _ in range(warm):
+            step()
+        torch.cuda.synchronize()
+        evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+        t0 = time.perf_counter()
+        for k in range(steps):
+            step(evs[k])
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        return (wall, sum(e[0].elapsed_time(e[1]) for e in evs) / steps,
+                sum(e[1].elapsed_time(e[2]) for e in evs) / steps)
+
+    # the memory-lean route first (no logits kept, the backward recomputes them), then the default
+    FL.set_saved_logits_limit(0)
+    r_wall, r_fwd_ms, r_bwd_ms = timed()
+    FL.set_saved_logits_limit(16 << 30)
+    wall, fwd_ms, bwd_ms = timed()
+    saved_gb = FL._saved_logits_bytes(T, V) / 1e9
     gemm = 2.0 * T * H * V
     tf_step = 3 * gemm / (wall / steps) / 1e12
     out = {
@@ -255,11 +266,17 @@ def bench_config5(args, dev):
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"config5: fused lm_head + logprob/entropy, hidden [{T}, {H}], W [{V}, {H}], fwd + bwd to "
                                "hidden and W", "tokens": T, "hidden": H, "vocab": V, "seed": SEED},
-        "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
-                    "backward (recompute + dlogits per 8192-column slab; d hidden and d weight per four slabs)": {"ms": bwd_ms, "TFLOP/s executed": 3 * gemm / bwd_ms / 1e9}},
+        "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> parking its fp32 tiles + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
+                    "backward (dlogits from the parked tiles, d hidden and d weight per 32768 columns)": {"ms": bwd_ms, "TFLOP/s executed": 2 * gemm / bwd_ms / 1e9}},
+        "saved_logits_GB": saved_gb,
+        "recompute_variant": {"what": "set_saved_logits_limit(0): nothing kept between forward and backward, the "
+                                      "backward recomputes the logits per 8192-column slab",
+                              "ms_per_step": r_wall * 1e3 / steps, "tokens_per_s": T * steps / r_wall,
+                              "forward_ms": r_fwd_ms, "backward_ms": r_bwd_ms,
+                              "algorithmic_TFLOP/s": 3 * gemm / (r_wall / steps) / 1e12},
         "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel", "achieved": tf_step, "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": tf_step / 2500.0, "traffic": None,
-                     "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step; the backward's recompute is not counted"},
+                     "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step (forward, d hidden, d weight)"},
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:  # the oracle's chunked fp32 matmul + log-softmax on the host cores, 256 tokens

@@ -462,11 +462,16 @@ int siirl_group_keep_mask(const void* metric, int metric_dtype, const int64_t* u
 /* Bytes of scratch for the two entry points below. */
 size_t siirl_fused_linear_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 size_t siirl_fused_linear_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int want_d_hidden, int want_d_weight);
+/* Bytes of the optional saved_logits buffer of the two entry points below: 4 bytes per logit, whole 256 x 256 tiles. */
+size_t siirl_fused_linear_saved_logits_bytes(int64_t T, int64_t V);
 
 /*
  * Forward: z = (hidden[T, H] . weight[V, H]^T) * inv_temperature is formed tile by tile on the matrix cores
- * (bf16 operands, fp32 accumulation) and reduced in the epilogue; the [T, V] logits are never stored.
+ * (bf16 operands, fp32 accumulation) and reduced in the epilogue; no [T, V] tensor is needed.
  * Outputs as siirl_logprob_entropy_fwd: logprob[T] (with labels), entropy[T], lse[T], ex[T], all fp32.
+ * saved_logits (may be NULL): siirl_fused_linear_saved_logits_bytes(T, V) bytes, 16-byte aligned, into which the
+ * fp32 accumulator tiles are parked in the kernel's own lane order for the backward; an opaque buffer, trading
+ * memory for the backward's recomputation.
  * dtype must be SIIRL_BF16; H a multiple of 64; hidden and weight row-major, contiguous, 16-byte aligned;
  * workspace 256-byte aligned.
  * Replaces: FusedLinearForPPO.forward  siirl/utils/experimental/torch_functional.py:20-32,70-133
@@ -475,24 +480,25 @@ size_t siirl_fused_linear_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, i
  */
 int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype, const int64_t* labels,
                                            int64_t T, int64_t H, int64_t V, float inv_temperature, float* logprob,
-                                           float* entropy, float* lse, float* ex, void* workspace,
+                                           float* entropy, float* lse, float* ex, float* saved_logits, void* workspace,
                                            size_t workspace_bytes, siirl_stream_t stream);
 
 /*
  * Backward: for upstream gradients g_logprob[T] / g_entropy[T] (either may be NULL) writes
  * d_hidden[T, H] and / or d_weight[V, H] in bf16 (either may be NULL).  The vocabulary is walked in slabs of
- * 8192 columns: the slab's logits are recomputed, dlogits = inv_T * (g_lp (onehot - p) - g_H p (z - ex)) is
- * written to scratch in both layouts, then d_hidden += dlogits . W_slab (fp32 accumulation across slabs,
- * rounded once) and d_weight_slab = dlogits^T . hidden.
+ * 8192 columns: the slab's logits are recomputed -- or, when saved_logits holds what the forward call with the
+ * same hidden, weight and inv_temperature parked there, read back --, dlogits = inv_T * (g_lp (onehot - p)
+ * - g_H p (z - ex)) is written to scratch in both layouts, then d_hidden += dlogits . W_slab (fp32 accumulation
+ * across slabs, rounded once) and d_weight_slab = dlogits^T . hidden.  Both routes give the same bits.
  * Replaces: FusedLinearForPPO.backward siirl/utils/experimental/torch_functional.py:35-67,135-188
  *           linear_cross_entropy bwd   siirl/utils/kernel/kernels.py:1378-1586 (the split-N d_logits strategy
  *                                      :1263-1375,1523-1581)
  */
 int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const void* weight, int dtype, const int64_t* labels,
                                            int64_t T, int64_t H, int64_t V, float inv_temperature, const float* lse,
-                                           const float* ex, const float* g_logprob, const float* g_entropy,
-                                           void* d_hidden, void* d_weight, void* workspace, size_t workspace_bytes,
-                                           siirl_stream_t stream);
+                                           const float* ex, const float* saved_logits, const float* g_logprob,
+                                           const float* g_entropy, void* d_hidden, void* d_weight, void* workspace,
+                                           size_t workspace_bytes, siirl_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -59,10 +59,11 @@ SIGNATURES = {
     "siirl_group_keep_mask": (_i32, [_p, _i32, _p, _i64, _p, _p, _p]),
     "siirl_fused_linear_fwd_workspace_bytes": (_sz, [_i64, _i64, _i64]),
     "siirl_fused_linear_bwd_workspace_bytes": (_sz, [_i64, _i64, _i64, _i32, _i32]),
-    "siirl_fused_linear_logprob_entropy_fwd": (_i32, [_p, _p, _i32, _p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _p, _sz,
-                                                      _p]),
+    "siirl_fused_linear_saved_logits_bytes": (_sz, [_i64, _i64]),
+    "siirl_fused_linear_logprob_entropy_fwd": (_i32, [_p, _p, _i32, _p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _p, _p,
+                                                      _sz, _p]),
     "siirl_fused_linear_logprob_entropy_bwd": (_i32, [_p, _p, _i32, _p, _i64, _i64, _i64, _f32, _p, _p, _p, _p, _p, _p,
-                                                      _p, _sz, _p]),
+                                                      _p, _p, _sz, _p]),
 }
 
 _lock = threading.Lock()

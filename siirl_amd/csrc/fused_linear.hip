@@ -20,6 +20,10 @@
 // bf16 store (d weight).  The backward walks the vocabulary in slabs: recompute the slab's logits, write
 // dlogits[T, slab] and its transpose, then dH += dlogits . W_slab and dW_slab = dlogits^T . hidden as two more
 // runs of the same core against packed transposed copies of W and hidden.
+// Optionally the forward also parks the fp32 accumulator tiles in memory (4 bytes per logit, in the accumulator's
+// own lane order, so stores and loads are whole 1 KB wave accesses); the backward then replays the tiles through
+// the same dlogits epilogue instead of recomputing the GEMM: a third of the backward's matrix work is traded for
+// one streaming pass.
 #include "common.hpp"
 
 namespace siirl {
@@ -54,6 +58,7 @@ constexpr int kDmaPerWave = kTileBytes / 1024 / (kThreads / 64);  // 1 KB per wa
 #define SIIRL_SLAB 8192
 #endif
 constexpr int kSlab = SIIRL_SLAB;                   // vocabulary columns per backward slab
+static_assert(kSlab % 256 == 0, "a slab is a whole number of workgroup tiles");
 #ifndef SIIRL_DH_GROUP
 #define SIIRL_DH_GROUP 4
 #endif
@@ -247,6 +252,46 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
 }
 #pragma clang diagnostic pop
 
+// ------------------------------------------------------------------------------ parked accumulator tiles
+
+// Tile (tm, tn) of the forward GEMM occupies kQuads * kThreads 16-byte slots; slot c * kThreads + tid holds
+// elements 4q .. 4q + 3 of thread tid's acc[i][j], c = (i * NJ + j) * 4 + q.  A wave instruction therefore moves
+// one contiguous KB, and the tile can be handed to any epilogue exactly as the main loop would have left it.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kQuads = MI * NJ * 4;
+constexpr int64_t kSavedTileBytes = (int64_t)kQuads * kThreads * 16;  // BM * BN * 4
+__device__ __forceinline__ f32x4* saved_tile(float* base, int tm, int tn, int tiles_n) {
+  return reinterpret_cast<f32x4*>(base) + ((int64_t)tm * tiles_n + tn) * (kQuads * kThreads);
+}
+
+// Runs an epilogue over parked tiles: workgroup b takes tile (tm_first + b / tiles_n, b % tiles_n) and calls the
+// epilogue with vocabulary row m0 counted from the first tile row of the launch.  (Measured at T=16384, V=152064:
+// 0.95 ms per 32768 columns, 4.5 TB/s of its 8 bytes per logit; splitting the workgroup into its two rows of waves,
+// each with half the LDS image so that two share a CU, was slower, 1.09 ms.)
+template <class Epi>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void replay_tiles_kernel(
+    const float* __restrict__ saved, int tiles_n, int tm_first, Epi epi) {
+  extern __shared__ __align__(16) char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int wm = w / WN, wn = w % WN;
+  const int tml = blockIdx.x / tiles_n, tn = blockIdx.x - tml * tiles_n;
+  const f32x4* src = saved_tile(const_cast<float*>(saved), tm_first + tml, tn, tiles_n) + tid;
+  floatx16 acc[MI][NJ];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const f32x4 v = __builtin_nontemporal_load(src + ((i * NJ + j) * 4 + q) * kThreads);
+        acc[i][j][q * 4] = v.x;
+        acc[i][j][q * 4 + 1] = v.y;
+        acc[i][j][q * 4 + 2] = v.z;
+        acc[i][j][q * 4 + 3] = v.w;
+      }
+  epi(acc, tml * BM, tn * BN, tml, 0, wm, wn, lane, tid, smem);
+}
+
 // ------------------------------------------------------------------------------ epilogue: softmax partials
 
 // The two fused GEMMs run "transposed": M is the vocabulary (A = W), N the tokens (B = hidden).  In the MFMA
@@ -260,8 +305,22 @@ struct SoftmaxPartialsEpi {
   float inv_T;
   int T, V;
   float* part;  // [tiles_m][3][T]
+  float* save;  // null, or the parked accumulator tiles (see saved_tile)
+  int tiles_n;
   __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
                                              int lane, int tid, char* smem) const {
+    if (save) {
+      f32x4* dst = saved_tile(save, tm, n0 / BN, tiles_n) + tid;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const f32x4 v = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
+            dst[((i * NJ + j) * 4 + q) * kThreads] = v;
+          }
+    }
     float* sh = reinterpret_cast<float*>(smem);  // [WM][BN][3]; the main loop's last barrier freed the LDS
     const float k = kLog2e;
     const float ninf = -__builtin_inff();
@@ -675,13 +734,19 @@ extern "C" size_t siirl_fused_linear_bwd_workspace_bytes(int64_t T, int64_t H, i
   return bwd_ws(T, H, V, want_d_hidden != 0, want_d_weight != 0).total;
 }
 
+extern "C" size_t siirl_fused_linear_saved_logits_bytes(int64_t T, int64_t V) {
+  if (T < 1 || V < 1) return 0;
+  return (size_t)(((V + BM - 1) / BM) * ((T + BN - 1) / BN) * kSavedTileBytes);
+}
+
 extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype,
                                                       const int64_t* labels, int64_t T, int64_t H, int64_t V,
                                                       float inv_temperature, float* logprob, float* entropy, float* lse,
-                                                      float* ex, void* workspace, size_t workspace_bytes,
-                                                      siirl_stream_t stream) {
+                                                      float* ex, float* saved_logits, void* workspace,
+                                                      size_t workspace_bytes, siirl_stream_t stream) {
   if (int rc = check_fused(hidden, weight, T, H, V, inv_temperature, dtype)) return rc;
   SIIRL_REQUIRE(lse != nullptr, "lse is NULL");
+  SIIRL_REQUIRE(((uintptr_t)saved_logits & 15) == 0, "saved_logits must be 16-byte aligned");
   SIIRL_REQUIRE((logprob == nullptr) == (labels == nullptr), "labels and logprob must be given together");
   SIIRL_REQUIRE(entropy == nullptr || ex != nullptr, "ex is required when entropy is requested");
   const FwdWs ws = fwd_ws(T, H, V);
@@ -700,7 +765,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   }
   u32x4* hp = reinterpret_cast<u32x4*>((char*)workspace + ws.hp);
   if (int rc = pack_hidden(h, T, H, hp, st)) return rc;
-  SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part};
+  SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part, saved_logits, (int)((T + BN - 1) / BN)};
   if (int rc = launch_gemm(w, H, hp, H / 16, (int)V, (int)T, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
   const int tiles_v = (int)((V + BM - 1) / BM);
   merge_partials_kernel<<<dim3((unsigned)((T + 63) / 64)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
@@ -712,11 +777,12 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
 extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const void* weight, int dtype,
                                                       const int64_t* labels, int64_t T, int64_t H, int64_t V,
                                                       float inv_temperature, const float* lse, const float* ex,
-                                                      const float* g_logprob, const float* g_entropy, void* d_hidden,
-                                                      void* d_weight, void* workspace, size_t workspace_bytes,
-                                                      siirl_stream_t stream) {
+                                                      const float* saved_logits, const float* g_logprob,
+                                                      const float* g_entropy, void* d_hidden, void* d_weight,
+                                                      void* workspace, size_t workspace_bytes, siirl_stream_t stream) {
   if (int rc = check_fused(hidden, weight, T, H, V, inv_temperature, dtype)) return rc;
   SIIRL_REQUIRE(lse != nullptr, "lse is NULL");
+  SIIRL_REQUIRE(((uintptr_t)saved_logits & 15) == 0, "saved_logits must be 16-byte aligned");
   SIIRL_REQUIRE(g_logprob != nullptr || g_entropy != nullptr, "no upstream gradient given");
   SIIRL_REQUIRE(g_logprob == nullptr || labels != nullptr, "labels is required with g_logprob");
   SIIRL_REQUIRE(g_entropy == nullptr || ex != nullptr, "ex is required with g_entropy");
@@ -737,7 +803,8 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
   const uint16_t* h = (const uint16_t*)hidden;
   const uint16_t* w = (const uint16_t*)weight;
 
-  if (int rc = pack_hidden(h, T, H, hp, st)) return rc;
+  if (!saved_logits)
+    if (int rc = pack_hidden(h, T, H, hp, st)) return rc;
   if (want_dh) {
     transpose_pack_b_kernel<<<dim3((unsigned)(ws.ldwt / 64), (unsigned)(ws.hpad / 64)), dim3(256), 0, st>>>(
         w, H, (int)V, (int)H, Wtp, ws.ldwt / 16);
@@ -751,13 +818,28 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
   int dh_splits = 1;
   const int64_t dh32_stride = (int64_t)(round_up((size_t)T * H * 4, 256) / 4);
   int slab_idx = 0;
+  const int tiles_t = (int)((T + BN - 1) / BN);
   for (int64_t v0 = 0; v0 < V; v0 += kSlab, ++slab_idx) {
     const int N = (int)((V - v0) < kSlab ? (V - v0) : kSlab);
     const int Npad = (int)round_up(N, BK);
     const int gs = slab_idx % kDhGroup;  // position of this slab in its group of D columns
-    DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
-                   D + (int64_t)gs * kSlab, ws.ldd_row, Dt + (int64_t)gs * kSlab * ws.ldt_row, ws.ldt_row, ws.ldt};
-    if (int rc = launch_gemm(w + v0 * H, H, hp, H / 16, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
+    if (!saved_logits) {
+      DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
+                     D + (int64_t)gs * kSlab, ws.ldd_row, Dt + (int64_t)gs * kSlab * ws.ldt_row, ws.ldt_row, ws.ldt};
+      if (int rc = launch_gemm(w + v0 * H, H, hp, H / 16, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
+    } else if (gs == 0) {
+      // the whole group's dlogits in one pass over the tiles the forward parked
+      const int64_t left = V - v0, cap = (int64_t)kDhGroup * kSlab;
+      const int Ng = (int)(left < cap ? left : cap);
+      DlogitsEpi epi{inv_temperature, (int)T, Ng, (int)round_up(Ng, BK), v0, lse, ex, g_logprob, g_entropy, labels,
+                     D, ws.ldd_row, Dt, ws.ldt_row, ws.ldt};
+      const void* fn = reinterpret_cast<const void*>(&replay_tiles_kernel<DlogitsEpi>);
+      if (int rc = allow_dynamic_lds(fn, kSmemBytes)) return rc;
+      const int64_t wgs = (int64_t)((Ng + BM - 1) / BM) * tiles_t;
+      replay_tiles_kernel<DlogitsEpi><<<dim3((unsigned)wgs), dim3(kThreads), kSmemBytes, st>>>(
+          saved_logits, tiles_t, (int)(v0 / BM), epi);
+      SIIRL_LAUNCH_CHECK("replay_tiles_kernel<DlogitsEpi>");
+    }
     if (want_dh && (gs == kDhGroup - 1 || v0 + kSlab >= V)) {
       // dH[T, H] += D[T, K] . Wt[H, g0 : g0 + K]^T over the group's columns (only the last slab can be partial)
       const int64_t g0 = v0 - (int64_t)gs * kSlab;

@@ -6,8 +6,12 @@
 * ``linear_cross_entropy`` -- mirror of ``siirl/utils/kernel/linear_cross_entropy.py:40-117``:
   ``(hidden, weight, labels, temperature, reduction, dist_process_group) -> (logprobs, entropy)``.
 
-Both run the MFMA kernels of ``csrc/fused_linear.hip`` through the C ABI.  Operands are bf16 on the GPU; the
-``[T, V]`` logits are never materialised.  Outputs are fp32 (the reference's Triton path returns fp32,
+Both run the MFMA kernels of ``csrc/fused_linear.hip`` through the C ABI.  Operands are bf16 on the GPU.  The
+forward needs no ``[T, V]`` tensor.  When a backward will follow and the buffer fits the limit set with
+``set_saved_logits_limit`` (default 16 GiB; 4 bytes per logit), the forward parks its fp32 logit tiles and the
+backward reads them back instead of running the projection a second time: the same bits, a quarter less matrix
+work per step.  With the limit at 0 the logits are never stored and the backward recomputes them slab by slab,
+which is the reference's memory behaviour.  Outputs are fp32 (the reference's Triton path returns fp32,
 ``kernels.py:586-593``; its chunked-torch path casts back to the input dtype, ``torch_functional.py:32``, which
 ``FusedLinearForPPO(cast_outputs=True)`` reproduces).  ``chunk_size`` is accepted and ignored: tiling is the
 kernel's business.
@@ -20,6 +24,21 @@ import typing
 import torch
 
 from . import ops as _ops_module  # noqa: F401  (registers torch.ops.siirl_hip.*)
+
+
+_SAVED_LOGITS_LIMIT = 16 << 30
+
+
+def set_saved_logits_limit(nbytes: int) -> None:
+    """Largest fp32 logit buffer (bytes) the forward may keep for the backward; 0 = always recompute."""
+    global _SAVED_LOGITS_LIMIT
+    if nbytes < 0:
+        raise ValueError(f"the limit must not be negative, got {nbytes}")
+    _SAVED_LOGITS_LIMIT = int(nbytes)
+
+
+def _saved_logits_bytes(T: int, V: int) -> int:
+    return ((V + 255) // 256) * ((T + 255) // 256) * (256 * 256 * 4)
 
 
 class _FusedLinearLogprobEntropy(torch.autograd.Function):
@@ -38,15 +57,17 @@ class _FusedLinearLogprobEntropy(torch.autograd.Function):
         if w.shape[1] != H or y.shape != (T,):
             raise ValueError(f"shape mismatch: hidden {tuple(h.shape)}, weight {tuple(w.shape)}, labels {tuple(y.shape)}")
         inv_t = 1.0 / float(temperature)
-        lp, ent, lse, ex = torch.ops.siirl_hip.fused_linear_logprob_entropy_fwd(h, w, y, inv_t)
-        ctx.save_for_backward(h, w, y, lse, ex)
+        save = (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) and \
+            _saved_logits_bytes(T, V) <= _SAVED_LOGITS_LIMIT
+        lp, ent, lse, ex, saved = torch.ops.siirl_hip.fused_linear_logprob_entropy_fwd(h, w, y, inv_t, bool(save))
+        ctx.save_for_backward(h, w, y, lse, ex, saved)
         ctx.inv_t = inv_t
         ctx.set_materialize_grads(False)
         return lp, ent
 
     @staticmethod
     def backward(ctx, g_lp, g_ent):
-        h, w, y, lse, ex = ctx.saved_tensors
+        h, w, y, lse, ex, saved = ctx.saved_tensors
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if (g_lp is None and g_ent is None) or not (need_h or need_w):
             return None, None, None, None
@@ -54,7 +75,7 @@ class _FusedLinearLogprobEntropy(torch.autograd.Function):
         f = lambda t: None if t is None else t.detach().to(device=dev, dtype=torch.float32).contiguous()  # noqa: E731
         g_lp, g_ent = f(g_lp), f(g_ent)
         d_h, d_w = torch.ops.siirl_hip.fused_linear_logprob_entropy_bwd(h, w, y, ctx.inv_t, lse, ex, g_lp, g_ent,
-                                                                        bool(need_h), bool(need_w))
+                                                                        bool(need_h), bool(need_w), saved)
         return (d_h if need_h else None), (d_w if need_w else None), None, None
 
 

@@ -401,10 +401,11 @@ def _bf16_2d(t: torch.Tensor, name: str):
 
 @torch.library.custom_op(f"{_NS}::fused_linear_logprob_entropy_fwd", mutates_args=())
 def fused_linear_logprob_entropy_fwd(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,
-                                     inv_temperature: float) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor,
-                                                                      torch.Tensor]:
-    """lm_head projection fused with log-prob / entropy -> (logprob, entropy, lse, ex), fp32 ``[T]``; the ``[T, V]``
-    logits are never written."""
+                                     inv_temperature: float, save_logits: bool = False
+                                     ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """lm_head projection fused with log-prob / entropy -> (logprob, entropy, lse, ex, saved), fp32 ``[T]``.
+    ``saved`` is empty unless ``save_logits``: then it holds the fp32 logit tiles in the kernel's own order (4 bytes
+    per logit) for the backward to read instead of recomputing them."""
     h, w = _bf16_2d(hidden, "hidden"), _bf16_2d(weight, "weight")
     T, H = h.shape
     V = w.shape[0]
@@ -413,29 +414,36 @@ def fused_linear_logprob_entropy_fwd(hidden: torch.Tensor, weight: torch.Tensor,
         raise ValueError(f"shape mismatch: hidden {tuple(h.shape)}, weight {tuple(w.shape)}, labels {tuple(labels.shape)}")
     L = _lib.lib()
     lp, ent, lse, ex = (torch.empty(T, dtype=torch.float32, device=dev) for _ in range(4))
+    saved = torch.empty(L.siirl_fused_linear_saved_logits_bytes(T, V) // 4 if save_logits else 0, dtype=torch.float32,
+                        device=dev)
     nws = L.siirl_fused_linear_fwd_workspace_bytes(T, H, V)
     ws = torch.empty(max(nws, 256), dtype=torch.uint8, device=dev)
     y = labels.contiguous()
     with torch.cuda.device(dev):
         rc = L.siirl_fused_linear_logprob_entropy_fwd(_lib.ptr(h), _lib.ptr(w), _lib.BF16, _lib.ptr(y), T, H, V,
                                                       inv_temperature, _lib.ptr(lp), _lib.ptr(ent), _lib.ptr(lse),
-                                                      _lib.ptr(ex), _lib.ptr(ws), nws, _lib.current_stream(dev))
+                                                      _lib.ptr(ex), _lib.ptr(saved) if save_logits else None,
+                                                      _lib.ptr(ws), nws, _lib.current_stream(dev))
     _lib.check(rc, "siirl_fused_linear_logprob_entropy_fwd")
-    return lp, ent, lse, ex
+    return lp, ent, lse, ex, saved
 
 
 @fused_linear_logprob_entropy_fwd.register_fake
-def _(hidden, weight, labels, inv_temperature):
+def _(hidden, weight, labels, inv_temperature, save_logits=False):
     mk = lambda: hidden.new_empty(hidden.shape[0], dtype=torch.float32)  # noqa: E731
-    return mk(), mk(), mk(), mk()
+    T, V = hidden.shape[0], weight.shape[0]
+    n = ((V + 255) // 256) * ((T + 255) // 256) * 65536 if save_logits else 0
+    return mk(), mk(), mk(), mk(), hidden.new_empty(n, dtype=torch.float32)
 
 
 @torch.library.custom_op(f"{_NS}::fused_linear_logprob_entropy_bwd", mutates_args=())
 def fused_linear_logprob_entropy_bwd(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,
                                      inv_temperature: float, lse: torch.Tensor, ex: torch.Tensor,
                                      g_logprob: Optional[torch.Tensor], g_entropy: Optional[torch.Tensor],
-                                     need_hidden: bool, need_weight: bool) -> Tuple[torch.Tensor, torch.Tensor]:
-    """-> (d_hidden, d_weight), bf16; a gradient that is not needed comes back empty."""
+                                     need_hidden: bool, need_weight: bool,
+                                     saved: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """-> (d_hidden, d_weight), bf16; a gradient that is not needed comes back empty.  ``saved``: the fifth output
+    of the forward op (empty or None: the logits are recomputed)."""
     h, w = _bf16_2d(hidden, "hidden"), _bf16_2d(weight, "weight")
     T, H = h.shape
     V = w.shape[0]
@@ -444,13 +452,21 @@ def fused_linear_logprob_entropy_bwd(hidden: torch.Tensor, weight: torch.Tensor,
     d_h = torch.empty(h.shape if need_hidden else (0,), dtype=h.dtype, device=dev)
     d_w = torch.empty(w.shape if need_weight else (0,), dtype=w.dtype, device=dev)
     L = _lib.lib()
+    if saved is not None and saved.numel() == 0:
+        saved = None
+    if saved is not None:
+        _require_gpu(saved, "saved")
+        if saved.dtype != torch.float32 or not saved.is_contiguous() or \
+                saved.numel() * 4 != L.siirl_fused_linear_saved_logits_bytes(T, V):
+            raise ValueError("saved is not the buffer the forward op returned for these shapes")
     nws = L.siirl_fused_linear_bwd_workspace_bytes(T, H, V, int(need_hidden), int(need_weight))
     ws = torch.empty(max(nws, 256), dtype=torch.uint8, device=dev)
     y = labels.contiguous()
     with torch.cuda.device(dev):
         rc = L.siirl_fused_linear_logprob_entropy_bwd(_lib.ptr(h), _lib.ptr(w), _lib.BF16, _lib.ptr(y), T, H, V,
-                                                      inv_temperature, _lib.ptr(lse), _lib.ptr(ex), _lib.ptr(g_lp),
-                                                      _lib.ptr(g_ent), _lib.ptr(d_h) if need_hidden else None,
+                                                      inv_temperature, _lib.ptr(lse), _lib.ptr(ex), _lib.ptr(saved),
+                                                      _lib.ptr(g_lp), _lib.ptr(g_ent),
+                                                      _lib.ptr(d_h) if need_hidden else None,
                                                       _lib.ptr(d_w) if need_weight else None, _lib.ptr(ws), nws,
                                                       _lib.current_stream(dev))
     _lib.check(rc, "siirl_fused_linear_logprob_entropy_bwd")
@@ -458,6 +474,6 @@ def fused_linear_logprob_entropy_bwd(hidden: torch.Tensor, weight: torch.Tensor,
 
 
 @fused_linear_logprob_entropy_bwd.register_fake
-def _(hidden, weight, labels, inv_temperature, lse, ex, g_logprob, g_entropy, need_hidden, need_weight):
+def _(hidden, weight, labels, inv_temperature, lse, ex, g_logprob, g_entropy, need_hidden, need_weight, saved=None):
     return (hidden.new_empty(hidden.shape if need_hidden else (0,)),
             weight.new_empty(weight.shape if need_weight else (0,)))

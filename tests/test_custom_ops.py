@@ -46,9 +46,12 @@ def test_fake_kernels_give_shapes_without_a_gpu(with_optional):
         assert adv.shape == (B, L) and adv.dtype == torch.float32
         keep, gsz = ns.group_keep_mask(mk((B,), torch.float64), mk((B,), torch.int64))
         assert keep.dtype == torch.uint8 and gsz.dtype == torch.int32 and keep.shape == gsz.shape == (B,)
-        lp, ent, lse, ex = ns.fused_linear_logprob_entropy_fwd(mk((T, H), torch.bfloat16), mk((V, H), torch.bfloat16),
-                                                               mk((T,), torch.int64), 1.0)
-        assert lp.shape == ent.shape == lse.shape == ex.shape == (T,) and lp.dtype == torch.float32
+        lp, ent, lse, ex, sv = ns.fused_linear_logprob_entropy_fwd(mk((T, H), torch.bfloat16),
+                                                                   mk((V, H), torch.bfloat16), mk((T,), torch.int64), 1.0)
+        assert lp.shape == ent.shape == lse.shape == ex.shape == (T,) and lp.dtype == torch.float32 and sv.numel() == 0
+        sv = ns.fused_linear_logprob_entropy_fwd(mk((T, H), torch.bfloat16), mk((V, H), torch.bfloat16),
+                                                 mk((T,), torch.int64), 1.0, True)[4]
+        assert sv.numel() == ((V + 255) // 256) * ((T + 255) // 256) * 65536 and sv.dtype == torch.float32
         dh, dw = ns.fused_linear_logprob_entropy_bwd(mk((T, H), torch.bfloat16), mk((V, H), torch.bfloat16),
                                                      mk((T,), torch.int64), 1.0, lse, ex, mk((T,), torch.float32), None,
                                                      True, False)
@@ -80,8 +83,11 @@ def test_opcheck_on_the_gpu():
     h, w = mk((T, H), torch.bfloat16), mk((V, H), torch.bfloat16)
     y = torch.randint(0, V, (T,), device=dev)
     torch.library.opcheck(ns.fused_linear_logprob_entropy_fwd, (h, w, y, 1.0), test_utils=checks)
-    lp, ent, lse, ex = ns.fused_linear_logprob_entropy_fwd(h, w, y, 1.0)
+    torch.library.opcheck(ns.fused_linear_logprob_entropy_fwd, (h, w, y, 1.0, True), test_utils=checks)
+    lp, ent, lse, ex, sv = ns.fused_linear_logprob_entropy_fwd(h, w, y, 1.0, True)
     torch.library.opcheck(ns.fused_linear_logprob_entropy_bwd, (h, w, y, 1.0, lse, ex, torch.ones(T, device=dev), None,
                                                                 True, True), test_utils=checks)
+    torch.library.opcheck(ns.fused_linear_logprob_entropy_bwd, (h, w, y, 1.0, lse, ex, torch.ones(T, device=dev), None,
+                                                                True, True, sv), test_utils=checks)
     x = mk((T, V), torch.bfloat16)
     torch.library.opcheck(ns.logprob_entropy_fwd, (x, y, 1.0, True), test_utils=checks)

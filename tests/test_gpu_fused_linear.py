@@ -109,3 +109,47 @@ def test_fused_vs_fixtures(dev):
     torch.autograd.backward([lp, ent], [torch.from_numpy(G["fl_g_lp"]).to(dev), torch.from_numpy(G["fl_g_h"]).to(dev)])
     _check_grad(hd.grad, torch.from_numpy(G["fl_dhidden"]), "d_hidden")
     _check_grad(wd.grad, torch.from_numpy(G["fl_dweight"]), "d_weight")
+
+
+@pytest.mark.parametrize("T,H,V", [(64, 64, 300), (257, 128, 32769), (1000, 192, 40000), (130, 128, 65537)])
+@pytest.mark.parametrize("which", ["both", "logprob", "entropy"])
+def test_saved_logits_route_equals_recompute(dev, T, H, V, which):
+    """The backward that reads the logit tiles the forward parked gives the bits of the backward that recomputes
+    them; the forward's outputs do not depend on whether it parks them."""
+    import siirl_amd.fused_linear as FL
+
+    g = torch.Generator().manual_seed(T + V)
+    h = (torch.randn(T, H, generator=g) * 0.7).to(torch.bfloat16).to(dev)
+    w = (torch.randn(V, H, generator=g) * 0.2).to(torch.bfloat16).to(dev)
+    y = torch.randint(0, V, (T,), generator=g).to(dev)
+    g_lp, g_h = torch.randn(T, generator=g).to(dev), torch.randn(T, generator=g).to(dev)
+    out = {}
+    try:
+        for name, limit in (("saved", 1 << 40), ("recompute", 0)):
+            FL.set_saved_logits_limit(limit)
+            hd, wd = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
+            lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y, 0.8)
+            outs, grads = {"both": ([lp, ent], [g_lp, g_h]), "logprob": ([lp], [g_lp]), "entropy": ([ent], [g_h])}[which]
+            torch.autograd.backward(outs, grads)
+            out[name] = (lp.detach(), ent.detach(), hd.grad, wd.grad)
+    finally:
+        FL.set_saved_logits_limit(16 << 30)
+    for a, b, what in zip(out["saved"], out["recompute"], ("logprob", "entropy", "d_hidden", "d_weight")):
+        assert torch.equal(a, b), what
+
+
+def test_saved_logits_limit_and_no_grad(dev):
+    import siirl_amd.fused_linear as FL
+
+    ns = torch.ops.siirl_hip
+    h = torch.randn(70, 64, device=dev).to(torch.bfloat16)
+    w = torch.randn(500, 64, device=dev).to(torch.bfloat16)
+    y = torch.randint(0, 500, (70,), device=dev)
+    lp, ent, lse, ex, sv = ns.fused_linear_logprob_entropy_fwd(h, w, y, 1.0, True)
+    assert sv.numel() == 2 * 1 * 65536
+    with pytest.raises(ValueError, match="saved"):
+        ns.fused_linear_logprob_entropy_bwd(h, w, y, 1.0, lse, ex, torch.ones(70, device=dev), None, True, True, sv[:-1])
+    with pytest.raises(ValueError):
+        FL.set_saved_logits_limit(-1)
+    assert FL._saved_logits_bytes(70, 500) == torch.ops.siirl_hip.fused_linear_logprob_entropy_fwd(
+        h, w, y, 1.0, True)[4].numel() * 4

@@ -266,8 +266,9 @@ __device__ __forceinline__ f32x4* saved_tile(float* base, int tm, int tn, int ti
 
 // Runs an epilogue over parked tiles: workgroup b takes tile (tm_first + b / tiles_n, b % tiles_n) and calls the
 // epilogue with vocabulary row m0 counted from the first tile row of the launch.  (Measured at T=16384, V=152064:
-// 0.95 ms per 32768 columns, 4.5 TB/s of its 8 bytes per logit; splitting the workgroup into its two rows of waves,
-// each with half the LDS image so that two share a CU, was slower, 1.09 ms.)
+// 0.87 ms per 32768 columns, 4.9 TB/s of its 8 bytes per logit, arithmetic and LDS writes about level with the
+// memory time; splitting the workgroup into its two rows of waves, each with half the LDS image so that two share
+// a CU, was 15 % slower.)
 template <class Epi>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void replay_tiles_kernel(
     const float* __restrict__ saved, int tiles_n, int tm_first, Epi epi) {
@@ -408,9 +409,15 @@ struct DlogitsEpi {
   static __device__ __forceinline__ int lds_at(int vrow, int tok_l) {
     return vrow * (BN * 2) + ((((tok_l >> 3) ^ vrow) & 31) << 4) + ((tok_l & 7) << 1);
   }
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
-                                             int lane, int tid, char* smem) const {
-    // the main loop's last barrier (and its vmcnt(0)) freed the ring: 256 x 512 B fit it exactly
+  // One lane's part of the tile.  With a = raw accumulator (z = a * inv_T) the gradient is
+  //   d = p * (c0 + c1 * a) + [v == y] * cy,   p = exp2(a * ek + nl),
+  // ek = inv_T * log2(e), nl = -lse * log2(e), c1 = -g_h * inv_T^2, c0 = inv_T * (g_h * ex - g_lp), cy = g_lp * inv_T:
+  // two fused multiply-adds, one exp2 and one multiply per logit.  A token past T has all coefficients zero (its
+  // accumulators are zero: p = 1, d = 0).  FULL: every vocabulary row of the tile is inside the slab.
+  template <bool FULL>
+  __device__ __forceinline__ void tile(floatx16 (&acc)[MI][NJ], int m0, int n0, int wm, int wn, int lane,
+                                       char* smem) const {
+    const float ek = inv_T * kLog2e;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
       const int tok_l = acc_col(wn, j, lane), tok = n0 + tok_l;
@@ -419,6 +426,7 @@ struct DlogitsEpi {
       const float g2 = (live && g_h) ? g_h[tok] : 0.f;
       const float nl = live ? -lse[tok] * kLog2e : 0.f;
       const float exv = (live && g_h) ? ex[tok] : 0.f;
+      const float c1 = -g2 * inv_T * inv_T, c0 = inv_T * (g2 * exv - g1), cy = g1 * inv_T;
       int y = -1;
       if (live && g_lp) {
         const int64_t yl = labels[tok] - v0;
@@ -434,14 +442,11 @@ struct DlogitsEpi {
           float d[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            d[e] = 0.f;
-            if (live && v + e < Vs) {
-              const float z = acc[i][j][q * 4 + e] * inv_T;
-              const float p = fast_exp2(fmaf(z, kLog2e, nl));
-              float g = p * (-g1 - g2 * (z - exv));
-              if (v + e == y) g += g1;
-              d[e] = g * inv_T;
-            }
+            const float a = acc[i][j][q * 4 + e];
+            const float p = fast_exp2(fmaf(a, ek, nl));
+            float g = p * fmaf(a, c1, c0);
+            if (v + e == y) g += cy;
+            d[e] = (FULL || v + e < Vs) ? g : 0.f;
           }
           const uint32_t lo = pack_bf16(d[0], d[1]), hi = pack_bf16(d[2], d[3]);
           if (live && v < Vpad) *reinterpret_cast<uint2*>(drow + v) = make_uint2(lo, hi);  // 8-byte aligned
@@ -451,6 +456,14 @@ struct DlogitsEpi {
           *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 3, tok_l)) = (uint16_t)(hi >> 16);
         }
     }
+  }
+  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
+                                             int lane, int tid, char* smem) const {
+    // the main loop's last barrier (and its vmcnt(0)) freed the ring: 256 x 512 B fit it exactly
+    if (m0 + BM <= Vs)
+      tile<true>(acc, m0, n0, wm, wn, lane, smem);
+    else
+      tile<false>(acc, m0, n0, wm, wn, lane, smem);
     __syncthreads();
     // Dt[v][token]: rows leave the LDS as 16-byte chunks, 32 consecutive threads per 512-byte row
 #pragma unroll 4

@@ -40,11 +40,16 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #endif
 static_assert(SIIRL_GEMM_BM == 256 || SIIRL_GEMM_BM == 128, "the workgroup tile has 256 or 128 rows");
 constexpr int BM = SIIRL_GEMM_BM, BN = 256, BK = 64;
+// Waves along N: 4 (8 waves of 128 x 64, two per SIMD) or 2 (4 waves of 128 x 128, one per SIMD, accumulators in
+// the AGPRs).  Measured at T=16384, H=3584, V=152064: the 4-wave grid is 5 % slower in the d-weight GEMM, 9 % in the
+// forward and 14 % in d-hidden, so halving the operand fetches per MFMA does not pay for losing the second wave.
 #ifndef SIIRL_GEMM_WAVES_N
 #define SIIRL_GEMM_WAVES_N 4
 #endif
 constexpr int WM = BM / 128, WN = SIIRL_GEMM_WAVES_N;  // wave grid over the workgroup tile
 constexpr int kThreads = WM * WN * 64;
+constexpr int kWavesPerSimd = kThreads / 256;  // one workgroup per CU (the LDS ring), four SIMDs
+static_assert(kThreads == 256 || kThreads == 512, "4 or 8 waves per workgroup");
 constexpr int MI = BM / (WM * 32), NJ = BN / (WN * 32);  // 32x32 MFMA tiles per wave
 constexpr int kLoadsPerThread = (BM * BK / 8) / kThreads;  // 16-byte chunks per operand tile per thread
 constexpr int kLoadRowStep = kThreads / 8;
@@ -113,7 +118,7 @@ __device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (N
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
 template <class Epi>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void gemm_nt_kernel(GemmArgs g, Epi epi) {
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void gemm_nt_kernel(GemmArgs g, Epi epi) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int wm = w / WN, wn = w % WN;
@@ -172,19 +177,27 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(b[j][2]) : "v"(offB[j]), "s"(base));
     asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(b[j][3]) : "v"(offB[j]), "s"(base));
   };
-  // waits until at most `n` of this wave's loads are in flight and ties the B registers to the wait
-#define SIIRL_BWAIT(n, b)                                                                                              \
-  asm volatile("s_waitcnt vmcnt(" #n ")"                                                                              \
-               : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[0][3]), "+v"(b[1][0]), "+v"(b[1][1]),            \
-                 "+v"(b[1][2]), "+v"(b[1][3])::"memory")
-  static_assert(NJ == 2 && BK == 64 && kDmaPerWave == 4, "the wait counts below assume 8 B loads and 4 DMA per step");
+  // waits until only this wave's last kDmaPerWave loads (one stage of DMA) are in flight and ties the B registers
+  // to the wait (at most 30 asm operands: the registers of N-tiles 2 and 3 are tied by a second, empty statement)
+  static_assert((NJ == 2 || NJ == 4) && BK == 64 && kDmaPerWave % 2 == 0, "see the load schedule of a K-step");
+  auto bwait = [&](u32x4 (&b)[NJ][BK / 16]) {
+    asm volatile("s_waitcnt vmcnt(%[n])"
+                 : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[0][3]), "+v"(b[1][0]), "+v"(b[1][1]),
+                   "+v"(b[1][2]), "+v"(b[1][3])
+                 : [n] "n"(kDmaPerWave)
+                 : "memory");
+    if constexpr (NJ == 4)
+      asm volatile(""
+                   : "+v"(b[NJ - 2][0]), "+v"(b[NJ - 2][1]), "+v"(b[NJ - 2][2]), "+v"(b[NJ - 2][3]), "+v"(b[NJ - 1][0]),
+                     "+v"(b[NJ - 1][1]), "+v"(b[NJ - 1][2]), "+v"(b[NJ - 1][3])::"memory");
+  };
 
-  bload(b0, 0, 0);
-  bload(b0, 0, 1);
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) bload(b0, 0, j);
   dma(0, 0);
   dma(1, KT > 1 ? 1 : 0);
   dma(2, KT > 2 ? 2 : 0);
-  SIIRL_BWAIT(4, b0);
+  bwait(b0);
   __syncthreads();
 
   const int m31 = lane & 31, gsel = lane >> 5, sw = (m31 >> 1) & 7;
@@ -212,7 +225,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], __builtin_bit_cast(bf16x8, bc[j][kk]), acc[i][j], 0, 0, 0);
   };
   fread(afa, 0, 0);
-  // One K-step.  The 12 vector-memory instructions are spread over the step (B for one N-tile before each of the
+  // One K-step.  The vector-memory instructions (12 with 8 waves) are spread over the step (B for one N-tile before each of the
   // first two MFMA groups, half of the DMA before each of the last two) instead of being issued in one burst, and
   // the wave raises its priority while it issues MFMAs so that its SIMD partner's loads do not delay them.
   auto mma_prio = [&](bf16x8 (&af)[MI], u32x4 (&bc)[NJ][BK / 16], int kk) {
@@ -223,10 +236,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   auto step = [&](int kt, u32x4 (&bc)[NJ][BK / 16], u32x4 (&bn)[NJ][BK / 16]) {
     const int stage = kt & 3;
     const int ktb = kt + 1 < KT ? kt + 1 : KT - 1, kta = kt + 3 < KT ? kt + 3 : KT - 1;
-    bload(bn, ktb, 0);
+#pragma unroll
+    for (int j = 0; j < NJ / 2; ++j) bload(bn, ktb, j);
     fread(afb, stage, 1);
     mma_prio(afa, bc, 0);
-    bload(bn, ktb, 1);
+#pragma unroll
+    for (int j = NJ / 2; j < NJ; ++j) bload(bn, ktb, j);
     fread(afa, stage, 2);
     mma_prio(afb, bc, 1);
     dma((stage + 3) & 3, kta, 0, kDmaPerWave / 2);
@@ -235,7 +250,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
     dma((stage + 3) & 3, kta, kDmaPerWave / 2, kDmaPerWave);
     fread(afa, (stage + 1) & 3, 0);
     mma_prio(afb, bc, 3);
-    SIIRL_BWAIT(4, bn);
+    bwait(bn);
     __syncthreads();
   };
   int kt = 0;
@@ -247,7 +262,6 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))
   // the clamped DMA of the last steps may still be in flight and the epilogue reuses the LDS
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
-#undef SIIRL_BWAIT
   epi(acc, m0, n0, tc.tm, split, wm, wn, lane, tid, smem);
 }
 #pragma clang diagnostic pop
@@ -270,7 +284,7 @@ __device__ __forceinline__ f32x4* saved_tile(float* base, int tm, int tn, int ti
 // memory time; splitting the workgroup into its two rows of waves, each with half the LDS image so that two share
 // a CU, was 15 % slower.)
 template <class Epi>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void replay_tiles_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void replay_tiles_kernel(
     const float* __restrict__ saved, int tiles_n, int tm_first, Epi epi) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;

@@ -223,3 +223,76 @@ def test_config2_slice_properties(dev):
     assert (a1 - a2).abs().max() < 1e-4 and (e1 - e2).abs().max() < 1e-4
     (dx,) = torch.autograd.grad([lp, ent], [xr], [torch.ones(T, device=dev), torch.ones(T, device=dev)])
     assert dx.float().sum(-1).abs().max() < 2e-2  # 152k bf16-rounded terms per row
+
+
+def _actor_post_logits(SF, logits, labels, checkpointed, reentrant=False):
+    """The actor's post-logits step (reference dp_actor.py:176-195): log-prob, then the entropy, optionally under
+    torch.utils.checkpoint as with entropy_checkpointing."""
+    import torch.utils.checkpoint as ckpt
+
+    lp = SF.logprobs_from_logits(logits, labels, inplace_backward=False)
+    if checkpointed:
+        ent = ckpt.checkpoint(SF.entropy_from_logits, logits, use_reentrant=reentrant)
+    else:
+        ent = SF.entropy_from_logits(logits)
+    return lp, ent
+
+
+@pytest.mark.parametrize("pairing", [True, False])
+@pytest.mark.parametrize("mode", ["plain", "checkpoint", "checkpoint_reentrant", "autocast", "autocast_checkpoint"])
+def test_checkpoint_and_autocast_contexts(dev, mode, pairing):
+    """The reference calls these functions under torch.autocast(bf16) (dp_actor.py:101) and wraps the entropy in
+    torch.utils.checkpoint (:193-195): the forward must be re-runnable and every context must give the bits of the
+    plain call."""
+    import contextlib
+
+    import siirl_amd.torch_functional as SF
+
+    x, y = _make(37, 5003, torch.bfloat16, 11)
+    g = torch.Generator().manual_seed(5)
+    w_lp, w_ent = torch.randn(37, generator=g).to(dev), torch.randn(37, generator=g).to(dev)
+
+    def run(mode):
+        xd = x.to(dev).requires_grad_(True)
+        ctx = torch.autocast("cuda", dtype=torch.bfloat16) if mode.startswith("autocast") else contextlib.nullcontext()
+        with ctx:
+            lp, ent = _actor_post_logits(SF, xd, y.to(dev), "checkpoint" in mode, reentrant=mode.endswith("reentrant"))
+            loss = (lp * w_lp).sum() - (ent * w_ent).sum()
+        loss.backward()
+        return lp.detach(), ent.detach(), xd.grad
+
+    SF.set_pairing(pairing)
+    try:
+        want = run("plain")
+        got = run(mode)
+    finally:
+        SF.set_pairing(True)
+    assert got[0].dtype == torch.float32 and got[1].dtype == torch.float32 and got[2].dtype == torch.bfloat16
+    for a, b, what in zip(got, want, ("logprob", "entropy", "dlogits")):
+        if what == "dlogits" and pairing and mode.endswith("reentrant"):
+            # the reentrant checkpoint re-runs the entropy on a detached copy, so its gradient comes from its own
+            # kernel and autograd adds the two bf16 results (as the reference's autograd does): each part carries
+            # its own rounding, so compare with the fp64 oracle in units of the parts' magnitudes
+            d1 = OF.logprob_entropy_backward(x, y, w_lp.cpu(), None, dtype=torch.float64)
+            d2 = OF.logprob_entropy_backward(x, y, None, -w_ent.cpu(), dtype=torch.float64)
+            tol = 2.0 ** -8 * (d1.abs() + d2.abs() + (d1 + d2).abs()) + 1e-7
+            assert ((a.double().cpu() - (d1 + d2)).abs() <= tol).all(), (mode, what)
+        else:
+            assert torch.equal(a, b), (mode, what)
+    lp_o = OF.logprobs_from_logits(x, y, dtype=torch.float32)
+    assert (got[0].cpu() - lp_o).abs().max() < ABS_TOL
+
+
+def test_no_grad_and_inference_mode(dev):
+    import siirl_amd.torch_functional as SF
+
+    x, y = _make(9, 777, torch.bfloat16, 2)
+    xd, yd = x.to(dev), y.to(dev)
+    ref = SF.logprobs_from_logits(xd, yd), SF.entropy_from_logits(xd)
+    with torch.no_grad():  # reference dp_actor.py:330 (compute_log_prob)
+        a = SF.logprobs_from_logits(xd.clone().requires_grad_(True), yd), SF.entropy_from_logits(xd)
+    with torch.inference_mode():
+        b = SF.logprobs_from_logits(xd, yd), SF.entropy_from_logits(xd)
+    for t in (*a, *b):
+        assert not t.requires_grad
+    assert torch.equal(a[0], ref[0]) and torch.equal(a[1], ref[1]) and torch.equal(b[0], ref[0]) and torch.equal(b[1], ref[1])

@@ -65,11 +65,13 @@ constexpr int kDmaPerWave = kTileBytes / 1024 / (kThreads / 64);  // 1 KB per wa
 constexpr int kSlab = SIIRL_SLAB;                   // vocabulary columns per backward slab
 static_assert(kSlab % 256 == 0, "a slab is a whole number of workgroup tiles");
 #ifndef SIIRL_DH_GROUP
-#define SIIRL_DH_GROUP 4
+#define SIIRL_DH_GROUP 8
 #endif
 constexpr int kDhGroup = SIIRL_DH_GROUP;      // slabs of dlogits kept before d hidden and d weight are updated: fewer
-                                              // fp32 read-modify-write passes over [T, H], and 4 x 448 d-weight
-                                              // tiles fill 7 rounds of the 256 CUs exactly
+                                              // fp32 read-modify-write passes over [T, H] (about 6 % of a d-hidden
+                                              // launch at 4 slabs), and 8 x 448 d-weight tiles fill 14 rounds of
+                                              // the 256 CUs exactly; measured 4 / 8 / all 19 slabs of V = 152064:
+                                              // 34.4 / 33.7 / 33.2 ms per backward
 constexpr int kLdPad = 64;                    // extra elements per row of D / Dt: keeps a tile's 256 rows off a
                                               // power-of-two stride, which would put them all in one memory channel
 
@@ -280,7 +282,7 @@ __device__ __forceinline__ f32x4* saved_tile(float* base, int tm, int tn, int ti
 
 // Runs an epilogue over parked tiles: workgroup b takes tile (tm_first + b / tiles_n, b % tiles_n) and calls the
 // epilogue with vocabulary row m0 counted from the first tile row of the launch.  (Measured at T=16384, V=152064:
-// 0.87 ms per 32768 columns, 4.9 TB/s of its 8 bytes per logit, arithmetic and LDS writes about level with the
+// 0.87 ms per 32768 columns (launches take 65536), 4.9 TB/s of its 8 bytes per logit, arithmetic and LDS writes about level with the
 // memory time; splitting the workgroup into its two rows of waves, each with half the LDS image so that two share
 // a CU, was 15 % slower.)
 template <class Epi>

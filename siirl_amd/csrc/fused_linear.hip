@@ -94,7 +94,9 @@ struct TileCoord {
 // kBlkM x kBlkN tiles (32 tiles: one XCD's resident set); block b goes to XCD b % 8 and its tiles to 32
 // consecutive workgroups of that XCD, so the workgroups sharing an L2 at any time share 8 A-tiles and 4
 // B-tiles instead of streaming 32 different A-tiles.  Blocks sweep M fastest inside a strip of kBlkN N-tiles,
-// which keeps a strip's B-tiles hot across the 8 XCDs.
+// which keeps a strip's B-tiles hot across the 8 XCDs.  (Sweeping N fastest instead, which would stream the big
+// operand from memory once rather than once per strip, measured 4 % slower forward and 8-17 % slower backward GEMMs
+// at T=16384, H=3584, V=152064: the L2 reuse inside a strip matters more than the bytes from memory.)
 constexpr int kXcd = 8, kBlkM = 8 * 256 / BM, kBlkN = 4;
 __host__ __device__ inline int64_t raster_grid(int tiles_m, int tiles_n) {
   const int64_t blocks = (int64_t)((tiles_m + kBlkM - 1) / kBlkM) * ((tiles_n + kBlkN - 1) / kBlkN);

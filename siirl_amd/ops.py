@@ -414,8 +414,12 @@ def fused_linear_logprob_entropy_fwd(hidden: torch.Tensor, weight: torch.Tensor,
         raise ValueError(f"shape mismatch: hidden {tuple(h.shape)}, weight {tuple(w.shape)}, labels {tuple(labels.shape)}")
     L = _lib.lib()
     lp, ent, lse, ex = (torch.empty(T, dtype=torch.float32, device=dev) for _ in range(4))
-    saved = torch.empty(L.siirl_fused_linear_saved_logits_bytes(T, V) // 4 if save_logits else 0, dtype=torch.float32,
-                        device=dev)
+    saved = torch.empty(0, dtype=torch.float32, device=dev)
+    if save_logits:
+        try:
+            saved = torch.empty(L.siirl_fused_linear_saved_logits_bytes(T, V) // 4, dtype=torch.float32, device=dev)
+        except torch.OutOfMemoryError:
+            save_logits = False  # no room to keep the logits: the backward recomputes them
     nws = L.siirl_fused_linear_fwd_workspace_bytes(T, H, V)
     ws = torch.empty(max(nws, 256), dtype=torch.uint8, device=dev)
     y = labels.contiguous()

@@ -153,3 +153,32 @@ def test_saved_logits_limit_and_no_grad(dev):
         FL.set_saved_logits_limit(-1)
     assert FL._saved_logits_bytes(70, 500) == torch.ops.siirl_hip.fused_linear_logprob_entropy_fwd(
         h, w, y, 1.0, True)[4].numel() * 4
+
+
+def test_parked_logits_allocation_failure_falls_back_to_recompute(dev, monkeypatch):
+    """When the buffer for the parked logits cannot be allocated the forward keeps nothing and the backward
+    recomputes: same results, no error."""
+    import siirl_amd._lib as L
+    import siirl_amd.fused_linear as FL
+
+    h = torch.randn(70, 64, device=dev).to(torch.bfloat16)
+    w = torch.randn(500, 64, device=dev).to(torch.bfloat16)
+    y = torch.randint(0, 500, (70,), device=dev)
+
+    def run():
+        hd, wd = h.clone().requires_grad_(True), w.clone().requires_grad_(True)
+        lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y)
+        (lp.sum() + ent.sum()).backward()
+        return lp.detach(), ent.detach(), hd.grad, wd.grad
+
+    want = run()
+    handle = L.lib()
+    real = handle.siirl_fused_linear_saved_logits_bytes
+    monkeypatch.setattr(handle, "siirl_fused_linear_saved_logits_bytes", lambda T, V: 1 << 52)
+    try:
+        assert torch.ops.siirl_hip.fused_linear_logprob_entropy_fwd(h, w, y, 1.0, True)[4].numel() == 0
+        got = run()
+    finally:
+        monkeypatch.setattr(handle, "siirl_fused_linear_saved_logits_bytes", real)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)

@@ -42,7 +42,8 @@ static_assert(SIIRL_GEMM_BM == 256 || SIIRL_GEMM_BM == 128, "the workgroup tile 
 constexpr int BM = SIIRL_GEMM_BM, BN = 256, BK = 64;
 // Waves along N: 4 (8 waves of 128 x 64, two per SIMD) or 2 (4 waves of 128 x 128, one per SIMD, accumulators in
 // the AGPRs).  Measured at T=16384, H=3584, V=152064: the 4-wave grid is 5 % slower in the d-weight GEMM, 9 % in the
-// forward and 14 % in d-hidden, so halving the operand fetches per MFMA does not pay for losing the second wave.
+// forward and 14 % in d-hidden: its matrix cores are busy 0.67 of the cycles at 1.74 GHz against 0.76 at 1.66 GHz, so
+// halving the operand fetches per MFMA frees little power and does not pay for losing the second wave per SIMD.
 #ifndef SIIRL_GEMM_WAVES_N
 #define SIIRL_GEMM_WAVES_N 4
 #endif

@@ -71,7 +71,9 @@ typedef enum siirl_kl_mode {
 
 /* ------------------------------------------------------------------------------------------ misc */
 
-/* ABI version of this header (major * 1000 + minor). */
+/* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
+ * from.  A host compiled against another version must not call the library. */
+#define SIIRL_HIP_ABI_VERSION 1001
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the

@@ -13,6 +13,7 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsiirl_hip.so"
 # dtype codes of siirl_dtype
 F32, BF16, F16, F64, I64, I32, U8 = range(7)
 MAX_EOS_TOKENS = 16  # SIIRL_MAX_EOS_TOKENS
+ABI_VERSION = 1001  # SIIRL_HIP_ABI_VERSION of include/siirl_hip.h that SIGNATURES below transcribes
 BWD_SKIP_ZERO_ROWS = 1
 
 _p, _i64, _i32, _f32, _u32, _sz, _f64 = (C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint32, C.c_size_t,
@@ -91,6 +92,10 @@ def lib():
                 for name, (res, args) in SIGNATURES.items():
                     fn = getattr(h, name)  # AttributeError if the symbol is not exported
                     fn.restype, fn.argtypes = res, args
+                if h.siirl_hip_abi_version() != ABI_VERSION:
+                    raise SiirlHipError(
+                        f"{LIB_PATH} was built from ABI version {h.siirl_hip_abi_version()}, this package binds "
+                        f"version {ABI_VERSION}: rebuild it with `python -m siirl_amd.build`")
                 _lib = h
     return _lib
 

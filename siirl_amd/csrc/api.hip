@@ -34,6 +34,6 @@ int allow_dynamic_lds(const void* kernel, int bytes) {
 
 }  // namespace siirl
 
-extern "C" int siirl_hip_abi_version(void) { return 1000; }
+extern "C" int siirl_hip_abi_version(void) { return SIIRL_HIP_ABI_VERSION; }
 
 extern "C" const char* siirl_hip_last_error(void) { return siirl::g_last_error.c_str(); }

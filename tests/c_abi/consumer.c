@@ -60,7 +60,7 @@ int main(void) {
   hipStream_t stream;
   CK(hipStreamCreate(&stream));
 
-  if (siirl_hip_abi_version() < 1000) {
+  if (siirl_hip_abi_version() != SIIRL_HIP_ABI_VERSION) {
     printf("FAIL abi version %d\n", siirl_hip_abi_version());
     return 4;
   }

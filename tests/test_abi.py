@@ -35,7 +35,8 @@ def test_header_symbols_are_exported_and_bound():
     for n in names:
         assert hasattr(h, n), f"{n} is declared in siirl_hip.h but not exported"
     assert sorted(L.SIGNATURES) == names, "ctypes table and header disagree"
-    assert h.siirl_hip_abi_version() >= 1000
+    assert h.siirl_hip_abi_version() == L.ABI_VERSION
+    assert f"#define SIIRL_HIP_ABI_VERSION {L.ABI_VERSION}\n" in open(HEADER).read()
 
 
 def test_every_entry_point_cites_the_reference():

@@ -163,6 +163,42 @@ def bench_config3(args, dev):
     loss_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / steps
     tokens = Bk * L
     loss_bytes = tokens * (2 * (4 * 4 + 8) + 4)  # forward and backward each read 4 fp32 operands + int64 mask; d_lp written
+
+    # the path's smaller building blocks on the same [kept, L] tensors, each timed alone (not part of the step)
+    import siirl_amd.torch_functional as SF
+
+    def timed_ms(fn, iters=10):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    lpd = lp.detach()
+    kl_ctrl = CA.FixedKLController(0.001)
+    td = {"token_level_scores": rk, "old_log_probs": old, "ref_log_prob": ref, "response_mask": mk}
+    lm = torch.randn(Bk, L, device=dev, generator=gen).requires_grad_(True)
+
+    def agg_fb():
+        CA.agg_loss(lm, mk, "seq-mean-token-mean").backward()
+        lm.grad = None
+
+    blocks = {
+        "masked_mean(values, mask) -> scalar (12 B/token)": (lambda: SF.masked_mean(lpd, mk), 12),
+        "masked_mean(values, mask, axis=-1) -> [B] (12 B/token)": (lambda: SF.masked_mean(lpd, mk, axis=-1), 12),
+        "kl_penalty low_var_kl forward (12 B/token)": (lambda: CA.kl_penalty(lpd, ref, "low_var_kl"), 12),
+        "apply_kl_penalty: rewards = scores - beta * kl * mask, batch KL, one host sync (24 B/token)":
+            (lambda: CA.apply_kl_penalty(td, kl_ctrl, "low_var_kl"), 24),
+        "agg_loss seq-mean-token-mean forward + backward (28 B/token)": (agg_fb, 28),
+    }
+    block_ms = {}
+    for name, (fn, bpt) in blocks.items():
+        ms = timed_ms(fn)
+        block_ms[name] = {"ms": ms, "GB/s": tokens * bpt / ms / 1e6}
     gbs = loss_bytes / loss_ms / 1e6
     out = {
         "metric": "DAPO loss path (filter + GRPO advantage + clipped loss fwd+bwd) tokens/sec @[B,L] fp32",
@@ -173,6 +209,7 @@ def bench_config3(args, dev):
                    "trajectories": B, "kept": Bk, "response_length": L, "seed": SEED},
         "kernels": {"keep mask + GRPO advantage": {"ms": grp_ms},
                     "actor loss forward + backward (loss_partials/finish/bwd kernels)": {"ms": loss_ms, "GB/s": gbs}},
+        "building_blocks": block_ms,
         "roofline": {"bound": "hbm", "kernel": "loss_partials_kernel + loss_bwd_kernel", "achieved": gbs, "peak": 8000.0,
                      "unit": "GB/s", "frac": gbs / 8000.0,
                      "traffic": MEASURED_TRAFFIC_BYTES_CONFIG3 if Bk == 5488 else None},

@@ -455,18 +455,38 @@ __global__ __launch_bounds__(kThreads) void agg_weights_kernel(LossArgs a, const
 
 // ---------------------------------------------------------------------------- KL penalty (elementwise)
 
+// four consecutive elements per thread and pass; `vec`: every operand is 16-byte aligned (one 16-byte access each)
 __global__ __launch_bounds__(kThreads) void kl_fwd_kernel(const float* __restrict__ lp, const float* __restrict__ ref,
-                                                          int64_t n, int mode, float* __restrict__ out) {
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads)
-    out[i] = kl_token(lp[i], ref[i], mode, 0).v;
+                                                          int64_t n, int mode, bool vec, float* __restrict__ out) {
+  const int64_t nq = (n + 3) / 4;
+  for (int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x; q < nq; q += (int64_t)gridDim.x * kThreads) {
+    const int64_t i = q * 4;
+    const int nv = (int)(n - i < 4 ? n - i : 4);
+    const bool v4 = vec && nv == 4;
+    const Quad a = load_quad(lp, i, v4, nv, 0.f), b = load_quad(ref, i, v4, nv, 0.f);
+    Quad o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o.v[e] = kl_token(a.v[e], b.v[e], mode, 0).v;
+    store_quad(out, i, v4, nv, o);
+  }
 }
 __global__ __launch_bounds__(kThreads) void kl_bwd_kernel(const float* __restrict__ g, const float* __restrict__ lp,
                                                           const float* __restrict__ ref, int64_t n, int mode, int st,
-                                                          float* __restrict__ d_lp, float* __restrict__ d_ref) {
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
-    const float d = g[i] * kl_token(lp[i], ref[i], mode, st).g;
-    if (d_lp) d_lp[i] = d;
-    if (d_ref) d_ref[i] = -d;  // every estimator depends on lp - ref only
+                                                          bool vec, float* __restrict__ d_lp, float* __restrict__ d_ref) {
+  const int64_t nq = (n + 3) / 4;
+  for (int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x; q < nq; q += (int64_t)gridDim.x * kThreads) {
+    const int64_t i = q * 4;
+    const int nv = (int)(n - i < 4 ? n - i : 4);
+    const bool v4 = vec && nv == 4;
+    const Quad gg = load_quad(g, i, v4, nv, 0.f), a = load_quad(lp, i, v4, nv, 0.f), b = load_quad(ref, i, v4, nv, 0.f);
+    Quad d, nd;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      d.v[e] = gg.v[e] * kl_token(a.v[e], b.v[e], mode, st).g;
+      nd.v[e] = -d.v[e];  // every estimator depends on lp - ref only
+    }
+    if (d_lp) store_quad(d_lp, i, v4, nv, d);
+    if (d_ref) store_quad(d_ref, i, v4, nv, nd);
   }
 }
 
@@ -498,23 +518,72 @@ __global__ __launch_bounds__(kThreads) void masked_finish_kernel(const float* __
   }
 }
 
+// many rows: one thread per row writes the row's results, one {sum, mask sum} record per workgroup; then one
+// workgroup folds the records (fp64 as above; the order of the additions differs from the one-level finish)
+__global__ __launch_bounds__(kThreads) void masked_rows_kernel(const float* __restrict__ partials, int nseg, int64_t B,
+                                                               float* __restrict__ row_sum,
+                                                               float* __restrict__ row_mean, double* __restrict__ rec) {
+  const int64_t b = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  double v = 0, m = 0;
+  if (b < B) {
+    for (int s = 0; s < nseg; ++s) {
+      v += partials[(b * nseg + s) * kNP + P_PG];
+      m += partials[(b * nseg + s) * kNP + P_M];
+    }
+    if (row_sum) row_sum[b] = (float)v;
+    if (row_mean) row_mean[b] = (float)(v / (m + 1e-8));
+  }
+  __shared__ double sh[kThreads / kWave + 1];
+  v = block_sum_d(v, sh);
+  m = block_sum_d(m, sh);
+  if (threadIdx.x == 0) {
+    rec[2 * (int64_t)blockIdx.x] = v;
+    rec[2 * (int64_t)blockIdx.x + 1] = m;
+  }
+}
+__global__ __launch_bounds__(kThreads) void masked_finish2_kernel(const double* __restrict__ rec, int nrec,
+                                                                  float* __restrict__ total2) {
+  double tv = 0, tm = 0;
+  for (int i = threadIdx.x; i < nrec; i += kThreads) {
+    tv += rec[2 * i];
+    tm += rec[2 * i + 1];
+  }
+  __shared__ double sh[kThreads / kWave + 1];
+  tv = block_sum_d(tv, sh);
+  tm = block_sum_d(tm, sh);
+  if (threadIdx.x == 0) {
+    total2[0] = (float)tv;
+    total2[1] = (float)(tv / (tm + 1e-8));
+  }
+}
+
 // ---------------------------------------------------------------------------- KL penalty in the reward
 
 // rewards = scores - beta * kld,  kld = kl(old, ref) * m ; row_kl[b] = masked_mean(kld, m) of the row
 __global__ __launch_bounds__(kThreads) void kl_reward_kernel(const float* __restrict__ scores,
                                                              const float* __restrict__ old_lp,
                                                              const float* __restrict__ ref, const void* mask,
-                                                             int mask_dtype, int64_t L, int kl_mode, float beta,
+                                                             int mask_dtype, int64_t L, int kl_mode, float beta, bool vec,
                                                              float* __restrict__ rewards, float* __restrict__ row_kl) {
   const int64_t b = blockIdx.x;
   float sv = 0.f, sm = 0.f;
-  for (int64_t t = threadIdx.x; t < L; t += kThreads) {
+  for (int64_t t = (int64_t)threadIdx.x * 4; t < L; t += kThreads * 4) {  // four tokens per thread and pass
     const int64_t idx = b * L + t;
-    const float m = load_mask(mask, mask_dtype, idx);
-    const float kld = kl_token(old_lp[idx], ref[idx], kl_mode, 0).v * m;
-    rewards[idx] = scores[idx] - beta * kld;
-    sv += contrib_where(kld, m);
-    sm += m;
+    const int nv = (int)(L - t < 4 ? L - t : 4);
+    const Quad m = load_mask_quad(mask, mask_dtype, idx, vec, nv);
+    const Quad o = load_quad(old_lp, idx, vec, nv, 0.f), r = load_quad(ref, idx, vec, nv, 0.f);
+    const Quad s = load_quad(scores, idx, vec, nv, 0.f);
+    Quad out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float kld = kl_token(o.v[e], r.v[e], kl_mode, 0).v * m.v[e];
+      out.v[e] = s.v[e] - beta * kld;
+      if (e < nv) {
+        sv += contrib_where(kld, m.v[e]);
+        sm += m.v[e];
+      }
+    }
+    store_quad(rewards, idx, vec, nv, out);
   }
   __shared__ float sh[kThreads / kWave + 1];
   sv = block_sum(sv, sh);
@@ -793,8 +862,10 @@ extern "C" int siirl_kl_penalty_fwd(const float* logprob, const float* ref_logpr
   SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
   if (n == 0) return SIIRL_OK;
   SIIRL_REQUIRE(logprob && ref_logprob && out, "NULL operand");
-  const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads < 8192 ? (n + kThreads - 1) / kThreads : 8192);
-  kl_fwd_kernel<<<dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream>>>(logprob, ref_logprob, n, kl_mode, out);
+  const int64_t want = ((n + 3) / 4 + kThreads - 1) / kThreads;
+  const unsigned blocks = (unsigned)(want < 16384 ? want : 16384);
+  const bool vec = (((uintptr_t)logprob | (uintptr_t)ref_logprob | (uintptr_t)out) & 15) == 0;
+  kl_fwd_kernel<<<dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream>>>(logprob, ref_logprob, n, kl_mode, vec, out);
   SIIRL_LAUNCH_CHECK("kl_fwd_kernel");
   return SIIRL_OK;
 }
@@ -806,9 +877,12 @@ extern "C" int siirl_kl_penalty_bwd(const float* g, const float* logprob, const 
   SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
   if (n == 0) return SIIRL_OK;
   SIIRL_REQUIRE(g && logprob && ref_logprob && (d_logprob || d_ref_logprob), "NULL operand");
-  const unsigned blocks = (unsigned)((n + kThreads - 1) / kThreads < 8192 ? (n + kThreads - 1) / kThreads : 8192);
+  const int64_t want = ((n + 3) / 4 + kThreads - 1) / kThreads;
+  const unsigned blocks = (unsigned)(want < 16384 ? want : 16384);
+  const bool vec = (((uintptr_t)g | (uintptr_t)logprob | (uintptr_t)ref_logprob | (uintptr_t)d_logprob |
+                     (uintptr_t)d_ref_logprob) & 15) == 0;
   kl_bwd_kernel<<<dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream>>>(g, logprob, ref_logprob, n, kl_mode,
-                                                                        straight_through, d_logprob, d_ref_logprob);
+                                                                        straight_through, vec, d_logprob, d_ref_logprob);
   SIIRL_LAUNCH_CHECK("kl_bwd_kernel");
   return SIIRL_OK;
 }
@@ -831,12 +905,25 @@ extern "C" int siirl_masked_reduce(const float* values, const void* mask, int ma
   if (workspace_bytes < ws_bytes_of(B, L) || workspace == nullptr)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes,
                 ws_bytes_of(B, L));
+  SIIRL_REQUIRE(((uintptr_t)workspace & 7) == 0, "workspace must be 8-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   float* partials = (float*)workspace;
   set_vec(a);
   if (int rc = launch_loss_partials(a, nullptr, partials, st)) return rc;
-  masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, total2);
-  SIIRL_LAUNCH_CHECK("masked_finish_kernel");
+  if (B <= kTwoLevelRows) {
+    masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, total2);
+    SIIRL_LAUNCH_CHECK("masked_finish_kernel");
+    return SIIRL_OK;
+  }
+  const size_t used = ((size_t)B * a.nseg * (kNP + kNPre) * sizeof(float) + 255) / 256 * 256;
+  double* rec = reinterpret_cast<double*>((char*)workspace + used);  // room for kFinRec >= 2 doubles per workgroup
+  const int nrec = (int)((B + kThreads - 1) / kThreads);
+  masked_rows_kernel<<<dim3((unsigned)nrec), dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, rec);
+  SIIRL_LAUNCH_CHECK("masked_rows_kernel");
+  if (total2) {
+    masked_finish2_kernel<<<1, dim3(kThreads), 0, st>>>(rec, nrec, total2);
+    SIIRL_LAUNCH_CHECK("masked_finish2_kernel");
+  }
   return SIIRL_OK;
 }
 
@@ -851,9 +938,13 @@ extern "C" int siirl_kl_in_reward(const float* token_level_scores, const float* 
                                           token_level_rewards && row_kl)), "NULL operand");
   hipStream_t st = (hipStream_t)stream;
   if (B > 0) {  // an empty batch has no rewards to write; its mean KL is the mean of nothing (NaN)
+    LossArgs a{};  // only to decide whether rows can move as 16-byte quads
+    a.old_lp = old_log_prob; a.ref = ref_log_prob; a.adv = token_level_scores; a.mask = mask; a.mask_dtype = mask_dtype;
+    a.L = L;
+    set_vec(a, token_level_rewards);
     kl_reward_kernel<<<dim3((unsigned)B), dim3(kThreads), 0, st>>>(token_level_scores, old_log_prob, ref_log_prob, mask,
-                                                                  mask_dtype, L, kl_mode, beta, token_level_rewards,
-                                                                  row_kl);
+                                                                  mask_dtype, L, kl_mode, beta, a.vec != 0,
+                                                                  token_level_rewards, row_kl);
     SIIRL_LAUNCH_CHECK("kl_reward_kernel");
   }
   mean_rows_kernel<<<1, dim3(kThreads), 0, st>>>(row_kl, B, current_kl);

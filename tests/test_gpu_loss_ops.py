@@ -404,3 +404,63 @@ def test_compute_entropy_loss(dev, mode):
     got.backward()
     want.backward()
     assert (xd.grad.cpu().double() - x64.grad).abs().max() < 1e-6
+
+
+@pytest.mark.parametrize("B,L", [(3, 37), (5, 1030), (4, 1031), (2, 4096), (1, 1)])
+@pytest.mark.parametrize("mdt", [torch.int64, torch.bool, torch.float32])
+def test_kl_in_reward_shapes(dev, B, L, mdt):
+    """apply_kl_penalty over row lengths that take the 16-byte path, the scalar tail and several passes per row."""
+    import siirl_amd.core_algos as CA
+
+    lp, old, ref, _, mask, _ = _batch(B, L, seed=B * 7 + L)
+    scores = torch.randn(B, L)
+    for kind in ("kl", "low_var_kl"):
+        data = {"token_level_scores": scores.to(dev), "old_log_probs": old.to(dev), "ref_log_prob": ref.to(dev),
+                "response_mask": mask.to(dev).to(mdt)}
+        data, metrics = CA.apply_kl_penalty(data, CA.FixedKLController(0.07), kl_penalty=kind)
+        odata = {"token_level_scores": scores.clone(), "old_log_probs": old, "ref_log_prob": ref, "response_mask": mask}
+        odata, ometrics = OC.apply_kl_penalty(odata, OC.FixedKLController(0.07), kind)
+        assert (data["token_level_rewards"].cpu() - odata["token_level_rewards"]).abs().max() < 1e-5
+        assert abs(metrics["actor/reward_kl_penalty"] - ometrics["actor/reward_kl_penalty"]) < 1e-5
+
+
+@pytest.mark.parametrize("B,L", [(2049, 33), (5000, 130), (2048, 64)])
+def test_masked_reductions_many_rows(dev, B, L):
+    """Above 2048 rows the per-row results and the totals are folded in two levels."""
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(B + L)
+    v = torch.randn(B, L, generator=g)
+    m = (torch.rand(B, L, generator=g) > 0.3).long()
+    m[B // 2] = 0
+    vd, md = v.to(dev), m.to(dev)
+    assert _close(SF.masked_sum(vd, md), OF.masked_sum(v.double(), m), 1e-3)
+    assert _close(SF.masked_mean(vd, md), OF.masked_mean(v.double(), m))
+    got = SF.masked_mean(vd, md, axis=-1).cpu().double()
+    assert (got - OF.masked_mean(v.double(), m, axis=-1)).abs().max() < 2e-5 and float(got[B // 2]) == 0.0
+    got = SF.masked_sum(vd, md, axis=-1).cpu().double()
+    assert (got - OF.masked_sum(v.double(), m, axis=-1)).abs().max() < 2e-4
+
+
+@pytest.mark.parametrize("n,offset", [(1501, 0), (1501, 1), (4096, 3), (2, 0), (262147, 0)])
+def test_kl_penalty_lengths_and_alignment(dev, n, offset):
+    """Element counts with a tail after the 16-byte groups, and operands that start off a 16-byte boundary."""
+    import siirl_amd.core_algos as CA
+
+    g = torch.Generator().manual_seed(n + offset)
+    lp_full, ref_full = torch.randn(n + offset, generator=g) - 1.0, torch.randn(n + offset, generator=g) - 1.0
+    w_full = torch.randn(n + offset, generator=g)
+    lp, ref, w = lp_full[offset:], ref_full[offset:], w_full[offset:]
+    x = lp_full.to(dev)[offset:].requires_grad_(True)
+    r = ref_full.to(dev)[offset:].requires_grad_(True)
+    for kind in ("low_var_kl", "mse"):
+        x.grad = r.grad = None
+        out = CA.kl_penalty(x, r, kind)
+        x64, r64 = lp.double().requires_grad_(True), ref.double().requires_grad_(True)
+        want = OC.kl_penalty(x64, r64, kind)
+        assert out.shape == (n,) and ((out.cpu().double() - want).abs() <= 2e-5 + 1e-6 * want.abs()).all()
+        out.backward(w_full.to(dev)[offset:])
+        want.backward(w.double())
+        for got, ref64 in ((x.grad, x64.grad), (r.grad, r64.grad)):
+            ok, err = _grad_close(got.cpu(), ref64)
+            assert ok, (kind, err)

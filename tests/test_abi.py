@@ -101,3 +101,19 @@ def test_argument_validation_without_gpu():
         L.check(-2, "x")
     with pytest.raises(L.SiirlHipError):
         L.check(-3, "x")
+
+
+def test_size_queries_agree_with_the_host_side():
+    """Pure size arithmetic (no GPU): the buffer the Python layer plans for the parked logits is the one the library
+    asks for, and the backward scratch grows with the requested gradients."""
+    L = _lib()
+    h = L.lib()
+    import siirl_amd.fused_linear as FL
+
+    for T, V in ((1, 1), (256, 256), (257, 255), (16384, 152064), (70, 500)):
+        assert h.siirl_fused_linear_saved_logits_bytes(T, V) == FL._saved_logits_bytes(T, V)
+    assert h.siirl_fused_linear_saved_logits_bytes(0, 5) == 0
+    both = h.siirl_fused_linear_bwd_workspace_bytes(512, 128, 4096, 1, 1)
+    assert both > h.siirl_fused_linear_bwd_workspace_bytes(512, 128, 4096, 1, 0) > 0
+    assert both > h.siirl_fused_linear_bwd_workspace_bytes(512, 128, 4096, 0, 1) > 0
+    assert h.siirl_fused_linear_fwd_workspace_bytes(512, 128, 4096) > 512 * 128 * 2

@@ -569,12 +569,25 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const uint16_t* __restrict_
 // 64 x 64 tile through LDS and emits its 512 chunks.
 __global__ __launch_bounds__(256) void transpose_pack_b_kernel(const uint16_t* __restrict__ in, int64_t ld_in, int R,
                                                                int C, u32x4* __restrict__ out, int64_t KB) {
-  __shared__ uint16_t tile[64][66];
+  __shared__ __align__(16) uint16_t tile[64][72];  // 144-byte rows: 16-byte aligned, 36 dwords (column reads spread)
   const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;  // r = k, c = n
-  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
-  for (int rr = ty; rr < 64; rr += 4) {
-    const int r = r0 + rr, cc = c0 + tx;
-    tile[rr][tx] = (r < R && cc < C) ? in[(int64_t)r * ld_in + cc] : (uint16_t)0;
+  // 16 bytes (8 columns) per thread and pass, 8 threads per row, 32 rows per pass; ld_in and c0 are multiples of 8
+  for (int q = threadIdx.x; q < 512; q += 256) {
+    const int rr = q >> 3, cc = (q & 7) * 8;
+    const int r = r0 + rr, c = c0 + cc;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (r < R) {
+      if (c + 8 <= C) {
+        v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(in + (int64_t)r * ld_in + c));
+      } else if (c < C) {
+        uint16_t t[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = c + e < C ? in[(int64_t)r * ld_in + c + e] : (uint16_t)0;
+        v = u32x4{(uint32_t)t[0] | ((uint32_t)t[1] << 16), (uint32_t)t[2] | ((uint32_t)t[3] << 16),
+                  (uint32_t)t[4] | ((uint32_t)t[5] << 16), (uint32_t)t[6] | ((uint32_t)t[7] << 16)};
+      }
+    }
+    *reinterpret_cast<u32x4*>(&tile[rr][cc]) = v;
   }
   __syncthreads();
   for (int q = threadIdx.x; q < 512; q += 256) {

@@ -287,7 +287,8 @@ __device__ __forceinline__ f32x4* saved_tile(float* base, int tm, int tn, int ti
 // epilogue with vocabulary row m0 counted from the first tile row of the launch.  (Measured at T=16384, V=152064:
 // 0.87 ms per 32768 columns (launches take 65536), 4.9 TB/s of its 8 bytes per logit, arithmetic and LDS writes about level with the
 // memory time; splitting the workgroup into its two rows of waves, each with half the LDS image so that two share
-// a CU, was 15 % slower.)
+// a CU, was 15 % slower, and 256 persistent workgroups that issue the next tile's loads before draining the LDS
+// image were 27 % slower.)
 template <class Epi>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void replay_tiles_kernel(
     const float* __restrict__ saved, int tiles_n, int tm_first, Epi epi) {

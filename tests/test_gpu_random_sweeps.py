@@ -108,3 +108,126 @@ def test_sweep_grpo_advantage_random_groups(dev):
         err = (got.cpu().double() - want.double()).abs()
         assert bool((err <= 1e-6 + 1e-5 * want.double().abs()).all()), (case, B, L, norm, err.max().item())
         assert bool((got.cpu()[mask == 0] == 0).all()), case
+
+
+# ----------------------------------------------------------------------------------- floating-point parts
+
+AGGS = ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"]
+
+
+def _loss_case(rng, case):
+    from types import SimpleNamespace
+
+    B, L = int(rng.integers(1, 20)), int(rng.integers(1, 600))
+    g = torch.Generator().manual_seed(int(rng.integers(1 << 30)))
+    lp = torch.randn(B, L, generator=g) - 1.5
+    old = lp + float(rng.choice([0.0, 0.05, 0.5, 3.0])) * torch.randn(B, L, generator=g)
+    adv = torch.randn(B, L, generator=g) * float(rng.choice([0.1, 1.0, 10.0]))
+    if case % 4 == 0:
+        adv[:, ::3] = 0.0
+    lens = torch.from_numpy(rng.integers(0 if case % 5 == 0 else 1, L + 1, B))
+    mask = (torch.arange(L)[None, :] < lens[:, None])
+    if case % 3 == 0:  # holes inside the responses
+        mask = mask & (torch.rand(B, L, generator=g) > 0.2)
+    mdt = [torch.int64, torch.bool, torch.float32, torch.int32][case % 4]
+    lo, hi = float(rng.choice([0.1, 0.2, 3e-4])), float(rng.choice([0.2, 0.28, 4e-4]))
+    cfg = SimpleNamespace(clip_ratio=lo, clip_ratio_low=lo, clip_ratio_high=hi, clip_ratio_c=float(rng.choice([1.5, 3.0, 10.0])))
+    isw = torch.rand(B, L, generator=g) + 0.5 if case % 6 == 0 else None
+    return B, L, lp, old, adv, mask.to(mdt), cfg, isw
+
+
+@pytest.mark.parametrize("loss", ["vanilla", "gspo"])
+def test_sweep_policy_loss(dev, loss):
+    """Random shapes, masks (empty rows, holes, every dtype), clip ranges and aggregation modes: the four returned
+    scalars within 2e-5 + 1e-5 relative of the fp64 oracle, d loss / d log_prob within 1e-6 + 1e-5 relative."""
+    import siirl_amd.core_algos as CA
+
+    rng = np.random.default_rng(201 if loss == "vanilla" else 202)
+    ofn = OC.compute_policy_loss_vanilla if loss == "vanilla" else OC.compute_policy_loss_gspo
+    fn = CA.compute_policy_loss_vanilla if loss == "vanilla" else CA.compute_policy_loss_gspo
+    for case in range(80):
+        B, L, lp, old, adv, mask, cfg, isw = _loss_case(rng, case)
+        mode = AGGS[case % 4]
+        if mode == "seq-mean-token-mean" or loss == "gspo":
+            mask = mask.clone()
+            mask[:, 0] = 1  # an all-masked row makes this mode NaN in the reference too; covered elsewhere
+        x64 = lp.double().requires_grad_(True)
+        want = ofn(old.double(), x64, adv.double(), mask.double() if mask.dtype != torch.bool else mask, mode, cfg,
+                   None if isw is None else isw.double())
+        x = lp.to(dev).requires_grad_(True)
+        got = fn(old.to(dev), x, adv.to(dev), mask.to(dev), mode, cfg, None if isw is None else isw.to(dev))
+        for k, (a, b) in enumerate(zip(got, want)):
+            assert abs(float(a) - float(b)) <= 2e-5 + 1e-5 * abs(float(b)), (case, loss, mode, k, float(a), float(b))
+        if float(mask.double().sum()) > 0:
+            got[0].backward()
+            want[0].backward()
+            err = (x.grad.cpu().double() - x64.grad).abs()
+            assert bool((err <= 1e-6 + 1e-5 * x64.grad.abs()).all()), (case, loss, mode, err.max().item())
+
+
+def test_sweep_gae_and_value_loss(dev):
+    import siirl_amd.core_algos as CA
+
+    rng = np.random.default_rng(203)
+    for case in range(60):
+        B, L = int(rng.integers(1, 40)), int(rng.integers(1, 700))
+        g = torch.Generator().manual_seed(case)
+        rewards, values = torch.randn(B, L, generator=g), torch.randn(B, L, generator=g)
+        lens = torch.from_numpy(rng.integers(1, L + 1, B))
+        mask = (torch.arange(L)[None, :] < lens[:, None]).long()
+        if B * L < 3 or int(mask.sum()) < 2:
+            continue
+        gamma, lam = float(rng.choice([1.0, 0.99, 0.9])), float(rng.choice([1.0, 0.95, 0.5]))
+        a_o, r_o = OC.compute_gae_advantage_return(rewards.double(), values.double(), mask, gamma, lam)
+        a, r = CA.compute_gae_advantage_return(rewards.to(dev), values.to(dev), mask.to(dev), gamma, lam)
+        scale = max(1.0, float(a_o.abs().max()))
+        assert (a.cpu().double() - a_o).abs().max() <= 2e-4 * scale, (case, B, L, gamma, lam)
+        assert (r.cpu().double() - r_o).abs().max() <= 1e-4 * max(1.0, float(r_o.abs().max())), (case, B, L)
+        mode = AGGS[case % 4]
+        vp64 = (values + 0.3 * torch.randn(B, L, generator=g)).double().requires_grad_(True)
+        want = OC.compute_value_loss(vp64, r_o, values.double(), mask.double(), 0.2, mode)
+        vp = vp64.detach().float().to(dev).requires_grad_(True)
+        got = CA.compute_value_loss(vp, r_o.float().to(dev), values.to(dev), mask.to(dev), 0.2, mode)
+        for a1, b1 in zip(got, want):
+            assert abs(float(a1) - float(b1)) <= 2e-5 + 2e-5 * abs(float(b1)), (case, mode, float(a1), float(b1))
+        got[0].backward()
+        want[0].backward()
+        err = (vp.grad.cpu().double() - vp64.grad).abs()
+        assert bool((err <= 1e-6 + 2e-5 * vp64.grad.abs()).all()), (case, mode, err.max().item())
+
+
+def test_sweep_logprob_entropy(dev):
+    """Random row counts, vocabulary sizes (odd, tiny, beyond one workgroup pass), dtypes, temperatures and row-strided
+    views: log-prob and entropy within 1e-3 of the fp32 oracle, dlogits within 1 ulp of the logits dtype of the fp64
+    oracle, plus the absolute error that fp32 rounding of lse and E[z] leaves (about 2^-23 * max|z| * |g|)."""
+    import siirl_amd.torch_functional as SF
+    from oracle import torch_functional as OF
+
+    rng = np.random.default_rng(204)
+    for case in range(90):
+        T = int(rng.integers(1, 50))
+        V = int(rng.choice([1, 2, 3, 7, 64, 255, 256, 257, 1000, 4097, 8191, 32000, 40001, int(rng.integers(1, 70000))]))
+        dt = [torch.bfloat16, torch.float32, torch.float16][case % 3]
+        temp = float(rng.choice([1.0, 0.6, 1.7]))
+        g = torch.Generator().manual_seed(case)
+        pad = int(rng.choice([0, 0, 8, 5]))
+        base = (torch.randn(T, V + pad, generator=g) * float(rng.choice([0.5, 3.0, 8.0]))).to(dt)
+        x = base[:, :V]  # a row-strided view when pad > 0
+        y = torch.randint(0, V, (T,), generator=g)
+        g_lp, g_h = torch.randn(T, generator=g), torch.randn(T, generator=g)
+        xd = base.to(dev)[:, :V].detach().requires_grad_(True)
+        lp, ent = SF.logprobs_and_entropy_from_logits(xd, y.to(dev), temperature=temp)
+        lp_o, ent_o, _, _ = OF.logprob_entropy_forward(x, y, temp, dtype=torch.float32)
+        assert (lp.detach().cpu() - lp_o).abs().max() < 1e-3 and (ent.detach().cpu() - ent_o).abs().max() < 1e-3, (case, T, V, dt)
+        torch.autograd.backward([lp, ent], [g_lp.to(dev), g_h.to(dev)])
+        d64 = OF.logprob_entropy_backward(x, y, g_lp, g_h, temp, dtype=torch.float64)
+        got = xd.grad.cpu()
+        assert got.dtype == dt and got.shape == (T, V)
+        eps = {torch.bfloat16: 2.0 ** -8, torch.float16: 2.0 ** -11, torch.float32: 2.0 ** -23}[dt]
+        # fp32 arithmetic rounds lse and E[z] to about 2^-23 * max|z|; where the softmax is saturated that is an
+        # absolute error of p, hence of the gradient, of that size times the upstream gradients
+        zmax = (x.double().abs().max(dim=-1).values / temp).unsqueeze(-1)
+        fp32_abs = 2.4e-7 * zmax * (g_lp.double().abs() + g_h.double().abs() * (1 + zmax)).unsqueeze(-1) / temp
+        tol = 2 * eps * d64.abs() + 1e-6 + fp32_abs + (1e-5 * d64.abs() if dt == torch.float32 else 0)
+        err = (got.double() - d64).abs()
+        assert bool((err <= tol).all()), (case, T, V, dt, temp, float((err - tol).max()))

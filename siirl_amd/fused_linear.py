@@ -8,7 +8,8 @@
 
 Both run the MFMA kernels of ``csrc/fused_linear.hip`` through the C ABI.  Operands are bf16 on the GPU.  The
 forward needs no ``[T, V]`` tensor.  When a backward will follow and the buffer fits the limit set with
-``set_saved_logits_limit`` (default 16 GiB; 4 bytes per logit), the forward parks its fp32 logit tiles and the
+``set_saved_logits_limit`` (default 16 GiB, or ``SIIRL_AMD_SAVED_LOGITS_LIMIT`` bytes from the environment; 4 bytes
+per logit), the forward parks its fp32 logit tiles and the
 backward reads them back instead of running the projection a second time: the same bits, a quarter less matrix
 work per step.  With the limit at 0 the logits are never stored and the backward recomputes them slab by slab,
 which is the reference's memory behaviour.  Outputs are fp32 (the reference's Triton path returns fp32,
@@ -19,6 +20,7 @@ kernel's business.
 
 from __future__ import annotations
 
+import os
 import typing
 
 import torch
@@ -26,7 +28,8 @@ import torch
 from . import ops as _ops_module  # noqa: F401  (registers torch.ops.siirl_hip.*)
 
 
-_SAVED_LOGITS_LIMIT = 16 << 30
+# bytes; the environment variable gives a deployment its own default without code changes
+_SAVED_LOGITS_LIMIT = int(os.environ.get("SIIRL_AMD_SAVED_LOGITS_LIMIT", 16 << 30))
 
 
 def set_saved_logits_limit(nbytes: int) -> None:

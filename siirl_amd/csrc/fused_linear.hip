@@ -628,18 +628,20 @@ __global__ __launch_bounds__(256) void label_logit_kernel(const uint16_t* __rest
   if (lane == 0) out[row] = s * inv_T;
 }
 
-// folds the per-tile partials of each token: lse, ex, entropy, logprob.  A workgroup handles 64 tokens; four
-// thread groups each merge every fourth tile online, then the four states are merged through LDS.
+// folds the per-tile partials of each token: lse, ex, entropy, logprob.  A workgroup handles kMergeTok tokens;
+// kMergeGrp thread groups each merge every kMergeGrp-th tile online, then the states are merged through LDS.
+constexpr int kMergeTok = 16, kMergeGrp = 16;
+static_assert(kMergeTok * kMergeGrp == 256, "one thread per (token, group)");
 __global__ __launch_bounds__(256) void merge_partials_kernel(const float* __restrict__ part, int nparts, int T,
                                                              const float* __restrict__ label_logit,
                                                              float* __restrict__ logprob, float* __restrict__ entropy,
                                                              float* __restrict__ lse_out, float* __restrict__ ex_out) {
-  __shared__ float sh[4][64][3];
-  const int tl = threadIdx.x & 63, grp = threadIdx.x >> 6;
-  const int row = blockIdx.x * 64 + tl;
+  __shared__ float sh[kMergeGrp][kMergeTok][3];
+  const int tl = threadIdx.x % kMergeTok, grp = threadIdx.x / kMergeTok;
+  const int row = blockIdx.x * kMergeTok + tl;
   float M = -__builtin_inff(), s = 0.f, t = 0.f;
   if (row < T) {
-    for (int p = grp; p < nparts; p += 4) {
+    for (int p = grp; p < nparts; p += kMergeGrp) {
       const float* q = part + (int64_t)p * 3 * T;
       const float m = q[row];
       if (m > -__builtin_inff()) {
@@ -658,10 +660,10 @@ __global__ __launch_bounds__(256) void merge_partials_kernel(const float* __rest
   if (grp != 0 || row >= T) return;
   float Mx = M;
 #pragma unroll
-  for (int g = 1; g < 4; ++g) Mx = fmaxf(Mx, sh[g][tl][0]);
+  for (int g = 1; g < kMergeGrp; ++g) Mx = fmaxf(Mx, sh[g][tl][0]);
   double ss = 0.0, tt = 0.0;
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
+  for (int g = 0; g < kMergeGrp; ++g) {
     const float m = sh[g][tl][0];
     if (m > -__builtin_inff()) {
       const float f = fast_exp2((m - Mx) * kLog2e);
@@ -817,7 +819,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part, saved_logits, (int)((T + BN - 1) / BN)};
   if (int rc = launch_gemm(w, H, hp, H / 16, (int)V, (int)T, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
   const int tiles_v = (int)((V + BM - 1) / BM);
-  merge_partials_kernel<<<dim3((unsigned)((T + 63) / 64)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
+  merge_partials_kernel<<<dim3((unsigned)((T + kMergeTok - 1) / kMergeTok)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
                                                                                logprob, entropy, lse, ex);
   SIIRL_LAUNCH_CHECK("merge_partials_kernel");
   return SIIRL_OK;

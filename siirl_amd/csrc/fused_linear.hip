@@ -1,5 +1,6 @@
 // lm_head projection fused with log-prob / entropy: logits = hidden[T,H] . W[V,H]^T are produced tile by tile on
-// the matrix cores and consumed in the epilogue, never written to memory.
+// the matrix cores and consumed in the epilogue; no [T, V] tensor is needed (the forward may park its tiles for the
+// backward, see below).
 //
 // Replaces FusedLinearForPPO (siirl/utils/experimental/torch_functional.py:20-211) and linear_cross_entropy
 // (siirl/utils/kernel/linear_cross_entropy.py:40-117 -> siirl/utils/kernel/kernels.py:507-696,1378-1586); the

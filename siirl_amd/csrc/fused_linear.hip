@@ -289,7 +289,7 @@ __device__ __forceinline__ f32x4* saved_tile(float* base, int tm, int tn, int ti
 // 0.87 ms per 32768 columns (launches take 65536), 4.9 TB/s of its 8 bytes per logit, arithmetic and LDS writes about level with the
 // memory time; splitting the workgroup into its two rows of waves, each with half the LDS image so that two share
 // a CU, was 15 % slower, and 256 persistent workgroups that issue the next tile's loads before draining the LDS
-// image were 27 % slower.)
+// image were 17-27 % slower, with full barriers or with barriers that order the LDS only.)
 template <class Epi>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void replay_tiles_kernel(
     const float* __restrict__ saved, int tiles_n, int tm_first, Epi epi) {

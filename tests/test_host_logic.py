@@ -104,3 +104,28 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_response_window_helpers_refuse_the_cpu_and_bad_arguments():
+    """The helpers of siirl/utils/model_utils/torch_functional.py:209-254,416-500,638-647: CPU tensors raise (no CPU
+    fallback), argument errors surface before any device work; remove_pad_token is host-side list building."""
+    import siirl_amd.fused_linear as FL
+    import siirl_amd.torch_functional as SF
+    from oracle import padding as OP
+
+    ids = torch.tensor([[5, 1, 0, 0], [7, 8, 9, 1]])
+    with pytest.raises(RuntimeError, match="GPU only"):
+        SF.get_response_mask(ids, 1)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        SF.get_eos_mask(ids, 1)
+    with pytest.raises(RuntimeError):
+        SF.get_unpad_data(torch.ones(2, 4, dtype=torch.long))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        SF.log_probs_from_logits_response(ids, torch.zeros(2, 4, 11), 2)
+    mask = torch.tensor([[0, 0, 1, 1], [1, 1, 1, 1]])
+    assert SF.remove_pad_token(ids, mask) == OP.remove_pad_token(ids.numpy(), mask.numpy()) == [[0, 0], [7, 8, 9, 1]]
+    with pytest.raises(RuntimeError, match="GPU only"):
+        FL.fused_linear_logprob_entropy(torch.zeros(2, 64, dtype=torch.bfloat16), torch.zeros(9, 64, dtype=torch.bfloat16),
+                                        torch.zeros(2, dtype=torch.long))
+    with pytest.raises(ValueError):
+        FL.set_saved_logits_limit(-5)

@@ -60,6 +60,13 @@ compute_data_metric                    numpy mean / max / min / var(ddof=1) of t
 merge_leftover / place_outcome_reward  the reference's leftover-cache test vectors
                                        (tests/dag_worker/test_dapo_pipeline.py:145-195); hand-computed
                                        penalties either side of the expected length
+micro_batch_step                       closed-form uniform-logits case written out with ``math``; a
+                                       torch-free scalar restatement of dp_actor.py:425-513: equal
+                                       loss, ``dlogits`` == its central differences (vanilla with
+                                       every aggregation, gspo, cpgd + drift, entropy / KL terms,
+                                       importance weights, on-policy); metric scalings
+compute_entropy_loss                   uniform rows -> log V under each aggregation;
+                                       ``Categorical.entropy`` aggregated by hand
 fused_linear_for_ppo_fwd / _bwd        equals logprob/entropy of ``(h @ W.T)/T`` in fp64 and
                                        autograd through that expression
 =====================================  ==========================================================

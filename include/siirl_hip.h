@@ -73,7 +73,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1001
+#define SIIRL_HIP_ABI_VERSION 1002
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -235,7 +235,27 @@ int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_prob, const
                          size_t workspace_bytes, siirl_stream_t stream);
 
 /*
- * Backward of the above for an upstream gradient g_loss[0] (device scalar) on out16[SIIRL_OUT_LOSS]:
+ * siirl_actor_loss_fwd for callers that cannot allocate or bring a workspace (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same operands, same kernels, same results bit for bit,
+ * with the scratch taken from a buffer of SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES that is part of the library's
+ * device image (one copy per GPU, held until the process ends).  The call allocates nothing and frees nothing.
+ * A [B, L] problem whose siirl_loss_workspace_bytes(B, L) exceeds the buffer (64 bytes per 2048-token segment of a
+ * row: about 65 000 segments) is refused with SIIRL_ERR_WORKSPACE.  All calls on one GPU share the buffer: calls
+ * that overlap in time on one GPU (different streams or threads) race; calls on one stream do not.  The first
+ * call on each GPU looks the buffer's address up (hipGetSymbolAddress) and must happen outside stream capture.
+ * This entry point has no counterpart in the reference.
+ */
+#define SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES (4u << 20)
+int siirl_actor_loss_fwd_static(const float* old_log_prob, const float* log_prob, const float* advantages,
+                                const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
+                                const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
+                                float clip_high, float clip_c, float log_ratio_clamp, int agg_mode,
+                                float entropy_coeff, int kl_mode, int kl_straight_through, float kl_coef,
+                                float policy_drift_coeff, float loss_scale, float* out16, float* row_msum,
+                                float* row_s, siirl_stream_t stream);
+
+/*
+ * Backward of siirl_actor_loss_fwd for an upstream gradient g_loss[0] (device scalar) on out16[SIIRL_OUT_LOSS]:
  * d_log_prob[B, L] and, when entropy was given, d_entropy[B, L].  Ties follow autograd: maximum / minimum
  * split the gradient 1/2 : 1/2, clamp passes it on the closed interval.
  */

@@ -15,6 +15,15 @@
 #include "common.hpp"
 #include "loss_token.hpp"
 
+#include <mutex>
+
+// Scratch of siirl_actor_loss_fwd_static, the entry point that allocates nothing: the segment partials, the row
+// pre-pass sums and the finish records that the other forward entry points take from the caller's workspace.  One
+// copy per GPU, held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress;
+// kernels receive the device address that call returns.
+constexpr size_t kStaticScratchBytes = SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
 namespace siirl {
 namespace {
 
@@ -797,6 +806,53 @@ extern "C" int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_
   SIIRL_REQUIRE(B == 0 || (loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
                 "row_s is required for the gspo and geo_mean losses");
   return run_forward(a, out16, row_msum, row_s, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+// Device address of `scratch` on each GPU, looked up on the first call made with that GPU current.
+constexpr int kMaxDevices = 64;
+static void* g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mu;
+
+static int static_scratch_address(void** out) {
+  int dev = -1;
+  SIIRL_HIP_CHECK(hipGetDevice(&dev));
+  SIIRL_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d is outside [0, %d)", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    SIIRL_HIP_CHECK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    SIIRL_REQUIRE(p != nullptr && ((uintptr_t)p & 255) == 0, "static scratch resolved to %p", p);
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_actor_loss_fwd_static(const float* old_log_prob, const float* log_prob, const float* advantages,
+                                           const void* mask, int mask_dtype, const float* is_weights,
+                                           const float* entropy, const float* ref_log_prob, int64_t B, int64_t L,
+                                           int loss_mode, float clip_low, float clip_high, float clip_c,
+                                           float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode,
+                                           int kl_straight_through, float kl_coef, float policy_drift_coeff,
+                                           float loss_scale, float* out16, float* row_msum, float* row_s,
+                                           siirl_stream_t stream) {
+  LossArgs a{};
+  if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
+                               ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode,
+                               entropy_coeff, kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale))
+    return rc;
+  SIIRL_REQUIRE(out16 && (B == 0 || row_msum), "NULL output");
+  SIIRL_REQUIRE(B == 0 || (loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
+                "row_s is required for the gspo and geo_mean losses");
+  const size_t need = B == 0 ? 0 : ws_bytes_of(B, L);
+  if (need > kStaticScratchBytes)
+    return fail(SIIRL_ERR_WORKSPACE,
+                "B=%lld x L=%lld needs %zu bytes of scratch, the static buffer holds %zu: use siirl_actor_loss_fwd "
+                "with a workspace of the caller's", (long long)B, (long long)L, need, kStaticScratchBytes);
+  void* ws = nullptr;
+  if (int rc = static_scratch_address(&ws)) return rc;
+  // every scratch slot that the finish kernels read is written by this call's earlier kernels: nothing to clear
+  return run_forward(a, out16, row_msum, row_s, ws, kStaticScratchBytes, (hipStream_t)stream);
 }
 
 extern "C" int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const float* log_prob,

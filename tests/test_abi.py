@@ -42,6 +42,10 @@ def test_header_symbols_are_exported_and_bound():
 def test_every_entry_point_cites_the_reference():
     text = open(HEADER).read()
     for n in _declared():
+        if n == "siirl_actor_loss_fwd_static":  # the allocation-free variant: says that the reference has no such thing
+            pos = text.index(n + "(")
+            assert "no counterpart in the reference" in text[text.rfind("/*", 0, pos):pos]
+            continue
         if n in ("siirl_hip_abi_version", "siirl_hip_last_error", "siirl_agg_loss_bwd", "siirl_actor_loss_bwd",
                  "siirl_kl_penalty_bwd") or n.endswith("_workspace_bytes") or n.endswith("_logits_bytes"):
             continue  # utilities and backward halves documented with their forward
@@ -77,6 +81,10 @@ def test_argument_validation_without_gpu():
     assert b"Unsupported loss mode" in h.siirl_hip_last_error()
     assert h.siirl_actor_loss_fwd(p, p, p, p, L.F32, None, None, None, 2, 4, 4, 0.2, 0.2, 3.0, 20.0, 0, 0.0, 0, 0, 0.0,
                                   0.0, 1.0, p, p, None, p, 1 << 20, None) == -1  # geo_mean needs row_s
+    # the allocation-free variant refuses what its fixed buffer cannot hold, before any device call
+    assert h.siirl_actor_loss_fwd_static(p, p, p, p, L.F32, None, None, None, 1 << 20, 4096, 0, 0.2, 0.2, 3.0, 20.0, 0,
+                                         0.0, 0, 0, 0.0, 0.0, 1.0, p, p, p, None) == -4
+    assert b"static buffer" in h.siirl_hip_last_error()
     assert h.siirl_value_loss_fwd(p, p, p, p, L.F32, 2, 4, 0.5, 7, p, p, p, 1 << 20, None) == -1
     assert h.siirl_gae_advantage_return(p, p, p, L.F32, 2, 4, 1.0, 1.0, p, p, p, p, 8, 0, None) == -1  # adv == returns
     q2 = ctypes.c_void_p(p.value + 64)

@@ -742,6 +742,109 @@ def bench_glue(args, dev):
     print(json.dumps(out), flush=True)
 
 
+def bench_host(args, dev):
+    """Host time per call of the drop-in functions (the cost of the boundary itself): operands small enough that
+    the GPU is never the bottleneck, the host clock read before any synchronisation.  One line of JSON: microseconds
+    per call, forward alone (no graph), forward in grad mode, and forward + ``backward()``; then the ten-call
+    micro-batch body of the reference actor (siirl/engine/actor/dp_actor.py:403-501) as one figure.  Not a
+    throughput benchmark and not the headline."""
+    import torch
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator(device=dev).manual_seed(SEED)
+    B, L, V = 8, 256, 512
+    lens = torch.randint(16, L + 1, (B,), device=dev, generator=g)
+    mask = (torch.arange(L, device=dev)[None] < lens[:, None]).long()
+    lp_leaf = (torch.randn(B, L, device=dev, generator=g) - 1.5).requires_grad_(True)
+    old = lp_leaf.detach() + 0.05 * torch.randn(B, L, device=dev, generator=g)
+    ref = lp_leaf.detach() + 0.1 * torch.randn(B, L, device=dev, generator=g)
+    adv = torch.randn(B, L, device=dev, generator=g)
+    logits = (torch.randn(B, L, V, device=dev, generator=g) * 2).requires_grad_(True)
+    labels = torch.randint(0, V, (B, L), device=dev, generator=g)
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.2, clip_ratio_c=3.0, entropy_coeff=0.01,
+                          use_kl_loss=True, kl_loss_coef=0.001, kl_loss_type="low_var_kl", loss_agg_mode="token-mean",
+                          loss_mode="vanilla")
+    ns = torch.ops.siirl_hip
+    f32 = lp_leaf.detach()
+    calls = {
+        "torch.ops.siirl_hip.logprob_entropy_fwd": lambda: ns.logprob_entropy_fwd(logits.detach(), labels, 1.0, True),
+        "torch.ops.siirl_hip.policy_loss_fwd": lambda: ns.policy_loss_fwd(old, f32, adv, mask, None, None, ref, 0, 0.2,
+                                                                          0.2, 3.0, 20.0, 0, 0.0, 3, False, 0.001, 0.0,
+                                                                          1.0),
+        "torch.ops.siirl_hip.kl_penalty_fwd": lambda: ns.kl_penalty_fwd(f32, ref, 3),
+        "torch.ops.siirl_hip.agg_loss_fwd": lambda: ns.agg_loss_fwd(f32, mask, 0),
+        "logprobs_from_logits": lambda: SF.logprobs_from_logits(logits, labels, inplace_backward=False),
+        "entropy_from_logits (own pass)": lambda: SF.entropy_from_logits(logits),
+        "compute_policy_loss_vanilla": lambda: CA.compute_policy_loss_vanilla(old, lp_leaf, adv, mask, "token-mean", cfg),
+        "agg_loss": lambda: CA.agg_loss(lp_leaf, mask, "token-mean"),
+        "kl_penalty": lambda: CA.kl_penalty(lp_leaf, ref, "low_var_kl"),
+        "masked_mean": lambda: SF.masked_mean(lp_leaf, mask),
+        "actor_loss (fused)": lambda: CA.actor_loss(old, lp_leaf, adv, mask, cfg, ref_log_prob=ref),
+    }
+
+    def host_us(fn, n=300):
+        for _ in range(30):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        el = time.perf_counter() - t0
+        torch.cuda.synchronize()
+        return el / n * 1e6
+
+    per_call = {}
+    for name, fn in calls.items():
+        with torch.no_grad():
+            a = host_us(fn)
+        per_call[name] = {"no_grad_us": round(a, 1), "grad_mode_us": round(host_us(fn), 1)}
+
+    def fwd_bwd(make_loss, leaf):
+        def run():
+            make_loss().backward()
+            leaf.grad = None
+        return host_us(run)
+
+    per_call["logprobs_from_logits"]["fwd_bwd_us"] = round(fwd_bwd(
+        lambda: SF.logprobs_from_logits(logits, labels, inplace_backward=False).sum(), logits), 1)
+    per_call["compute_policy_loss_vanilla"]["fwd_bwd_us"] = round(fwd_bwd(
+        lambda: CA.compute_policy_loss_vanilla(old, lp_leaf, adv, mask, "token-mean", cfg)[0], lp_leaf), 1)
+    per_call["actor_loss (fused)"]["fwd_bwd_us"] = round(fwd_bwd(
+        lambda: CA.actor_loss(old, lp_leaf, adv, mask, cfg, ref_log_prob=ref).loss, lp_leaf), 1)
+
+    def micro_batch():  # dp_actor.py:403-501 with the drop-in functions: the reference's own ten calls
+        lp = SF.logprobs_from_logits(logits, labels, inplace_backward=False)
+        ent = SF.entropy_from_logits(logits)
+        pg, clipfrac, kl, lower = CA.compute_policy_loss_vanilla(old_log_prob=old, log_prob=lp, advantages=adv,
+                                                                 response_mask=mask, loss_agg_mode="token-mean",
+                                                                 config=cfg)
+        ent_loss = CA.agg_loss(loss_mat=ent, loss_mask=mask, loss_agg_mode="token-mean")
+        policy = pg - ent_loss * cfg.entropy_coeff
+        kld = CA.kl_penalty(logprob=lp, ref_logprob=ref, kl_penalty="low_var_kl")
+        kl_loss = CA.agg_loss(loss_mat=kld, loss_mask=mask, loss_agg_mode="token-mean")
+        policy = policy + kl_loss * cfg.kl_loss_coef
+        (policy * 0.125).backward()
+        logits.grad = None
+
+    def micro_batch_fused():  # the same arithmetic through actor_loss
+        lp = SF.logprobs_from_logits(logits, labels, inplace_backward=False)
+        ent = SF.entropy_from_logits(logits)
+        CA.actor_loss(old, lp, adv, mask, cfg, entropy=ent, ref_log_prob=ref, loss_scale_factor=0.125).loss.backward()
+        logits.grad = None
+
+    out = {"metric": "host microseconds per call of the drop-in functions (GPU work negligible)", "unit": "us",
+           "n_gpus": 1, "data": "synthetic", "config": {"workload": f"host: [B, L] = [{B}, {L}] fp32 operands, logits "
+                                                                    f"[{B}, {L}, {V}] fp32, int64 mask"},
+           "per_call": per_call,
+           "micro_batch_drop_in_us": round(host_us(micro_batch, 200), 1),
+           "micro_batch_actor_loss_us": round(host_us(micro_batch_fused, 200), 1),
+           "cpu": cpu_model()}
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -752,7 +855,7 @@ def main():
                     help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 2 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "critic", "glue"],
+    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "critic", "glue", "host"],
                     help="config2 (default): the headline logprob+entropy fwd+bwd; config1: fp32 GRPO step at V = 32000; "
                          "config4: GSPO long-context sequence; config3: DAPO [B, L] loss path; "
                          "config5: fused lm_head variant; critic: reward placement + GAE + value loss + metrics; "
@@ -792,6 +895,8 @@ def main():
         return bench_critic(args, dev)
     if args.workload == "glue":
         return bench_glue(args, dev)
+    if args.workload == "host":
+        return bench_host(args, dev)
     SF.set_skip_zero_rows(False)  # dense: every row is read and written, as the algorithmic byte count assumes
 
     logits, labels, g_lp, g_ent, mask = make_workload(dev, seqs=args.seqs)

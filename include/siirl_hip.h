@@ -73,7 +73,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1002
+#define SIIRL_HIP_ABI_VERSION 1003
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -295,13 +295,22 @@ int siirl_kl_penalty_bwd(const float* g, const float* logprob, const float* ref_
 
 /*
  * masked_sum / masked_mean over a [B, L] fp32 matrix: row_sum[b] = sum_t where(mask, v, 0) * mask,
- * row_mean[b] = row_sum[b] / (sum_t mask + 1e-8), total2 = {sum over all, sum / (sum(mask) + 1e-8)}.
- * Any of the three outputs may be NULL.  Workspace as for the loss entry points.
- * Replaces: masked_sum / masked_mean siirl/utils/model_utils/torch_functional.py:146-168 (axis None or -1).
+ * row_mean[b] = row_sum[b] / (sum_t mask + 1e-8), total2 = {sum over all, sum / (sum(mask) + 1e-8)},
+ * row_msum[b] = sum_t mask, mask_total[0] = sum(mask) (the denominators, kept for the backward).
+ * Any output may be NULL.  Workspace as for the loss entry points.  A reduction over other axes is this one after
+ * the caller has moved the reduced axes last.
+ * Replaces: masked_sum / masked_mean siirl/utils/model_utils/torch_functional.py:146-168.
  */
 int siirl_masked_reduce(const float* values, const void* mask, int mask_dtype, int64_t B, int64_t L, float* row_sum,
-                        float* row_mean, float* total2, void* workspace, size_t workspace_bytes,
-                        siirl_stream_t stream);
+                        float* row_mean, float* total2, float* row_msum, float* mask_total, void* workspace,
+                        size_t workspace_bytes, siirl_stream_t stream);
+
+/*
+ * Backward of the above: d_values[b, t] = g[per_row ? b : 0] * mask[b, t], divided by (mask_sums[per_row ? b : 0]
+ * + 1e-8) when mask_sums is given (the mean; NULL for the sum).  g holds B entries (per_row) or one.
+ */
+int siirl_masked_reduce_bwd(const float* g, const void* mask, int mask_dtype, int64_t B, int64_t L, int per_row,
+                            const float* mask_sums, float* d_values, siirl_stream_t stream);
 
 /*
  * KL penalty folded into the reward: kld = kl_penalty(old_log_prob, ref_log_prob) * mask,

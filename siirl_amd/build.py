@@ -1,6 +1,8 @@
-"""Builds ``siirl_amd/lib/libsiirl_hip.so`` from ``siirl_amd/csrc/*.hip`` with hipcc for gfx950.
+"""Builds ``siirl_amd/lib/libsiirl_hip.so`` from ``siirl_amd/csrc/*.hip`` with hipcc for gfx950, and
+``siirl_amd/lib/libsiirl_torch.so`` (the ``TORCH_LIBRARY(siirl_hip, ...)`` layer, host-only C++ over the C ABI of the
+first) from ``siirl_amd/csrc/torch_ops.cpp`` with g++ against the installed torch's headers.
 
-Usage: ``python -m siirl_amd.build [--force]``.  The library is built in-tree so that it travels with
+Usage: ``python -m siirl_amd.build [--force]``.  The libraries are built in-tree so that they travel with
 the source tree to a GPU machine; nothing is compiled at import time."""
 
 from __future__ import annotations
@@ -16,6 +18,8 @@ PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIBDIR = PKG / "lib"
 LIBNAME = "libsiirl_hip.so"
+TORCH_LIBNAME = "libsiirl_torch.so"
+CXX = os.environ.get("CXX", "g++")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
@@ -78,6 +82,34 @@ def build(force: bool = False, verbose: bool = True) -> Path:
             raise RuntimeError("link of libsiirl_hip.so failed")
         if verbose:
             print(f"[siirl_amd.build] linked {out}", flush=True)
+    build_torch_layer(force=force or bool(jobs), verbose=verbose)
+    return out
+
+
+def build_torch_layer(force: bool = False, verbose: bool = True) -> Path:
+    """``csrc/torch_ops.cpp`` -> ``lib/libsiirl_torch.so``: no device code, so the host compiler builds it; it links
+    torch's own libraries and ``libsiirl_hip.so`` (found next to it through ``$ORIGIN``)."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    src = CSRC / "torch_ops.cpp"
+    out = LIBDIR / TORCH_LIBNAME
+    deps = [src, *(PKG.parent / "include").glob("*.h"), LIBDIR / LIBNAME]
+    if not force and not _stale(out, deps):
+        return out
+    torch_lib = Path(torch.__file__).resolve().parent / "lib"
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [CXX, "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__", "-DUSE_ROCM",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}", "-Wno-deprecated-declarations",
+           *(f"-I{p}" for p in ce.include_paths()), f"-I{rocm}/include", str(src), "-o", str(out),
+           f"-L{torch_lib}", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+           f"-L{LIBDIR}", "-lsiirl_hip", "-Wl,-rpath,$ORIGIN", "-Wl,--no-as-needed"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose:
+        print(f"[siirl_amd.build] {CXX} torch_ops.cpp: {'ok' if r.returncode == 0 else 'FAILED'}", flush=True)
+    if r.returncode != 0:
+        print(r.stderr, file=sys.stderr)
+        raise RuntimeError("build of libsiirl_torch.so failed")
     return out
 
 

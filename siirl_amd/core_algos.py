@@ -29,6 +29,7 @@ from . import _lib
 from . import ops as _ops_module  # noqa: F401  (registers torch.ops.siirl_hip.*)
 
 _OPS = torch.ops.siirl_hip
+_actor_loss_op = _OPS.actor_loss.default  # one C++ autograd node: fused forward, elementwise backward, 13 scalars out
 from . import torch_functional as siirl_F
 
 __all__ = [
@@ -375,34 +376,12 @@ def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_i
 # ------------------------------------------------------------------------------------ aggregation
 
 
-class _AggLoss(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, loss_mat, loss_mask, agg_code):
-        dev = loss_mat.device
-        v = _as_2d(_f32(loss_mat, dev))
-        B, L = v.shape
-        m, mcode = _mask_arg(_as_2d(loss_mask), dev)
-        out16, row_msum = _OPS.agg_loss_fwd(v, m, agg_code)
-        ctx.save_for_backward(m, out16, row_msum)
-        ctx.meta = (mcode, B, L, agg_code, loss_mat.shape, loss_mat.dtype)
-        return out16[O_PG]
-
-    @staticmethod
-    def backward(ctx, g):
-        m, out16, row_msum = ctx.saved_tensors
-        mcode, B, L, agg_code, shape, dtype = ctx.meta
-        dev = out16.device
-        g = g.detach().to(torch.float32).reshape(1).contiguous()
-        d = _OPS.agg_loss_bwd(g, m, out16, row_msum, agg_code)
-        return d.reshape(shape).to(dtype), None, None
-
-
 def agg_loss(loss_mat: torch.Tensor, loss_mask: torch.Tensor, loss_agg_mode: str):
     """Aggregate a ``[B, L]`` loss into a scalar (reference ``core_algos.py:536-569``); unknown modes raise
     ``ValueError``.  ``seq-mean-token-mean`` of a row with an empty mask is NaN, as in the reference."""
     code = _agg_code(loss_agg_mode)
     _gpu_of(loss_mat)
-    return _AggLoss.apply(loss_mat, loss_mask, code)
+    return _OPS.agg_loss(loss_mat, loss_mask, code)
 
 
 def compute_entropy_loss(logits: torch.Tensor, response_mask: torch.Tensor, loss_agg_mode: str = "token-mean"):
@@ -415,69 +394,6 @@ def compute_entropy_loss(logits: torch.Tensor, response_mask: torch.Tensor, loss
 # ------------------------------------------------------------------------------------ policy loss
 
 
-class _ActorLoss(torch.autograd.Function):
-    """One fused forward (partials + finish) and one elementwise backward for the whole micro-batch loss.
-    ``policy_only``: the four policy-loss scalars are the outputs and the gradient enters through pg_loss;
-    otherwise the scaled total enters through ``loss``.  The other scalars are metrics (no gradient)."""
-
-    @staticmethod
-    def forward(ctx, log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, ref_log_prob, cfg):
-        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, drift_coef, scale,
-         policy_only) = cfg
-        dev = log_prob.device
-        lp = _as_2d(_f32(log_prob, dev))
-        B, L = lp.shape
-        old = _as_2d(_f32(old_log_prob, dev))
-        adv = _as_2d(_f32(advantages, dev))
-        m, mcode = _mask_arg(_as_2d(response_mask), dev)
-        isw = None if is_weights is None else _as_2d(_f32(is_weights, dev))
-        ent = None if entropy is None else _as_2d(_f32(entropy, dev))
-        ref = None if ref_log_prob is None else _as_2d(_f32(ref_log_prob, dev))
-        for name, t in (("old_log_prob", old), ("advantages", adv), ("response_mask", m), ("rollout_is_weights", isw),
-                        ("entropy", ent), ("ref_log_prob", ref)):
-            if t is not None and tuple(t.shape) != (B, L):
-                raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {(B, L)}")
-        out16, row_msum, row_s = _OPS.policy_loss_fwd(old, lp, adv, m, isw, ent, ref, loss_mode, eps_lo, eps_hi, clip_c,
-                                                      dclamp, agg_code, ent_coef, kl_code, bool(kl_st), kl_coef,
-                                                      drift_coef, scale)
-        ctx.save_for_backward(lp, old, adv, m, out16, row_msum, row_s,
-                              *(t for t in (isw, ent, ref) if t is not None))
-        ctx.flags = (isw is not None, ent is not None, ref is not None)
-        ctx.meta = (mcode, B, L, cfg, log_prob.shape, log_prob.dtype,
-                    None if entropy is None else (entropy.shape, entropy.dtype))
-        ctx.set_materialize_grads(False)
-        outs = tuple(out16[i] for i in range(13))
-        diff = (O_PG,) if policy_only else (O_LOSS,)
-        ctx.mark_non_differentiable(*(o for i, o in enumerate(outs) if i not in diff))
-        ctx.diff_index = diff[0]
-        return outs
-
-    @staticmethod
-    def backward(ctx, *grads):
-        g = grads[ctx.diff_index]
-        if g is None:
-            return (None,) * 8
-        lp, old, adv, m, out16, row_msum, row_s, *rest = ctx.saved_tensors
-        has_isw, has_ent, has_ref = ctx.flags
-        rest = list(rest)
-        isw = rest.pop(0) if has_isw else None
-        ent = rest.pop(0) if has_ent else None
-        ref = rest.pop(0) if has_ref else None
-        mcode, B, L, cfg, lp_shape, lp_dtype, ent_meta = ctx.meta
-        (loss_mode, eps_lo, eps_hi, clip_c, dclamp, agg_code, ent_coef, kl_code, kl_st, kl_coef, drift_coef, scale,
-         _) = cfg
-        dev = lp.device
-        g = g.detach().to(torch.float32).reshape(1).contiguous()
-        d_lp, d_ent = _OPS.policy_loss_bwd(g, old, lp, adv, m, isw, ent, ref, loss_mode, eps_lo, eps_hi, clip_c, dclamp,
-                                           agg_code, ent_coef, kl_code, bool(kl_st), kl_coef, drift_coef, scale, out16,
-                                           row_msum, row_s)
-        if not has_ent:
-            d_ent = None
-        g_lp = d_lp.reshape(lp_shape).to(lp_dtype)
-        g_ent = None if d_ent is None else d_ent.reshape(ent_meta[0]).to(ent_meta[1])
-        return g_lp, g_ent, None, None, None, None, None, None
-
-
 def _clip_params(config):
     clip_ratio = config.clip_ratio
     lo = config.clip_ratio_low if getattr(config, "clip_ratio_low", None) is not None else clip_ratio
@@ -488,8 +404,8 @@ def _clip_params(config):
 def _policy_only(loss_mode, old_log_prob, log_prob, advantages, response_mask, agg_code, lo, hi, c, dclamp,
                  rollout_is_weights):
     _gpu_of(log_prob)
-    cfg = (loss_mode, lo, hi, float(c), float(dclamp), agg_code, 0.0, 0, 0, 0.0, 0.0, 1.0, True)
-    outs = _ActorLoss.apply(log_prob, None, old_log_prob, advantages, response_mask, rollout_is_weights, None, cfg)
+    outs = _actor_loss_op(log_prob, None, old_log_prob, advantages, response_mask, rollout_is_weights, None, loss_mode,
+                          lo, hi, float(c), float(dclamp), agg_code, 0.0, 0, False, 0.0, 0.0, 1.0, True)
     return outs[O_PG], outs[O_CLIPFRAC], outs[O_PPOKL], outs[O_CLIPLOWER]
 
 
@@ -576,53 +492,12 @@ def compute_policy_loss_geo_mean(old_log_prob: torch.Tensor, log_prob: torch.Ten
                         AGG_MODES["token-mean"], lo, hi, 3.0, 20.0, rollout_is_weights)
 
 
-class _ValueLoss(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, vpreds, returns, values, response_mask, cliprange_value, agg_code):
-        dev = vpreds.device
-        vp = _as_2d(_f32(vpreds, dev))
-        B, L = vp.shape
-        ret = _as_2d(_f32(returns, dev))
-        val = _as_2d(_f32(values, dev))
-        m, mcode = _mask_arg(_as_2d(response_mask), dev)
-        for name, t in (("returns", ret), ("values", val), ("response_mask", m)):
-            if tuple(t.shape) != (B, L):
-                raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {(B, L)}")
-        out16 = torch.empty(16, dtype=torch.float32, device=dev)
-        row_msum = torch.empty(B, dtype=torch.float32, device=dev)
-        ws, nws = _workspace(B, L, dev)
-        with torch.cuda.device(dev):
-            rc = _lib.lib().siirl_value_loss_fwd(_lib.ptr(vp), _lib.ptr(ret), _lib.ptr(val), _lib.ptr(m), mcode, B, L,
-                                                 float(cliprange_value), agg_code, _lib.ptr(out16),
-                                                 _lib.ptr(row_msum), _lib.ptr(ws), nws, _lib.current_stream(dev))
-        _lib.check(rc, "siirl_value_loss_fwd")
-        ctx.save_for_backward(vp, ret, val, m, out16, row_msum)
-        ctx.meta = (mcode, B, L, float(cliprange_value), agg_code, vpreds.shape, vpreds.dtype)
-        loss, frac = out16[O_LOSS], out16[O_CLIPFRAC]
-        ctx.mark_non_differentiable(frac)
-        return loss, frac
-
-    @staticmethod
-    def backward(ctx, g, _):
-        vp, ret, val, m, out16, row_msum = ctx.saved_tensors
-        mcode, B, L, clip, agg_code, shape, dtype = ctx.meta
-        dev = vp.device
-        g = g.detach().to(torch.float32).reshape(1).contiguous()
-        d = torch.empty(B, L, dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
-            rc = _lib.lib().siirl_value_loss_bwd(_lib.ptr(g), _lib.ptr(vp), _lib.ptr(ret), _lib.ptr(val), _lib.ptr(m),
-                                                 mcode, B, L, clip, agg_code, _lib.ptr(out16), _lib.ptr(row_msum),
-                                                 _lib.ptr(d), _lib.current_stream(dev))
-        _lib.check(rc, "siirl_value_loss_bwd")
-        return d.reshape(shape).to(dtype), None, None, None, None, None
-
-
 def compute_value_loss(vpreds: torch.Tensor, returns: torch.Tensor, values: torch.Tensor, response_mask: torch.Tensor,
                        cliprange_value: float, loss_agg_mode: str = "token-mean"):
     """Clipped value loss of the critic (reference ``core_algos.py:1173-1212``).  Returns ``(vf_loss,
     vf_clipfrac)`` as 0-d device tensors; ``vf_loss`` carries the gradient to ``vpreds``."""
     _gpu_of(vpreds)
-    return _ValueLoss.apply(vpreds, returns, values, response_mask, cliprange_value, _agg_code(loss_agg_mode))
+    return _OPS.value_loss(vpreds, returns, values, response_mask, float(cliprange_value), _agg_code(loss_agg_mode))
 
 
 def compute_policy_loss(old_log_prob, log_prob, advantages, response_mask, cliprange=None, cliprange_low=None,
@@ -646,41 +521,13 @@ def compute_policy_loss(old_log_prob, log_prob, advantages, response_mask, clipr
 # ------------------------------------------------------------------------------------ KL penalty
 
 
-class _KlPenalty(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, logprob, ref_logprob, code, straight_through):
-        dev = logprob.device
-        lp, ref = _f32(logprob, dev), _f32(ref_logprob, dev)
-        if ref.shape != lp.shape:
-            ref = ref.expand(lp.shape).contiguous()
-        out = _OPS.kl_penalty_fwd(lp, ref, code)
-        ctx.save_for_backward(lp, ref)
-        ctx.meta = (code, straight_through, logprob.dtype, ref_logprob.dtype, ref_logprob.shape)
-        return out.to(logprob.dtype) if logprob.dtype != torch.float32 else out
-
-    @staticmethod
-    def backward(ctx, g):
-        lp, ref = ctx.saved_tensors
-        code, st, lp_dtype, ref_dtype, ref_shape = ctx.meta
-        dev = lp.device
-        g = _f32(g, dev)
-        need_lp, need_ref = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        d_lp, d_ref = _OPS.kl_penalty_bwd(g, lp, ref, code, bool(st), bool(need_lp), bool(need_ref))
-        d_lp = d_lp if need_lp else None
-        d_ref = d_ref if need_ref else None
-        if d_ref is not None and tuple(ref_shape) != tuple(lp.shape):
-            d_ref = d_ref.sum_to_size(ref_shape)
-        return (None if d_lp is None else d_lp.to(lp_dtype), None if d_ref is None else d_ref.to(ref_dtype),
-                None, None)
-
-
 def kl_penalty_forward(logprob: torch.Tensor, ref_logprob: torch.Tensor, kl_penalty) -> torch.Tensor:
     """Per-token KL estimator (reference ``core_algos.py:1241-1276``): ``kl``/``k1``, ``abs``, ``mse``/``k2``,
     ``low_var_kl``/``k3``; anything else, ``full`` included, raises ``NotImplementedError``."""
     if kl_penalty not in KL_MODES:
         raise NotImplementedError
     _gpu_of(logprob, ref_logprob)
-    return _KlPenalty.apply(logprob, ref_logprob, KL_MODES[kl_penalty], False)
+    return _OPS.kl_penalty(logprob, ref_logprob, KL_MODES[kl_penalty], False)
 
 
 def kl_penalty(logprob: torch.Tensor, ref_logprob: torch.Tensor, kl_penalty) -> torch.Tensor:
@@ -698,7 +545,7 @@ def kl_penalty_straight_through(logprob: torch.Tensor, ref_logprob: torch.Tensor
     if name not in KL_MODES:
         raise NotImplementedError
     _gpu_of(logprob, ref_logprob)
-    return _KlPenalty.apply(logprob, ref_logprob, KL_MODES[name], True)
+    return _OPS.kl_penalty(logprob, ref_logprob, KL_MODES[name], True)
 
 
 # ------------------------------------------------------------------------------------ fused actor loss
@@ -768,10 +615,10 @@ def actor_loss(old_log_prob, log_prob, advantages, response_mask, config, entrop
         if kl_type not in KL_MODES:
             raise NotImplementedError
         kl_code, kl_coef = KL_MODES[kl_type], float(getattr(config, "kl_loss_coef", 0.001))
-    cfg = (_LOSS_CODES[mode], lo, hi, c, 20.0, agg_code, ent_coef if use_ent else 0.0,
-           kl_code, 0, kl_coef, drift, float(loss_scale_factor), False)
-    outs = _ActorLoss.apply(log_prob, entropy if use_ent else None, old_log_prob, advantages, response_mask,
-                            None if mode == "cpgd" else rollout_is_weights, ref_log_prob if use_kl else None, cfg)
+    outs = _actor_loss_op(log_prob, entropy if use_ent else None, old_log_prob, advantages, response_mask,
+                          None if mode == "cpgd" else rollout_is_weights, ref_log_prob if use_kl else None,
+                          _LOSS_CODES[mode], lo, hi, c, 20.0, agg_code, ent_coef if use_ent else 0.0, kl_code, False,
+                          kl_coef, drift, float(loss_scale_factor), False)
     return ActorLossOutput(outs, float(loss_scale_factor), kl_coef, use_kl, use_ent)
 
 

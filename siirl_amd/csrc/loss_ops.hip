@@ -505,7 +505,9 @@ __global__ __launch_bounds__(kThreads) void kl_bwd_kernel(const float* __restric
 __global__ __launch_bounds__(kThreads) void masked_finish_kernel(const float* __restrict__ partials, int nseg,
                                                                  int64_t B, float* __restrict__ row_sum,
                                                                  float* __restrict__ row_mean,
-                                                                 float* __restrict__ total2) {
+                                                                 float* __restrict__ total2,
+                                                                 float* __restrict__ row_msum,
+                                                                 float* __restrict__ mask_total) {
   double tv = 0, tm = 0;
   for (int64_t b = threadIdx.x; b < B; b += kThreads) {
     double v = 0, m = 0;
@@ -515,6 +517,7 @@ __global__ __launch_bounds__(kThreads) void masked_finish_kernel(const float* __
     }
     if (row_sum) row_sum[b] = (float)v;
     if (row_mean) row_mean[b] = (float)(v / (m + 1e-8));
+    if (row_msum) row_msum[b] = (float)m;
     tv += v;
     tm += m;
   }
@@ -525,13 +528,15 @@ __global__ __launch_bounds__(kThreads) void masked_finish_kernel(const float* __
     total2[0] = (float)tv;
     total2[1] = (float)(tv / (tm + 1e-8));
   }
+  if (threadIdx.x == 0 && mask_total) mask_total[0] = (float)tm;
 }
 
 // many rows: one thread per row writes the row's results, one {sum, mask sum} record per workgroup; then one
 // workgroup folds the records (fp64 as above; the order of the additions differs from the one-level finish)
 __global__ __launch_bounds__(kThreads) void masked_rows_kernel(const float* __restrict__ partials, int nseg, int64_t B,
                                                                float* __restrict__ row_sum,
-                                                               float* __restrict__ row_mean, double* __restrict__ rec) {
+                                                               float* __restrict__ row_mean,
+                                                               float* __restrict__ row_msum, double* __restrict__ rec) {
   const int64_t b = (int64_t)blockIdx.x * kThreads + threadIdx.x;
   double v = 0, m = 0;
   if (b < B) {
@@ -541,6 +546,7 @@ __global__ __launch_bounds__(kThreads) void masked_rows_kernel(const float* __re
     }
     if (row_sum) row_sum[b] = (float)v;
     if (row_mean) row_mean[b] = (float)(v / (m + 1e-8));
+    if (row_msum) row_msum[b] = (float)m;
   }
   __shared__ double sh[kThreads / kWave + 1];
   v = block_sum_d(v, sh);
@@ -551,7 +557,8 @@ __global__ __launch_bounds__(kThreads) void masked_rows_kernel(const float* __re
   }
 }
 __global__ __launch_bounds__(kThreads) void masked_finish2_kernel(const double* __restrict__ rec, int nrec,
-                                                                  float* __restrict__ total2) {
+                                                                  float* __restrict__ total2,
+                                                                  float* __restrict__ mask_total) {
   double tv = 0, tm = 0;
   for (int i = threadIdx.x; i < nrec; i += kThreads) {
     tv += rec[2 * i];
@@ -560,9 +567,26 @@ __global__ __launch_bounds__(kThreads) void masked_finish2_kernel(const double* 
   __shared__ double sh[kThreads / kWave + 1];
   tv = block_sum_d(tv, sh);
   tm = block_sum_d(tm, sh);
-  if (threadIdx.x == 0) {
+  if (threadIdx.x == 0 && total2) {
     total2[0] = (float)tv;
     total2[1] = (float)(tv / (tm + 1e-8));
+  }
+  if (threadIdx.x == 0 && mask_total) mask_total[0] = (float)tm;
+}
+
+// backward of masked_sum / masked_mean: d[b, t] = g[b or 0] * m[b, t] (/ (mask sum of the reduced extent + 1e-8))
+__global__ __launch_bounds__(kThreads) void masked_bwd_kernel(const float* __restrict__ g, const void* mask,
+                                                              int mask_dtype, int64_t B, int64_t L, int per_row,
+                                                              const float* __restrict__ den, float* __restrict__ d) {
+  const int64_t n = B * L;
+  const float all = per_row ? 0.f : (den ? g[0] / (den[0] + 1e-8f) : g[0]);
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+    float w = all;
+    if (per_row) {
+      const int64_t b = i / L;
+      w = den ? g[b] / (den[b] + 1e-8f) : g[b];
+    }
+    d[i] = w * load_mask(mask, mask_dtype, i);
   }
 }
 
@@ -944,17 +968,19 @@ extern "C" int siirl_kl_penalty_bwd(const float* g, const float* logprob, const 
 }
 
 extern "C" int siirl_masked_reduce(const float* values, const void* mask, int mask_dtype, int64_t B, int64_t L,
-                                   float* row_sum, float* row_mean, float* total2, void* workspace,
-                                   size_t workspace_bytes, siirl_stream_t stream) {
+                                   float* row_sum, float* row_mean, float* total2, float* row_msum,
+                                   float* mask_total, void* workspace, size_t workspace_bytes,
+                                   siirl_stream_t stream) {
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   SIIRL_REQUIRE(B == 0 || (values && mask), "NULL operand");
-  SIIRL_REQUIRE(row_sum || row_mean || total2, "no output requested");
+  SIIRL_REQUIRE(row_sum || row_mean || total2 || row_msum || mask_total, "no output requested");
   LossArgs a{};
   a.lp = values; a.mask = mask; a.mask_dtype = mask_dtype; a.kind = KIND_AGG; a.agg_mode = SIIRL_AGG_TOKEN_MEAN;
   a.aux_agg_mode = a.agg_mode; a.scale = 1.f; a.B = B; a.L = L; a.nseg = nseg_of(L);
   if (B == 0) {  // sums of nothing
-    masked_finish_kernel<<<1, dim3(kThreads), 0, (hipStream_t)stream>>>(nullptr, a.nseg, 0, row_sum, row_mean, total2);
+    masked_finish_kernel<<<1, dim3(kThreads), 0, (hipStream_t)stream>>>(nullptr, a.nseg, 0, row_sum, row_mean, total2,
+                                                                        row_msum, mask_total);
     SIIRL_LAUNCH_CHECK("masked_finish_kernel");
     return SIIRL_OK;
   }
@@ -967,19 +993,35 @@ extern "C" int siirl_masked_reduce(const float* values, const void* mask, int ma
   set_vec(a);
   if (int rc = launch_loss_partials(a, nullptr, partials, st)) return rc;
   if (B <= kTwoLevelRows) {
-    masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, total2);
+    masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, total2, row_msum,
+                                                       mask_total);
     SIIRL_LAUNCH_CHECK("masked_finish_kernel");
     return SIIRL_OK;
   }
   const size_t used = ((size_t)B * a.nseg * (kNP + kNPre) * sizeof(float) + 255) / 256 * 256;
   double* rec = reinterpret_cast<double*>((char*)workspace + used);  // room for kFinRec >= 2 doubles per workgroup
   const int nrec = (int)((B + kThreads - 1) / kThreads);
-  masked_rows_kernel<<<dim3((unsigned)nrec), dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, rec);
+  masked_rows_kernel<<<dim3((unsigned)nrec), dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, row_msum,
+                                                                      rec);
   SIIRL_LAUNCH_CHECK("masked_rows_kernel");
-  if (total2) {
-    masked_finish2_kernel<<<1, dim3(kThreads), 0, st>>>(rec, nrec, total2);
+  if (total2 || mask_total) {
+    masked_finish2_kernel<<<1, dim3(kThreads), 0, st>>>(rec, nrec, total2, mask_total);
     SIIRL_LAUNCH_CHECK("masked_finish2_kernel");
   }
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_masked_reduce_bwd(const float* g, const void* mask, int mask_dtype, int64_t B, int64_t L,
+                                       int per_row, const float* mask_sums, float* d_values, siirl_stream_t stream) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  if (B == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(g && mask && d_values, "NULL operand");
+  const int64_t want = (B * L + kThreads - 1) / kThreads;
+  const unsigned blocks = (unsigned)(want < 16384 ? want : 16384);
+  masked_bwd_kernel<<<dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream>>>(g, mask, mask_dtype, B, L, per_row,
+                                                                            mask_sums, d_values);
+  SIIRL_LAUNCH_CHECK("masked_bwd_kernel");
   return SIIRL_OK;
 }
 

@@ -6,13 +6,12 @@
 * ``linear_cross_entropy`` -- mirror of ``siirl/utils/kernel/linear_cross_entropy.py:40-117``:
   ``(hidden, weight, labels, temperature, reduction, dist_process_group) -> (logprobs, entropy)``.
 
-Both run the MFMA kernels of ``csrc/fused_linear.hip`` through the C ABI.  Operands are bf16 on the GPU.  The
-forward needs no ``[T, V]`` tensor.  When a backward will follow and the buffer fits the limit set with
-``set_saved_logits_limit`` (default 16 GiB, or ``SIIRL_AMD_SAVED_LOGITS_LIMIT`` bytes from the environment; 4 bytes
-per logit), the forward parks its fp32 logit tiles and the
-backward reads them back instead of running the projection a second time: the same bits, a quarter less matrix
-work per step.  With the limit at 0 the logits are never stored and the backward recomputes them slab by slab,
-which is the reference's memory behaviour.  Outputs are fp32 (the reference's Triton path returns fp32,
+Both run the MFMA kernels of ``csrc/fused_linear.hip`` through the C ABI.  Operands are bf16 on the GPU.  Neither
+pass holds a ``[T, V]`` tensor: the backward recomputes the logits slab by slab, which is the reference's memory
+behaviour.  Opt-in trade of memory for time: with ``set_saved_logits_limit(nbytes)`` (or
+``SIIRL_AMD_SAVED_LOGITS_LIMIT`` bytes in the environment; default 0 = never), a forward that a backward will follow
+parks its fp32 logit tiles (4 bytes per logit) when they fit the limit and the backward reads them back instead of
+running the projection a second time: the same bits, a quarter less matrix work per step.  Outputs are fp32 (the reference's Triton path returns fp32,
 ``kernels.py:586-593``; its chunked-torch path casts back to the input dtype, ``torch_functional.py:32``, which
 ``FusedLinearForPPO(cast_outputs=True)`` reproduces).  ``chunk_size`` is accepted and ignored: tiling is the
 kernel's business.
@@ -29,11 +28,12 @@ from . import ops as _ops_module  # noqa: F401  (registers torch.ops.siirl_hip.*
 
 
 # bytes; the environment variable gives a deployment its own default without code changes
-_SAVED_LOGITS_LIMIT = int(os.environ.get("SIIRL_AMD_SAVED_LOGITS_LIMIT", 16 << 30))
+_SAVED_LOGITS_LIMIT = int(os.environ.get("SIIRL_AMD_SAVED_LOGITS_LIMIT", 0))
 
 
 def set_saved_logits_limit(nbytes: int) -> None:
-    """Largest fp32 logit buffer (bytes) the forward may keep for the backward; 0 = always recompute."""
+    """Largest fp32 logit buffer (bytes) the forward may keep for the backward; 0 (the default) = never keep one,
+    always recompute."""
     global _SAVED_LOGITS_LIMIT
     if nbytes < 0:
         raise ValueError(f"the limit must not be negative, got {nbytes}")
@@ -44,42 +44,11 @@ def _saved_logits_bytes(T: int, V: int) -> int:
     return ((V + 255) // 256) * ((T + 255) // 256) * (256 * 256 * 4)
 
 
-class _FusedLinearLogprobEntropy(torch.autograd.Function):
-    @staticmethod
-    def forward(ctx, hidden, weight, labels, temperature):
-        if not hidden.is_cuda or not weight.is_cuda:
-            raise RuntimeError("siirl_amd: the fused lm_head path runs on the GPU only (no CPU fallback)")
-        if hidden.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
-            raise TypeError("siirl_amd: the fused lm_head path takes bfloat16 hidden states and weights")
-        dev = hidden.device
-        h = hidden.detach().contiguous()
-        w = weight.detach().contiguous()
-        y = labels.detach().to(device=dev, dtype=torch.int64).contiguous()
-        T, H = h.shape
-        V = w.shape[0]
-        if w.shape[1] != H or y.shape != (T,):
-            raise ValueError(f"shape mismatch: hidden {tuple(h.shape)}, weight {tuple(w.shape)}, labels {tuple(y.shape)}")
-        inv_t = 1.0 / float(temperature)
-        save = (ctx.needs_input_grad[0] or ctx.needs_input_grad[1]) and \
-            _saved_logits_bytes(T, V) <= _SAVED_LOGITS_LIMIT
-        lp, ent, lse, ex, saved = torch.ops.siirl_hip.fused_linear_logprob_entropy_fwd(h, w, y, inv_t, bool(save))
-        ctx.save_for_backward(h, w, y, lse, ex, saved)
-        ctx.inv_t = inv_t
-        ctx.set_materialize_grads(False)
-        return lp, ent
-
-    @staticmethod
-    def backward(ctx, g_lp, g_ent):
-        h, w, y, lse, ex, saved = ctx.saved_tensors
-        need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-        if (g_lp is None and g_ent is None) or not (need_h or need_w):
-            return None, None, None, None
-        dev = h.device
-        f = lambda t: None if t is None else t.detach().to(device=dev, dtype=torch.float32).contiguous()  # noqa: E731
-        g_lp, g_ent = f(g_lp), f(g_ent)
-        d_h, d_w = torch.ops.siirl_hip.fused_linear_logprob_entropy_bwd(h, w, y, ctx.inv_t, lse, ex, g_lp, g_ent,
-                                                                        bool(need_h), bool(need_w), saved)
-        return (d_h if need_h else None), (d_w if need_w else None), None, None
+def _apply(hidden2d, weight, labels1d, temperature):
+    if not hidden2d.is_cuda or not weight.is_cuda:
+        raise RuntimeError("siirl_amd: the fused lm_head path runs on the GPU only (no CPU fallback)")
+    return torch.ops.siirl_hip.fused_linear_logprob_entropy(hidden2d, weight, labels1d, 1.0 / float(temperature),
+                                                            _SAVED_LOGITS_LIMIT)
 
 
 def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,
@@ -89,8 +58,7 @@ def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, lab
     lead = hidden.shape[:-1]
     if labels.shape != lead:
         raise ValueError(f"labels shape {tuple(labels.shape)} does not match hidden {tuple(hidden.shape)}")
-    lp, ent = _FusedLinearLogprobEntropy.apply(hidden.reshape(-1, hidden.shape[-1]), weight, labels.reshape(-1),
-                                               float(temperature))
+    lp, ent = _apply(hidden.reshape(-1, hidden.shape[-1]), weight, labels.reshape(-1), temperature)
     return lp.reshape(lead), ent.reshape(lead)
 
 
@@ -127,7 +95,7 @@ def linear_cross_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: tor
     if dist_process_group is not None:
         raise NotImplementedError("siirl_amd: vocab-parallel linear_cross_entropy (dist_process_group) is not built")
     h2 = hidden.reshape(-1, hidden.shape[-1])
-    lp, ent = _FusedLinearLogprobEntropy.apply(h2, weight, labels.reshape(-1), temperature)
+    lp, ent = _apply(h2, weight, labels.reshape(-1), temperature)
     if red == "sum":
         lp = lp.sum()
     elif red == "mean":

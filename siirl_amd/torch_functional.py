@@ -6,25 +6,30 @@ argument meaning.  The arithmetic runs in ``libsiirl_hip.so``; tensors must live
 Differences a caller can observe, all deliberate:
 
 * results for 16-bit logits are fp32 (what the reference returns on its flash-attn dispatch,
-  ``torch_functional.py:73-79,85-90``); accumulation is always fp32;
-* ``logprobs_from_logits(..., inplace_backward=False)`` also computes the entropy in the same pass over
-  the row and parks it, so that the ``entropy_from_logits(logits)`` call that the actor issues next on
-  the same tensor (``siirl/engine/actor/dp_actor.py:179-195``) costs no second pass and both gradients
-  are written by one backward kernel.  ``set_pairing(False)`` turns this off.
+  ``torch_functional.py:73-79,85-90``); accumulation is always fp32; float64 logits are computed in fp32
+  (rounded once on entry) and the results returned as float64;
+* ``logprobs_from_logits`` also computes the entropy in the same pass over the row and keeps it with the
+  returned log-probs, so that the ``entropy_from_logits(logits)`` call that the actor issues next on the same
+  tensor (``siirl/engine/actor/dp_actor.py:179-195,254-260``) costs no second pass and both gradients are written
+  by one backward kernel.  ``set_pairing(False)`` turns this off;
+* the backward writes zeros, without reading the row, where both upstream gradients of a row are zero
+  (``set_skip_zero_rows``): a NaN or Inf in a padded row's logits therefore does not reach ``dlogits`` as it would
+  through the reference's autograd.
 """
 
 from __future__ import annotations
 
 import weakref
-from typing import Optional
 
 import torch
 
-from . import ops  # noqa: F401  (registers torch.ops.siirl_hip.*)
+from . import ops  # noqa: F401  (loads torch.ops.siirl_hip.*)
 
-_fwd = torch.ops.siirl_hip.logprob_entropy_fwd
-_bwd = torch.ops.siirl_hip.logprob_entropy_bwd
-_bwd_ = torch.ops.siirl_hip.logprob_entropy_bwd_
+_OPS = torch.ops.siirl_hip
+_fwd = _OPS.logprob_entropy_fwd
+_bwd = _OPS.logprob_entropy_bwd
+_bwd_ = _OPS.logprob_entropy_bwd_
+_lpe = _OPS.logprob_entropy.default
 
 _SKIP_ZERO_ROWS = True
 
@@ -37,7 +42,8 @@ def set_skip_zero_rows(flag: bool) -> None:
 
 
 class _LogprobEntropy(torch.autograd.Function):
-    """(logits, labels) -> (logprob, entropy) with one forward pass and one backward pass over the rows."""
+    """(logits, labels) -> (logprob, entropy) over the plain operators: the form ``torch.compile`` traces (the
+    operators are opaque to Dynamo and have fake kernels).  Eager calls use the C++ node ``logprob_entropy``."""
 
     @staticmethod
     def forward(ctx, logits, labels, inv_temperature, want_entropy, inplace_backward):
@@ -71,14 +77,24 @@ class _LogprobEntropy(torch.autograd.Function):
         return _bwd(*args), None, None, None, None
 
 
+_FLOATS = (torch.float32, torch.bfloat16, torch.float16)
+
+
 def _check_logits(logits):
+    """-> (logits the kernels accept, dtype to cast the results to or None)."""
     if not isinstance(logits, torch.Tensor) or logits.dim() < 1:
         raise TypeError("logits must be a tensor of shape (..., vocab_size)")
-    if logits.dtype not in (torch.float32, torch.bfloat16, torch.float16):
-        raise TypeError(f"logits dtype {logits.dtype} is not supported (float32, bfloat16, float16)")
+    if logits.dtype not in _FLOATS and logits.dtype != torch.float64:
+        raise TypeError(f"logits dtype {logits.dtype} is not supported (float32, float64, bfloat16, float16)")
+    if not logits.is_cuda:
+        raise RuntimeError(f"siirl_amd: `logits` is on {logits.device}; these ops run on the GPU only (no CPU fallback)")
+    back = None
+    if logits.dtype == torch.float64:
+        # the reference's fp32 / fp64 branch (torch_functional.py:103-107) serves float64: computed here in fp32
+        logits, back = logits.to(torch.float32), torch.float64
     if logits.shape[-1] > 1 and logits.stride(-1) != 1:
         logits = logits.contiguous()
-    return logits
+    return logits, back
 
 
 def logprobs_and_entropy_from_logits(logits: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
@@ -86,37 +102,113 @@ def logprobs_and_entropy_from_logits(logits: torch.Tensor, labels: torch.Tensor,
     """Both per-token outputs of the actor's post-logits step in one pass: ``(logprob, entropy)`` of
     ``logits / temperature``.  The division is folded into the kernels, ``logits`` is left untouched
     (the reference divides in place first, ``siirl/engine/actor/dp_actor.py:176``)."""
-    logits = _check_logits(logits)
-    return _LogprobEntropy.apply(logits, labels, 1.0 / float(temperature), True, inplace_backward)
+    logits, back = _check_logits(logits)
+    if torch.compiler.is_compiling():
+        lp, ent = _LogprobEntropy.apply(logits, labels, 1.0 / float(temperature), True, inplace_backward)
+    else:
+        lp, ent = _lpe(logits, labels, 1.0 / float(temperature), True, bool(inplace_backward), _SKIP_ZERO_ROWS, None)
+    return (lp, ent) if back is None else (lp.to(back), ent.to(back))
 
 
-# ------------------------------------------------------------------------------ pairing slot
+# ------------------------------------------------------------------------------ pairing
+#
+# logprobs_from_logits computes the entropy of the same rows in its one pass (the row is in registers anyway) and
+# hangs it on the returned log-prob tensor; entropy_from_logits(logits) on the same tensor object, at the same
+# version and grad mode, hands it out.  Both then belong to ONE autograd node, which autograd runs once with both
+# upstream gradients: one backward pass over the rows, and an in-place backward that cannot overtake a second reader.
+# The slot below only holds weak references: the parked entropy lives exactly as long as the log-probs it came with,
+# so an unclaimed one pins nothing once the caller drops those.
 
 _PAIRING = True
-_slot = None  # (weakref to logits, _version, grad_enabled, entropy)
+_slot = None  # (weakref logits, version, grad mode, weakref entropy or None, defer flag or None, output dtype or None)
+_entropy_reader = None  # (weakref to the last separately computed entropy that carries a graph, its logits' storage)
 
 
 def set_pairing(flag: bool) -> None:
-    global _PAIRING, _slot
-    _PAIRING, _slot = bool(flag), None
+    global _PAIRING, _slot, _traced_slot, _entropy_reader
+    _PAIRING, _slot, _traced_slot, _entropy_reader = bool(flag), None, None, None
 
 
-def _park(logits, entropy):
-    global _slot
-    _slot = (weakref.ref(logits), logits._version, torch.is_grad_enabled(), entropy)
+def _version(t):
+    return 0 if t.is_inference() else t._version
 
 
 def _claim(logits):
+    """The parked entropy for exactly this tensor, or None.  A miss on a tensor that shares memory with logits whose
+    log-prob node was built for an in-place backward turns that backward out-of-place: the caller is about to give
+    those logits a second reader (its own entropy node, or a checkpoint's recomputation), which an in-place backward
+    running first would feed with gradients instead of logits."""
     global _slot
     if _slot is None:
         return None
-    ref, version, grad_mode, entropy = _slot
-    if ref() is logits and logits._version == version and torch.is_grad_enabled() == grad_mode:
+    ref, version, grad_mode, ent_ref, defer, back = _slot
+    parked = ref()
+    if parked is None:
         _slot = None
-        return entropy
-    if ref() is None:
-        _slot = None
+        return None
+    if ent_ref is not None and parked is logits and _version(logits) == version and \
+            torch.is_grad_enabled() == grad_mode:
+        ent = ent_ref()
+        if ent is not None:
+            _slot = None
+            return ent if back is None else ent.to(back)
+    if defer is not None and parked.untyped_storage().data_ptr() == logits.untyped_storage().data_ptr():
+        defer[0] = 1
     return None
+
+
+def _has_reader(logits) -> bool:
+    """True while an entropy computed on its own from the same memory is alive with a graph: its node has saved the
+    logits, so a log-prob node built now must not overwrite them."""
+    global _entropy_reader
+    if _entropy_reader is None:
+        return False
+    ent_ref, storage = _entropy_reader
+    if ent_ref() is None:
+        _entropy_reader = None
+        return False
+    return storage == logits.untyped_storage().data_ptr()
+
+
+def _logprobs(logits, labels, inplace_backward, caller_logits, back):
+    global _slot
+    tracked = logits.requires_grad and torch.is_grad_enabled()
+    if inplace_backward and tracked and _has_reader(logits):
+        inplace_backward = False
+    defer = torch.zeros(1, dtype=torch.int32) if (inplace_backward and tracked) else None
+    lp, ent = _lpe(logits, labels, 1.0, _PAIRING, inplace_backward, _SKIP_ZERO_ROWS, defer)
+    if _PAIRING:
+        lp._siirl_paired_entropy = ent  # keeps the entropy (and through it the node) alive as long as the log-probs
+        _slot = (weakref.ref(caller_logits), _version(caller_logits), torch.is_grad_enabled(), weakref.ref(ent), defer,
+                 back)
+    elif defer is not None:
+        _slot = (weakref.ref(caller_logits), 0, True, None, defer, back)
+    return lp
+
+
+# The same pairing for code that torch.compile traces: plain module state that Dynamo can follow.
+_traced_slot = None
+
+
+def _traced_logprobs(logits, labels, inplace_backward):
+    global _traced_slot
+    if _PAIRING and not inplace_backward:
+        lp, ent = _LogprobEntropy.apply(logits, labels, 1.0, True, False)
+        _traced_slot = (weakref.ref(logits), logits._version, torch.is_grad_enabled(), ent)
+        return lp
+    lp, _ = _LogprobEntropy.apply(logits, labels, 1.0, False, bool(inplace_backward))
+    return lp
+
+
+def _traced_entropy(logits):
+    global _traced_slot
+    if _PAIRING and _traced_slot is not None:
+        ref, version, grad_mode, entropy = _traced_slot
+        _traced_slot = None
+        if ref() is logits and logits._version == version and torch.is_grad_enabled() == grad_mode:
+            return entropy
+    _, ent = _LogprobEntropy.apply(logits, None, 1.0, True, False)
+    return ent
 
 
 # ------------------------------------------------------------------------------ reference API
@@ -131,18 +223,23 @@ def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_bac
     """Log-probability of ``labels`` under ``softmax(logits)``, shape ``logits.shape[:-1]``
     (reference ``torch_functional.py:56-82``).  With ``inplace_backward=True`` the backward pass
     overwrites ``logits`` with its gradient, as the reference's flash-attn path does (``:85-90``)."""
-    logits = _check_logits(logits)
-    if _PAIRING and not inplace_backward:
-        lp, ent = _LogprobEntropy.apply(logits, labels, 1.0, True, False)
-        _park(logits, ent)
-        return lp
-    lp, _ = _LogprobEntropy.apply(logits, labels, 1.0, False, bool(inplace_backward))
-    return lp
+    x, back = _check_logits(logits)
+    if torch.compiler.is_compiling():
+        lp = _traced_logprobs(x, labels, inplace_backward)
+    else:
+        # a converted copy (fp64, non-unit vocab stride) is private to this call: nothing to overwrite in place
+        lp = _logprobs(x, labels, bool(inplace_backward) and x is logits, logits, back)
+    return lp if back is None else lp.to(back)
 
 
 def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor):
-    """reference ``torch_functional.py:99-116``; same kernel, never in place."""
-    return logprobs_from_logits(logits, labels, inplace_backward=False)
+    """reference ``torch_functional.py:99-116``; same kernel, never in place, nothing parked."""
+    x, back = _check_logits(logits)
+    if torch.compiler.is_compiling():
+        lp, _ = _LogprobEntropy.apply(x, labels, 1.0, False, False)
+    else:
+        lp, _ = _lpe(x, labels, 1.0, False, False, _SKIP_ZERO_ROWS, None)
+    return lp if back is None else lp.to(back)
 
 
 logprobs_from_logits_naive = logprobs_from_logits_v2  # reference :93-96
@@ -150,12 +247,18 @@ logprobs_from_logits_naive = logprobs_from_logits_v2  # reference :93-96
 
 def entropy_from_logits(logits: torch.Tensor):
     """Entropy of ``softmax(logits)`` per row (reference ``torch_functional.py:128-132``)."""
-    logits = _check_logits(logits)
-    parked = _claim(logits) if _PAIRING else None
+    x, back = _check_logits(logits)
+    if torch.compiler.is_compiling():
+        ent = _traced_entropy(x)
+        return ent if back is None else ent.to(back)
+    global _entropy_reader
+    parked = _claim(logits)
     if parked is not None:
         return parked
-    _, ent = _LogprobEntropy.apply(logits, None, 1.0, True, False)
-    return ent
+    _, ent = _lpe(x, None, 1.0, True, False, _SKIP_ZERO_ROWS, None)
+    if ent.requires_grad:
+        _entropy_reader = (weakref.ref(ent), x.untyped_storage().data_ptr())
+    return ent if back is None else ent.to(back)
 
 
 def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 2048):
@@ -163,55 +266,38 @@ def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 20
     kernel has none, so the whole tensor goes in one launch.  2-D input, fp32 output, as there."""
     if logits.dim() != 2:
         raise ValueError("entropy_from_logits_with_chunking expects a 2-D tensor")
-    return entropy_from_logits(logits)
+    ent = entropy_from_logits(logits)
+    return ent if ent.dtype == torch.float32 else ent.to(torch.float32)
 
 
 # ------------------------------------------------------------------------------ masked reductions
 
 
 def _masked_reduce(values: torch.Tensor, mask: torch.Tensor, axis, want_mean: bool):
-    from . import _lib
-    from . import core_algos as CA
-
     if not values.is_cuda:
         raise RuntimeError("siirl_amd: masked reductions run on the GPU only (no CPU fallback)")
-    nd = values.dim()
-    if isinstance(axis, (tuple, list)):
-        axis = axis[0] if len(axis) == 1 else (None if sorted(a % nd for a in axis) == list(range(nd)) else axis)
-    per_row = axis is not None
-    if per_row and (not isinstance(axis, int) or axis % nd != nd - 1):
-        raise NotImplementedError("siirl_amd: masked_sum / masked_mean reduce over all elements or over the last axis")
-    if values.requires_grad and torch.is_grad_enabled():
-        if want_mean and not per_row:  # identical arithmetic to agg_loss(..., 'token-mean'), which has a backward
-            return CA.agg_loss(values, mask.expand_as(values), "token-mean")
-        raise NotImplementedError("siirl_amd: only masked_mean over all elements is differentiable here")
-    dev = values.device
-    mask = mask.expand_as(values)
-    v = CA._as_2d(CA._f32(values, dev)) if nd >= 1 else CA._f32(values, dev).reshape(1, 1)
-    m, mcode = CA._mask_arg(CA._as_2d(mask) if nd >= 1 else mask.reshape(1, 1), dev)
-    B, L = v.shape
-    ws, nws = CA._workspace(B, L, dev)
-    row = torch.empty(B, dtype=torch.float32, device=dev) if per_row else None
-    tot = None if per_row else torch.empty(2, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
-        rc = _lib.lib().siirl_masked_reduce(_lib.ptr(v), _lib.ptr(m), mcode, B, L,
-                                            _lib.ptr(row) if (per_row and not want_mean) else None,
-                                            _lib.ptr(row) if (per_row and want_mean) else None, _lib.ptr(tot),
-                                            _lib.ptr(ws), nws, _lib.current_stream(dev))
-    _lib.check(rc, "siirl_masked_reduce")
-    if per_row:
-        return row.reshape(values.shape[:-1])
-    return tot[1] if want_mean else tot[0]
+    if axis is None:
+        axes = []
+    elif isinstance(axis, (tuple, list)):
+        axes = [int(a) for a in axis]
+        if not axes:  # torch's sum over an empty tuple of axes reduces everything
+            axes = list(range(values.dim()))
+    else:
+        axes = [int(axis)]
+    if axis is not None and values.dim() and len(set(a % values.dim() for a in axes)) == values.dim():
+        axes = []
+    return _OPS.masked_reduce(values, mask, axes, want_mean)
 
 
 def masked_sum(values: torch.Tensor, mask: torch.Tensor, axis=None):
-    """``sum(where(mask, values, 0) * mask)`` over everything or over the last axis (reference
-    ``torch_functional.py:146-151``); fp32 result."""
+    """``sum(where(mask, values, 0) * mask)`` over everything or over ``axis`` (an int or a tuple of ints;
+    reference ``torch_functional.py:146-151``); fp32 result, differentiable in ``values``."""
     return _masked_reduce(values, mask, axis, want_mean=False)
 
 
 def masked_mean(values: torch.Tensor, mask: torch.Tensor, axis=None):
-    """``masked_sum / (mask.sum + 1e-8)`` (reference ``torch_functional.py:154-168``)."""
+    """``masked_sum / (mask.sum(axis) + 1e-8)`` (reference ``torch_functional.py:154-168``); differentiable in
+    ``values``."""
     return _masked_reduce(values, mask, axis, want_mean=True)
 
 

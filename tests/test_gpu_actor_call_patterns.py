@@ -1,0 +1,264 @@
+"""The call sequences of the reference actor around the log-prob / entropy functions, on the GPU against the CPU
+oracle: the padded path (``siirl/engine/actor/dp_actor.py:254-260``: default in-place log-prob, then the entropy of the
+same tensor, plain or under ``torch.utils.checkpoint``), orders of the two calls that an autograd engine could run
+either way round, the lifetime of what the pairing keeps, float64 logits, and the general masked reductions
+(``siirl/utils/model_utils/torch_functional.py:103-107,146-168``)."""
+
+import gc
+
+import pytest
+import torch
+
+from oracle import torch_functional as OF
+
+pytestmark = pytest.mark.gpu
+
+
+def _bf16_close(got, want64, parts=None):
+    """<= 1 bf16 ulp of the fp64 value (or of the separately rounded parts' magnitudes), or tiny."""
+    mag = want64.abs() if parts is None else sum(p.abs() for p in parts) + want64.abs()
+    tol = 2.0 ** -7 * mag + 1e-6
+    err = (got.double() - want64).abs()
+    return bool((err <= tol).all()), err.max().item()
+
+
+def _padded_inputs(seed, B=3, S=11, L=6, V=517):
+    g = torch.Generator().manual_seed(seed)
+    full = (torch.randn(B, S, V, generator=g) * 2).to(torch.bfloat16)
+    y = torch.randint(0, V, (B, L), generator=g)
+    w_lp, w_ent = torch.randn(B, L, generator=g), torch.randn(B, L, generator=g)
+    return full, y, w_lp, w_ent, L
+
+
+@pytest.mark.parametrize("pairing", [True, False])
+@pytest.mark.parametrize("mode", ["plain", "checkpoint", "checkpoint_reentrant", "no_entropy"])
+def test_padded_actor_pattern(dev, mode, pairing):
+    """dp_actor.py:254-260: ``logits = logits[:, -L-1:-1, :]``; ``logprobs_from_logits(logits, responses)`` with the
+    default ``inplace_backward=True``; then ``entropy_from_logits(logits)`` on the same tensor, optionally through
+    ``torch.utils.checkpoint``.  Both gradients must reach the model's logits whatever the node order."""
+    import torch.utils.checkpoint as ckpt
+
+    import siirl_amd.torch_functional as SF
+
+    full, y, w_lp, w_ent, L = _padded_inputs(3)
+    SF.set_pairing(pairing)
+    try:
+        leaf = full.to(dev).requires_grad_(True)
+        out = leaf * 1.0  # the model's output: not a leaf
+        logits = out[:, -L - 1:-1, :]
+        lp = SF.logprobs_from_logits(logits, y.to(dev))
+        if mode == "no_entropy":
+            loss = (lp * w_lp.to(dev)).sum()
+        else:
+            if mode == "plain":
+                ent = SF.entropy_from_logits(logits)
+            else:
+                ent = ckpt.checkpoint(SF.entropy_from_logits, logits, use_reentrant=mode.endswith("reentrant"))
+            if pairing and mode != "checkpoint_reentrant":
+                assert ent.grad_fn is lp.grad_fn  # one node: one pass writes both gradients
+            loss = (lp * w_lp.to(dev)).sum() + (ent * w_ent.to(dev)).sum()
+        loss.backward()
+    finally:
+        SF.set_pairing(True)
+    xs = full[:, -L - 1:-1, :]
+    lp64, ent64, _, _ = OF.logprob_entropy_forward(xs, y, dtype=torch.float64)
+    assert (lp.detach().cpu().double() - lp64).abs().max() < 2e-5
+    d_lp = OF.logprob_entropy_backward(xs, y, w_lp, None, dtype=torch.float64)
+    if mode == "no_entropy":
+        want, parts = d_lp, None
+    else:
+        assert (ent.detach().cpu().double() - ent64).abs().max() < 2e-5
+        d_ent = OF.logprob_entropy_backward(xs, y, None, w_ent, dtype=torch.float64)
+        want = d_lp + d_ent
+        parts = None if (pairing and mode != "checkpoint_reentrant") else (d_lp, d_ent)
+    got = leaf.grad.cpu()
+    ok, err = _bf16_close(got[:, -L - 1:-1, :], want, parts)
+    assert ok, (mode, pairing, err)
+    assert torch.count_nonzero(got[:, :-L - 1]) == 0 and torch.count_nonzero(got[:, -1]) == 0
+
+
+@pytest.mark.parametrize("pairing", [True, False])
+def test_entropy_first_then_inplace_logprob(dev, pairing):
+    """The entropy node is built BEFORE an in-place log-prob node on the same tensor: the engine then runs the log-prob
+    node first.  It must not overwrite the logits the entropy node has saved."""
+    import siirl_amd.torch_functional as SF
+
+    full, y, w_lp, w_ent, L = _padded_inputs(4)
+    SF.set_pairing(pairing)
+    try:
+        leaf = full.to(dev).requires_grad_(True)
+        logits = (leaf * 1.0)[:, -L - 1:-1, :]
+        ent = SF.entropy_from_logits(logits)
+        lp = SF.logprobs_from_logits(logits, y.to(dev))  # default in-place
+        ((lp * w_lp.to(dev)).sum() + (ent * w_ent.to(dev)).sum()).backward()
+    finally:
+        SF.set_pairing(True)
+    xs = full[:, -L - 1:-1, :]
+    d_lp = OF.logprob_entropy_backward(xs, y, w_lp, None, dtype=torch.float64)
+    d_ent = OF.logprob_entropy_backward(xs, y, None, w_ent, dtype=torch.float64)
+    ok, err = _bf16_close(leaf.grad.cpu()[:, -L - 1:-1, :], d_lp + d_ent, (d_lp, d_ent))
+    assert ok, err
+
+
+def test_second_view_of_the_same_logits_downgrades_the_inplace_node(dev):
+    """entropy_from_logits on ANOTHER view object of the memory whose log-prob node is in-place: no pairing (different
+    tensor object), so the in-place node must turn out-of-place; the logits stay intact after backward."""
+    import siirl_amd.torch_functional as SF
+
+    full, y, w_lp, w_ent, L = _padded_inputs(5)
+    leaf = full.to(dev).requires_grad_(True)
+    out = leaf * 1.0
+    a, b = out[:, -L - 1:-1, :], out[:, -L - 1:-1, :]
+    before = out.detach().clone()
+    lp = SF.logprobs_from_logits(a, y.to(dev))
+    ent = SF.entropy_from_logits(b)
+    assert ent.grad_fn is not lp.grad_fn
+    ((lp * w_lp.to(dev)).sum() + (ent * w_ent.to(dev)).sum()).backward()
+    assert torch.equal(out.detach(), before)
+    xs = full[:, -L - 1:-1, :]
+    d_lp = OF.logprob_entropy_backward(xs, y, w_lp, None, dtype=torch.float64)
+    d_ent = OF.logprob_entropy_backward(xs, y, None, w_ent, dtype=torch.float64)
+    ok, err = _bf16_close(leaf.grad.cpu()[:, -L - 1:-1, :], d_lp + d_ent, (d_lp, d_ent))
+    assert ok, err
+
+
+def test_inplace_backward_still_overwrites_when_alone(dev):
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(6)
+    x = (torch.randn(10, 2049, generator=g) * 3).to(torch.bfloat16)
+    y = torch.randint(0, 2049, (10,), generator=g)
+    leaf = x.to(dev).requires_grad_(True)
+    xd = leaf * 1.0
+    lp = SF.logprobs_from_logits(xd, y.to(dev))
+    g_lp = torch.linspace(-1, 1, 10)
+    lp.backward(g_lp.to(dev))
+    want = OF.logprob_entropy_backward(x, y, g_lp, None, dtype=torch.float64)
+    ok, err = _bf16_close(leaf.grad.cpu(), want)
+    assert ok, err
+    ok2, _ = _bf16_close(xd.detach().cpu(), want)  # the logits buffer now holds the gradient
+    assert ok2
+
+
+def test_pairing_keeps_nothing_alive(dev):
+    """What logprobs_from_logits parks for a later entropy_from_logits is reachable only through the returned
+    log-probs: dropping them (with or without a backward) releases the [T, V] logits the node has saved."""
+    import siirl_amd.torch_functional as SF
+
+    T, V = 512, 32768  # 32 MiB of bf16 logits
+    y = torch.randint(0, V, (T,), device=dev)
+    gc.collect()
+    torch.cuda.synchronize()
+    base = torch.cuda.memory_allocated(dev)
+    for variant in ("dropped", "backward", "v2", "entropy_unclaimed_inplace"):
+        x = torch.randn(T, V, device=dev, dtype=torch.bfloat16).requires_grad_(True)
+        xd = x * 1.0
+        if variant == "v2":
+            lp = SF.logprobs_from_logits_v2(xd, y)
+        elif variant == "entropy_unclaimed_inplace":
+            lp = SF.logprobs_from_logits(xd, y)
+        else:
+            lp = SF.logprobs_from_logits(xd, y, inplace_backward=False)
+        assert torch.cuda.memory_allocated(dev) - base >= 2 * T * V * 2
+        if variant != "dropped":
+            lp.sum().backward()
+        del lp, xd, x
+        gc.collect()
+        assert torch.cuda.memory_allocated(dev) - base < (1 << 20), variant
+    # and a parked entropy that nobody claims does not survive its log-probs
+    x = torch.randn(64, 1000, device=dev, dtype=torch.bfloat16)
+    lp = SF.logprobs_from_logits(x, y[:64] % 1000, inplace_backward=False)
+    ent_ref = SF._slot[3]
+    assert ent_ref() is not None
+    del lp
+    gc.collect()
+    assert ent_ref() is None and SF.entropy_from_logits(x).shape == (64,)
+
+
+def test_v2_and_naive_park_nothing(dev):
+    import siirl_amd.torch_functional as SF
+
+    x = torch.randn(8, 100, device=dev)
+    y = torch.randint(0, 100, (8,), device=dev)
+    SF.set_pairing(True)  # clears the slot
+    a = SF.logprobs_from_logits_v2(x, y)
+    b = SF.logprobs_from_logits_naive(x, y)
+    assert SF._slot is None and torch.equal(a, b)
+    assert not hasattr(a, "_siirl_paired_entropy")
+    c = SF.logprobs_from_logits(x, y)
+    assert SF._slot is not None and torch.equal(a, c)
+    e = SF.entropy_from_logits(x)
+    assert e is c._siirl_paired_entropy and SF._slot is None
+
+
+def test_float64_logits(dev):
+    """The reference's fp32 / fp64 branch (torch_functional.py:103-107) takes float64 logits; here they are rounded
+    to fp32 once, computed as fp32 and returned as float64, gradient included."""
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(6, 301, generator=g, dtype=torch.float64) * 2
+    y = torch.randint(0, 301, (6,), generator=g)
+    xd = x.to(dev).requires_grad_(True)
+    lp = SF.logprobs_from_logits(xd, y.to(dev))
+    ent = SF.entropy_from_logits(xd)
+    lp2 = SF.logprobs_from_logits_v2(xd, y.to(dev))
+    assert lp.dtype == ent.dtype == lp2.dtype == torch.float64
+    lp64, ent64, _, _ = OF.logprob_entropy_forward(x, y, dtype=torch.float64)
+    assert (lp.detach().cpu() - lp64).abs().max() < 1e-5 and (ent.detach().cpu() - ent64).abs().max() < 1e-5
+    assert torch.equal(lp.detach(), lp2.detach())
+    w1, w2 = torch.randn(6, generator=g, dtype=torch.float64), torch.randn(6, generator=g, dtype=torch.float64)
+    ((lp * w1.to(dev)).sum() + (ent * w2.to(dev)).sum()).backward()
+    want = OF.logprob_entropy_backward(x, y, w1, w2, dtype=torch.float64)
+    assert xd.grad.dtype == torch.float64 and (xd.grad.cpu() - want).abs().max() < 1e-5
+    assert SF.entropy_from_logits_with_chunking(xd.detach()).dtype == torch.float32
+
+
+MASK_KINDS = ["int64", "bool", "float", "bf16"]
+
+
+def _mask(shape, kind, g):
+    m = torch.rand(shape, generator=g) > 0.35
+    return {"int64": m.long(), "bool": m, "float": m.float(), "bf16": m.to(torch.bfloat16)}[kind]
+
+
+@pytest.mark.parametrize("kind", MASK_KINDS)
+@pytest.mark.parametrize("axis", [None, -1, 1, 0, (0, 2), (1, 2), (0, 1, 2), 2])
+def test_masked_sum_and_mean_any_axis_with_backward(dev, axis, kind):
+    """masked_sum / masked_mean over any axis (reference torch_functional.py:146-168) and their gradient
+    (g * mask, divided by (mask.sum(axis) + 1e-8) for the mean), against the oracle and its autograd."""
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(13)
+    v = torch.randn(4, 5, 6, generator=g)
+    m = _mask((4, 5, 6), kind, g)
+    m[1, :, 2] = 0  # an empty reduction somewhere: 0 / 1e-8
+    for fn, ofn in ((SF.masked_sum, OF.masked_sum), (SF.masked_mean, OF.masked_mean)):
+        vd = v.to(dev).requires_grad_(True)
+        got = fn(vd, m.to(dev), axis=axis)
+        vo = v.double().requires_grad_(True)
+        mo = m if kind == "bool" else m.double()
+        want = ofn(vo, mo, axis=axis)
+        assert got.shape == want.shape, (got.shape, want.shape)
+        assert torch.allclose(got.detach().cpu().double(), want.detach(), rtol=1e-5, atol=1e-6)
+        w = torch.randn(want.shape, generator=g, dtype=torch.float64)
+        (got * w.to(dev).float()).sum().backward()
+        (want * w).sum().backward()
+        assert torch.allclose(vd.grad.cpu().double(), vo.grad, rtol=1e-5, atol=1e-7)
+
+
+def test_masked_reductions_broadcast_mask_and_no_grad(dev):
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(14)
+    v = torch.randn(7, 9, generator=g)
+    m = (torch.rand(1, 9, generator=g) > 0.5).long()  # broadcast over rows
+    got = SF.masked_mean(v.to(dev), m.to(dev), axis=-1)
+    want = OF.masked_mean(v.double(), m.expand(7, 9).double(), axis=-1)
+    assert not got.requires_grad and torch.allclose(got.cpu().double(), want, rtol=1e-5, atol=1e-6)
+    tot = SF.masked_sum(v.to(dev), m.to(dev))
+    assert tot.dim() == 0 and abs(tot.item() - OF.masked_sum(v.double(), m.expand(7, 9).double()).item()) < 1e-4
+    nan_outside = v.clone()
+    nan_outside[:, m[0] == 0] = float("nan")  # where(mask, v, 0): values outside the mask never matter
+    got2 = SF.masked_mean(nan_outside.to(dev), m.to(dev), axis=-1)
+    assert torch.equal(got2, got)

@@ -75,7 +75,7 @@ def test_no_cpu_fallback():
         with pytest.raises(RuntimeError, match="no GPU"):
             CA.compute_grpo_outcome_advantage(z, z, np.zeros(2, dtype=np.int64))
     with pytest.raises(TypeError):
-        SF.logprobs_from_logits(z.double(), torch.zeros(2, dtype=torch.long))
+        SF.logprobs_from_logits(z.long(), torch.zeros(2, dtype=torch.long))
 
 
 def test_row_blocks():

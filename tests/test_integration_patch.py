@@ -1,0 +1,61 @@
+"""The start-up patch of the integration guide, applied to stand-ins for the reference's two modules (CPU only):
+the actor-side functions and registry entries are replaced, the masked reductions that the reference also calls on
+host tensors (compute_gae_advantage_return -> masked_whiten -> masked_mean, clip_cov, kl_cov) are left alone."""
+import types
+
+import torch
+
+
+def _stub_modules():
+    F = types.ModuleType("ref_torch_functional")
+    A = types.ModuleType("ref_core_algos")
+
+    def masked_mean(values, mask, axis=None):  # the reference's, torch_functional.py:154-168
+        return (values * mask).sum(axis=axis) / (mask.sum(axis=axis) + 1e-8)
+
+    def masked_whiten(values, mask):  # resolves the module global, as the reference's does
+        return values - F.masked_mean(values, mask)
+
+    for name in ("logprobs_from_logits", "entropy_from_logits", "entropy_from_logits_with_chunking", "masked_sum"):
+        setattr(F, name, lambda *a, **k: "reference")
+    F.masked_mean, F.masked_whiten = masked_mean, masked_whiten
+    for name in ("agg_loss", "kl_penalty", "compute_policy_loss", "compute_policy_loss_vanilla",
+                 "compute_policy_loss_gspo", "compute_grpo_outcome_advantage", "apply_kl_penalty", "compute_policy_loss_gpg"):
+        setattr(A, name, lambda *a, **k: "reference")
+    A.POLICY_LOSS_REGISTRY = {"vanilla": A.compute_policy_loss_vanilla, "gspo": A.compute_policy_loss_gspo,
+                              "gpg": A.compute_policy_loss_gpg}
+    A.ADV_ESTIMATOR_REGISTRY = {"grpo": A.compute_grpo_outcome_advantage, "gae": object()}
+    return F, A
+
+
+def test_patch_replaces_the_actor_side_and_leaves_host_side_reductions():
+    import siirl_amd.core_algos as CA
+    import siirl_amd.torch_functional as SF
+    from siirl_amd.integration import CORE_ALGOS_NAMES, TORCH_FUNCTIONAL_NAMES, patch_reference
+
+    F, A = _stub_modules()
+    gae_before, gpg_before, masked_sum_before = A.ADV_ESTIMATOR_REGISTRY["gae"], A.compute_policy_loss_gpg, F.masked_sum
+    undo = patch_reference(F, A)
+    for name in TORCH_FUNCTIONAL_NAMES:
+        assert getattr(F, name) is getattr(SF, name)
+    for name in CORE_ALGOS_NAMES:
+        assert getattr(A, name) is getattr(CA, name)
+    assert A.POLICY_LOSS_REGISTRY["vanilla"] is CA.compute_policy_loss_vanilla
+    assert A.POLICY_LOSS_REGISTRY["gspo"] is CA.compute_policy_loss_gspo
+    assert A.POLICY_LOSS_REGISTRY["gpg"] is gpg_before
+    assert A.ADV_ESTIMATOR_REGISTRY["grpo"] is CA.compute_grpo_outcome_advantage
+    assert A.ADV_ESTIMATOR_REGISTRY["gae"] is gae_before
+    assert len(undo) == len(TORCH_FUNCTIONAL_NAMES) + len(CORE_ALGOS_NAMES)
+    # the reference's host-side whitening still resolves the reference's own masked_mean and runs on CPU tensors
+    assert F.masked_sum is masked_sum_before
+    v, m = torch.tensor([[1.0, 2.0, 3.0]]), torch.tensor([[1.0, 1.0, 0.0]])
+    assert torch.allclose(F.masked_whiten(v, m), v - 1.5)
+
+
+def test_integration_guide_names_the_same_recipe():
+    import os
+
+    text = open(os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "INTEGRATION.md")).read()
+    assert "patch_reference" in text
+    block = text[text.index("patch_reference"):]
+    assert '"masked_mean"' not in block.split("```")[0]

@@ -288,11 +288,13 @@ def bench_config5(args, dev):
         return (wall, sum(e[0].elapsed_time(e[1]) for e in evs) / steps,
                 sum(e[1].elapsed_time(e[2]) for e in evs) / steps)
 
-    # the memory-lean route first (no logits kept, the backward recomputes them), then the default
+    # the route the configuration names (no [T, V] tensor kept: the backward recomputes the logits) is the headline;
+    # the opt-in route that parks the fp32 logit tiles between forward and backward is reported beside it
     FL.set_saved_logits_limit(0)
-    r_wall, r_fwd_ms, r_bwd_ms = timed()
-    FL.set_saved_logits_limit(16 << 30)
     wall, fwd_ms, bwd_ms = timed()
+    FL.set_saved_logits_limit(16 << 30)
+    p_wall, p_fwd_ms, p_bwd_ms = timed()
+    FL.set_saved_logits_limit(0)
     saved_gb = FL._saved_logits_bytes(T, V) / 1e9
     gemm = 2.0 * T * H * V
     tf_step = 3 * gemm / (wall / steps) / 1e12
@@ -302,18 +304,22 @@ def bench_config5(args, dev):
         "ms_per_step": wall * 1e3 / steps, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"config5: fused lm_head + logprob/entropy, hidden [{T}, {H}], W [{V}, {H}], fwd + bwd to "
-                               "hidden and W", "tokens": T, "hidden": H, "vocab": V, "seed": SEED},
-        "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> parking its fp32 tiles + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
-                    "backward (dlogits from the parked tiles, d hidden and d weight per 65536 columns)": {"ms": bwd_ms, "TFLOP/s executed": 2 * gemm / bwd_ms / 1e9}},
-        "saved_logits_GB": saved_gb,
-        "recompute_variant": {"what": "set_saved_logits_limit(0): nothing kept between forward and backward, the "
-                                      "backward recomputes the logits per 8192-column slab",
-                              "ms_per_step": r_wall * 1e3 / steps, "tokens_per_s": T * steps / r_wall,
-                              "forward_ms": r_fwd_ms, "backward_ms": r_bwd_ms,
-                              "algorithmic_TFLOP/s": 3 * gemm / (r_wall / steps) / 1e12},
+                               "hidden and W, no [T, V] tensor kept (logits recomputed per 8192-column slab in the "
+                               "backward)", "tokens": T, "hidden": H, "vocab": V, "seed": SEED},
+        "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
+                    "backward (recompute + dlogits per slab, d hidden and d weight per 65536 columns)":
+                        {"ms": bwd_ms, "TFLOP/s executed": 3 * gemm / bwd_ms / 1e9}},
+        "parked_variant": {"what": "set_saved_logits_limit(16 GiB): the forward parks its fp32 logit tiles "
+                                   f"({saved_gb:.2f} GB) and the backward reads them back instead of recomputing; "
+                                   "opt-in, NOT the configuration's route",
+                           "ms_per_step": p_wall * 1e3 / steps, "tokens_per_s": T * steps / p_wall,
+                           "forward_ms": p_fwd_ms, "backward_ms": p_bwd_ms,
+                           "algorithmic_TFLOP/s": 3 * gemm / (p_wall / steps) / 1e12,
+                           "frac_of_peak": 3 * gemm / (p_wall / steps) / 1e12 / 2500.0},
         "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel", "achieved": tf_step, "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": tf_step / 2500.0, "traffic": None,
-                     "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step (forward, d hidden, d weight)"},
+                     "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step (forward, d hidden, d weight); the "
+                             "backward's recomputation of the logits (a fourth GEMM) is executed but not counted"},
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:  # the oracle's chunked fp32 matmul + log-softmax on the host cores, 256 tokens
@@ -452,8 +458,8 @@ def bench_config1(args, dev):
                                f"sequences, eps 0.2, token-mean, low_var_kl x 0.001", "tokens": tokens, "seed": SEED},
         "roofline": {"bound": "hbm", "kernel": "lpe_fwd_kernel + lpe_bwd_flat_kernel (whole step, wall clock)",
                      "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None,
-                     "note": "64 micro-batches of 262 MB each, about ten launches per micro-batch issued from Python: "
-                             "launch-bound as much as bandwidth-bound"},
+                     "note": "64 micro-batches of 262 MB each; per micro-batch two logits passes (0.12 ms at the "
+                             "config 2 rates) and the [8, 256] loss kernels, issued through the C++ torch.library layer"},
         "fused_step_variant": {"what": "siirl_actor_step_fused per micro-batch (one pass over the logits)",
                                "ms_per_step": fused_wall * 1e3 / steps, "tokens_per_s": tokens * steps / fused_wall,
                                "ms_per_step_as_one_hip_graph": graph_ms},
@@ -969,21 +975,41 @@ def main():
                            loss_agg_mode="token-mean", loss_mode="vanilla")
     x3 = logits.detach().view(Bq, Lq, V)
 
-    def fused():
-        return CA.fused_actor_step(x3, labels.view(Bq, Lq), old_lp, adv, mask.view(Bq, Lq), acfg, ref_log_prob=ref_lp)
+    def fused_ms_with(m2d):
+        def fused():
+            return CA.fused_actor_step(x3, labels.view(Bq, Lq), old_lp, adv, m2d, acfg, ref_log_prob=ref_lp)
 
-    for _ in range(2):
-        fused()
-    torch.cuda.synchronize()
-    t2 = time.perf_counter()
-    for _ in range(args.steps):
-        fused()
-    torch.cuda.synchronize()
-    fused_ms = (time.perf_counter() - t2) * 1e3 / args.steps
+        for _ in range(2):
+            fused()
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        for _ in range(args.steps):
+            fused()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t2) * 1e3 / args.steps
+
+    # bytes of the one-launch kernel by its own count: every row is read once (es*V) and written once (es*V); a row
+    # with a non-zero aggregation weight is read a second time except for the 8192 16-byte vectors (128 KiB) that stay
+    # in LDS between the passes; a zero-weight row (padding) is written as zeros without the second read
+    row_bytes = es * V
+    refetch = max(0.0, 1.0 - 131072.0 / row_bytes)
+    m2 = mask.view(Bq, Lq)
+    f_valid = float(m2.float().mean().item())
+    masked_ms = fused_ms_with(m2)
+    dense_ms = fused_ms_with(torch.ones_like(m2))
+    masked_bytes = T * row_bytes * (2.0 + refetch * f_valid)
+    dense_bytes = T * row_bytes * (2.0 + refetch)
     fused_step = {"what": "siirl_actor_step_fused: logits -> log-prob, entropy, PPO-clip + KL + entropy loss -> dlogits "
-                          "in one launch, padding rows included; plus the [B, L] scalar/metric pass",
-                  "ms_per_step": fused_ms, "tokens_per_s": T / fused_ms * 1e3,
-                  "GB/s_of_the_two_launch_byte_count": (fwd_bytes + bwd_bytes) / fused_ms / 1e6}
+                          "in one launch, plus the [B, L] scalar/metric pass",
+                  "bytes_model": "per row es*V read + es*V written + es*V*(1 - 128 KiB / (es*V)) read again when the "
+                                 "row's loss weight is non-zero (the rest of the row waits in LDS)",
+                  "config2_mask": {"valid_row_fraction": f_valid, "ms_per_step": masked_ms,
+                                   "tokens_per_s": T / masked_ms * 1e3, "bytes": masked_bytes,
+                                   "GB/s": masked_bytes / masked_ms / 1e6},
+                  "dense_mask": {"valid_row_fraction": 1.0, "ms_per_step": dense_ms, "tokens_per_s": T / dense_ms * 1e3,
+                                 "bytes": dense_bytes, "GB/s": dense_bytes / dense_ms / 1e6},
+                  "note": "the config 2 mask leaves part of the rows without a second read; compare the dense figure "
+                          "with the two-launch headline, which is dense"}
 
     out = {
         "metric": METRIC,
@@ -1007,7 +1033,9 @@ def main():
                     "lpe_bwd_flat_kernel": {"ms": bwd_ms, "GB/s": bwd_gbs, "bytes": bwd_bytes}},
         "roofline": {"bound": "hbm", "kernel": "lpe_bwd_flat_kernel", "achieved": bwd_gbs, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": bwd_gbs / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES if args.seqs == SEQS else None},
+                     "traffic": MEASURED_TRAFFIC_BYTES if args.seqs == SEQS else None,
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command in separate runs "
+                                       "(profiles/lpe_config2_hbm_traffic.md); a constant here, not read in this process"},
         "row_skip_variant": row_skip,
         "fused_step_variant": fused_step,
     }

@@ -87,7 +87,8 @@ const char* siirl_hip_last_error(void);
  * With z = x * inv_temperature, per row:
  *     lse[r]     = logsumexp(z)
  *     ex[r]      = sum softmax(z) * z
- *     logprob[r] = z[labels[r]] - lse[r]          (NaN when labels[r] is outside [0, V))
+ *     logprob[r] = z[labels[r]] - lse[r]          (0 when labels[r] == -100, the ignore_index of flash-attn's
+ *                                                  cross_entropy_loss; NaN for any other label outside [0, V))
  *     entropy[r] = lse[r] - ex[r]
  * Outputs are fp32.  labels and logprob may both be NULL (entropy only); entropy may be NULL;
  * lse is required; ex is required when entropy is requested and may be NULL otherwise.
@@ -110,6 +111,7 @@ int siirl_logprob_entropy_fwd(const void* logits, int logits_dtype, int64_t T, i
  *     p = exp(z - lse[r]),  z = x * inv_T,
  * in the dtype of the logits (round to nearest even).  g_logprob or g_entropy may be NULL (that
  * branch contributes nothing); labels is required iff g_logprob is given; ex iff g_entropy is.
+ * A row whose label is -100 (ignored) takes no gradient from g_logprob.
  * dlogits may be the logits buffer itself (in-place backward, same stride), otherwise the two must
  * not overlap.  lse / ex are the forward's outputs for the same inv_temperature.
  *

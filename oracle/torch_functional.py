@@ -44,6 +44,17 @@ def logprobs_from_logits(logits, labels, inplace_backward=True, *, dtype=None, l
     return picked - torch.logsumexp(x, dim=-1)
 
 
+def logprobs_from_logits_flash_attn(logits, labels, *, dtype=None):
+    """The reference's flash-attn dispatch (``torch_functional.py:73-90``): ``-cross_entropy_loss(logits, labels)[0]``.
+    flash-attn (2.7.3 / 2.8.2, not in the reference tree) computes the per-row cross entropy in fp32 with its default
+    ``ignore_index=-100``: an ignored row has loss 0 and receives no gradient.  Stated here with torch's own
+    ``F.cross_entropy``, which has the same default and the same convention.  Parity with flash-attn's Triton kernel
+    itself is unpinned (third party); this function is pinned by the library routine it calls."""
+    x = logits.to(_work_dtype(logits, dtype))
+    flat = -F.cross_entropy(x.reshape(-1, x.shape[-1]), labels.reshape(-1), reduction="none")
+    return flat.reshape(labels.shape)
+
+
 def entropy_from_logits(logits, *, dtype=None, literal_bf16=False):
     """``H = logsumexp(x) - sum(softmax(x) * x)`` (reference ``torch_functional.py:128-132``)."""
     if literal_bf16:

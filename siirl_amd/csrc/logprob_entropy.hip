@@ -16,6 +16,11 @@
 namespace siirl {
 namespace {
 
+// A label equal to this value is ignored: log-prob 0 and no gradient through it.  It is the default ignore_index of
+// flash-attn's cross_entropy_loss, which the reference's logprobs_from_logits dispatches to when flash-attn is
+// installed (siirl/utils/model_utils/torch_functional.py:73-90).  Any other label outside [0, V) yields NaN.
+constexpr int64_t kIgnoreIndex = -100;
+
 // Tuning knobs.  Measured on MI355X at T=32768, V=152064, bf16: non-temporal loads are worth 12% on the
 // forward (a pure read stream); on the backward (read + write) the hints are within run-to-run noise;
 // 256 threads with 4 loads in flight per lane beat 512/1024 threads and deeper unrolling on both.
@@ -239,7 +244,7 @@ __global__ __launch_bounds__(kFwdThreads) void lpe_fwd_kernel(const typename E::
     }
     if (logprob != nullptr) {
       const int64_t y = labels[row];
-      float lp = __builtin_nanf("");
+      float lp = y == kIgnoreIndex ? 0.f : __builtin_nanf("");
       if (y >= 0 && y < (int64_t)V) lp = E::load1(x + y) * inv_T - lse;
       logprob[row] = lp;
     }
@@ -274,7 +279,7 @@ __global__ __launch_bounds__(kBwdThreads) void lpe_bwd_kernel(const typename E::
   const int tid = threadIdx.x;
   const RowSplit<E> sp(x, d, V);
 
-  const float g1 = g_lp ? g_lp[row] : 0.f;
+  const float g1 = (g_lp && labels[row] != kIgnoreIndex) ? g_lp[row] : 0.f;
   const float g2 = HAS_ENT ? g_ent[row] : 0.f;
   const u32x4* xv = reinterpret_cast<const u32x4*>(x + sp.head);
   u32x4* dv = reinterpret_cast<u32x4*>(d + sp.head);
@@ -387,7 +392,7 @@ __global__ __launch_bounds__(kBwdThreads) void lpe_bwd_flat_kernel(const typenam
     const int64_t row = row0 + q;
     rc[q] = RowCoef{0.f, 0.f, 0.f, 0.f, -1, 0, true};
     if (row < T) {
-      const float g1 = g_lp ? g_lp[row] : 0.f;
+      const float g1 = (g_lp && labels[row] != kIgnoreIndex) ? g_lp[row] : 0.f;
       const float g2 = HAS_ENT ? g_ent[row] : 0.f;
       rc[q].zero = (flags & SIIRL_BWD_SKIP_ZERO_ROWS) && g1 == 0.f && g2 == 0.f;
       rc[q].nl = -lse[row] * kLog2e;
@@ -559,15 +564,17 @@ __global__ __launch_bounds__(kFusedThreads) void lpe_fused_kernel(const typename
   }
   __syncthreads();
   int y = -1;
+  bool ignored = false;
   {
     const int64_t yl = labels ? labels[row] : -1;
     if (yl >= 0 && yl < (int64_t)V) y = (int)yl;
+    ignored = labels && yl == kIgnoreIndex;
   }
   if (tid == 0) {
     for (int w = 1; w < kFusedThreads / kWave; ++w) merge(st, sm[w * 3], sm[w * 3 + 1], sm[w * 3 + 2], k);
     const float lse = st.mx * inv_T + logf(st.s);
     const float exv = ENT ? inv_T * (st.t / st.s) : 0.f;
-    const float lp = y >= 0 ? E::load1(x + y) * inv_T - lse : __builtin_nanf("");
+    const float lp = y >= 0 ? E::load1(x + y) * inv_T - lse : (ignored ? 0.f : __builtin_nanf(""));
     bc[0] = lse;
     bc[1] = exv;
     bc[2] = lp;
@@ -581,6 +588,7 @@ __global__ __launch_bounds__(kFusedThreads) void lpe_fused_kernel(const typename
   float g1, g2;
   coef(row, lp, lse - exv, g1, g2);
   if (!ENT) g2 = 0.f;
+  if (ignored) g1 = 0.f;
   BwdCoef c;
   c.k = k;
   c.nl = -lse * kLog2e;

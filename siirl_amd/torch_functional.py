@@ -337,13 +337,14 @@ def _whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool):
 
 
 def masked_var(values: torch.Tensor, mask: torch.Tensor, unbiased: bool = True):
-    """Variance over the masked elements (reference ``torch_functional.py:171-187``), 0-d fp32."""
+    """Variance over the masked elements (reference ``torch_functional.py:171-187``), 0-d fp32.  The biased form of
+    a mask that selects one element, or none, is 0 as there (``masked_mean`` of zeros, or ``0 / 1e-8``)."""
     _, stats = _whiten(values, mask, True)
     n = float(stats[2])
     if unbiased:
         _check_whiten_count(n)
         return stats[1]
-    return stats[1] * ((n - 1.0) / n) if n > 1 else stats[1]
+    return stats[1] * ((n - 1.0) / n) if n > 1 else torch.zeros_like(stats[1])
 
 
 def masked_whiten(values: torch.Tensor, mask: torch.Tensor, shift_mean: bool = True):

@@ -214,6 +214,57 @@ def test_float64_logits(dev):
     assert SF.entropy_from_logits_with_chunking(xd.detach()).dtype == torch.float32
 
 
+def test_ignored_label_minus_100(dev):
+    """A label of -100 (the default ignore_index of flash-attn's cross_entropy_loss, the reference's dispatch target
+    at torch_functional.py:73-90) gives log-prob 0 and takes no gradient; the row's entropy is unaffected."""
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(17)
+    x = (torch.randn(9, 1031, generator=g) * 2).to(torch.bfloat16)
+    y = torch.randint(0, 1031, (9,), generator=g)
+    y[2] = y[7] = -100
+    w1, w2 = torch.randn(9, generator=g), torch.randn(9, generator=g)
+    for inplace in (False, True):
+        leaf = x.to(dev).requires_grad_(True)
+        xd = leaf * 1.0
+        lp = SF.logprobs_from_logits(xd, y.to(dev), inplace_backward=inplace)
+        ent = SF.entropy_from_logits(xd)
+        want = OF.logprobs_from_logits_flash_attn(x, y, dtype=torch.float64)
+        assert lp[2].item() == 0.0 and lp[7].item() == 0.0
+        assert (lp.detach().cpu().double() - want).abs().max() < 2e-5
+        ((lp * w1.to(dev)).sum() + (ent * w2.to(dev)).sum()).backward()
+        xo = x.double().requires_grad_(True)
+        (OF.logprobs_from_logits_flash_attn(xo, y) * w1.double()).sum().backward()
+        d_ent = OF.logprob_entropy_backward(x, y.clamp(min=0), None, w2, dtype=torch.float64)
+        ok, err = _bf16_close(leaf.grad.cpu(), xo.grad + d_ent)
+        assert ok, (inplace, err)
+    # the strided (row-per-workgroup) backward and the single-launch step treat it the same way
+    wide = torch.zeros(9, 1040, dtype=torch.bfloat16)
+    wide[:, 3:1034] = x
+    wd = wide.to(dev).requires_grad_(True)
+    lp2 = SF.logprobs_from_logits(wd[:, 3:1034], y.to(dev), inplace_backward=False)
+    (lp2 * w1.to(dev)).sum().backward()
+    xo = x.double().requires_grad_(True)
+    (OF.logprobs_from_logits_flash_attn(xo, y) * w1.double()).sum().backward()
+    ok, err = _bf16_close(wd.grad.cpu()[:, 3:1034], xo.grad)
+    assert ok and lp2[2].item() == 0.0, err
+    other = SF.logprobs_from_logits(x.to(dev), torch.full((9,), -7).to(dev))
+    assert torch.isnan(other).all()  # any other label outside [0, V) is an error value, not an ignored row
+
+
+def test_biased_masked_var_of_one_element(dev):
+    """reference torch_functional.py:171-187 with unbiased=False: a mask selecting one element (or none) gives 0."""
+    import siirl_amd.torch_functional as SF
+
+    v = torch.tensor([[1.0, 5.0, -2.0]], device=dev)
+    assert SF.masked_var(v, torch.tensor([[0, 1, 0]], device=dev), unbiased=False).item() == 0.0
+    assert SF.masked_var(v, torch.tensor([[0, 0, 0]], device=dev), unbiased=False).item() == 0.0
+    two = SF.masked_var(v, torch.tensor([[1, 1, 0]], device=dev), unbiased=False).item()
+    assert abs(two - 4.0) < 1e-6
+    with pytest.raises(ValueError):
+        SF.masked_var(v, torch.tensor([[0, 1, 0]], device=dev), unbiased=True)
+
+
 MASK_KINDS = ["int64", "bool", "float", "bf16"]
 
 

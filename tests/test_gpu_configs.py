@@ -75,8 +75,9 @@ def test_config1_grpo_step_fp32(dev):
         # fused single-launch composition
         fused = CA.actor_loss(old.to(dev), lp, adv[rows], mask[rows].to(dev), cfg, ref_log_prob=ref.to(dev),
                               loss_scale_factor=scale)
-        assert abs(float(loss) - float(loss_o)) < 1e-3 and abs(float(fused.loss) - float(loss_o)) < 1e-3
-        assert abs(float(loss) - float(fused.loss)) < 1e-6
+        loss_v, fused_v = loss.detach().item(), fused.loss.detach().item()
+        assert abs(loss_v - float(loss_o)) < 1e-3 and abs(fused_v - float(loss_o)) < 1e-3
+        assert abs(loss_v - fused_v) < 1e-6
         m = fused.metrics()
         for k in ("actor/pg_loss", "actor/pg_clipfrac", "actor/ppo_kl", "actor/pg_clipfrac_lower", "actor/kl_loss",
                   "actor/pg_clip_mean", "actor/pg_clip_min", "actor/pg_clip_max"):
@@ -177,7 +178,7 @@ def test_config3_dapo_loss_path(dev):
     lp_c, old_c, mask_c = lp.cpu(), old.cpu(), mask_k.cpu().long()
     want = OC.compute_policy_loss_vanilla(old_c, lp_c, adv_o, mask_c, "token-mean", cfg)
     for a, b in zip((pg, cf, kl, cfl), want):
-        assert abs(float(a) - float(b)) < 1e-3, (float(a), float(b))
+        assert abs(a.detach().item() - float(b)) < 1e-3, (a.detach().item(), float(b))
     # gradient: full fp64 autograd on the first 256 kept rows with the batch-wide token count as the normaliser
     sub = slice(0, 256)
     x64 = lp_c[sub].double().requires_grad_(True)
@@ -216,7 +217,7 @@ def test_config4_gspo_long_context(dev):
     want = OC.compute_policy_loss_gspo(old.cpu().double(), lp.detach().cpu().double(), adv.cpu().double(), mask.cpu(),
                                        "token-mean", cfg)
     for a, b in zip((pg, cf, kl, cfl), want):
-        assert abs(float(a) - float(b)) < 1e-3, (float(a), float(b))
+        assert abs(a.detach().item() - float(b)) < 1e-3, (a.detach().item(), float(b))
     sample = torch.randperm(L, device=dev, generator=gen)[:40]
     lp_o = OF.logprobs_from_logits(x[sample].cpu(), y[sample].cpu())
     assert (lp.detach()[0, sample].cpu() - lp_o).abs().max() < 1e-3

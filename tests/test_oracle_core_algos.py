@@ -86,11 +86,11 @@ def test_vanilla_known_cases():
     mask = torch.ones(1, 6, dtype=torch.int64)
     A = torch.tensor([[1.0, -1.0, 2.0, -2.0, 0.5, -0.5]], dtype=torch.float64)
     pg, cf, kl, cfl = OC.compute_policy_loss_vanilla(old, old.clone(), A, mask, "token-mean", cfg)
-    assert abs(float(pg) + float(A.mean())) < 1e-9 and float(cf) == 0 and float(kl) == 0 and float(cfl) == 0
+    assert abs(float(pg.detach()) + float(A.mean())) < 1e-9 and float(cf) == 0 and float(kl) == 0 and float(cfl) == 0
     lp = torch.log(torch.tensor([[1.5, 0.5, 4.0, 1.1, 1.5, 4.0]], dtype=torch.float64)).requires_grad_(True)
     A2 = torch.tensor([[2.0, -1.0, -1.0, 1.0, -1.0, 1.0]], dtype=torch.float64)
     pg, cf, kl, cfl = OC.compute_policy_loss_vanilla(old, lp, A2, mask, "seq-mean-token-sum", cfg)
-    assert abs(float(pg) - (-2.56 + 0.8 + 3.0 - 1.1 + 1.5 - 1.28)) < 1e-9
+    assert abs(float(pg.detach()) - (-2.56 + 0.8 + 3.0 - 1.1 + 1.5 - 1.28)) < 1e-9
     assert abs(float(cf) - 0.5) < 1e-7 and abs(float(cfl) - 1 / 6) < 1e-7
     assert abs(float(kl) + float(lp.detach().mean())) < 1e-7
     pg.backward()
@@ -99,7 +99,7 @@ def test_vanilla_known_cases():
     lp2 = torch.tensor([[25.0]], dtype=torch.float64, requires_grad=True)
     pg, *_ = OC.compute_policy_loss_vanilla(torch.zeros(1, 1, dtype=torch.float64), lp2, torch.tensor([[-1e-9]], dtype=torch.float64),
                                             torch.ones(1, 1), "token-mean", _cfg(c=1e12))
-    assert abs(float(pg) - 1e-9 * math.exp(20)) < 1e-6
+    assert abs(float(pg.detach()) - 1e-9 * math.exp(20)) < 1e-6
     pg.backward()
     assert float(lp2.grad) == 0.0
     with pytest.raises(AssertionError):
@@ -141,7 +141,7 @@ def test_gspo_reduces_to_ppo_for_length_one_and_known_case():
     A = torch.tensor([[2.0, 2.0, 2.0]], dtype=torch.float64)
     pg, cf, kl, _ = OC.compute_policy_loss_gspo(old, lp, A, m, "token-mean", _cfg(0.1, 0.1))
     rho = math.exp(0.2)
-    assert abs(float(pg) - (-2 * 1.1)) < 1e-9 and rho > 1.1 and abs(float(cf) - 1.0) < 1e-7
+    assert abs(float(pg.detach()) - (-2 * 1.1)) < 1e-9 and rho > 1.1 and abs(float(cf) - 1.0) < 1e-7
     assert abs(float(kl) + 0.2) < 1e-7
 
 

@@ -114,3 +114,19 @@ def test_masked_reductions():
     assert torch.allclose(OF.masked_mean(v, m, axis=-1), torch.tensor([1.5, 5.5]), atol=1e-6)
     assert float(OF.masked_mean(v, torch.zeros_like(m))) == 0.0  # 0 / 1e-8
     assert float(OF.gather_from_labels(v, torch.tensor([1, 2]))[1]) == 6.0
+
+
+def test_flash_attn_dispatch_statement_ignores_minus_100():
+    """oracle.logprobs_from_logits_flash_attn: equal to the v2 statement on ordinary labels; a label of -100 gives 0
+    and a zero gradient row (the convention of the cross-entropy routine it calls)."""
+    g = torch.Generator().manual_seed(4)
+    x = torch.randn(5, 13, generator=g, dtype=torch.float64, requires_grad=True)
+    y = torch.randint(0, 13, (5,), generator=g)
+    a = OF.logprobs_from_logits_flash_attn(x, y)
+    b = OF.logprobs_from_logits(x, y)
+    assert torch.allclose(a, b, atol=1e-12)
+    y[3] = -100
+    c = OF.logprobs_from_logits_flash_attn(x, y)
+    assert c[3].item() == 0.0 and torch.allclose(c[[0, 1, 2, 4]], b[[0, 1, 2, 4]].detach(), atol=1e-12)
+    (gx,) = torch.autograd.grad(c.sum(), x)
+    assert gx[3].abs().max().item() == 0.0 and gx[0].abs().max().item() > 0

@@ -6,14 +6,32 @@ import torch
 import siirl_amd.ops  # noqa: F401  (registers the ops)
 
 OPS = ("logprob_entropy_fwd", "logprob_entropy_bwd", "logprob_entropy_bwd_", "grpo_advantage", "group_keep_mask",
-       "agg_loss_fwd", "agg_loss_bwd", "policy_loss_fwd", "policy_loss_bwd", "kl_penalty_fwd", "kl_penalty_bwd",
+       "agg_loss_fwd", "agg_loss_bwd", "masked_reduce_fwd", "masked_reduce_bwd", "policy_loss_fwd", "policy_loss_bwd", "kl_penalty_fwd", "kl_penalty_bwd",
        "fused_linear_logprob_entropy_fwd", "fused_linear_logprob_entropy_bwd")
 
 
+DIFFERENTIABLE = ("logprob_entropy", "actor_loss", "agg_loss", "masked_reduce", "value_loss", "kl_penalty",
+                  "fused_linear_logprob_entropy")
+
+
 def test_ops_are_registered():
-    for name in OPS:
+    for name in OPS + DIFFERENTIABLE:
         op = getattr(torch.ops.siirl_hip, name)
         assert op.default._schema.name == f"siirl_hip::{name}"
+    # the in-place backward declares what it overwrites
+    assert "Tensor(a!) logits" in str(torch.ops.siirl_hip.logprob_entropy_bwd_.default._schema)
+
+
+def test_the_layer_is_the_cpp_library():
+    """The operators come from lib/libsiirl_torch.so (TORCH_LIBRARY(siirl_hip) in csrc/torch_ops.cpp), not from
+    Python-side registrations: they dispatch to a C++ kernel for the GPU key and have none for the CPU."""
+    import siirl_amd.ops as ops
+
+    assert ops.TORCH_LIB_PATH.exists() and ops.TORCH_LIB_PATH.name == "libsiirl_torch.so"
+    assert torch._C._dispatch_has_kernel_for_dispatch_key("siirl_hip::logprob_entropy_fwd", "CUDA")
+    assert not torch._C._dispatch_has_kernel_for_dispatch_key("siirl_hip::logprob_entropy_fwd", "CPU")
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.siirl_hip.kl_penalty_fwd(torch.zeros(2, 3), torch.zeros(2, 3), 0)
 
 
 def _loss_args(mk, B, L, with_optional):
@@ -38,6 +56,11 @@ def test_fake_kernels_give_shapes_without_a_gpu(with_optional):
         o, r = ns.agg_loss_fwd(mk((B, L), torch.float32), mk((B, L), torch.bool), 0)
         assert o.shape == (16,) and r.shape == (B,)
         assert ns.agg_loss_bwd(mk((1,), torch.float32), mk((B, L), torch.bool), o, r, 0).shape == (B, L)
+        r, ms = ns.masked_reduce_fwd(mk((B, L), torch.float32), mk((B, L), torch.int64), True, True)
+        assert r.shape == (B,) and ms.shape == (B,)
+        r, ms = ns.masked_reduce_fwd(mk((B, L), torch.float32), mk((B, L), torch.int64), False, False)
+        assert r.shape == (2,) and ms.shape == (1,)
+        assert ns.masked_reduce_bwd(mk((B,), torch.float32), mk((B, L), torch.bool), True, None).shape == (B, L)
         assert ns.kl_penalty_fwd(mk((B, L), torch.float32), mk((B, L), torch.float32), 3).shape == (B, L)
         d1, d2 = ns.kl_penalty_bwd(mk((B, L), torch.float32), mk((B, L), torch.float32), mk((B, L), torch.float32), 3,
                                    False, True, False)
@@ -76,6 +99,14 @@ def test_opcheck_on_the_gpu():
     lm, m = mk((B, L), torch.float32), torch.ones(B, L, dtype=torch.bool, device=dev)
     torch.library.opcheck(ns.agg_loss_fwd, (lm, m, 2), test_utils=checks)
     torch.library.opcheck(ns.kl_penalty_fwd, (lm, mk((B, L), torch.float32), 3), test_utils=checks)
+    torch.library.opcheck(ns.masked_reduce_fwd, (lm, m, True, True), test_utils=checks)
+    torch.library.opcheck(ns.masked_reduce_fwd, (lm, m, False, True), test_utils=checks)
+    _, msum = ns.masked_reduce_fwd(lm, m, True, True)
+    torch.library.opcheck(ns.masked_reduce_bwd, (torch.ones(B, device=dev), m, True, msum), test_utils=checks)
+    torch.library.opcheck(ns.logprob_entropy_bwd_, (mk((T, V), torch.bfloat16), torch.randint(0, V, (T,), device=dev),
+                                                     1.0, torch.zeros(T, device=dev), torch.zeros(T, device=dev),
+                                                     torch.ones(T, device=dev), torch.ones(T, device=dev), False),
+                          test_utils=checks)
     uid = torch.arange(B, device=dev) // 2
     torch.library.opcheck(ns.grpo_advantage, (lm, torch.ones(B, L, dtype=torch.int64, device=dev), uid, 1e-6, True),
                           test_utils=checks)

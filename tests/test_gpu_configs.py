@@ -247,7 +247,7 @@ def test_config4_gspo_long_context(dev):
     xd = logits.to(dev).requires_grad_(True)
     lpd = SF.logprobs_from_logits(xd, labels.to(dev))
     res = CA.actor_loss(oldm.to(dev), lpd, advm.to(dev), m.to(dev), ocfg)
-    assert abs(float(res.loss) - float(loss_o)) < 1e-3
+    assert abs(float(res.loss.detach()) - float(loss_o)) < 1e-3
     assert abs(float(res.pg_clipfrac) - met_o["actor/pg_clipfrac"]) < 1e-3
     res.loss.backward()
     ok, err = _bf16_grad_close(xd.grad.cpu(), dlog_o)

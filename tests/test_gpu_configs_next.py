@@ -50,7 +50,7 @@ def test_config3_value_loss_two_routes(dev):
     tok = torch.max((vp2 - returns) ** 2, (vc - returns) ** 2)
     loss2 = 0.5 * CA.agg_loss(tok, m, "seq-mean-token-mean")
     (g2,) = torch.autograd.grad(loss2, vp2)
-    assert abs(float(loss) - float(loss2)) < 1e-5 * abs(float(loss2)) + 1e-7
+    assert abs(float(loss.detach()) - float(loss2.detach())) < 1e-5 * abs(float(loss2.detach())) + 1e-7
     assert (g1 - g2).abs().max() <= 1e-9 + 1e-5 * g2.abs().max()
 
 
@@ -128,7 +128,7 @@ def test_config2_fused_step_equals_two_launch_path(dev):
     ent = F.entropy_from_logits(xr)
     two = CA.actor_loss(old, lp, adv, m, cfg, entropy=ent, ref_log_prob=ref, loss_scale_factor=0.25)
     two.loss.backward()
-    assert abs(float(two.loss.detach()) - float(out.loss)) < 1e-6
+    assert abs(float(two.loss.detach()) - float(out.loss.detach())) < 1e-6
     diff = (xr.grad.float() - out.dlogits.float()).abs()
     assert bool((diff <= 1e-12 + 2 ** -7 * xr.grad.float().abs()).all()), diff.max()
     # rows past the response lengths carry no gradient; rows sum to ~0 (softmax gradients)

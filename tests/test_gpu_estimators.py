@@ -20,7 +20,8 @@ AGGS = ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-tok
 
 
 def _close(got, want64, tol=2e-5):
-    return abs(float(got) - float(want64)) <= tol + 1e-5 * abs(float(want64))
+    got, want64 = float(got.detach()), float(want64.detach())
+    return abs(got - want64) <= tol + 1e-5 * abs(want64)
 
 
 def _grad_close(got, want64):
@@ -138,9 +139,9 @@ def test_value_loss(dev, mode, B, L):
     loss, frac = CA.compute_value_loss(x, returns.to(dev), values.to(dev), m.to(dev), clip, mode)
     x64 = vpreds.double().requires_grad_(True)
     loss_o, frac_o = OC.compute_value_loss(x64, returns.double(), values.double(), m, clip, mode)
-    assert _close(loss, loss_o) and _close(frac, frac_o), (float(loss), float(loss_o), float(frac), float(frac_o))
+    assert _close(loss, loss_o) and _close(frac, frac_o), (float(loss.detach()), float(loss_o), float(frac), float(frac_o))
     l32, f32 = OC.compute_value_loss(vpreds, returns, values, m, clip, mode)
-    assert abs(float(loss) - float(l32)) < 1e-3 and abs(float(frac) - float(f32)) < 1e-3
+    assert abs(float(loss.detach()) - float(l32)) < 1e-3 and abs(float(frac) - float(f32)) < 1e-3
     loss.backward()
     loss_o.backward()
     ok, err = _grad_close(x.grad.cpu(), x64.grad)
@@ -160,7 +161,7 @@ def test_value_loss_ties_follow_autograd(dev):
     loss, frac = CA.compute_value_loss(x, returns.to(dev), values.to(dev), m.to(dev), clip, "token-mean")
     x32 = vpreds.clone().requires_grad_(True)
     loss_o, frac_o = OC.compute_value_loss(x32, returns, values, m, clip, "token-mean")
-    assert abs(float(loss) - float(loss_o)) < 1e-6 and float(frac) == float(frac_o)
+    assert abs(float(loss.detach()) - float(loss_o)) < 1e-6 and float(frac) == float(frac_o)
     loss.backward()
     loss_o.backward()
     assert torch.allclose(x.grad.cpu(), x32.grad, rtol=1e-5, atol=1e-7), (x.grad.cpu(), x32.grad)
@@ -308,7 +309,7 @@ def test_actor_loss_with_drift(dev, loss_mode, agg):
     drift = OC.policy_drift_loss(old.double(), x64, m, agg)
     want = (pg - 0.01 * OC.agg_loss(e64, m, agg) + 0.05 * OC.agg_loss(OC.kl_penalty(x64, ref.double(), "low_var_kl"), m, agg)
             + 0.3 * drift) * 0.25
-    assert _close(out.loss, want), (float(out.loss), float(want))
+    assert _close(out.loss, want), (float(out.loss.detach()), float(want))
     assert _close(out.policy_drift_loss, drift)
     out.loss.backward()
     want.backward()

@@ -45,7 +45,7 @@ def _check(dev, logits, resp, mask, old, ref, adv, isw, cfg, T=1.0, scale=1.0, o
         loss_scale_factor=scale, on_policy=on_policy, rollout_is_weights=isw.double() if use_isw else None,
         dtype=torch.float64)
     assert out.dlogits.shape == x.shape and out.dlogits.dtype == x.dtype
-    assert abs(float(out.loss) - float(loss_o)) < 1e-3 * max(1.0, abs(float(loss_o)))
+    assert abs(float(out.loss.detach()) - float(loss_o)) < 1e-3 * max(1.0, abs(float(loss_o)))
     valid = mask.bool()
     assert (out.log_prob.cpu()[valid].double() - lp_o[valid]).abs().max() < 1e-3
     if ent_o is not None:
@@ -102,7 +102,7 @@ def test_fused_step_strided_view_and_two_pass_agreement(dev):
     two.loss.backward()
     diff = (x.grad.float() - out.dlogits.float()).abs()
     assert bool((diff <= 1e-7 + 2 ** -7 * x.grad.float().abs()).all()), diff.max()
-    assert abs(float(two.loss) - float(out.loss)) < 1e-5
+    assert abs(float(two.loss.detach()) - float(out.loss.detach())) < 1e-5
 
 
 def test_fused_step_masked_rows_are_zero_and_errors(dev):

@@ -381,7 +381,7 @@ def test_empty_batch_matches_reference_semantics(dev):
     assert float(SF.masked_mean(e, m)) == 0.0 and float(SF.masked_sum(e, m)) == 0.0
     v = torch.empty(0, L, device=dev, requires_grad=True)
     loss, clipfrac = CA.compute_value_loss(v, e, e, m, 0.5, "token-mean")
-    assert float(loss) == 0.0 and float(clipfrac) == 0.0
+    assert float(loss.detach()) == 0.0 and float(clipfrac) == 0.0
     loss.backward()
     assert v.grad.shape == (0, L)
 

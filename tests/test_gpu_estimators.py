@@ -19,8 +19,12 @@ pytestmark = pytest.mark.gpu
 AGGS = ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"]
 
 
+def _scalar(v):
+    return float(v.detach()) if isinstance(v, torch.Tensor) else float(v)
+
+
 def _close(got, want64, tol=2e-5):
-    got, want64 = float(got.detach()), float(want64.detach())
+    got, want64 = _scalar(got), _scalar(want64)
     return abs(got - want64) <= tol + 1e-5 * abs(want64)
 
 

@@ -42,8 +42,9 @@ def set_skip_zero_rows(flag: bool) -> None:
 
 
 class _LogprobEntropy(torch.autograd.Function):
-    """(logits, labels) -> (logprob, entropy) over the plain operators: the form ``torch.compile`` traces (the
-    operators are opaque to Dynamo and have fake kernels).  Eager calls use the C++ node ``logprob_entropy``."""
+    """(logits, labels) -> (logprob, entropy) over the plain operators, which are opaque to Dynamo and have fake
+    kernels: the form a ``torch.compile(fullgraph=True)`` region can hold (``logprob_entropy_traceable``).  Everything
+    else uses the C++ node ``logprob_entropy``."""
 
     @staticmethod
     def forward(ctx, logits, labels, inv_temperature, want_entropy, inplace_backward):
@@ -102,12 +103,33 @@ def logprobs_and_entropy_from_logits(logits: torch.Tensor, labels: torch.Tensor,
     """Both per-token outputs of the actor's post-logits step in one pass: ``(logprob, entropy)`` of
     ``logits / temperature``.  The division is folded into the kernels, ``logits`` is left untouched
     (the reference divides in place first, ``siirl/engine/actor/dp_actor.py:176``)."""
-    logits, back = _check_logits(logits)
     if torch.compiler.is_compiling():
-        lp, ent = _LogprobEntropy.apply(logits, labels, 1.0 / float(temperature), True, inplace_backward)
-    else:
-        lp, ent = _lpe(logits, labels, 1.0 / float(temperature), True, bool(inplace_backward), _SKIP_ZERO_ROWS, None)
+        return _outside_graph(logprobs_and_entropy_from_logits)(logits, labels, temperature, inplace_backward)
+    logits, back = _check_logits(logits)
+    lp, ent = _lpe(logits, labels, 1.0 / float(temperature), True, bool(inplace_backward), _SKIP_ZERO_ROWS, None)
     return (lp, ent) if back is None else (lp.to(back), ent.to(back))
+
+
+def logprob_entropy_traceable(logits: torch.Tensor, labels=None, temperature: float = 1.0, want_entropy: bool = True):
+    """``(logprob, entropy)`` as one Python ``autograd.Function`` over the plain ``torch.ops.siirl_hip`` operators
+    (opaque to Dynamo, with fake kernels): for a region compiled with ``torch.compile(fullgraph=True)``, where a
+    graph break is not allowed.  No pairing state, never in place; an output that was not asked for is empty."""
+    if logits.dtype not in _FLOATS:
+        raise TypeError(f"logits dtype {logits.dtype} is not supported (float32, bfloat16, float16)")
+    return _LogprobEntropy.apply(logits, labels, 1.0 / float(temperature), bool(want_entropy), False)
+
+
+# Under ``torch.compile`` the reference-named functions below leave the graph for the duration of the call (the
+# reference compiles ``entropy_from_logits`` alone, siirl/engine/actor/dp_actor.py:80-84, default ``fullgraph=False``):
+# the eager body runs as it would uncompiled, with the pairing and the in-place bookkeeping intact.
+_disabled = {}
+
+
+def _outside_graph(fn):
+    wrapped = _disabled.get(fn)
+    if wrapped is None:
+        wrapped = _disabled[fn] = torch.compiler.disable(fn)
+    return wrapped
 
 
 # ------------------------------------------------------------------------------ pairing
@@ -125,8 +147,8 @@ _entropy_reader = None  # (weakref to the last separately computed entropy that 
 
 
 def set_pairing(flag: bool) -> None:
-    global _PAIRING, _slot, _traced_slot, _entropy_reader
-    _PAIRING, _slot, _traced_slot, _entropy_reader = bool(flag), None, None, None
+    global _PAIRING, _slot, _entropy_reader
+    _PAIRING, _slot, _entropy_reader = bool(flag), None, None
 
 
 def _version(t):
@@ -186,31 +208,6 @@ def _logprobs(logits, labels, inplace_backward, caller_logits, back):
     return lp
 
 
-# The same pairing for code that torch.compile traces: plain module state that Dynamo can follow.
-_traced_slot = None
-
-
-def _traced_logprobs(logits, labels, inplace_backward):
-    global _traced_slot
-    if _PAIRING and not inplace_backward:
-        lp, ent = _LogprobEntropy.apply(logits, labels, 1.0, True, False)
-        _traced_slot = (weakref.ref(logits), logits._version, torch.is_grad_enabled(), ent)
-        return lp
-    lp, _ = _LogprobEntropy.apply(logits, labels, 1.0, False, bool(inplace_backward))
-    return lp
-
-
-def _traced_entropy(logits):
-    global _traced_slot
-    if _PAIRING and _traced_slot is not None:
-        ref, version, grad_mode, entropy = _traced_slot
-        _traced_slot = None
-        if ref() is logits and logits._version == version and torch.is_grad_enabled() == grad_mode:
-            return entropy
-    _, ent = _LogprobEntropy.apply(logits, None, 1.0, True, False)
-    return ent
-
-
 # ------------------------------------------------------------------------------ reference API
 
 
@@ -223,22 +220,20 @@ def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_bac
     """Log-probability of ``labels`` under ``softmax(logits)``, shape ``logits.shape[:-1]``
     (reference ``torch_functional.py:56-82``).  With ``inplace_backward=True`` the backward pass
     overwrites ``logits`` with its gradient, as the reference's flash-attn path does (``:85-90``)."""
-    x, back = _check_logits(logits)
     if torch.compiler.is_compiling():
-        lp = _traced_logprobs(x, labels, inplace_backward)
-    else:
-        # a converted copy (fp64, non-unit vocab stride) is private to this call: nothing to overwrite in place
-        lp = _logprobs(x, labels, bool(inplace_backward) and x is logits, logits, back)
+        return _outside_graph(logprobs_from_logits)(logits, labels, inplace_backward)
+    x, back = _check_logits(logits)
+    # a converted copy (fp64, non-unit vocab stride) is private to this call: nothing to overwrite in place
+    lp = _logprobs(x, labels, bool(inplace_backward) and x is logits, logits, back)
     return lp if back is None else lp.to(back)
 
 
 def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor):
     """reference ``torch_functional.py:99-116``; same kernel, never in place, nothing parked."""
-    x, back = _check_logits(logits)
     if torch.compiler.is_compiling():
-        lp, _ = _LogprobEntropy.apply(x, labels, 1.0, False, False)
-    else:
-        lp, _ = _lpe(x, labels, 1.0, False, False, _SKIP_ZERO_ROWS, None)
+        return _outside_graph(logprobs_from_logits_v2)(logits, labels)
+    x, back = _check_logits(logits)
+    lp, _ = _lpe(x, labels, 1.0, False, False, _SKIP_ZERO_ROWS, None)
     return lp if back is None else lp.to(back)
 
 
@@ -247,11 +242,10 @@ logprobs_from_logits_naive = logprobs_from_logits_v2  # reference :93-96
 
 def entropy_from_logits(logits: torch.Tensor):
     """Entropy of ``softmax(logits)`` per row (reference ``torch_functional.py:128-132``)."""
-    x, back = _check_logits(logits)
-    if torch.compiler.is_compiling():
-        ent = _traced_entropy(x)
-        return ent if back is None else ent.to(back)
     global _entropy_reader
+    if torch.compiler.is_compiling():
+        return _outside_graph(entropy_from_logits)(logits)
+    x, back = _check_logits(logits)
     parked = _claim(logits)
     if parked is not None:
         return parked

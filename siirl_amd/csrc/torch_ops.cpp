@@ -82,9 +82,11 @@ Tensor empty_f32(at::IntArrayRef shape, const Tensor& like) {
   return at::empty(shape, like.options().dtype(at::kFloat).memory_format(c10::nullopt));
 }
 
-// fp32, contiguous, on `dev`, detached from any graph
+// fp32, contiguous, on `dev`.  Called below the autograd keys (inside a node's forward / backward), where no
+// conversion records a graph; a tensor that already qualifies is returned as it is.
 Tensor f32c(const Tensor& t, const c10::Device& dev) {
-  Tensor r = t.detach();
+  if (t.scalar_type() == at::kFloat && t.device() == dev && t.is_contiguous()) return t;
+  Tensor r = t;
   if (r.device() != dev) r = r.to(dev);
   if (r.scalar_type() != at::kFloat) r = r.to(at::kFloat);
   return r.contiguous();
@@ -96,7 +98,7 @@ optional<Tensor> f32c(const optional<Tensor>& t, const c10::Device& dev) {
 
 // a mask in a dtype the kernels read as is (anything else becomes fp32), contiguous, on `dev`
 Tensor mask_arg(const Tensor& mask, const c10::Device& dev) {
-  Tensor m = mask.detach();
+  Tensor m = mask;
   if (m.device() != dev) m = m.to(dev);
   switch (m.scalar_type()) {
     case at::kBool: case at::kByte: case at::kInt: case at::kLong: case at::kFloat: case at::kBFloat16: case at::kHalf:
@@ -558,29 +560,36 @@ struct LossCfg {
   bool kl_st;
 };
 
-std::tuple<Tensor, Tensor, Tensor> policy_loss_fwd_impl(const Tensor& old, const Tensor& lp, const Tensor& adv,
-                                                        const Tensor& mask, const optional<Tensor>& isw,
-                                                        const optional<Tensor>& ent, const optional<Tensor>& ref,
-                                                        const LossCfg& c) {
+void policy_loss_fwd_launch(const Tensor& old, const Tensor& lp, const Tensor& adv, const Tensor& mask,
+                            const optional<Tensor>& isw, const optional<Tensor>& ent, const optional<Tensor>& ref,
+                            const LossCfg& c, float* out16, float* row_msum, float* row_s, void* ws, size_t nws) {
   require_f32c(lp, "log_prob");
   require_f32c(old, "old_log_prob");
   require_f32c(adv, "advantages");
   require_f32c(isw, "is_weights");
   require_f32c(ent, "entropy");
   require_f32c(ref, "ref_log_prob");
-  TORCH_CHECK_VALUE(lp.dim() == 2, "log_prob must be [B, L]");
   const int64_t B = lp.size(0), L = lp.size(1);
-  Tensor out16 = empty_f32({16}, lp), row_msum = empty_f32({B}, lp), row_s = empty_f32({B}, lp);
-  size_t nws;
-  Tensor ws = loss_workspace(B, L, lp, &nws);
   DeviceGuard guard(lp.device());
   check_rc(siirl_actor_loss_fwd(ptr<float>(old), ptr<float>(lp), ptr<float>(adv), ptr(mask), mask_code(mask),
                                 ptr<float>(isw), ptr<float>(ent), ptr<float>(ref), B, L, (int)c.loss_mode,
                                 (float)c.clip_low, (float)c.clip_high, (float)c.clip_c, (float)c.log_ratio_clamp,
                                 (int)c.agg_mode, (float)c.entropy_coeff, (int)c.kl_mode, (int)c.kl_st, (float)c.kl_coef,
-                                (float)c.drift_coef, (float)c.scale, ptr<float>(out16), ptr<float>(row_msum),
-                                ptr<float>(row_s), ptr(ws), nws, stream_of(lp)),
+                                (float)c.drift_coef, (float)c.scale, out16, row_msum, row_s, ws, nws, stream_of(lp)),
            "siirl_actor_loss_fwd");
+}
+
+std::tuple<Tensor, Tensor, Tensor> policy_loss_fwd_impl(const Tensor& old, const Tensor& lp, const Tensor& adv,
+                                                        const Tensor& mask, const optional<Tensor>& isw,
+                                                        const optional<Tensor>& ent, const optional<Tensor>& ref,
+                                                        const LossCfg& c) {
+  TORCH_CHECK_VALUE(lp.dim() == 2, "log_prob must be [B, L]");
+  const int64_t B = lp.size(0), L = lp.size(1);
+  Tensor out16 = empty_f32({16}, lp), row_msum = empty_f32({B}, lp), row_s = empty_f32({B}, lp);
+  size_t nws;
+  Tensor ws = loss_workspace(B, L, lp, &nws);
+  policy_loss_fwd_launch(old, lp, adv, mask, isw, ent, ref, c, ptr<float>(out16), ptr<float>(row_msum),
+                         ptr<float>(row_s), ptr(ws), nws);
   return {out16, row_msum, row_s};
 }
 
@@ -671,7 +680,16 @@ struct ActorLossFn : public torch::autograd::Function<ActorLossFn> {
     if (ref) same(*ref, "ref_log_prob");
     const LossCfg c{loss_mode, agg_mode, kl_mode, clip_low, clip_high, clip_c, log_ratio_clamp, entropy_coeff,
                     kl_coef, drift_coef, scale, kl_st};
-    auto [out16, row_msum, row_s] = policy_loss_fwd_impl(old, lp, adv, m, isw, ent, ref, c);
+    // one allocation for the result block, the two per-row vectors kept for the backward, and the scratch
+    // (64 floats | B | B | workspace at a 256-byte boundary of a 512-byte aligned block)
+    TORCH_CHECK_VALUE(lp.dim() == 2, "log_prob must be [B, L]");
+    const int64_t B = lp.size(0), L = lp.size(1);
+    const size_t nws = siirl_loss_workspace_bytes(B, L);
+    const int64_t head = (64 + 2 * B + 63) / 64 * 64;  // floats before the workspace
+    Tensor buf = empty_f32({head + (int64_t)((nws + 3) / 4)}, lp);
+    Tensor out16 = buf.narrow(0, 0, 16), row_msum = buf.narrow(0, 64, B), row_s = buf.narrow(0, 64 + B, B);
+    policy_loss_fwd_launch(old, lp, adv, m, isw, ent, ref, c, ptr<float>(out16), ptr<float>(row_msum),
+                           ptr<float>(row_s), ptr<float>(buf) + head, nws);
     ctx->save_for_backward({lp, old, adv, m, out16, row_msum, row_s, isw ? *isw : Tensor(), ent ? *ent : Tensor(),
                             ref ? *ref : Tensor()});
     ctx->saved_data["i"] = std::vector<int64_t>{loss_mode, agg_mode, kl_mode, (int64_t)kl_st, (int64_t)policy_only,

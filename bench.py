@@ -298,6 +298,26 @@ def bench_config5(args, dev):
     saved_gb = FL._saved_logits_bytes(T, V) / 1e9
     gemm = 2.0 * T * H * V
     tf_step = 3 * gemm / (wall / steps) / 1e12
+
+    # the same forward launch on quiet operands (all zeros): identical instruction stream, fewer wires toggling.
+    # The gap to the timing on the configuration's random operands is what the power limit costs.
+    def forward_ms(hh, ww, n=5):
+        with torch.no_grad():
+            for _ in range(2):
+                fused_linear_logprob_entropy(hh, ww, y)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                fused_linear_logprob_entropy(hh, ww, y)
+            e1.record()
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    fwd_random_ms = forward_ms(h.detach(), w.detach())
+    hz, wz = torch.zeros_like(h), torch.zeros_like(w)
+    fwd_zero_ms = forward_ms(hz, wz)
+    del hz, wz
     out = {
         "metric": "fused lm_head+logprob/entropy fwd+bwd tokens/sec @vocab152k bf16; % MFMA roofline",
         "value": T * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
@@ -316,6 +336,10 @@ def bench_config5(args, dev):
                            "forward_ms": p_fwd_ms, "backward_ms": p_bwd_ms,
                            "algorithmic_TFLOP/s": 3 * gemm / (p_wall / steps) / 1e12,
                            "frac_of_peak": 3 * gemm / (p_wall / steps) / 1e12 / 2500.0},
+        "power_limit_probe": {"what": "the forward alone (no grad) on the configuration's random operands and on "
+                                      "all-zero operands: same instructions, quieter data",
+                              "forward_ms_random_operands": fwd_random_ms, "TFLOP/s_random": gemm / fwd_random_ms / 1e9,
+                              "forward_ms_zero_operands": fwd_zero_ms, "TFLOP/s_zero": gemm / fwd_zero_ms / 1e9},
         "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel", "achieved": tf_step, "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": tf_step / 2500.0, "traffic": None,
                      "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step (forward, d hidden, d weight); the "

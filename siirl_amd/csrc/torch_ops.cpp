@@ -141,6 +141,7 @@ struct RowBlock { int64_t off, rows, stride; };
 void row_blocks(const Tensor& x, std::vector<RowBlock>& out) {
   const int64_t V = x.size(-1);
   TORCH_CHECK_VALUE(x.stride(-1) == 1 || V <= 1, "siirl_amd: the vocab axis of logits must have stride 1");
+  if (x.numel() == 0) return;  // no rows: no blocks (an empty leading axis must not yield one)
   std::vector<std::pair<int64_t, int64_t>> dims;  // (size, stride) of the leading axes, size-1 axes dropped
   for (int64_t d = 0; d + 1 < x.dim(); ++d)
     if (x.size(d) != 1) dims.emplace_back(x.size(d), x.stride(d));
@@ -181,6 +182,7 @@ std::vector<int64_t> lead_shape(const Tensor& logits) {
 void check_logits(const Tensor& logits) {
   require_gpu(logits, "logits");
   TORCH_CHECK_TYPE(logits.dim() >= 1, "logits must be a tensor of shape (..., vocab_size)");
+  TORCH_CHECK_VALUE(logits.size(-1) >= 1, "logits have an empty vocabulary axis (V=0)");
   const auto t = logits.scalar_type();
   TORCH_CHECK_TYPE(t == at::kFloat || t == at::kBFloat16 || t == at::kHalf, "logits dtype ", t,
                    " is not supported (float32, bfloat16, float16)");
@@ -465,6 +467,7 @@ std::tuple<Tensor, Tensor> masked_reduce_fwd(const Tensor& values, const Tensor&
   Tensor ws = loss_workspace(B, L, values, &nws);
   Tensor out = empty_f32({per_row ? B : 2}, values);
   Tensor msum = empty_f32({per_row ? B : 1}, values);
+  if (per_row && B == 0) return {out, msum};  // no rows: nothing to reduce, nothing to launch
   DeviceGuard guard(values.device());
   check_rc(siirl_masked_reduce(ptr<float>(values), ptr(mask), mask_code(mask), B, L,
                                (per_row && !want_mean) ? ptr<float>(out) : nullptr,

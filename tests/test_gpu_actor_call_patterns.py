@@ -313,3 +313,29 @@ def test_masked_reductions_broadcast_mask_and_no_grad(dev):
     nan_outside[:, m[0] == 0] = float("nan")  # where(mask, v, 0): values outside the mask never matter
     got2 = SF.masked_mean(nan_outside.to(dev), m.to(dev), axis=-1)
     assert torch.equal(got2, got)
+
+
+def test_empty_inputs(dev):
+    """No rows at all, in every shape the callers can produce: results are empty tensors of the right shape, the
+    backward gives an empty gradient, nothing is launched on memory that does not exist."""
+    import siirl_amd.torch_functional as SF
+
+    V = 100
+    for shape in ((0, V), (0, 5, V), (3, 0, V)):
+        x = torch.zeros(*shape, device=dev, dtype=torch.bfloat16, requires_grad=True)
+        y = torch.zeros(shape[:-1], dtype=torch.long, device=dev)
+        lp = SF.logprobs_from_logits(x, y, inplace_backward=False)
+        ent = SF.entropy_from_logits(x)
+        assert lp.shape == shape[:-1] and ent.shape == shape[:-1]
+        (lp.sum() + ent.sum()).backward()
+        assert x.grad.shape == x.shape
+    # a strided view whose outer axis is empty (no collapse into one block)
+    base = torch.zeros(0, 7, V, device=dev)
+    assert SF.logprobs_from_logits(base[:, 1:4, :], torch.zeros(0, 3, dtype=torch.long, device=dev)).shape == (0, 3)
+    with pytest.raises(ValueError, match="V=0"):
+        SF.entropy_from_logits(torch.zeros(4, 0, device=dev))
+    e = torch.zeros(0, 6, device=dev)
+    assert float(SF.masked_sum(e, e)) == 0.0 and float(SF.masked_mean(e, e)) == 0.0
+    assert SF.masked_mean(e, e, axis=-1).shape == (0,)
+    z = torch.zeros(4, 0, device=dev)
+    assert torch.equal(SF.masked_sum(z, z, axis=-1), torch.zeros(4, device=dev))

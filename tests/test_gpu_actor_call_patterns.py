@@ -339,3 +339,30 @@ def test_empty_inputs(dev):
     assert SF.masked_mean(e, e, axis=-1).shape == (0,)
     z = torch.zeros(4, 0, device=dev)
     assert torch.equal(SF.masked_sum(z, z, axis=-1), torch.zeros(4, device=dev))
+
+
+def test_one_call_replacement_of_div_logprob_entropy(dev):
+    """``logprobs_and_entropy_from_logits(logits, labels, temperature=T, inplace_backward=True)`` against the
+    reference's three lines ``logits.div_(T)``; ``logprobs_from_logits``; ``entropy_from_logits``
+    (dp_actor.py:176-195): same values, and the gradient w.r.t. the UNDIVIDED logits, written in place."""
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(23)
+    x = (torch.randn(12, 3001, generator=g) * 3).to(torch.bfloat16)
+    y = torch.randint(0, 3001, (12,), generator=g)
+    w1, w2 = torch.randn(12, generator=g), torch.randn(12, generator=g)
+    T = 0.6
+    leaf = x.to(dev).requires_grad_(True)
+    xd = leaf * 1.0
+    lp, ent = SF.logprobs_and_entropy_from_logits(xd, y.to(dev), temperature=T, inplace_backward=True)
+    ((lp * w1.to(dev)).sum() + (ent * w2.to(dev)).sum()).backward()
+    xo = x.double().requires_grad_(True)
+    z = xo / T  # what div_ leaves in the reference's tensor
+    lp_o, ent_o = OF.logprobs_from_logits(z, y, dtype=torch.float64), OF.entropy_from_logits(z, dtype=torch.float64)
+    ((lp_o * w1.double()).sum() + (ent_o * w2.double()).sum()).backward()
+    assert (lp.detach().cpu().double() - lp_o.detach()).abs().max() < 5e-5
+    assert (ent.detach().cpu().double() - ent_o.detach()).abs().max() < 5e-5
+    ok, err = _bf16_close(leaf.grad.cpu(), xo.grad)
+    assert ok, err
+    ok2, _ = _bf16_close(xd.detach().cpu(), xo.grad)  # written in place over the logits
+    assert ok2

@@ -1035,6 +1035,34 @@ def main():
                   "note": "the config 2 mask leaves part of the rows without a second read; compare the dense figure "
                           "with the two-launch headline, which is dense"}
 
+    # what the actor's `logits.div_(temperature)` before the calls (siirl/engine/actor/dp_actor.py:176) costs: a pass
+    # over [T, V] in the forward and autograd's division of the gradient in the backward, against the one call that
+    # takes the temperature as a factor.  Reported beside the headline, never as `value`.
+    temp = 0.7
+
+    def temperature_flow(one_call):
+        def run():
+            if one_call:
+                lp, ent = SF.logprobs_and_entropy_from_logits(x, labels, temperature=temp)
+            else:
+                z = x / temp  # stands for div_ on the model's output: the same read + write
+                lp = SF.logprobs_from_logits(z, labels, inplace_backward=False)
+                ent = SF.entropy_from_logits(z)
+            torch.autograd.backward([lp, ent], [g_lp, g_ent])
+            x.grad = None
+
+        for _ in range(2):
+            run()
+        torch.cuda.synchronize()
+        t3 = time.perf_counter()
+        for _ in range(5):
+            run()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t3) * 1e3 / 5
+
+    division_ms, folded_ms = temperature_flow(False), temperature_flow(True)
+    torch.cuda.empty_cache()
+
     out = {
         "metric": METRIC,
         "value": tokens_per_s,
@@ -1062,6 +1090,10 @@ def main():
                                        "(profiles/lpe_config2_hbm_traffic.md); a constant here, not read in this process"},
         "row_skip_variant": row_skip,
         "fused_step_variant": fused_step,
+        "temperature_flow": {"what": f"temperature {temp}: `logits / T`, logprobs_from_logits, entropy_from_logits, "
+                                     "backward (the reference's lines) against logprobs_and_entropy_from_logits("
+                                     "logits, labels, temperature=T), backward",
+                             "division_then_calls_ms": division_ms, "one_call_ms": folded_ms},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(logits.detach(), labels, g_lp, g_ent)

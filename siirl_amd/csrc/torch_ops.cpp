@@ -172,6 +172,20 @@ void row_blocks(const Tensor& x, std::vector<RowBlock>& out) {
   }
 }
 
+// The blocks as a flat list {offset, rows, stride, ...}: host-side arithmetic on sizes and strides only, any device.
+std::vector<int64_t> row_blocks_op(const Tensor& x) {
+  TORCH_CHECK_VALUE(x.dim() >= 1, "row blocks need at least one axis");
+  std::vector<RowBlock> blocks;
+  row_blocks(x, blocks);
+  std::vector<int64_t> flat;
+  for (const auto& b : blocks) {
+    flat.push_back(b.off);
+    flat.push_back(b.rows);
+    flat.push_back(b.stride);
+  }
+  return flat;
+}
+
 std::vector<int64_t> lead_shape(const Tensor& logits) {
   auto s = logits.sizes();
   return std::vector<int64_t>(s.begin(), s.end() - 1);
@@ -1040,6 +1054,8 @@ TORCH_LIBRARY(siirl_hip, m) {
   m.def("fused_linear_logprob_entropy_bwd(Tensor hidden, Tensor weight, Tensor labels, float inv_temperature, "
         "Tensor lse, Tensor ex, Tensor? g_logprob, Tensor? g_entropy, bool need_hidden, bool need_weight, "
         "Tensor? saved=None) -> (Tensor, Tensor)");
+  // how the log-prob operators cut a (..., V) view into launches; no device work (used by the host-side tests)
+  m.def("row_blocks(Tensor x) -> int[]", &row_blocks_op);
   // differentiable operators (autograd nodes in C++; eager use only)
   m.def("logprob_entropy(Tensor logits, Tensor? labels, float inv_temperature, bool want_entropy, "
         "bool inplace_backward, bool skip_zero_rows, Tensor? defer=None) -> (Tensor, Tensor)", &logprob_entropy);

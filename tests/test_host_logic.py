@@ -96,6 +96,49 @@ def test_row_blocks():
     assert list(row_blocks(w[:, :, 1:3, :])) == [(120 * a + 40 * b, 2, 10) for a in range(2) for b in range(3)]
 
 
+def _views(seed):
+    """Random (..., V) views with unit inner stride: slices, steps, size-1 and size-0 axes, expanded leading axes."""
+    import random
+
+    rnd = random.Random(seed)
+    nd = rnd.randint(1, 4)
+    shape = [rnd.choice((0, 1, 2, 3, 5)) if rnd.random() < 0.9 else 1 for _ in range(nd - 1)] + [rnd.choice((1, 4, 9))]
+    base = torch.zeros(shape)
+    v = base
+    for d in range(nd):
+        n = v.shape[d]
+        if n >= 2 and rnd.random() < 0.6:
+            lo = rnd.randint(0, n - 1)
+            hi = rnd.randint(lo + 1, n)
+            step = rnd.choice((1, 1, 2)) if d < nd - 1 else 1
+            v = v[(slice(None),) * d + (slice(lo, hi, step),)]
+    if nd >= 2 and rnd.random() < 0.2:
+        v = v.unsqueeze(0)
+    return v
+
+
+def test_cpp_row_blocks_agree_with_the_python_statement():
+    """The C++ layer cuts a logits view into uniformly strided row blocks before it launches anything; an error there
+    would send a kernel to memory the view does not own.  Same answer as the Python statement of the rule on 2000
+    random views, and every block stays inside the view's storage."""
+    from siirl_amd.ops import row_blocks
+
+    for seed in range(2000):
+        v = _views(seed)
+        want = [t for blk in row_blocks(v) if blk[1] for t in blk]
+        got = list(torch.ops.siirl_hip.row_blocks(v))
+        got = [t for i in range(0, len(got), 3) if got[i + 1] for t in got[i:i + 3]]
+        assert got == want, (seed, tuple(v.shape), v.stride(), got, want)
+        V = v.shape[-1]
+        limit = v.untyped_storage().nbytes() // v.element_size() - v.storage_offset()
+        rows = 0
+        for i in range(0, len(got), 3):
+            off, n, stride = got[i:i + 3]
+            assert off >= 0 and off + (n - 1) * stride + V <= limit
+            rows += n
+        assert rows == (v.numel() // V if V else 0)
+
+
 def test_bench_refuses_more_than_one_gpu():
     import subprocess
     import sys

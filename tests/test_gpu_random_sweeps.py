@@ -231,3 +231,58 @@ def test_sweep_logprob_entropy(dev):
         tol = 2 * eps * d64.abs() + 1e-6 + fp32_abs + (1e-5 * d64.abs() if dt == torch.float32 else 0)
         err = (got.double() - d64).abs()
         assert bool((err <= tol).all()), (case, T, V, dt, temp, float((err - tol).max()))
+
+
+def test_sweep_logprob_entropy_over_random_views(dev):
+    """Log-prob, entropy and their gradient over randomly sliced (..., V) views -- row-strided, outer-strided, with
+    size-1 axes, rows that are not 16-byte aligned, an ignored label here and there -- in the three logits dtypes,
+    against the fp64 oracle.  Tolerances: 2e-5 on the fp32 outputs against the fp64 value of the same (rounded)
+    inputs; dlogits within 1 ulp of a 16-bit logits dtype (2^-7 relative for bf16, 2^-10 for fp16) and 5e-6 relative
+    for fp32 (fp32 arithmetic with a hardware exp2 against the fp64 value)."""
+    import random
+
+    import siirl_amd.torch_functional as SF
+    from oracle import torch_functional as OF
+
+    rel = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 5e-6}
+    for case in range(160):
+        rnd = random.Random(7000 + case)
+        g = torch.Generator().manual_seed(7000 + case)
+        dtype = (torch.bfloat16, torch.float32, torch.float16)[case % 3]
+        nd = rnd.randint(1, 3)
+        V = rnd.choice((1, 7, 8, 33, 250, 1031))
+        lead = [rnd.choice((1, 2, 3, 5, 9)) for _ in range(nd)]
+        pad = [rnd.randint(0, 3) for _ in range(nd)] + [rnd.choice((0, 0, 1, 8, 13))]
+        base = (torch.randn(*[n + 2 * p for n, p in zip(lead, pad[:-1])], V + 2 * pad[-1], generator=g) * 2.5).to(dtype)
+        idx = tuple(slice(p, p + n) for n, p in zip(lead, pad[:-1])) + (slice(pad[-1], pad[-1] + V),)
+        xs = base[idx]
+        y = torch.randint(0, V, lead, generator=g)
+        if case % 9 == 0:
+            y.view(-1)[0] = -100
+        w1, w2 = torch.randn(lead, generator=g), torch.randn(lead, generator=g)
+        leaf = base.to(dev).requires_grad_(True)
+        view = leaf[idx]
+        pairing = case % 2 == 0
+        SF.set_pairing(pairing)
+        try:
+            lp = SF.logprobs_from_logits(view, y.to(dev), inplace_backward=False)
+            ent = SF.entropy_from_logits(view)
+            ((lp * w1.to(dev)).sum() + (ent * w2.to(dev)).sum()).backward()
+        finally:
+            SF.set_pairing(True)
+        lp_o = OF.logprobs_from_logits_flash_attn(xs, y, dtype=torch.float64)
+        ent_o = OF.entropy_from_logits(xs, dtype=torch.float64)
+        assert (lp.detach().cpu().double() - lp_o).abs().max() < 2e-5, (case, "logprob")
+        assert (ent.detach().cpu().double() - ent_o).abs().max() < 2e-5, (case, "entropy")
+        xo = xs.double().requires_grad_(True)
+        (OF.logprobs_from_logits_flash_attn(xo, y) * w1.double()).sum().backward()
+        d_lp = xo.grad
+        d_ent = OF.logprob_entropy_backward(xs, y.clamp(min=0), None, w2, dtype=torch.float64)
+        want = d_lp + d_ent
+        got = leaf.grad.cpu()
+        mag = want.abs() if pairing else d_lp.abs() + d_ent.abs() + want.abs()
+        err = (got[idx].double() - want).abs()
+        assert bool((err <= rel[dtype] * mag + 1e-6).all()), (case, dtype, tuple(xs.shape), xs.stride(), err.max().item())
+        outside = got.clone()
+        outside[idx] = 0
+        assert torch.count_nonzero(outside) == 0, (case, "gradient outside the view")

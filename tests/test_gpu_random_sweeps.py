@@ -286,3 +286,75 @@ def test_sweep_logprob_entropy_over_random_views(dev):
         outside = got.clone()
         outside[idx] = 0
         assert torch.count_nonzero(outside) == 0, (case, "gradient outside the view")
+
+
+def test_sweep_loss_functions_over_shapes_dtypes_and_layouts(dev):
+    """The [B, L] loss functions as callers may hand them operands: 1-D, 2-D and 3-D tensors, log-probs in fp32 /
+    bf16 / fp64, masks in every dtype (and non-contiguous), operands that are transposed views; values against the
+    fp64 oracle on the same (rounded) inputs to 1e-5 relative + 1e-6, gradients to 1e-5 relative + 1e-7 (the gradient
+    of a 16-bit log-prob comes back in that dtype: 2^-7 relative), shapes and dtypes of the gradients as autograd
+    expects them."""
+    import random
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    from oracle import core_algos as OC
+
+    aggs = ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"]
+    for case in range(120):
+        rnd = random.Random(9100 + case)
+        g = torch.Generator().manual_seed(9100 + case)
+        nd = rnd.choice((1, 2, 2, 3))
+        shape = [rnd.choice((1, 2, 3, 7)) for _ in range(nd - 1)] + [rnd.choice((1, 5, 64, 300, 2500))]
+        lp_dtype = (torch.float32, torch.bfloat16, torch.float64)[case % 3]
+        lp0 = (torch.randn(shape, generator=g) * 0.7 - 1.5).to(lp_dtype)
+        old = lp0.float() + torch.randn(shape, generator=g) * 0.15
+        ref = lp0.float() + torch.randn(shape, generator=g) * 0.3
+        adv = torch.randn(shape, generator=g)
+        mask_b = torch.rand(shape, generator=g) > 0.3
+        mask_b.view(-1)[0] = True
+        mask = {0: mask_b, 1: mask_b.long(), 2: mask_b.float(), 3: mask_b.to(torch.int32), 4: mask_b.to(torch.bfloat16)}[case % 5]
+        agg = aggs[case % 4]
+        if agg == "seq-mean-token-mean":  # keep every row non-empty: an empty one is NaN by definition
+            m2 = mask_b.reshape(-1, shape[-1])
+            m2[:, 0] = True
+            mask = m2.reshape(shape).to(mask.dtype)
+            mask_b = mask.bool()
+        cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=rnd.choice((0.1, 0.2)), clip_ratio_high=rnd.choice((0.2, 0.28)),
+                              clip_ratio_c=rnd.choice((1.5, 3.0)))
+        ocfg = OC.LossConfig(0.2, cfg.clip_ratio_low, cfg.clip_ratio_high, cfg.clip_ratio_c)
+        transposed = nd == 2 and case % 4 == 1  # hand over non-contiguous views of contiguous transposes
+        to_dev = (lambda t: t.t().contiguous().to(dev).t()) if transposed else (lambda t: t.to(dev))
+        lp = to_dev(lp0).requires_grad_(True)
+        which = case % 3
+        if which == 0:
+            pg, cf, kl, cfl = CA.compute_policy_loss_vanilla(to_dev(old), lp, to_dev(adv), to_dev(mask), agg, cfg)
+            total = pg
+        elif which == 1:
+            kld = CA.kl_penalty(lp, to_dev(ref), "low_var_kl")
+            total = CA.agg_loss(kld, to_dev(mask), agg)
+        else:
+            total = CA.agg_loss(lp * 1.0, to_dev(mask), agg)
+        total.backward()
+        assert lp.grad.shape == lp.shape and lp.grad.dtype == lp_dtype
+        # oracle on the same rounded inputs, 2-D view
+        L = shape[-1]
+        x64 = lp0.double().reshape(-1, L).requires_grad_(True)
+        m64 = mask_b.reshape(-1, L).double()
+        if which == 0:
+            want, cf_o, kl_o, cfl_o = OC.compute_policy_loss_vanilla(old.double().reshape(-1, L), x64,
+                                                                     adv.double().reshape(-1, L), m64, agg, ocfg)
+            for a, b in ((cf, cf_o), (kl, kl_o), (cfl, cfl_o)):
+                assert abs(a.item() - float(b)) < 1e-5 + 1e-5 * abs(float(b)), (case, "metric")
+        elif which == 1:
+            want = OC.agg_loss(OC.kl_penalty(x64, ref.double().reshape(-1, L), "low_var_kl"), m64, agg)
+        else:
+            want = OC.agg_loss(x64, m64, agg)
+        want.backward()
+        # a 16-bit log-prob makes kl_penalty return 16-bit values (as the reference's arithmetic would): bf16 accuracy
+        vtol = 2.0 ** -7 if (lp_dtype == torch.bfloat16 and which == 1) else 1e-5
+        assert abs(total.item() - want.item()) < 1e-6 + vtol * abs(want.item()), (case, which, agg, total.item(), want.item())
+        gw = x64.grad.reshape(shape)
+        rel = 2.0 ** -6 if lp_dtype == torch.bfloat16 else 1e-5
+        err = (lp.grad.cpu().double() - gw).abs()
+        assert bool((err <= rel * gw.abs() + 1e-7).all()), (case, which, agg, lp_dtype, tuple(shape), err.max().item())

@@ -139,7 +139,9 @@ def _outside_graph(fn):
 # version and grad mode, hands it out.  Both then belong to ONE autograd node, which autograd runs once with both
 # upstream gradients: one backward pass over the rows, and an in-place backward that cannot overtake a second reader.
 # The slot below only holds weak references: the parked entropy lives exactly as long as the log-probs it came with,
-# so an unclaimed one pins nothing once the caller drops those.
+# so an unclaimed one pins nothing once the caller drops those.  It is plain module state, one slot per process: the
+# reference's actor is one Python thread per process (a Ray worker per GPU); two threads interleaving these calls on
+# tensors of one storage should switch the pairing off.
 
 _PAIRING = True
 _slot = None  # (weakref logits, version, grad mode, weakref entropy or None, defer flag or None, output dtype or None)

@@ -242,6 +242,14 @@ def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor):
 logprobs_from_logits_naive = logprobs_from_logits_v2  # reference :93-96
 
 
+def logprobs_from_logits_flash_attn(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True):
+    """reference ``torch_functional.py:85-90`` (the negated flash-attn cross-entropy): fp32 log-probs of 2-D
+    ``logits`` whatever their dtype, 0 for a label of -100, backward in place when ``inplace_backward``."""
+    if logits.dim() != 2 or labels.dim() != 1:
+        raise ValueError("siirl_amd: logprobs_from_logits_flash_attn takes [tokens, vocab] logits and [tokens] labels")
+    return logprobs_from_logits(logits, labels, inplace_backward=inplace_backward)
+
+
 def entropy_from_logits(logits: torch.Tensor):
     """Entropy of ``softmax(logits)`` per row (reference ``torch_functional.py:128-132``)."""
     global _entropy_reader

@@ -250,6 +250,11 @@ def test_ignored_label_minus_100(dev):
     assert ok and lp2[2].item() == 0.0, err
     other = SF.logprobs_from_logits(x.to(dev), torch.full((9,), -7).to(dev))
     assert torch.isnan(other).all()  # any other label outside [0, V) is an error value, not an ignored row
+    # the flash-attn spelling itself (torch_functional.py:85-90): fp32 out of bf16 logits, 2-D operands only
+    fa = SF.logprobs_from_logits_flash_attn(x.to(dev), y.to(dev), inplace_backward=False)
+    assert fa.dtype == torch.float32 and torch.equal(fa, SF.logprobs_from_logits(x.to(dev), y.to(dev)))
+    with pytest.raises(ValueError):
+        SF.logprobs_from_logits_flash_attn(x.to(dev).view(3, 3, 1031), y.to(dev).view(3, 3))
 
 
 def test_biased_masked_var_of_one_element(dev):
@@ -366,3 +371,56 @@ def test_one_call_replacement_of_div_logprob_entropy(dev):
     assert ok, err
     ok2, _ = _bf16_close(xd.detach().cpu(), xo.grad)  # written in place over the logits
     assert ok2
+
+
+def test_embodied_actor_pattern(dev):
+    """siirl/engine/actor/embodied_actor.py:211-222,454-477: a 256-column action window of the vocabulary
+    (``logits[..., -256-64:-64]``, then ``.div(temperature)``), default in-place log-probs and the entropy of the same
+    tensor, both flattened to ``(1, -1)``; ``compute_policy_loss_vanilla`` on a slice of the trajectory with a bool
+    mask, the loss rescaled by the slice's share of the valid steps, ``backward()`` per slice."""
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as SA
+    import siirl_amd.torch_functional as SF
+    from oracle import core_algos as OA
+
+    g = torch.Generator().manual_seed(41)
+    steps, toks, Vfull, T = 6, 7, 512, 1.3
+    full = (torch.randn(steps, toks, Vfull, generator=g) * 2).to(torch.bfloat16)
+    resp = torch.randint(0, 256, (steps, toks), generator=g)
+    n = steps * toks
+    old = torch.randn(1, n, generator=g) * 0.1 - 5.5
+    adv = torch.randn(1, n, generator=g)
+    mask = (torch.arange(n) < 31).unsqueeze(0)  # finish_step * action_token_len
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=3.0)
+    half = steps // 2
+
+    def run(mod_f, mod_a, window_of, to):
+        total = mask.sum()
+        out = []
+        for i in range(0, steps, half):
+            logits = window_of(i)
+            lp = mod_f.logprobs_from_logits(logits, to(resp[i:i + half])).reshape((1, -1))
+            ent = mod_f.entropy_from_logits(logits).reshape((1, -1))
+            sl = slice(i * toks, (i + half) * toks)
+            m = to(mask[:, sl])
+            pg, clipfrac, kl, _ = mod_a.compute_policy_loss_vanilla(old_log_prob=to(old[:, sl]), log_prob=lp,
+                                                                    advantages=to(adv[:, sl]), response_mask=m, config=cfg)
+            loss = pg * m.sum() / to(total) / 2
+            loss.backward()
+            out.append((loss.detach().cpu().double(), clipfrac.detach().cpu().double(), kl.detach().cpu().double(),
+                        ent.detach().cpu().double()))
+        return out
+
+    leaf = full.to(dev).requires_grad_(True)
+    got = run(SF, SA, lambda i: (leaf * 1.0)[i:i + half][..., -256 - 64:-64].div(T), lambda t: t.to(dev))
+    # the oracle starts from the same bf16 quotient and is differentiated with respect to it in float64
+    quot = [full[i:i + half][..., -256 - 64:-64].div(T).double().requires_grad_(True) for i in range(0, steps, half)]
+    want = run(OF, OA, lambda i: quot[i // half], lambda t: t.double() if t.is_floating_point() else t)
+    for a, b in zip(got, want):
+        for x, y in zip(a, b):
+            assert (x - y).abs().max() < 1e-4, (x, y)
+    d_window = torch.cat([q.grad for q in quot]) / T  # autograd of `.div(T)`; two bf16 roundings on the GPU side
+    ok, err = _bf16_close(leaf.grad.cpu()[..., -256 - 64:-64], d_window, parts=(d_window,))
+    assert ok, err
+    assert torch.count_nonzero(leaf.grad[..., -64:]) == 0 and torch.count_nonzero(leaf.grad[..., :-320]) == 0

@@ -19,6 +19,7 @@ Differences a caller can observe, all deliberate:
 
 from __future__ import annotations
 
+import threading
 import weakref
 
 import torch
@@ -139,18 +140,23 @@ def _outside_graph(fn):
 # version and grad mode, hands it out.  Both then belong to ONE autograd node, which autograd runs once with both
 # upstream gradients: one backward pass over the rows, and an in-place backward that cannot overtake a second reader.
 # The slot below only holds weak references: the parked entropy lives exactly as long as the log-probs it came with,
-# so an unclaimed one pins nothing once the caller drops those.  It is plain module state, one slot per process: the
-# reference's actor is one Python thread per process (a Ray worker per GPU); two threads interleaving these calls on
-# tensors of one storage should switch the pairing off.
+# so an unclaimed one pins nothing once the caller drops those.  The slot is per Python thread (the reference's actor
+# is one thread per process, a Ray worker per GPU): calls of another thread neither claim nor disturb it.
 
 _PAIRING = True
-_slot = None  # (weakref logits, version, grad mode, weakref entropy or None, defer flag or None, output dtype or None)
-_entropy_reader = None  # (weakref to the last separately computed entropy that carries a graph, its logits' storage)
+
+
+class _PairingState(threading.local):
+    slot = None    # (weakref logits, version, grad mode, weakref entropy or None, defer flag or None, output dtype)
+    reader = None  # (weakref to the last separately computed entropy that carries a graph, its logits' storage)
+
+
+_st = _PairingState()
 
 
 def set_pairing(flag: bool) -> None:
-    global _PAIRING, _slot, _entropy_reader
-    _PAIRING, _slot, _entropy_reader = bool(flag), None, None
+    global _PAIRING
+    _PAIRING, _st.slot, _st.reader = bool(flag), None, None
 
 
 def _version(t):
@@ -162,19 +168,18 @@ def _claim(logits):
     log-prob node was built for an in-place backward turns that backward out-of-place: the caller is about to give
     those logits a second reader (its own entropy node, or a checkpoint's recomputation), which an in-place backward
     running first would feed with gradients instead of logits."""
-    global _slot
-    if _slot is None:
+    if _st.slot is None:
         return None
-    ref, version, grad_mode, ent_ref, defer, back = _slot
+    ref, version, grad_mode, ent_ref, defer, back = _st.slot
     parked = ref()
     if parked is None:
-        _slot = None
+        _st.slot = None
         return None
     if ent_ref is not None and parked is logits and _version(logits) == version and \
             torch.is_grad_enabled() == grad_mode:
         ent = ent_ref()
         if ent is not None:
-            _slot = None
+            _st.slot = None
             return ent if back is None else ent.to(back)
     if defer is not None and parked.untyped_storage().data_ptr() == logits.untyped_storage().data_ptr():
         defer[0] = 1
@@ -184,18 +189,16 @@ def _claim(logits):
 def _has_reader(logits) -> bool:
     """True while an entropy computed on its own from the same memory is alive with a graph: its node has saved the
     logits, so a log-prob node built now must not overwrite them."""
-    global _entropy_reader
-    if _entropy_reader is None:
+    if _st.reader is None:
         return False
-    ent_ref, storage = _entropy_reader
+    ent_ref, storage = _st.reader
     if ent_ref() is None:
-        _entropy_reader = None
+        _st.reader = None
         return False
     return storage == logits.untyped_storage().data_ptr()
 
 
 def _logprobs(logits, labels, inplace_backward, caller_logits, back):
-    global _slot
     tracked = logits.requires_grad and torch.is_grad_enabled()
     if inplace_backward and tracked and _has_reader(logits):
         inplace_backward = False
@@ -203,10 +206,10 @@ def _logprobs(logits, labels, inplace_backward, caller_logits, back):
     lp, ent = _lpe(logits, labels, 1.0, _PAIRING, inplace_backward, _SKIP_ZERO_ROWS, defer)
     if _PAIRING:
         lp._siirl_paired_entropy = ent  # keeps the entropy (and through it the node) alive as long as the log-probs
-        _slot = (weakref.ref(caller_logits), _version(caller_logits), torch.is_grad_enabled(), weakref.ref(ent), defer,
+        _st.slot = (weakref.ref(caller_logits), _version(caller_logits), torch.is_grad_enabled(), weakref.ref(ent), defer,
                  back)
     elif defer is not None:
-        _slot = (weakref.ref(caller_logits), 0, True, None, defer, back)
+        _st.slot = (weakref.ref(caller_logits), 0, True, None, defer, back)
     return lp
 
 
@@ -252,7 +255,6 @@ def logprobs_from_logits_flash_attn(logits: torch.Tensor, labels: torch.Tensor, 
 
 def entropy_from_logits(logits: torch.Tensor):
     """Entropy of ``softmax(logits)`` per row (reference ``torch_functional.py:128-132``)."""
-    global _entropy_reader
     if torch.compiler.is_compiling():
         return _outside_graph(entropy_from_logits)(logits)
     x, back = _check_logits(logits)
@@ -261,7 +263,7 @@ def entropy_from_logits(logits: torch.Tensor):
         return parked
     _, ent = _lpe(x, None, 1.0, True, False, _SKIP_ZERO_ROWS, None)
     if ent.requires_grad:
-        _entropy_reader = (weakref.ref(ent), x.untyped_storage().data_ptr())
+        _st.reader = (weakref.ref(ent), x.untyped_storage().data_ptr())
     return ent if back is None else ent.to(back)
 
 

@@ -168,7 +168,7 @@ def test_pairing_keeps_nothing_alive(dev):
     # and a parked entropy that nobody claims does not survive its log-probs
     x = torch.randn(64, 1000, device=dev, dtype=torch.bfloat16)
     lp = SF.logprobs_from_logits(x, y[:64] % 1000, inplace_backward=False)
-    ent_ref = SF._slot[3]
+    ent_ref = SF._st.slot[3]
     assert ent_ref() is not None
     del lp
     gc.collect()
@@ -183,12 +183,51 @@ def test_v2_and_naive_park_nothing(dev):
     SF.set_pairing(True)  # clears the slot
     a = SF.logprobs_from_logits_v2(x, y)
     b = SF.logprobs_from_logits_naive(x, y)
-    assert SF._slot is None and torch.equal(a, b)
+    assert SF._st.slot is None and torch.equal(a, b)
     assert not hasattr(a, "_siirl_paired_entropy")
     c = SF.logprobs_from_logits(x, y)
-    assert SF._slot is not None and torch.equal(a, c)
+    assert SF._st.slot is not None and torch.equal(a, c)
     e = SF.entropy_from_logits(x)
-    assert e is c._siirl_paired_entropy and SF._slot is None
+    assert e is c._siirl_paired_entropy and SF._st.slot is None
+
+
+def test_pairing_state_is_per_thread(dev):
+    """Two Python threads that interleave the calls on their own tensors each get their own pairing: a thread's
+    entropy call claims only what that thread's log-prob call parked."""
+    import threading
+
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator().manual_seed(5)
+    xs = [(torch.randn(16, 300, generator=g) * 2).to(dev) for _ in range(2)]
+    y = torch.randint(0, 300, (16,), generator=g).to(dev)
+    step = [threading.Event() for _ in range(3)]
+    out = {}
+
+    def first():
+        lp = SF.logprobs_from_logits(xs[0], y, inplace_backward=False)
+        step[0].set()
+        step[1].wait(10)
+        out["claimed_after_other_thread_parked"] = SF.entropy_from_logits(xs[0]) is lp._siirl_paired_entropy
+        step[2].set()
+
+    def second():
+        step[0].wait(10)
+        out["sees_no_slot_of_the_first"] = SF._st.slot is None
+        lp = SF.logprobs_from_logits(xs[1], y, inplace_backward=False)
+        step[1].set()
+        step[2].wait(10)
+        out["own_slot_survived"] = SF.entropy_from_logits(xs[1]) is lp._siirl_paired_entropy
+
+    threads = [threading.Thread(target=first), threading.Thread(target=second)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(30)
+    assert out == {"claimed_after_other_thread_parked": True, "sees_no_slot_of_the_first": True,
+                   "own_slot_survived": True}
+    want = OF.entropy_from_logits(xs[1].cpu(), dtype=torch.float64)
+    assert (SF.entropy_from_logits(xs[1]).cpu().double() - want).abs().max() < 2e-5
 
 
 def test_float64_logits(dev):

@@ -55,6 +55,9 @@ def _check(dev, logits, resp, mask, old, ref, adv, isw, cfg, T=1.0, scale=1.0, o
     tol = 1e-7 + 1.01 * ULP[logits.dtype] * d_o.abs()
     if logits.dtype == torch.float32:  # fp32 arithmetic: lse and E[z] carry about 2^-23 * |z| of rounding into p
         tol = tol + 2e-7 + 4e-6 * d_o.abs()
+    # at a label whose probability is within 1e-4 of one, `g * (1 - p)` cancels in fp32 (here and in the reference's
+    # autograd alike): a few fp32 ulps of the token's upstream gradient g, bounded through its advantage
+    tol = tol + (2.0 ** -21 * scale * (1 + 5 * adv.double().abs())).unsqueeze(-1)
     assert bool((err <= tol).all()), (err.max().item(), (err / tol).max().item())
     m = out.metrics()
     for k in ("actor/pg_loss", "actor/pg_clipfrac", "actor/ppo_kl", "actor/pg_clipfrac_lower"):
@@ -155,10 +158,13 @@ def test_fwd_bwd_entry_equals_two_launches(dev, T, V, dtype):
 
 def test_fused_step_random_sweep(dev):
     """Seeded random shapes, dtypes, loss modes, aggregation modes, coefficients and temperatures through the
-    single-pass step, each against the oracle's micro-batch step (tolerances of _check)."""
+    single-pass step, each against the oracle's micro-batch step (tolerances of _check).  ``SIIRL_TEST_SEED=<int>`` in
+    the environment shifts the seeds."""
+    import os
     import random
 
-    rnd = random.Random(77)
+    shift = 100003 * int(os.environ.get("SIIRL_TEST_SEED", "0"))
+    rnd = random.Random(77 + shift)
     aggs = ["token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"]
     for case in range(40):
         B, L = rnd.randint(1, 5), rnd.randint(1, 24)
@@ -170,7 +176,7 @@ def test_fused_step_random_sweep(dev):
                              use_kl_loss=rnd.random() < 0.5, kl_loss_coef=0.05,
                              kl_loss_type=rnd.choice(["low_var_kl", "kl", "mse", "abs"]), loss_mode=mode,
                              loss_agg_mode=rnd.choice(aggs), use_cpgd_loss=(mode == "cpgd"), policy_drift_coeff=0.2)
-        inp = _inputs(B, L, V, dtype, seed=1000 + case)
+        inp = _inputs(B, L, V, dtype, seed=1000 + case + shift)
         print(f"[sweep case {case}] B={B} L={L} V={V} {dtype} {mode} {cfg.loss_agg_mode} kl={cfg.use_kl_loss}", flush=True)
         _check(dev, *inp, cfg, T=rnd.choice([1.0, 0.8, 1.3]), scale=rnd.choice([1.0, 0.25]),
                on_policy=(mode == "vanilla" and rnd.random() < 0.2), use_isw=(mode != "cpgd" and rnd.random() < 0.5))

@@ -24,11 +24,14 @@ def dynamic_sampling_keep_indices(metric_values, uids):
     deviation computed *in the dtype of the values* with numpy's pairwise summation, so a group
     of equal non-dyadic fp64 values such as ``[0.1, 0.1, 0.1]`` has std 1.4e-17 > 0 and is kept,
     while the same values in fp32 give exactly 0.  Returns ``(indices, kept_uids, n_groups)``."""
+    def key(u):  # reference ``dapo.py:70,91``: tensor / numpy scalars through int(), any other object as it is
+        return int(u) if hasattr(u, "item") else u
+
     groups = OrderedDict()
     for i in range(len(uids)):
-        groups.setdefault(int(uids[i]), []).append(metric_values[i])
+        groups.setdefault(key(uids[i]), []).append(metric_values[i])
     kept = {u for u, vals in groups.items() if np.std(vals) > 0 or len(vals) == 1}
-    idx = [i for i in range(len(uids)) if int(uids[i]) in kept]
+    idx = [i for i in range(len(uids)) if key(uids[i]) in kept]
     return idx, kept, len(groups)
 
 

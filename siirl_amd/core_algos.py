@@ -210,13 +210,20 @@ def compute_response_mask(data):
 
 
 def _uid_tensor(index, n, dev) -> torch.Tensor:
+    """int64 group codes: integer arrays as they are; anything else goes through ``int()`` per entry as in the
+    reference (``core_algos.py:326``: numeric strings, floats, integers beyond 64 bits) and is numbered in order of
+    first appearance -- only equality of the keys matters."""
     if isinstance(index, torch.Tensor):
         out = index.detach().reshape(-1).to(device=dev, dtype=torch.int64)
     else:
         arr = np.asarray(index)
-        if arr.dtype.kind not in "iu":
-            arr = np.asarray([int(v) for v in arr.reshape(-1)], dtype=np.int64)  # numeric strings, floats
-        out = torch.from_numpy(np.ascontiguousarray(arr.reshape(-1).astype(np.int64))).to(dev)
+        if arr.dtype.kind in "iu" and (arr.dtype.kind == "i" or arr.size == 0 or int(arr.max()) < 2 ** 63):
+            arr = arr.reshape(-1).astype(np.int64)
+        else:
+            seq = list(index) if isinstance(index, (list, tuple)) else list(arr.reshape(-1))
+            codes: dict = {}
+            arr = np.fromiter((codes.setdefault(int(v), len(codes)) for v in seq), dtype=np.int64, count=len(seq))
+        out = torch.from_numpy(np.ascontiguousarray(arr)).to(dev)
     if out.numel() != n:
         raise ValueError(f"index has {out.numel()} entries for a batch of {n}")
     return out.contiguous()

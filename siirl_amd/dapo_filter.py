@@ -58,12 +58,20 @@ def _metric_tensor(values, dev) -> torch.Tensor:
 
 
 def _uid_tensor(uids, dev) -> torch.Tensor:
+    """int64 group codes on ``dev``.  Integer uids (the reference's ``preprocess_dataloader`` makes int64 ones,
+    ``sample.py:127-131``) are used as they are; anything else the reference's dict would accept as a key (strings,
+    integers beyond 64 bits, ``filter_interface/dapo.py:68-72``: ``int(uid)`` for numpy / tensor scalars, the object
+    itself otherwise) is numbered on the host in order of first appearance -- only equality matters downstream."""
     if isinstance(uids, torch.Tensor):
         return uids.detach().reshape(-1).to(device=dev, dtype=torch.int64).contiguous()
-    arr = np.asarray(uids).reshape(-1)
-    if arr.dtype.kind not in "iu":
-        raise TypeError("uids must be integers (the reference creates int64 uids, sample.py:127-131)")
-    return torch.from_numpy(np.ascontiguousarray(arr.astype(np.int64))).to(dev)
+    arr = np.asarray(uids)
+    if arr.dtype.kind in "iu" and (arr.dtype.kind == "i" or arr.size == 0 or int(arr.max()) < 2 ** 63):
+        return torch.from_numpy(np.ascontiguousarray(arr.reshape(-1).astype(np.int64))).to(dev)
+    seq = list(uids) if isinstance(uids, (list, tuple)) else list(arr.reshape(-1))
+    codes: dict = {}
+    out = np.fromiter((codes.setdefault(int(v) if hasattr(v, "item") else v, len(codes)) for v in seq),
+                      dtype=np.int64, count=len(seq))
+    return torch.from_numpy(out).to(dev)
 
 
 def group_keep_mask(metric_values, uids, device=None, return_group_size: bool = False):

@@ -95,6 +95,37 @@ def test_grpo_known_answers_and_invariants(dev):
     assert not a3.is_cuda and (a3 - a1.cpu()).abs().max() == 0
 
 
+def test_uids_that_are_not_int64(dev):
+    """The reference keys its groups with Python objects (core_algos.py:326 ``int(index[i])``; filter_interface/dapo.py:70
+    the uid itself unless it is a tensor / numpy scalar): uuid strings and 128-bit integers work there, so they do
+    here -- numbered on the host in order of first appearance, same groups."""
+    import uuid
+
+    import siirl_amd.core_algos as CA
+    from siirl_amd import dapo_filter as DF
+
+    g = torch.Generator().manual_seed(12)
+    names = [uuid.UUID(int=int(torch.randint(0, 2 ** 62, (1,), generator=g)) << 64 | 7 * k) for k in range(5)]
+    order = torch.randint(0, 5, (23,), generator=g).tolist()
+    big = [names[k].int for k in order]            # 128-bit Python integers
+    text = [str(names[k]) for k in order]          # uuid strings
+    small = np.asarray(order, dtype=np.int64)
+    rewards, mask, _ = _grpo_inputs(23, 1, 7, seed=5, reward="gauss")
+    want, _ = OC.compute_grpo_outcome_advantage(rewards, mask, small)
+    got_big, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), big)
+    got_obj, _ = CA.compute_grpo_outcome_advantage(rewards.to(dev), mask.to(dev), np.asarray(big, dtype=object))
+    assert (got_big.cpu() - want).abs().max() < 1e-5 and torch.equal(got_big, got_obj)
+    metric = torch.randint(0, 2, (23,), generator=g).double().numpy()
+    want_keep = OD.keep_mask(metric, small)
+    for uids in (big, text, np.asarray(text), np.asarray(big, dtype=object)):
+        if isinstance(uids, np.ndarray) and uids.dtype.kind == "U":
+            with pytest.raises(ValueError):  # numpy strings have .item: the reference calls int() on them
+                DF.group_keep_mask(metric, uids, device=dev)
+            continue
+        assert np.array_equal(DF.group_keep_mask(metric, uids, device=dev).cpu().numpy(), want_keep)
+        assert np.array_equal(OD.keep_mask(metric, uids), want_keep)
+
+
 def test_compute_advantage_dispatch(dev):
     import siirl_amd.core_algos as CA
 

@@ -463,3 +463,54 @@ def test_embodied_actor_pattern(dev):
     ok, err = _bf16_close(leaf.grad.cpu()[..., -256 - 64:-64], d_window, parts=(d_window,))
     assert ok, err
     assert torch.count_nonzero(leaf.grad[..., -64:]) == 0 and torch.count_nonzero(leaf.grad[..., :-320]) == 0
+
+
+def test_ops_run_on_the_current_stream(dev):
+    """Every operator is issued on torch's current stream: inputs produced late on a busy side stream are seen, with no
+    synchronisation in between (a launch on any other stream would read the zeros the buffers held before)."""
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.torch_functional as SF
+    from siirl_amd.fused_linear import fused_linear_logprob_entropy
+
+    g = torch.Generator().manual_seed(23)
+    T, V, H = 64, 3001, 128
+    x_host = (torch.randn(T, V, generator=g) * 2).to(torch.bfloat16)
+    h_host = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    w_host = (torch.randn(V, H, generator=g) * 0.1).to(torch.bfloat16)
+    y = torch.randint(0, V, (T,), generator=g).to(dev)
+    old = (torch.randn(8, 8, generator=g) * 0.1 - 8.0).to(dev)
+    adv = torch.randn(8, 8, generator=g).to(dev)
+    mask = torch.ones(8, 8, dtype=torch.long, device=dev)
+    uid = torch.arange(4).repeat_interleave(2).to(dev)
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.2, clip_ratio_c=3.0)
+    src = [t.to(dev) for t in (x_host, h_host, w_host)]
+    torch.cuda.synchronize()
+
+    def work(x, h, w):
+        leaf = x.detach().requires_grad_(True)
+        lp = SF.logprobs_from_logits(leaf, y, inplace_backward=False)
+        ent = SF.entropy_from_logits(leaf)
+        pg, _, kl, _ = CA.compute_policy_loss_vanilla(old, lp.view(8, 8), adv, mask, "token-mean", cfg)
+        (pg - 0.01 * CA.agg_loss(ent.view(8, 8), mask, "seq-mean-token-mean")).backward()
+        a, _ = CA.compute_grpo_outcome_advantage(lp.detach().view(8, 8), mask, uid)
+        mm = SF.masked_mean(ent.detach().view(8, 8), mask, axis=-1)
+        flp, fent = fused_linear_logprob_entropy(h, w, y)
+        return [leaf.grad, lp.detach(), ent.detach(), pg.detach(), kl, a, mm, flp, fent]
+
+    want = work(*src)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    bufs = [torch.zeros_like(t) for t in src]
+    busy = torch.randn(4096, 4096, device=dev)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for _ in range(40):  # keeps the side stream busy for tens of milliseconds
+            busy = busy @ busy * 1e-3
+        for b, s in zip(bufs, src):
+            b.copy_(s)
+        got = work(*bufs)
+    side.synchronize()
+    for i, (a, b) in enumerate(zip(got, want)):
+        assert torch.equal(a, b), i

@@ -172,3 +172,31 @@ def test_response_window_helpers_refuse_the_cpu_and_bad_arguments():
                                         torch.zeros(2, dtype=torch.long))
     with pytest.raises(ValueError):
         FL.set_saved_logits_limit(-5)
+
+
+def test_uid_codes_for_keys_that_are_not_int64():
+    """Host side of the group operators: uids the reference would use as dict keys (core_algos.py:326,
+    filter_interface/dapo.py:70) become int64 codes with the same equalities."""
+    import numpy as np
+    import torch
+
+    from siirl_amd import core_algos as CA
+    from siirl_amd import dapo_filter as DF
+
+    big = [2 ** 100 + 3, 5, 2 ** 100 + 3, -7, 5]
+    want = [0, 1, 0, 2, 1]
+    assert CA._uid_tensor(big, 5, "cpu").tolist() == want
+    assert CA._uid_tensor(np.asarray(big, dtype=object), 5, "cpu").tolist() == want
+    assert CA._uid_tensor(["10", "2", "10", "3", "2"], 5, "cpu").tolist() == want  # int() per entry, as the reference
+    assert CA._uid_tensor(np.asarray([2 ** 63 + 1, 4, 2 ** 63 + 1], dtype=np.uint64), 3, "cpu").tolist() == [0, 1, 0]
+    assert CA._uid_tensor(np.asarray([9, -4, 9]), 3, "cpu").tolist() == [9, -4, 9]  # integer arrays pass through
+    assert CA._uid_tensor(torch.tensor([9, -4, 9]), 3, "cpu").tolist() == [9, -4, 9]
+    with pytest.raises(ValueError):
+        CA._uid_tensor(["a", "b"], 2, "cpu")  # the reference's int("a")
+    with pytest.raises(ValueError):
+        CA._uid_tensor([1, 2, 3], 2, "cpu")
+    assert DF._uid_tensor(["a", "b", "a", "c"], "cpu").tolist() == [0, 1, 0, 2]  # the filter keys Python objects as is
+    assert DF._uid_tensor(big, "cpu").tolist() == want
+    assert DF._uid_tensor(np.asarray([3, 3, 1]), "cpu").tolist() == [3, 3, 1]
+    with pytest.raises(ValueError):
+        DF._uid_tensor(np.asarray(["a", "b"]), "cpu")  # numpy strings have .item: int() as in the reference

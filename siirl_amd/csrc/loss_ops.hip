@@ -435,6 +435,7 @@ int launch_loss_bwd(const LossArgs& a, const float* g_out, const float* saved_ou
     case KIND_VANILLA: loss_bwd_kernel<KIND_VANILLA><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
     case KIND_GSPO: loss_bwd_kernel<KIND_GSPO><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
     case KIND_AGG: loss_bwd_kernel<KIND_AGG><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
+    case KIND_VALUE: loss_bwd_kernel<KIND_VALUE><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
     default: loss_bwd_kernel<-1><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent);
   }
   SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
@@ -676,6 +677,7 @@ int launch_loss_partials(const LossArgs& a, const float* row_s, float* partials,
     case KIND_VANILLA: loss_partials_kernel<KIND_VANILLA><<<grid, block, 0, st>>>(a, row_s, partials); break;
     case KIND_GSPO: loss_partials_kernel<KIND_GSPO><<<grid, block, 0, st>>>(a, row_s, partials); break;
     case KIND_AGG: loss_partials_kernel<KIND_AGG><<<grid, block, 0, st>>>(a, row_s, partials); break;
+    case KIND_VALUE: loss_partials_kernel<KIND_VALUE><<<grid, block, 0, st>>>(a, row_s, partials); break;
     default: loss_partials_kernel<-1><<<grid, block, 0, st>>>(a, row_s, partials);
   }
   SIIRL_LAUNCH_CHECK("loss_partials_kernel");

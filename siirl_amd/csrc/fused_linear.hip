@@ -53,8 +53,6 @@ constexpr int kThreads = WM * WN * 64;
 constexpr int kWavesPerSimd = kThreads / 256;  // one workgroup per CU (the LDS ring), four SIMDs
 static_assert(kThreads == 256 || kThreads == 512, "4 or 8 waves per workgroup");
 constexpr int MI = BM / (WM * 32), NJ = BN / (WN * 32);  // 32x32 MFMA tiles per wave
-constexpr int kLoadsPerThread = (BM * BK / 8) / kThreads;  // 16-byte chunks per operand tile per thread
-constexpr int kLoadRowStep = kThreads / 8;
 constexpr int kRowBytes = BK * 2;             // unpadded rows, 16-byte chunks XOR-swizzled by (row / 2) % 8
 constexpr int kTileBytes = BM * kRowBytes;    // 32768
 constexpr int kStageBytes = kTileBytes;       // A tile only: B goes global -> registers

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kThreads) void cu_seqlens_kernel(const int32_t* __r
     sh[threadIdx.x] = v;
     __syncthreads();
     for (int off = 1; off < kThreads; off <<= 1) {  // Hillis-Steele inclusive scan
-      const int32_t add = threadIdx.x >= off ? sh[threadIdx.x - off] : 0;
+      const int32_t add = (int)threadIdx.x >= off ? sh[threadIdx.x - off] : 0;
       __syncthreads();
       sh[threadIdx.x] += add;
       __syncthreads();

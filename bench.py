@@ -754,7 +754,6 @@ def bench_glue(args, dev):
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:
-        import numpy as np
         from oracle import padding as OP
 
         am_c, ids_c, v_c = am.cpu().numpy(), ids.cpu().numpy(), vals.detach().cpu().numpy()

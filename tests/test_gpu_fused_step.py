@@ -3,7 +3,6 @@ the C ABI) vs the CPU oracle's micro-batch step and vs the two-launch path.
 
 Tolerances: log-prob / entropy / loss within 1e-3 absolute of the fp32 oracle (observed ~1e-5 against fp64);
 dlogits within one unit in the last place of the logits dtype of the fp64 oracle's gradient (plus 1e-7 absolute)."""
-import ctypes as C
 from dataclasses import replace
 
 import pytest

@@ -129,6 +129,34 @@ int mask_code(const Tensor& mask) {
   return dtype_code(mask.scalar_type());
 }
 
+// The plain operators hand raw pointers to kernels whose grids are sized from ONE operand: every other operand must
+// live on that operand's device and hold as many elements as the kernel will read or write.
+void require_on(const Tensor& t, const Tensor& like, const char* name) {
+  TORCH_CHECK(t.device() == like.device(), "siirl_amd: `", name, "` is on ", t.device(), ", expected ", like.device());
+}
+void require_mask(const Tensor& mask, const Tensor& like, const char* name = "mask") {
+  require_on(mask, like, name);
+  TORCH_CHECK_VALUE(mask.sizes() == like.sizes(), "siirl_amd: `", name, "` has shape ", mask.sizes(), ", expected ",
+                    like.sizes());
+}
+void require_f32_like(const Tensor& t, const Tensor& like, const char* name) {
+  require_on(t, like, name);
+  TORCH_CHECK_VALUE(t.scalar_type() == at::kFloat && t.is_contiguous() && t.sizes() == like.sizes(), "siirl_amd: `", name,
+                    "` must be a contiguous float32 tensor of shape ", like.sizes(), ", got ", t.scalar_type(), " ",
+                    t.sizes());
+}
+void require_f32_like(const optional<Tensor>& t, const Tensor& like, const char* name) {
+  if (has(t)) require_f32_like(*t, like, name);
+}
+void require_f32_n(const Tensor& t, int64_t n, const Tensor& like, const char* name) {
+  require_on(t, like, name);
+  TORCH_CHECK_VALUE(t.scalar_type() == at::kFloat && t.is_contiguous() && t.numel() == n, "siirl_amd: `", name,
+                    "` must be a contiguous float32 tensor of ", n, " elements, got ", t.scalar_type(), " ", t.sizes());
+}
+void require_f32_n(const optional<Tensor>& t, int64_t n, const Tensor& like, const char* name) {
+  if (has(t)) require_f32_n(*t, n, like, name);
+}
+
 Tensor loss_workspace(int64_t B, int64_t L, const Tensor& like, size_t* n) {
   *n = siirl_loss_workspace_bytes(B, L);
   return at::empty({(int64_t)*n}, like.options().dtype(at::kByte).memory_format(c10::nullopt));
@@ -263,6 +291,17 @@ void lpe_bwd_launch(const Tensor& logits, const optional<Tensor>& labels_in, dou
   }
   TORCH_CHECK_VALUE(!has(g_lp) || labels.defined(), "labels are required with g_logprob");
   TORCH_CHECK_VALUE(!has(g_ent) || has(ex), "ex is required with g_entropy");
+  const int64_t rows = logits.numel() / V;
+  auto per_row = [&](int64_t n, const char* name) {
+    TORCH_CHECK_VALUE(n == rows, "siirl_amd: `", name, "` has ", n, " elements for ", rows, " rows of logits");
+  };
+  per_row(lse.numel(), "lse");
+  if (has(ex)) per_row(ex->numel(), "ex");
+  if (has(g_lp)) per_row(g_lp->numel(), "g_logprob");
+  if (has(g_ent)) per_row(g_ent->numel(), "g_entropy");
+  if (labels.defined()) per_row(labels.numel(), "labels");
+  require_on(out, logits, "dlogits");
+  TORCH_CHECK_TYPE(out.scalar_type() == logits.scalar_type(), "siirl_amd: dlogits must have the dtype of logits");
   std::vector<RowBlock> in_blocks, out_blocks;
   row_blocks(logits, in_blocks);
   const bool inplace = out.is_same(logits) || (out.data_ptr() == logits.data_ptr() && out.strides() == logits.strides());
@@ -379,6 +418,8 @@ Tensor grpo_advantage(const Tensor& rewards, const Tensor& mask, const Tensor& u
   const int64_t B = rewards.size(0), L = rewards.size(1);
   TORCH_CHECK_VALUE(uid.scalar_type() == at::kLong && uid.numel() == B && mask.dim() == 2 && mask.size(0) == B &&
                         mask.size(1) == L, "siirl_amd: uid must be int64 [B] and mask [B, L]");
+  require_on(mask, rewards, "mask");
+  require_on(uid, rewards, "uid");
   Tensor adv = empty_f32({B, L}, rewards);
   Tensor scratch = empty_f32({2 * std::max<int64_t>(B, 1)}, rewards);
   Tensor u = uid.contiguous();
@@ -395,6 +436,7 @@ std::tuple<Tensor, Tensor> group_keep_mask(const Tensor& metric, const Tensor& u
   const int64_t B = uid.numel();
   TORCH_CHECK_VALUE(metric.numel() == B && uid.scalar_type() == at::kLong,
                     "siirl_amd: metric and uid must have one entry per trajectory, uid int64");
+  require_on(uid, metric, "uid");
   Tensor keep = at::empty({B}, metric.options().dtype(at::kByte));
   Tensor gsz = at::empty({B}, metric.options().dtype(at::kInt));
   Tensor met = metric.contiguous(), u = uid.contiguous();
@@ -410,6 +452,7 @@ std::tuple<Tensor, Tensor> group_keep_mask(const Tensor& metric, const Tensor& u
 std::tuple<Tensor, Tensor> agg_loss_fwd(const Tensor& loss_mat, const Tensor& mask, int64_t agg_mode) {
   require_f32c(loss_mat, "loss_mat");
   TORCH_CHECK_VALUE(loss_mat.dim() == 2, "loss_mat must be [B, L]");
+  require_mask(mask, loss_mat);
   const int64_t B = loss_mat.size(0), L = loss_mat.size(1);
   Tensor out16 = empty_f32({16}, loss_mat), row_msum = empty_f32({B}, loss_mat);
   size_t nws;
@@ -425,6 +468,10 @@ Tensor agg_loss_bwd(const Tensor& g, const Tensor& mask, const Tensor& out16, co
   TORCH_CHECK_VALUE(mask.dim() == 2, "mask must be [B, L]");
   const int64_t B = mask.size(0), L = mask.size(1);
   require_f32c(g, "g");
+  TORCH_CHECK_VALUE(g.numel() == 1, "siirl_amd: `g` is the gradient of the scalar loss (one element)");
+  require_f32_n(out16, 16, g, "out16");
+  require_f32_n(row_msum, B, g, "row_msum");
+  require_on(mask, g, "mask");
   Tensor d = empty_f32({B, L}, out16);
   DeviceGuard guard(out16.device());
   check_rc(siirl_agg_loss_bwd(ptr<float>(g), ptr(mask), mask_code(mask), ptr<float>(out16), ptr<float>(row_msum), B, L,
@@ -476,6 +523,7 @@ Tensor agg_loss(const Tensor& loss_mat, const Tensor& loss_mask, int64_t agg_mod
 std::tuple<Tensor, Tensor> masked_reduce_fwd(const Tensor& values, const Tensor& mask, bool per_row, bool want_mean) {
   require_f32c(values, "values");
   TORCH_CHECK_VALUE(values.dim() == 2 && mask.sizes() == values.sizes(), "values and mask must be [B, L]");
+  require_on(mask, values, "mask");
   const int64_t B = values.size(0), L = values.size(1);
   size_t nws;
   Tensor ws = loss_workspace(B, L, values, &nws);
@@ -498,6 +546,8 @@ Tensor masked_reduce_bwd(const Tensor& g, const Tensor& mask, bool per_row, cons
   const int64_t B = mask.size(0), L = mask.size(1);
   require_f32c(g, "g");
   require_f32c(mask_sums, "mask_sums");
+  require_on(mask, g, "mask");
+  if (has(mask_sums)) require_on(*mask_sums, g, "mask_sums");
   TORCH_CHECK_VALUE(g.numel() == (per_row ? B : 1) && (!has(mask_sums) || mask_sums->numel() == g.numel()),
                     "g and mask_sums must have one entry per reduced row");
   Tensor d = empty_f32({B, L}, g);
@@ -586,6 +636,13 @@ void policy_loss_fwd_launch(const Tensor& old, const Tensor& lp, const Tensor& a
   require_f32c(isw, "is_weights");
   require_f32c(ent, "entropy");
   require_f32c(ref, "ref_log_prob");
+  TORCH_CHECK_VALUE(lp.dim() == 2, "log_prob must be [B, L]");
+  require_f32_like(old, lp, "old_log_prob");
+  require_f32_like(adv, lp, "advantages");
+  require_f32_like(isw, lp, "is_weights");
+  require_f32_like(ent, lp, "entropy");
+  require_f32_like(ref, lp, "ref_log_prob");
+  require_mask(mask, lp);
   const int64_t B = lp.size(0), L = lp.size(1);
   DeviceGuard guard(lp.device());
   check_rc(siirl_actor_loss_fwd(ptr<float>(old), ptr<float>(lp), ptr<float>(adv), ptr(mask), mask_code(mask),
@@ -622,7 +679,18 @@ std::tuple<Tensor, Tensor> policy_loss_bwd_impl(const Tensor& g, const Tensor& o
   require_f32c(isw, "is_weights");
   require_f32c(ent, "entropy");
   require_f32c(ref, "ref_log_prob");
+  TORCH_CHECK_VALUE(lp.dim() == 2, "log_prob must be [B, L]");
+  require_f32_like(old, lp, "old_log_prob");
+  require_f32_like(adv, lp, "advantages");
+  require_f32_like(isw, lp, "is_weights");
+  require_f32_like(ent, lp, "entropy");
+  require_f32_like(ref, lp, "ref_log_prob");
+  require_mask(mask, lp);
   const int64_t B = lp.size(0), L = lp.size(1);
+  require_f32_n(g, 1, lp, "g_loss");
+  require_f32_n(out16, 16, lp, "out16");
+  require_f32_n(row_msum, B, lp, "row_msum");
+  require_f32_n(row_s, B, lp, "row_s");
   Tensor d_lp = empty_f32({B, L}, lp);
   const std::vector<int64_t> full{B, L}, none{0};
   Tensor d_ent = empty_f32(has(ent) ? at::IntArrayRef(full) : at::IntArrayRef(none), lp);
@@ -836,6 +904,7 @@ Tensor kl_penalty_fwd(const Tensor& lp, const Tensor& ref, int64_t kl_mode) {
   require_f32c(lp, "log_prob");
   require_f32c(ref, "ref_log_prob");
   TORCH_CHECK_VALUE(ref.sizes() == lp.sizes(), "siirl_amd: log_prob and ref_log_prob must have one shape");
+  require_on(ref, lp, "ref_log_prob");
   Tensor out = at::empty_like(lp);
   DeviceGuard guard(lp.device());
   check_rc(siirl_kl_penalty_fwd(ptr<float>(lp), ptr<float>(ref), lp.numel(), (int)kl_mode, ptr<float>(out),
@@ -848,7 +917,8 @@ std::tuple<Tensor, Tensor> kl_penalty_bwd(const Tensor& g, const Tensor& lp, con
                                           bool straight_through, bool need_lp, bool need_ref) {
   require_f32c(g, "g");
   require_f32c(lp, "log_prob");
-  require_f32c(ref, "ref_log_prob");
+  require_f32_like(ref, lp, "ref_log_prob");
+  require_f32_like(g, lp, "g");
   const std::vector<int64_t> none{0};
   Tensor d_lp = empty_f32(need_lp ? lp.sizes() : at::IntArrayRef(none), lp);
   Tensor d_ref = empty_f32(need_ref ? lp.sizes() : at::IntArrayRef(none), lp);
@@ -916,6 +986,8 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> fused_linear_fwd(const Tensor
   const int64_t T = hidden.size(0), H = hidden.size(1), V = weight.size(0);
   TORCH_CHECK_VALUE(weight.size(1) == H && labels.dim() == 1 && labels.size(0) == T && labels.scalar_type() == at::kLong,
                     "shape mismatch: hidden ", hidden.sizes(), ", weight ", weight.sizes(), ", labels ", labels.sizes());
+  require_on(weight, hidden, "weight");
+  require_on(labels, hidden, "labels");
   Tensor lp = empty_f32({T}, hidden), ent = empty_f32({T}, hidden), lse = empty_f32({T}, hidden),
          ex = empty_f32({T}, hidden);
   Tensor saved = empty_f32({0}, hidden);
@@ -948,13 +1020,21 @@ std::tuple<Tensor, Tensor> fused_linear_bwd(const Tensor& hidden, const Tensor& 
   require_f32c(g_lp, "g_logprob");
   require_f32c(g_ent, "g_entropy");
   const int64_t T = hidden.size(0), H = hidden.size(1), V = weight.size(0);
+  TORCH_CHECK_VALUE(weight.size(1) == H && labels.dim() == 1 && labels.size(0) == T && labels.scalar_type() == at::kLong,
+                    "shape mismatch: hidden ", hidden.sizes(), ", weight ", weight.sizes(), ", labels ", labels.sizes());
+  require_on(weight, hidden, "weight");
+  require_on(labels, hidden, "labels");
+  require_f32_n(lse, T, hidden, "lse");
+  require_f32_n(ex, T, hidden, "ex");
+  require_f32_n(g_lp, T, hidden, "g_logprob");
+  require_f32_n(g_ent, T, hidden, "g_entropy");
   const std::vector<int64_t> none{0};
   Tensor d_h = at::empty(need_hidden ? hidden.sizes() : at::IntArrayRef(none), hidden.options());
   Tensor d_w = at::empty(need_weight ? weight.sizes() : at::IntArrayRef(none), weight.options());
   optional<Tensor> saved;
   if (has(saved_in) && saved_in->numel() != 0) {
     saved = saved_in;
-    require_gpu(*saved, "saved");
+    require_on(*saved, hidden, "saved");
     TORCH_CHECK_VALUE(saved->scalar_type() == at::kFloat && saved->is_contiguous() &&
                           (size_t)saved->numel() * 4 == siirl_fused_linear_saved_logits_bytes(T, V),
                       "saved is not the buffer the forward op returned for these shapes");

@@ -122,3 +122,96 @@ def test_opcheck_on_the_gpu():
                                                                 True, True, sv), test_utils=checks)
     x = mk((T, V), torch.bfloat16)
     torch.library.opcheck(ns.logprob_entropy_fwd, (x, y, 1.0, True), test_utils=checks)
+
+
+@pytest.mark.gpu
+def test_plain_operators_refuse_misplaced_or_short_operands():
+    """The plain operators pass raw pointers to kernels sized from one operand: a secondary operand on the host, or
+    with fewer elements than the kernel would touch, must raise on the host, before anything is launched."""
+    dev = torch.device("cuda:0")
+    ns = torch.ops.siirl_hip
+    B, L, T, V, H = 4, 24, 16, 300, 64
+    f = lambda *s: torch.randn(*s, device=dev) * 0.1  # noqa: E731
+    ones = torch.ones(B, L, dtype=torch.int64, device=dev)
+    uid = torch.arange(B, device=dev) // 2
+    bad = (RuntimeError, ValueError, TypeError)
+
+    with pytest.raises(bad):
+        ns.grpo_advantage(f(B, L), ones.cpu(), uid, 1e-6, True)
+    with pytest.raises(bad):
+        ns.grpo_advantage(f(B, L), ones, uid.cpu(), 1e-6, True)
+    with pytest.raises(bad):
+        ns.group_keep_mask(torch.rand(B, device=dev, dtype=torch.float64), uid.cpu())
+    with pytest.raises(bad):
+        ns.agg_loss_fwd(f(B, L), ones[:, : L // 2].contiguous(), 0)
+    with pytest.raises(bad):
+        ns.agg_loss_fwd(f(B, L), ones.cpu(), 0)
+    out16, row_msum = ns.agg_loss_fwd(f(B, L), ones, 0)
+    g1 = torch.ones(1, device=dev)
+    with pytest.raises(bad):
+        ns.agg_loss_bwd(g1, ones, out16[:8].contiguous(), row_msum, 0)
+    with pytest.raises(bad):
+        ns.agg_loss_bwd(g1, ones, out16, row_msum[:-1].contiguous(), 0)
+    with pytest.raises(bad):
+        ns.agg_loss_bwd(g1, ones, out16.cpu(), row_msum, 0)
+    with pytest.raises(bad):
+        ns.masked_reduce_fwd(f(B, L), ones.cpu(), True, True)
+    with pytest.raises(bad):
+        ns.masked_reduce_bwd(torch.ones(B, device=dev), ones.cpu(), True, None)
+
+    args = list(_loss_args(lambda s, d: f(*s) if d.is_floating_point else torch.ones(s, dtype=d, device=dev), B, L, True))
+    for i in (0, 2, 3, 4, 5, 6):  # every operand but log_prob itself, in turn: wrong extent, then wrong device
+        short = list(args)
+        short[i] = args[i][:, : L // 2].contiguous()
+        with pytest.raises(bad):
+            ns.policy_loss_fwd(*short)
+        host = list(args)
+        host[i] = args[i].cpu()
+        with pytest.raises(bad):
+            ns.policy_loss_fwd(*host)
+    o16, rm, rs = ns.policy_loss_fwd(*args)
+    with pytest.raises(bad):
+        ns.policy_loss_bwd(g1, *args, o16, rm[:-1].contiguous(), rs)
+    with pytest.raises(bad):
+        ns.policy_loss_bwd(g1.cpu(), *args, o16, rm, rs)
+    short = list(args)
+    short[1] = args[1][:, : L // 2].contiguous()  # log_prob shorter than the others
+    with pytest.raises(bad):
+        ns.policy_loss_bwd(g1, *short, o16, rm, rs)
+
+    with pytest.raises(bad):
+        ns.kl_penalty_fwd(f(B, L), f(B, L).cpu(), 3)
+    with pytest.raises(bad):
+        ns.kl_penalty_bwd(f(B, L // 2), f(B, L), f(B, L), 3, False, True, False)
+
+    x = f(T, V).to(torch.bfloat16)
+    y = torch.randint(0, V, (T,), device=dev)
+    lp, ent, lse, ex = ns.logprob_entropy_fwd(x, y, 1.0, True)
+    gl = torch.ones(T, device=dev)
+    with pytest.raises(bad):
+        ns.logprob_entropy_bwd(x, y, 1.0, lse[:-1].contiguous(), ex, gl, gl, False)
+    with pytest.raises(bad):
+        ns.logprob_entropy_bwd(x, y, 1.0, lse, ex, gl[:-1].contiguous(), gl, False)
+    with pytest.raises(bad):
+        ns.logprob_entropy_bwd(x, y[:-1].contiguous(), 1.0, lse, ex, gl, gl, False)
+    with pytest.raises(bad):
+        ns.logprob_entropy_bwd(x, y, 1.0, lse, ex[:-1].contiguous(), gl, gl, False)
+
+    h, w = f(T, H).to(torch.bfloat16), f(V, H).to(torch.bfloat16)
+    with pytest.raises(bad):
+        ns.fused_linear_logprob_entropy_fwd(h, w, y.cpu(), 1.0)
+    with pytest.raises(bad):
+        ns.fused_linear_logprob_entropy_fwd(h, w.cpu(), y, 1.0)
+    lp, ent, lse, ex, _ = ns.fused_linear_logprob_entropy_fwd(h, w, y, 1.0)
+    with pytest.raises(bad):
+        ns.fused_linear_logprob_entropy_bwd(h, w, y, 1.0, lse[:-1].contiguous(), ex, gl, None, True, True)
+    with pytest.raises(bad):
+        ns.fused_linear_logprob_entropy_bwd(h, w, y, 1.0, lse, ex, gl[:-1].contiguous(), None, True, True)
+    with pytest.raises(bad):
+        ns.fused_linear_logprob_entropy_bwd(h, w, y.cpu(), 1.0, lse, ex, gl, None, True, True)
+    with pytest.raises(bad):
+        ns.fused_linear_logprob_entropy_bwd(h, w, y, 1.0, lse.cpu(), ex, gl, None, True, True)
+    # and the well-formed calls still run
+    torch.cuda.synchronize()
+    dh, dw = ns.fused_linear_logprob_entropy_bwd(h, w, y, 1.0, lse, ex, gl, None, True, True)
+    assert torch.isfinite(dh.float()).all() and torch.isfinite(dw.float()).all()

@@ -52,13 +52,15 @@ typedef enum siirl_agg_mode {
   SIIRL_AGG_SEQ_MEAN_TOKEN_SUM_NORM = 3 /* "seq-mean-token-sum-norm" */
 } siirl_agg_mode;
 
-/* registered policy losses, siirl/dag_worker/core_algos.py:572,710,795,865,1074 */
+/* registered policy losses, siirl/dag_worker/core_algos.py:572,710,795,865,898,998,1074 */
 typedef enum siirl_loss_mode {
   SIIRL_LOSS_VANILLA = 0,  /* "vanilla" */
   SIIRL_LOSS_GSPO = 1,     /* "gspo" */
   SIIRL_LOSS_CPGD = 2,     /* "cpgd" */
   SIIRL_LOSS_GPG = 3,      /* "gpg" */
-  SIIRL_LOSS_GEO_MEAN = 4  /* "geo_mean" (GMPO) */
+  SIIRL_LOSS_GEO_MEAN = 4, /* "geo_mean" (GMPO) */
+  SIIRL_LOSS_KL_COV = 5,   /* "kl_cov"   (siirl_actor_loss_cov_fwd / _bwd only) */
+  SIIRL_LOSS_CLIP_COV = 6  /* "clip_cov" (siirl_actor_loss_cov_fwd / _bwd only) */
 } siirl_loss_mode;
 
 /* kl_penalty estimators, siirl/dag_worker/core_algos.py:1241-1276 */
@@ -73,7 +75,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1003
+#define SIIRL_HIP_ABI_VERSION 1004
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -268,6 +270,54 @@ int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const f
                          float entropy_coeff, int kl_mode, int kl_straight_through, float kl_coef,
                          float policy_drift_coeff, float loss_scale, const float* out16, const float* row_msum,
                          const float* row_s, float* d_log_prob, float* d_entropy, siirl_stream_t stream);
+
+/*
+ * The two covariance losses (Clip-Cov, KL-Cov) pick a few tokens of the batch by the covariance of advantage and
+ * log-probability and treat them differently.  This entry point writes the scores that the pick is made from,
+ *   cov[b, t] = (A - mean A) * (log_prob - mean log_prob),
+ * SIIRL_LOSS_KL_COV: plain means over the tokens with mask > 0, cov = -inf where mask <= 0 (the caller takes the
+ * max(1, int(n * kl_cov_ratio)) largest); SIIRL_LOSS_CLIP_COV: masked means sum(v * m) / (sum(m) + 1e-8), cov = -inf
+ * where mask == 0 and where the PPO clip already bites (-A * clamp(ratio, 1 - clip_low, 1 + clip_high) > -A * ratio,
+ * ratio = exp(log_prob - old_log_prob)); the caller draws its tokens among clip_cov_lb < cov < clip_cov_ub.
+ * stats[4] (device) receives {count of mask > 0, sum of the mask, mean A, mean log_prob}.  old_log_prob may be NULL
+ * for SIIRL_LOSS_KL_COV.  workspace: siirl_cov_workspace_bytes(), 8-byte aligned.
+ * Replaces: siirl/dag_worker/core_algos.py:952-971 (clip_cov) and :1047-1055 (kl_cov).
+ */
+size_t siirl_cov_workspace_bytes(void);
+int siirl_cov_scores(const float* old_log_prob, const float* log_prob, const float* advantages, const void* mask,
+                     int mask_dtype, int64_t B, int64_t L, int loss_mode, float clip_low, float clip_high, float* cov,
+                     float* stats, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
+
+/*
+ * siirl_actor_loss_fwd for the two covariance losses: the same composition (entropy, KL and drift terms, ratio
+ * statistics, loss_scale) around a policy term that takes one more [B, L] fp32 operand, token_aux:
+ *   SIIRL_LOSS_KL_COV:   tok = -A * ratio + token_aux * |log_prob - old_log_prob|  (token_aux = ppo_kl_coef on the
+ *        selected tokens, 0 elsewhere); out16[SIIRL_OUT_PPO_KL] is masked_mean(|log_prob - old_log_prob|), the two
+ *        clip fractions are 0;
+ *   SIIRL_LOSS_CLIP_COV: tok = max(-A * ratio, -A * clamp(ratio, 1 - clip_low, 1 + clip_high)) where token_aux == 0
+ *        and 0 where token_aux != 0 (the dropped tokens); out16[SIIRL_OUT_PG_CLIPFRAC] is the masked share of dropped
+ *        tokens, out16[SIIRL_OUT_PPO_KL] masked_mean(-(log_prob - old_log_prob)).
+ * Neither clamps the log-ratio, neither has a dual clip; both multiply by is_weights when given and aggregate with
+ * agg_mode.  Workspace as for siirl_actor_loss_fwd.
+ * Replaces: compute_policy_loss_clip_cov siirl/dag_worker/core_algos.py:898-995 (after the draw, :983-995) and
+ *           compute_policy_loss_kl_cov :998-1071 (after the selection, :1061-1071).
+ */
+int siirl_actor_loss_cov_fwd(const float* old_log_prob, const float* log_prob, const float* advantages,
+                             const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
+                             const float* ref_log_prob, const float* token_aux, int64_t B, int64_t L, int loss_mode,
+                             float clip_low, float clip_high, int agg_mode, float entropy_coeff, int kl_mode,
+                             int kl_straight_through, float kl_coef, float policy_drift_coeff, float loss_scale,
+                             float* out16, float* row_msum, void* workspace, size_t workspace_bytes,
+                             siirl_stream_t stream);
+
+/* Backward of siirl_actor_loss_cov_fwd, as siirl_actor_loss_bwd; |x| passes sign(x), 0 at 0. */
+int siirl_actor_loss_cov_bwd(const float* g_loss, const float* old_log_prob, const float* log_prob,
+                             const float* advantages, const void* mask, int mask_dtype, const float* is_weights,
+                             const float* entropy, const float* ref_log_prob, const float* token_aux, int64_t B,
+                             int64_t L, int loss_mode, float clip_low, float clip_high, int agg_mode,
+                             float entropy_coeff, int kl_mode, int kl_straight_through, float kl_coef,
+                             float policy_drift_coeff, float loss_scale, const float* out16, const float* row_msum,
+                             float* d_log_prob, float* d_entropy, siirl_stream_t stream);
 
 /*
  * Clipped value loss of the critic over [B, L] fp32 operands:

@@ -45,6 +45,13 @@ compute_policy_loss_cpgd / drift       hand-computed tokens with log(1 +- eps) b
 compute_policy_loss_gpg                identity with agg_loss(-lp * A [* w])
 compute_policy_loss_geo_mean           explicit product of token ratios ** (1 / L); L = 1 cases
                                        for each clipping side; weights as their geometric mean
+compute_policy_loss_kl_cov             worked case with math (covariances, the picked token, loss);
+                                       brute-force sort of the products; closed-form gradient
+compute_policy_loss_clip_cov           candidate set by hand; loss after a given draw with math;
+                                       generator state shows one randperm(len(candidates)); no
+                                       candidates -> the plain clip loss
+compute_cpgd_outcome_advantage         the GRPO oracle (STD_weight, naive); hand case for
+                                       clip_filter_like_weight
 kl_penalty                             closed forms per mode; k3 >= 0; straight-through identities
 apply_kl_penalty / KL controllers      hand-computed controller step
 dynamic_sampling_keep_indices          worked example of the reference's docs

@@ -32,11 +32,13 @@ class ActorConfig:
     loss_mode: str = "vanilla"
     use_cpgd_loss: bool = False
     policy_drift_coeff: float = 0.0
+    policy_loss: Optional[core_algos.CovLossConfig] = None  # the covariance losses' parameters
 
 
 _LOSSES = {"vanilla": core_algos.compute_policy_loss_vanilla, "gspo": core_algos.compute_policy_loss_gspo,
            "cpgd": core_algos.compute_policy_loss_cpgd, "gpg": core_algos.compute_policy_loss_gpg,
-           "geo_mean": core_algos.compute_policy_loss_geo_mean}
+           "geo_mean": core_algos.compute_policy_loss_geo_mean, "clip_cov": core_algos.compute_policy_loss_clip_cov,
+           "kl_cov": core_algos.compute_policy_loss_kl_cov}
 
 
 def micro_batch_step(logits, responses, old_log_prob, advantages, response_mask, config: ActorConfig,

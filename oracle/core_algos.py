@@ -3,7 +3,8 @@
 Restates on the CPU the arithmetic of ``siirl/dag_worker/core_algos.py`` of the reference
 (GAE ``:229-276``, GRPO outcome advantage ``:279-348``, ``agg_loss`` ``:536-569``, the ``cpgd``
 loss ``:572-629``, the ``vanilla`` loss ``:710-792``, the ``gspo`` loss ``:795-862``, ``gpg``
-``:865-895``, ``geo_mean`` ``:1074-1153``, the value loss ``:1173-1212``, ``kl_penalty``
+``:865-895``, ``clip_cov`` ``:898-995``, ``kl_cov`` ``:998-1071``, ``geo_mean`` ``:1074-1153``, the CPGD outcome
+advantage ``:461-517``, the value loss ``:1173-1212``, ``kl_penalty``
 ``:1215-1276``, KL controllers ``:167-226``, ``apply_kl_penalty`` ``:1358-1397``) and the CPGD
 drift term of ``siirl/engine/actor/dp_actor.py:488-494``.  Works in the dtype of its inputs, so the
 same code serves as the fp32 statement and, on fp64 inputs, as the high-precision check.
@@ -256,6 +257,145 @@ def compute_policy_loss_geo_mean(old_log_prob, log_prob, advantages, response_ma
     pg_clipfrac = masked_mean((clipped * (advantages > 0)).to(d.dtype), response_mask)
     pg_clipfrac_lower = masked_mean((clipped * (advantages < 0)).to(d.dtype), response_mask)
     return torch.mean(seq), pg_clipfrac, ppo_kl, pg_clipfrac_lower
+
+
+@dataclass
+class CovLossConfig:
+    """``config.policy_loss`` of the two covariance losses (reference ``siirl/params/model_args.py``, read at
+    ``core_algos.py:943-948,1034-1035``); ``None`` selects the default the loss function states."""
+
+    clip_cov_ratio: Optional[float] = None
+    clip_cov_lb: Optional[float] = None
+    clip_cov_ub: Optional[float] = None
+    kl_cov_ratio: Optional[float] = None
+    ppo_kl_coef: Optional[float] = None
+
+
+def clip_cov_candidates(old_log_prob, log_prob, advantages, response_mask, eps_lo, eps_hi, lb, ub):
+    """The covariance matrix and the candidate set of Clip-Cov (reference ``core_algos.py:952-975``):
+    ``cov = (A - masked_mean(A)) * (lp - masked_mean(lp))``, minus infinity where the mask is zero or where the
+    PPO clip already bites (``l2 > l1``); candidates are the tokens with ``lb < cov < ub``, listed in row-major order."""
+    ratio = torch.exp(log_prob - old_log_prob)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - eps_lo, 1 + eps_hi)
+    clip_by_origin = (l2 > l1) & (response_mask > 0)
+    cov = (advantages - masked_mean(advantages, response_mask)) * (
+        log_prob.detach() - masked_mean(log_prob.detach(), response_mask))
+    cov = cov.clone()
+    cov[response_mask == 0] = -torch.inf
+    cov[clip_by_origin] = -torch.inf
+    cand = (cov < ub) & (cov > lb) & (response_mask > 0)
+    return cov, torch.nonzero(cand)
+
+
+def compute_policy_loss_clip_cov(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode="token-mean",
+                                 config=None, rollout_is_weights=None, dropped=None):
+    """Clip-Cov (reference ``core_algos.py:898-995``): the PPO clip surrogate without dual clip and without the
+    +-20 clamp of the log-ratio, with the loss of ``max(int(ratio * sum(mask)), 1)`` randomly chosen candidate tokens
+    (``torch.randperm`` on the host, the global generator) set to zero; ``pg_clipfrac`` is the masked share of
+    dropped tokens.  ``dropped`` (an ``[n, 2]`` index tensor) overrides the random choice, for tests of the arithmetic
+    after the draw.  Returns ``(pg_loss, pg_clipfrac, ppo_kl, 0)``."""
+    assert config is not None and config.policy_loss is not None
+    pl = config.policy_loss
+    ratio_cfg = pl.clip_cov_ratio if pl.clip_cov_ratio is not None else 0.0002
+    eps_lo, eps_hi = _clip_bounds(config)
+    ub = pl.clip_cov_ub if pl.clip_cov_ub is not None else 5.0
+    lb = pl.clip_cov_lb if pl.clip_cov_lb is not None else 1.0
+    assert ratio_cfg > 0, "clip_ratio should be larger than 0."
+
+    d = log_prob - old_log_prob
+    ratio = torch.exp(d)
+    ppo_kl = masked_mean(-d, response_mask)
+    l1 = -advantages * ratio
+    l2 = -advantages * torch.clamp(ratio, 1 - eps_lo, 1 + eps_hi)
+    if dropped is None:
+        _, cand = clip_cov_candidates(old_log_prob, log_prob, advantages, response_mask, eps_lo, eps_hi, lb, ub)
+        clip_num = max(int(ratio_cfg * response_mask.sum().item()), 1)
+        if len(cand) > 0:
+            perm = torch.randperm(len(cand))
+            dropped = cand[perm[: min(clip_num, len(cand))]]
+        else:
+            dropped = torch.empty((0, 2), dtype=torch.long)
+    corr = torch.ones_like(advantages)
+    corr[dropped[:, 0], dropped[:, 1]] = 0
+    pg_clipfrac = masked_mean((corr == 0).to(d.dtype), response_mask)
+    tok = torch.maximum(l1, l2) * corr
+    if rollout_is_weights is not None:
+        tok = tok * rollout_is_weights
+    return agg_loss(tok, response_mask, loss_agg_mode), pg_clipfrac, ppo_kl, torch.zeros((), dtype=d.dtype)
+
+
+def kl_cov_selection(log_prob, advantages, response_mask, kl_cov_ratio):
+    """Flat indices (into ``[B * L]``) of the tokens KL-Cov penalises (reference ``core_algos.py:1047-1060``): over
+    the tokens with a positive mask, ``cov = (A - mean A) * (lp - mean lp)`` with plain means, and the
+    ``max(1, int(n * ratio))`` largest values are taken."""
+    valid = response_mask > 0
+    valid_idx = torch.nonzero(valid.reshape(-1), as_tuple=True)[0]
+    a = advantages[valid].detach().reshape(-1)
+    lp = log_prob[valid].detach().reshape(-1)
+    if min(kl_cov_ratio, len(a)) == 0:
+        return valid_idx[:0], None
+    cov = (a - a.mean()) * (lp - lp.mean())
+    k = max(1, int(len(cov) * kl_cov_ratio))
+    return valid_idx[torch.topk(cov, k, largest=True).indices], cov
+
+
+def compute_policy_loss_kl_cov(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode="token-mean",
+                               config=None, rollout_is_weights=None):
+    """KL-Cov (reference ``core_algos.py:998-1071``): the unclipped surrogate ``-A * ratio``; the tokens selected by
+    ``kl_cov_selection`` additionally pay ``ppo_kl_coef * |lp - old|``.  Returns ``(pg_loss, 0, masked_mean(|lp - old|), 0)``."""
+    assert config is not None and config.policy_loss is not None
+    pl = config.policy_loss
+    kl_cov_ratio = pl.kl_cov_ratio if pl.kl_cov_ratio is not None else 0.0002
+    coef = pl.ppo_kl_coef if pl.ppo_kl_coef is not None else 1.0
+    assert kl_cov_ratio > 0, "kl_cov_ratio should be larger than 0."
+
+    d = log_prob - old_log_prob
+    abs_kl = d.abs()
+    ratio = torch.exp(d)
+    ppo_kl_abs = masked_mean(abs_kl, response_mask)
+    plain = -advantages * ratio
+    with_kl = -advantages * ratio + coef * abs_kl
+    chosen, _ = kl_cov_selection(log_prob, advantages, response_mask, kl_cov_ratio)
+    pick = torch.zeros(advantages.numel(), dtype=torch.bool)
+    pick[chosen] = True
+    tok = torch.where(pick.reshape(advantages.shape), with_kl, plain)
+    if rollout_is_weights is not None:
+        tok = tok * rollout_is_weights
+    zero = torch.zeros((), dtype=d.dtype)
+    return agg_loss(tok, response_mask, loss_agg_mode), zero, ppo_kl_abs, zero
+
+
+def compute_cpgd_outcome_advantage(token_level_rewards, response_mask, index, epsilon=1e-6,
+                                   weight_factor_in_cpgd="STD_weight"):
+    """CPGD's outcome advantage (reference ``core_algos.py:461-517``): the group statistics of the GRPO estimator (a
+    group of one: mean 0, std 1), then ``(s - mean) / (std + eps)`` (``STD_weight``), ``s - mean`` (``naive``) or
+    ``(s - mean) * min(B / #groups with std != 0, 3)`` (``clip_filter_like_weight``)."""
+    scores = token_level_rewards.sum(dim=-1)
+    keys = [index[i].item() if hasattr(index[i], "item") else index[i] for i in range(scores.shape[0])]
+    members = OrderedDict()
+    for i, k in enumerate(keys):
+        members.setdefault(k, []).append(i)
+    mean, std = {}, {}
+    for k, rows in members.items():
+        if len(rows) == 1:
+            mean[k], std[k] = torch.zeros((), dtype=scores.dtype), torch.ones((), dtype=scores.dtype)
+        else:
+            mean[k], std[k] = scores[rows].mean(), scores[rows].std()
+    bsz = scores.shape[0]
+    out = scores.clone()
+    for i, k in enumerate(keys):
+        if weight_factor_in_cpgd == "STD_weight":
+            out[i] = (scores[i] - mean[k]) / (std[k] + epsilon)
+        elif weight_factor_in_cpgd == "clip_filter_like_weight":
+            live = sum(int(v != 0) for v in std.values())  # no live group: B / 0 = inf there, clamped to 3
+            out[i] = (scores[i] - mean[k]) * (min(bsz / live, 3.0) if live else 3.0)
+        elif weight_factor_in_cpgd == "naive":
+            out[i] = scores[i] - mean[k]
+        else:
+            raise NotImplementedError
+    out = out.unsqueeze(-1) * response_mask
+    return out, out
 
 
 def compute_value_loss(vpreds, returns, values, response_mask, cliprange_value, loss_agg_mode="token-mean"):

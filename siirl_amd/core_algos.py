@@ -37,7 +37,8 @@ __all__ = [
     "AdaptiveKLController", "FixedKLController", "get_kl_controller", "compute_response_mask",
     "compute_gae_advantage_return", "compute_grpo_outcome_advantage", "compute_rewards", "agg_loss",
     "compute_policy_loss", "compute_policy_loss_vanilla", "compute_policy_loss_gspo", "compute_policy_loss_cpgd",
-    "compute_policy_loss_gpg", "compute_policy_loss_geo_mean", "compute_entropy_loss", "compute_value_loss", "kl_penalty",
+    "compute_policy_loss_gpg", "compute_policy_loss_geo_mean", "compute_policy_loss_clip_cov",
+    "compute_policy_loss_kl_cov", "compute_cpgd_outcome_advantage", "compute_entropy_loss", "compute_value_loss", "kl_penalty",
     "kl_penalty_forward",
     "apply_kl_penalty", "compute_advantage", "actor_loss", "ActorLossOutput", "fused_actor_step",
     "FusedActorStepOutput", "agg_weights",
@@ -45,8 +46,9 @@ __all__ = [
 
 AGG_MODES = {"token-mean": 0, "seq-mean-token-sum": 1, "seq-mean-token-mean": 2, "seq-mean-token-sum-norm": 3}
 KL_MODES = {"kl": 0, "k1": 0, "abs": 1, "mse": 2, "k2": 2, "low_var_kl": 3, "k3": 3}
-LOSS_VANILLA, LOSS_GSPO, LOSS_CPGD, LOSS_GPG, LOSS_GEO_MEAN = range(5)
-_LOSS_CODES = {"vanilla": LOSS_VANILLA, "gspo": LOSS_GSPO, "cpgd": LOSS_CPGD, "gpg": LOSS_GPG, "geo_mean": LOSS_GEO_MEAN}
+LOSS_VANILLA, LOSS_GSPO, LOSS_CPGD, LOSS_GPG, LOSS_GEO_MEAN, LOSS_KL_COV, LOSS_CLIP_COV = range(7)
+_LOSS_CODES = {"vanilla": LOSS_VANILLA, "gspo": LOSS_GSPO, "cpgd": LOSS_CPGD, "gpg": LOSS_GPG, "geo_mean": LOSS_GEO_MEAN,
+               "kl_cov": LOSS_KL_COV, "clip_cov": LOSS_CLIP_COV}
 # indices into the 16-float result block (SIIRL_OUT_* of include/siirl_hip.h)
 (O_LOSS, O_PG, O_CLIPFRAC, O_PPOKL, O_CLIPLOWER, O_ENT, O_KL, O_RMEAN, O_RMIN, O_RMAX, O_MTOTAL, O_POLICY,
  O_DRIFT) = range(13)
@@ -292,6 +294,47 @@ def compute_grpo_outcome_advantage(token_level_rewards: torch.Tensor, response_m
     return adv, adv
 
 
+def _group_codes(index, n, dev) -> torch.Tensor:
+    """int64 group codes for keys that are compared as they are (``core_algos.py:495``: ``id2score[index[i]]``):
+    integer tensors / arrays unchanged, anything else numbered in order of first appearance."""
+    if isinstance(index, torch.Tensor) and not index.dtype.is_floating_point:
+        return _uid_tensor(index, n, dev)
+    arr = np.asarray(index)
+    if arr.dtype.kind in "iu":
+        return _uid_tensor(arr, n, dev)
+    seq = [v.item() if hasattr(v, "item") else v for v in (index if isinstance(index, (list, tuple)) else arr.reshape(-1))]
+    codes: dict = {}
+    return _uid_tensor(np.fromiter((codes.setdefault(v, len(codes)) for v in seq), dtype=np.int64, count=len(seq)), n, dev)
+
+
+def compute_cpgd_outcome_advantage(token_level_rewards: torch.Tensor, response_mask: torch.Tensor, index,
+                                   epsilon: float = 1e-6, weight_factor_in_cpgd: str = "STD_weight"):
+    """CPGD's outcome advantage (reference ``core_algos.py:461-517``; the reference's dispatcher cannot reach it,
+    ``:1475-1480``, callers use it directly).  Group statistics as in the GRPO estimator (a group of one: mean 0,
+    std 1); ``STD_weight``: ``(s - mean) / (std + eps)``; ``naive``: ``s - mean``; ``clip_filter_like_weight``:
+    ``(s - mean) * min(B / #groups whose std is not zero, 3)``.  Returns the same ``[B, L]`` fp32 tensor twice."""
+    if weight_factor_in_cpgd not in ("STD_weight", "clip_filter_like_weight", "naive"):
+        raise NotImplementedError
+    dev, back = _staging_device(token_level_rewards, response_mask)
+    B, L = token_level_rewards.shape
+    r = _f32(token_level_rewards, dev)
+    m, mcode = _mask_arg(response_mask, dev)
+    uid = _group_codes(index, B, dev)
+    adv = _OPS.grpo_advantage(r, m, uid, float(epsilon), weight_factor_in_cpgd == "STD_weight")
+    if weight_factor_in_cpgd == "clip_filter_like_weight" and B > 0:
+        # a group is live when its scores are not all equal (or it has one member: std is set to 1); each member of
+        # a live group of n contributes 1 / n to the count
+        # (in float64 the mean of equal float32 scores is exact, so "all equal" and "std == 0" coincide as they do
+        # for torch.std)
+        keep, gsz = _OPS.group_keep_mask(r.sum(dim=-1).to(torch.float64), uid)
+        live = torch.round((keep.to(torch.float64) / gsz.to(torch.float64)).sum())
+        factor = torch.clamp((B / live).to(torch.float32), max=3.0)  # no live group: inf, clamped
+        adv = adv * factor
+    if back:
+        adv = adv.to(token_level_rewards.device)
+    return adv, adv
+
+
 def compute_rewards(token_level_scores, old_log_prob, ref_log_prob, kl_ratio):
     """reference ``core_algos.py:520-533``: ``scores - (old - ref) * kl_ratio`` (k1 estimator, no mask)."""
     dev = _gpu_of(token_level_scores, old_log_prob, ref_log_prob)
@@ -499,6 +542,118 @@ def compute_policy_loss_geo_mean(old_log_prob: torch.Tensor, log_prob: torch.Ten
                         AGG_MODES["token-mean"], lo, hi, 3.0, 20.0, rollout_is_weights)
 
 
+def _cov_operands(old_log_prob, log_prob, advantages, response_mask):
+    dev = _gpu_of(log_prob)
+    lp = _as_2d(_f32(log_prob, dev))
+    old = None if old_log_prob is None else _as_2d(_f32(old_log_prob, dev))
+    adv = _as_2d(_f32(advantages, dev))
+    m, _ = _mask_arg(_as_2d(response_mask), dev)
+    if m.shape != lp.shape:
+        m = m.expand(lp.shape).contiguous()
+    return dev, old, lp, adv, m
+
+
+def _kl_cov_weights(log_prob, advantages, response_mask, kl_cov_ratio: float, ppo_kl_coef: float) -> torch.Tensor:
+    """``[B, L]`` fp32: ``ppo_kl_coef`` on the ``max(1, int(n * kl_cov_ratio))`` tokens of largest covariance among
+    the ``n`` tokens with a positive mask (reference ``core_algos.py:1047-1060``), 0 elsewhere.  One host sync (the
+    count ``n``), as the reference's ``len(all_valid_adv)``."""
+    dev, _, lp, adv, m = _cov_operands(None, log_prob, advantages, response_mask)
+    cov, stats = _OPS.cov_scores(None, lp, adv, m, LOSS_KL_COV, 0.0, 0.0)
+    aux = torch.zeros_like(cov)
+    n = int(stats[0].item())
+    if min(kl_cov_ratio, n) != 0:  # reference :1052-1054
+        k = max(1, int(n * kl_cov_ratio))
+        if k > n:
+            raise RuntimeError(f"kl_cov_ratio {kl_cov_ratio} selects {k} of {n} valid tokens")  # torch.topk: k out of range
+        idx = torch.topk(cov.reshape(-1), k, largest=True).indices
+        aux.reshape(-1)[idx] = float(ppo_kl_coef)
+    return aux
+
+
+def _clip_cov_dropped(old_log_prob, log_prob, advantages, response_mask, lo, hi, clip_cov_ratio, lb, ub) -> torch.Tensor:
+    """``[B, L]`` fp32, 1 on the tokens Clip-Cov drops (reference ``core_algos.py:963-983``): candidates are the
+    unmasked tokens the PPO clip leaves alone with ``lb < cov < ub``, in row-major order; of them
+    ``max(int(ratio * sum(mask)), 1)`` are drawn with one ``torch.randperm`` on the host's global generator, the
+    reference's own draw.  Two host syncs (mask sum, candidate count), as there."""
+    dev, old, lp, adv, m = _cov_operands(old_log_prob, log_prob, advantages, response_mask)
+    cov, stats = _OPS.cov_scores(old, lp, adv, m, LOSS_CLIP_COV, lo, hi)
+    clip_num = max(int(clip_cov_ratio * stats[1].item()), 1)
+    cand = torch.nonzero((cov < ub) & (cov > lb) & (m > 0))
+    aux = torch.zeros_like(cov)
+    if len(cand) > 0:
+        perm = torch.randperm(len(cand))
+        chosen = cand[perm[: min(clip_num, len(cand))].to(dev)]
+        aux[chosen[:, 0], chosen[:, 1]] = 1.0
+    return aux
+
+
+def _policy_loss_cfg(config):
+    assert config is not None
+    pl = getattr(config, "policy_loss", None)
+    assert pl is not None
+    return pl
+
+
+def _clip_cov_params(config):
+    pl = _policy_loss_cfg(config)
+    ratio = pl.clip_cov_ratio if getattr(pl, "clip_cov_ratio", None) is not None else 0.0002
+    ub = pl.clip_cov_ub if getattr(pl, "clip_cov_ub", None) is not None else 5.0
+    lb = pl.clip_cov_lb if getattr(pl, "clip_cov_lb", None) is not None else 1.0
+    assert ratio > 0, "clip_ratio should be larger than 0."
+    return float(ratio), float(lb), float(ub)
+
+
+def _kl_cov_params(config):
+    pl = _policy_loss_cfg(config)
+    ratio = pl.kl_cov_ratio if getattr(pl, "kl_cov_ratio", None) is not None else 0.0002
+    coef = pl.ppo_kl_coef if getattr(pl, "ppo_kl_coef", None) is not None else 1.0
+    assert ratio > 0, "kl_cov_ratio should be larger than 0."
+    return float(ratio), float(coef)
+
+
+def _cov_policy_only(loss_mode, old_log_prob, log_prob, advantages, response_mask, agg_code, lo, hi, rollout_is_weights,
+                     aux):
+    outs = _actor_loss_op(log_prob, None, old_log_prob, advantages, response_mask, rollout_is_weights, None, loss_mode,
+                          lo, hi, 3.0, 20.0, agg_code, 0.0, 0, False, 0.0, 0.0, 1.0, True, aux)
+    return outs
+
+
+@register_policy_loss("clip_cov")
+def compute_policy_loss_clip_cov(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                                 response_mask: torch.Tensor, loss_agg_mode: str = "token-mean", config=None,
+                                 rollout_is_weights: Optional[torch.Tensor] = None):
+    """Clip-Cov (reference ``core_algos.py:898-995``): the PPO clip surrogate (no dual clip, no clamp of the
+    log-ratio) with the loss of a few randomly drawn high-covariance tokens set to zero.  ``config.policy_loss``
+    carries ``clip_cov_ratio`` (0.0002), ``clip_cov_lb`` (1.0), ``clip_cov_ub`` (5.0).  The draw is the reference's
+    own ``torch.randperm`` on the host generator: with the same seed and inputs the same tokens are dropped.
+    Returns ``(pg_loss, pg_clipfrac = masked share of dropped tokens, ppo_kl, 0)``.  The reference's assertion that
+    ``config`` is not its ``ActorArguments`` (``:940``) has no counterpart here."""
+    ratio, lb, ub = _clip_cov_params(config)
+    lo, hi = _clip_params(config)
+    agg_code = _agg_code(loss_agg_mode)
+    aux = _clip_cov_dropped(old_log_prob, log_prob, advantages, response_mask, lo, hi, ratio, lb, ub)
+    outs = _cov_policy_only(LOSS_CLIP_COV, old_log_prob, log_prob, advantages, response_mask, agg_code, lo, hi,
+                            rollout_is_weights, aux)
+    return outs[O_PG], outs[O_CLIPFRAC], outs[O_PPOKL], outs[O_CLIPLOWER]
+
+
+@register_policy_loss("kl_cov")
+def compute_policy_loss_kl_cov(old_log_prob: torch.Tensor, log_prob: torch.Tensor, advantages: torch.Tensor,
+                               response_mask: torch.Tensor, loss_agg_mode: str = "token-mean", config=None,
+                               rollout_is_weights: Optional[torch.Tensor] = None):
+    """KL-Cov (reference ``core_algos.py:998-1071``): the unclipped surrogate ``-A * ratio``; the
+    ``max(1, int(n * kl_cov_ratio))`` valid tokens of largest covariance between advantage and log-prob additionally
+    pay ``ppo_kl_coef * |log_prob - old_log_prob|``.  ``config.policy_loss`` carries ``kl_cov_ratio`` (0.0002) and
+    ``ppo_kl_coef`` (1.0).  Returns ``(pg_loss, 0, masked_mean(|log_prob - old_log_prob|), 0)``.  Tokens whose
+    covariances are equal at the cut are taken in the order ``torch.topk`` yields on the device."""
+    ratio, coef = _kl_cov_params(config)
+    agg_code = _agg_code(loss_agg_mode)
+    aux = _kl_cov_weights(log_prob, advantages, response_mask, ratio, coef)
+    outs = _cov_policy_only(LOSS_KL_COV, old_log_prob, log_prob, advantages, response_mask, agg_code, 0.2, 0.2,
+                            rollout_is_weights, aux)
+    return outs[O_PG], outs[O_CLIPFRAC], outs[O_PPOKL], outs[O_CLIPLOWER]
+
+
 def compute_value_loss(vpreds: torch.Tensor, returns: torch.Tensor, values: torch.Tensor, response_mask: torch.Tensor,
                        cliprange_value: float, loss_agg_mode: str = "token-mean"):
     """Clipped value loss of the critic (reference ``core_algos.py:1173-1212``).  Returns ``(vf_loss,
@@ -593,7 +748,7 @@ def actor_loss(old_log_prob, log_prob, advantages, response_mask, config, entrop
     ``siirl/engine/actor/dp_actor.py:455-500``), fused:
     ``loss = (pg_loss - entropy_coeff * agg(entropy) + kl_loss_coef * agg(kl_penalty(log_prob, ref))) * scale``.
     ``config`` carries ``clip_ratio*``, ``entropy_coeff``, ``use_kl_loss``, ``kl_loss_coef``, ``kl_loss_type``,
-    ``loss_agg_mode``, ``policy_loss.loss_mode`` (or ``loss_mode``; vanilla, gspo, cpgd, gpg or geo_mean) and
+    ``loss_agg_mode``, ``policy_loss.loss_mode`` (or ``loss_mode``; vanilla, gspo, cpgd, gpg, geo_mean, kl_cov or clip_cov) and
     ``use_cpgd_loss`` / ``policy_drift_coeff``.  The entropy term is used when ``entropy`` is given and
     ``entropy_coeff != 0``; the KL term when ``config.use_kl_loss``; the drift term
     ``policy_drift_coeff * agg(clamp(exp(lp - old) - 1, max=2) * lp)`` (``dp_actor.py:488-494``) when
@@ -622,10 +777,15 @@ def actor_loss(old_log_prob, log_prob, advantages, response_mask, config, entrop
         if kl_type not in KL_MODES:
             raise NotImplementedError
         kl_code, kl_coef = KL_MODES[kl_type], float(getattr(config, "kl_loss_coef", 0.001))
+    aux = None
+    if mode == "kl_cov":
+        aux = _kl_cov_weights(log_prob, advantages, response_mask, *_kl_cov_params(config))
+    elif mode == "clip_cov":
+        aux = _clip_cov_dropped(old_log_prob, log_prob, advantages, response_mask, lo, hi, *_clip_cov_params(config))
     outs = _actor_loss_op(log_prob, entropy if use_ent else None, old_log_prob, advantages, response_mask,
                           None if mode == "cpgd" else rollout_is_weights, ref_log_prob if use_kl else None,
                           _LOSS_CODES[mode], lo, hi, c, 20.0, agg_code, ent_coef if use_ent else 0.0, kl_code, False,
-                          kl_coef, drift, float(loss_scale_factor), False)
+                          kl_coef, drift, float(loss_scale_factor), False, aux)
     return ActorLossOutput(outs, float(loss_scale_factor), kl_coef, use_kl, use_ent)
 
 

@@ -139,6 +139,7 @@ __global__ __launch_bounds__(kStream) void loss_partials_kernel(LossArgs a, cons
     const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
     const Quad ent4 = a.ent ? load_quad(a.ent, idx0, vec, nv, 0.f) : const_quad(0.f);
     const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
+    const Quad aux4 = (KIND < 0 && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (e >= nv) break;
@@ -149,7 +150,7 @@ __global__ __launch_bounds__(kStream) void loss_partials_kernel(LossArgs a, cons
         continue;
       }
       const float lp = lp4.v[e];
-      const PgOut o = pg_token(kind, lp, old4.v[e], adv4.v[e], isw4.v[e], seq_s, a);
+      const PgOut o = pg_token(kind, lp, old4.v[e], adv4.v[e], isw4.v[e], seq_s, a, aux4.v[e]);
       if (kind != KIND_GEO) acc[P_PG] += contrib(o.tok, m, a.agg_mode);  // GEO: the loss is per sequence (row_s)
       acc[P_CLIP] += contrib_where(o.clip, m);
       acc[P_NEGD] += contrib_where(o.negd, m);
@@ -404,10 +405,11 @@ __global__ __launch_bounds__(kStream) void loss_bwd_kernel(LossArgs a, const flo
     const Quad adv4 = load_quad(a.adv, idx0, vec, nv, 0.f);
     const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
     const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
+    const Quad aux4 = (KIND < 0 && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float m = m4.v[e], lp = lp4.v[e];
-      const PgOut o = pg_token(kind, lp, old4.v[e], adv4.v[e], isw4.v[e], seq_s, a);
+      const PgOut o = pg_token(kind, lp, old4.v[e], adv4.v[e], isw4.v[e], seq_s, a, aux4.v[e]);
       float d;
       if (kind == KIND_GEO)  // d mean_b(row loss) / d x = row loss * m / (n + 1e-8) / B
         d = geo_c * m * o.dtok;
@@ -633,6 +635,77 @@ __global__ __launch_bounds__(kThreads) void mean_rows_kernel(const float* __rest
   if (threadIdx.x == 0) out[0] = (float)(s / (double)B);
 }
 
+// ---------------------------------------------------------------------------- covariance scores (clip_cov, kl_cov)
+
+// Sums over the whole [B, L] batch that the two covariance losses centre their operands with, in a fixed grid so
+// that the result does not depend on the launch: per workgroup {count of m > 0, sum A and sum lp over m > 0,
+// sum m, sum A*m, sum lp*m} (floats per thread, doubles from the wave up), folded by one workgroup.
+constexpr int kCovGrid = 1024;
+constexpr int kCovSums = 6;
+__global__ __launch_bounds__(kThreads) void cov_sums_kernel(const float* __restrict__ lp, const float* __restrict__ adv,
+                                                            const void* mask, int mask_dtype, int64_t n,
+                                                            double* __restrict__ part) {
+  float s[kCovSums] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+    const float m = load_mask(mask, mask_dtype, i);
+    const float a = adv[i], l = lp[i];
+    if (m > 0.f) { s[0] += 1.f; s[1] += a; s[2] += l; }
+    s[3] += m;
+    s[4] += contrib_where(a, m);  // masked_mean: where(mask, v, 0) * mask
+    s[5] += contrib_where(l, m);
+  }
+  __shared__ double sh[kThreads / kWave + 1];
+  for (int k = 0; k < kCovSums; ++k) {
+    const double t = block_sum((double)s[k], sh);
+    if (threadIdx.x == 0) part[(int64_t)blockIdx.x * kCovSums + k] = t;
+  }
+}
+// stats[0..3] = {count of m > 0, sum of the mask, mean A, mean lp}; plain means over m > 0 (kl_cov, core_algos.py:1055)
+// or masked means sum(v * m) / (sum(m) + 1e-8) in fp32 (clip_cov, :967-969)
+__global__ __launch_bounds__(kThreads) void cov_stats_kernel(const double* __restrict__ part, int nparts, int masked_means,
+                                                             float* __restrict__ stats) {
+  __shared__ double sh[kThreads / kWave + 1];
+  double t[kCovSums];
+  for (int k = 0; k < kCovSums; ++k) {
+    double v = 0.0;
+    for (int i = threadIdx.x; i < nparts; i += kThreads) v += part[(int64_t)i * kCovSums + k];
+    t[k] = block_sum(v, sh);
+  }
+  if (threadIdx.x == 0) {
+    stats[0] = (float)t[0];
+    stats[1] = (float)t[3];
+    if (masked_means) {
+      const float den = (float)t[3] + 1e-8f;
+      stats[2] = (float)t[4] / den;
+      stats[3] = (float)t[5] / den;
+    } else {
+      stats[2] = (float)(t[1] / t[0]);  // no token with m > 0: 0 / 0, and no score is finite anyway
+      stats[3] = (float)(t[2] / t[0]);
+    }
+  }
+}
+// cov[b, t] = (A - mean A) * (lp - mean lp), minus infinity where m <= 0 (kl_cov: m > 0 selects; clip_cov: m == 0 is
+// excluded) and, for clip_cov, where the PPO clip already bites (l2 > l1 under a positive mask)
+__global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __restrict__ old_lp, const float* __restrict__ lp,
+                                                              const float* __restrict__ adv, const void* mask,
+                                                              int mask_dtype, int64_t n, int clip_mode, float lo, float hi,
+                                                              const float* __restrict__ stats, float* __restrict__ cov) {
+  const float ma = stats[2], ml = stats[3];
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
+    const float m = load_mask(mask, mask_dtype, i);
+    const float a = adv[i], l = lp[i];
+    float c = (a - ma) * (l - ml);
+    if (clip_mode) {
+      const float r = expf(l - old_lp[i]);
+      const float l1 = -a * r, l2 = -a * clampf(r, lo, hi);
+      if (m == 0.f || (l2 > l1 && m > 0.f)) c = -__builtin_inff();
+    } else if (!(m > 0.f)) {
+      c = -__builtin_inff();
+    }
+    cov[i] = c;
+  }
+}
+
 // ---------------------------------------------------------------------------- host
 
 int nseg_of(int64_t L) { return (int)((L + kSeg - 1) / kSeg); }
@@ -643,7 +716,7 @@ void set_vec(LossArgs& a, const void* o1 = nullptr, const void* o2 = nullptr) {
   const size_t msz = a.mask_dtype == SIIRL_I64 ? 8 : (a.mask_dtype == SIIRL_U8 ? 1 : (a.mask_dtype == SIIRL_F32 || a.mask_dtype == SIIRL_I32 ? 4 : 2));
   const bool mask_ok = ((uintptr_t)a.mask & (msz * 4 > 16 ? 15 : msz * 4 - 1)) == 0;
   a.vec = (a.L % 4 == 0) && mask_ok && ok16(a.old_lp) && ok16(a.lp) && ok16(a.adv) && ok16(a.isw) && ok16(a.ent) &&
-          ok16(a.ref) && ok16(o1) && ok16(o2);
+          ok16(a.ref) && ok16(a.aux) && ok16(o1) && ok16(o2);
 }
 
 size_t ws_bytes_of(int64_t B, int64_t L) {
@@ -787,12 +860,17 @@ static int fill_actor_args(LossArgs& a, const float* old_log_prob, const float* 
                            const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
                            const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
                            float clip_high, float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode,
-                           int kl_straight_through, float kl_coef, float policy_drift_coeff, float loss_scale) {
+                           int kl_straight_through, float kl_coef, float policy_drift_coeff, float loss_scale,
+                           const float* token_aux = nullptr, bool cov = false) {
   if (int rc = check_dims(B, L)) return rc;
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   if (int rc = check_agg(agg_mode)) return rc;
-  SIIRL_REQUIRE(loss_mode >= SIIRL_LOSS_VANILLA && loss_mode <= SIIRL_LOSS_GEO_MEAN, "Unsupported loss mode: %d",
-                loss_mode);
+  if (!cov)
+    SIIRL_REQUIRE(loss_mode >= SIIRL_LOSS_VANILLA && loss_mode <= SIIRL_LOSS_GEO_MEAN, "Unsupported loss mode: %d",
+                  loss_mode);
+  else
+    SIIRL_REQUIRE(loss_mode == SIIRL_LOSS_KL_COV || loss_mode == SIIRL_LOSS_CLIP_COV,
+                  "loss mode %d takes no per-token selection (kl_cov and clip_cov do)", loss_mode);
   SIIRL_REQUIRE(B == 0 || (old_log_prob && log_prob && advantages && mask), "NULL operand");
   if (loss_mode == SIIRL_LOSS_VANILLA || loss_mode == SIIRL_LOSS_CPGD)
     SIIRL_REQUIRE(clip_c > 1.0f, "clip_ratio_c must be greater than 1.0, got %f", (double)clip_c);
@@ -804,8 +882,8 @@ static int fill_actor_args(LossArgs& a, const float* old_log_prob, const float* 
   SIIRL_REQUIRE(log_ratio_clamp > 0.f, "log_ratio_clamp must be positive (20 in the reference, +inf for none)");
   if (ref_log_prob) SIIRL_REQUIRE(kl_mode >= 0 && kl_mode <= 3, "unknown kl mode %d", kl_mode);
   a.old_lp = old_log_prob; a.lp = log_prob; a.adv = advantages; a.mask = mask; a.mask_dtype = mask_dtype;
-  a.isw = is_weights; a.ent = entropy; a.ref = ref_log_prob;
-  static const int kind_of[] = {KIND_VANILLA, KIND_GSPO, KIND_CPGD, KIND_GPG, KIND_GEO};
+  a.isw = is_weights; a.ent = entropy; a.ref = ref_log_prob; a.aux = token_aux;
+  static const int kind_of[] = {KIND_VANILLA, KIND_GSPO, KIND_CPGD, KIND_GPG, KIND_GEO, KIND_KL_COV, KIND_CLIP_COV};
   a.kind = kind_of[loss_mode];
   a.agg_mode = loss_mode == SIIRL_LOSS_GSPO ? SIIRL_AGG_SEQ_MEAN_TOKEN_MEAN : agg_mode;
   a.aux_agg_mode = agg_mode;
@@ -900,6 +978,80 @@ extern "C" int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_pr
   SIIRL_REQUIRE(entropy == nullptr || d_entropy != nullptr, "d_entropy is required when entropy is given");
   set_vec(a, d_log_prob, d_entropy);
   return launch_loss_bwd(a, g_loss, out16, row_msum, row_s, d_log_prob, d_entropy, (hipStream_t)stream);
+}
+
+extern "C" size_t siirl_cov_workspace_bytes(void) { return (size_t)kCovGrid * kCovSums * sizeof(double); }
+
+extern "C" int siirl_cov_scores(const float* old_log_prob, const float* log_prob, const float* advantages,
+                                const void* mask, int mask_dtype, int64_t B, int64_t L, int loss_mode, float clip_low,
+                                float clip_high, float* cov, float* stats, void* workspace, size_t workspace_bytes,
+                                siirl_stream_t stream) {
+  if (int rc = check_dims(B, L)) return rc;
+  if (int rc = check_mask_dtype(mask_dtype)) return rc;
+  SIIRL_REQUIRE(loss_mode == SIIRL_LOSS_KL_COV || loss_mode == SIIRL_LOSS_CLIP_COV,
+                "covariance scores belong to the kl_cov and clip_cov losses (loss mode %d given)", loss_mode);
+  SIIRL_REQUIRE(stats != nullptr, "NULL stats");
+  SIIRL_REQUIRE(B == 0 || (log_prob && advantages && mask && cov), "NULL operand");
+  SIIRL_REQUIRE(B == 0 || loss_mode != SIIRL_LOSS_CLIP_COV || old_log_prob, "clip_cov needs old_log_prob");
+  if (workspace == nullptr || workspace_bytes < siirl_cov_workspace_bytes())
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes,
+                siirl_cov_workspace_bytes());
+  SIIRL_REQUIRE(((uintptr_t)workspace & 7) == 0, "workspace must be 8-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n = B * L;
+  const int clip_mode = loss_mode == SIIRL_LOSS_CLIP_COV;
+  const int grid = (int)(n == 0 ? 1 : ((n + kThreads - 1) / kThreads < kCovGrid ? (n + kThreads - 1) / kThreads : kCovGrid));
+  double* part = (double*)workspace;
+  cov_sums_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(log_prob, advantages, mask, mask_dtype, n, part);
+  SIIRL_LAUNCH_CHECK("cov_sums_kernel");
+  cov_stats_kernel<<<1, dim3(kThreads), 0, st>>>(part, grid, clip_mode, stats);
+  SIIRL_LAUNCH_CHECK("cov_stats_kernel");
+  if (n == 0) return SIIRL_OK;
+  cov_scores_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(old_log_prob, log_prob, advantages, mask, mask_dtype,
+                                                                    n, clip_mode, 1.f - clip_low, 1.f + clip_high, stats,
+                                                                    cov);
+  SIIRL_LAUNCH_CHECK("cov_scores_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_actor_loss_cov_fwd(const float* old_log_prob, const float* log_prob, const float* advantages,
+                                        const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
+                                        const float* ref_log_prob, const float* token_aux, int64_t B, int64_t L,
+                                        int loss_mode, float clip_low, float clip_high, int agg_mode, float entropy_coeff,
+                                        int kl_mode, int kl_straight_through, float kl_coef, float policy_drift_coeff,
+                                        float loss_scale, float* out16, float* row_msum, void* workspace,
+                                        size_t workspace_bytes, siirl_stream_t stream) {
+  LossArgs a{};
+  SIIRL_REQUIRE(token_aux != nullptr || B == 0, "token_aux is NULL");
+  if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
+                               ref_log_prob, B, L, loss_mode, clip_low, clip_high, 3.0f, 20.0f, agg_mode, entropy_coeff,
+                               kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale,
+                               token_aux, true))
+    return rc;
+  SIIRL_REQUIRE(out16 && (B == 0 || row_msum), "NULL output");
+  return run_forward(a, out16, row_msum, nullptr, workspace, workspace_bytes, (hipStream_t)stream);
+}
+
+extern "C" int siirl_actor_loss_cov_bwd(const float* g_loss, const float* old_log_prob, const float* log_prob,
+                                        const float* advantages, const void* mask, int mask_dtype,
+                                        const float* is_weights, const float* entropy, const float* ref_log_prob,
+                                        const float* token_aux, int64_t B, int64_t L, int loss_mode, float clip_low,
+                                        float clip_high, int agg_mode, float entropy_coeff, int kl_mode,
+                                        int kl_straight_through, float kl_coef, float policy_drift_coeff,
+                                        float loss_scale, const float* out16, const float* row_msum, float* d_log_prob,
+                                        float* d_entropy, siirl_stream_t stream) {
+  LossArgs a{};
+  SIIRL_REQUIRE(token_aux != nullptr || B == 0, "token_aux is NULL");
+  if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
+                               ref_log_prob, B, L, loss_mode, clip_low, clip_high, 3.0f, 20.0f, agg_mode, entropy_coeff,
+                               kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale,
+                               token_aux, true))
+    return rc;
+  if (B == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(g_loss && out16 && row_msum && d_log_prob, "NULL operand");
+  SIIRL_REQUIRE(entropy == nullptr || d_entropy != nullptr, "d_entropy is required when entropy is given");
+  set_vec(a, d_log_prob, d_entropy);
+  return launch_loss_bwd(a, g_loss, out16, row_msum, nullptr, d_log_prob, d_entropy, (hipStream_t)stream);
 }
 
 static int fill_value_args(LossArgs& a, const float* vpreds, const float* returns, const float* values,

@@ -3,7 +3,8 @@
 // estimators, aggregation weights, and small load helpers.
 //
 // Follows siirl/dag_worker/core_algos.py: agg_loss :536-569, cpgd :572-629, vanilla :710-792, gspo :795-862,
-// gpg :865-895, geo_mean :1074-1153, value loss :1173-1212, kl_penalty :1215-1276; drift term
+// gpg :865-895, clip_cov :898-995, kl_cov :998-1071, geo_mean :1074-1153, value loss :1173-1212, kl_penalty
+// :1215-1276; drift term
 // siirl/engine/actor/dp_actor.py:488-494.
 #pragma once
 #include "common.hpp"
@@ -28,6 +29,8 @@ struct LossArgs {
   const float* isw;      // [B,L] or null
   const float* ent;      // [B,L] or null
   const float* ref;      // [B,L] or null
+  const float* aux;      // [B,L], the covariance losses only: kl_cov the coefficient of |lp - old| per token
+                         // (ppo_kl_coef where selected, else 0), clip_cov non-zero where the token's loss is dropped
   int mask_dtype;
   int kind;              // KIND_*
   int agg_mode;          // aggregation of the policy term (GSPO: forced to seq-mean-token-mean)
@@ -40,7 +43,8 @@ struct LossArgs {
   int nseg;
   int vec;  // L % 4 == 0 and every operand 16-byte aligned: tokens are moved four at a time
 };
-enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6 };
+enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6,
+       KIND_KL_COV = 7, KIND_CLIP_COV = 8 };
 
 // torch.clamp / torch.maximum / torch.minimum semantics (NaN propagates)
 __device__ __forceinline__ float clampf(float x, float lo, float hi) { return x < lo ? lo : (x > hi ? hi : x); }
@@ -155,9 +159,9 @@ struct PgOut {
 
 // seq_s: GSPO's sequence-level mean log-ratio (unused otherwise).  For KIND_GEO tok is the token's clipped
 // log-ratio x (the loss itself is per sequence); for KIND_VALUE lp = vpreds, old = values, A = returns and
-// eps_lo = cliprange_value.
+// eps_lo = cliprange_value.  aux: the token's entry of LossArgs::aux (0 for the losses that have none).
 __device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A, float isw, float seq_s,
-                                          const LossArgs& a) {
+                                          const LossArgs& a, float aux = 0.f) {
   const float eps_lo = a.eps_lo, eps_hi = a.eps_hi, clip_c = a.clip_c, dclamp = a.dclamp;
   PgOut o;
   const float raw = lp - old;
@@ -201,6 +205,32 @@ __device__ __forceinline__ PgOut pg_token(int kind, float lp, float old, float A
     const bool clipped = raw != dc;
     o.clip = (clipped && A > 0.f) ? 1.f : 0.f;
     o.lower = (clipped && A < 0.f) ? 1.f : 0.f;
+    return o;
+  }
+  if (kind == KIND_KL_COV) {
+    // -A * ratio, unclipped; a selected token also pays aux * |lp - old|.  The ppo_kl slot reports mean |lp - old|.
+    const float ad = fabsf(raw);
+    o.negd = ad; o.clip = 0.f; o.lower = 0.f;
+    const float base = -A * o.r_raw;
+    const float sg = raw > 0.f ? 1.f : (raw < 0.f ? -1.f : raw);  // torch.sign: 0 at 0, NaN stays NaN
+    o.tok = (aux != 0.f ? base + aux * ad : base) * isw;
+    o.dtok = (aux != 0.f ? base + aux * sg : base) * isw;
+    return o;
+  }
+  if (kind == KIND_CLIP_COV) {
+    // the PPO clip surrogate without dual clip and without the clamp of the log-ratio; a dropped token (aux != 0)
+    // contributes nothing and is what the clip-fraction slot counts
+    o.negd = -raw; o.lower = 0.f;
+    const float r = o.r_raw;
+    const float l1 = -A * r;
+    const float l2 = -A * clampf(r, lo, hi);
+    const float corr = aux != 0.f ? 0.f : 1.f;
+    o.clip = 1.f - corr;
+    o.tok = tmax(l1, l2) * corr * isw;
+    const float dl2 = (r >= lo && r <= hi) ? l1 : 0.f;  // d l1 / d lp = l1
+    const float w1 = l1 > l2 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    const float w2 = l2 > l1 ? 1.f : (l1 == l2 ? 0.5f : 0.f);
+    o.dtok = (w1 * l1 + w2 * dl2) * corr * isw;
     return o;
   }
   if (kind == KIND_VALUE) {

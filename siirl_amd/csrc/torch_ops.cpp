@@ -627,9 +627,12 @@ struct LossCfg {
   bool kl_st;
 };
 
+bool is_cov_loss(int64_t loss_mode) { return loss_mode == SIIRL_LOSS_KL_COV || loss_mode == SIIRL_LOSS_CLIP_COV; }
+
 void policy_loss_fwd_launch(const Tensor& old, const Tensor& lp, const Tensor& adv, const Tensor& mask,
                             const optional<Tensor>& isw, const optional<Tensor>& ent, const optional<Tensor>& ref,
-                            const LossCfg& c, float* out16, float* row_msum, float* row_s, void* ws, size_t nws) {
+                            const optional<Tensor>& aux, const LossCfg& c, float* out16, float* row_msum, float* row_s,
+                            void* ws, size_t nws) {
   require_f32c(lp, "log_prob");
   require_f32c(old, "old_log_prob");
   require_f32c(adv, "advantages");
@@ -643,8 +646,19 @@ void policy_loss_fwd_launch(const Tensor& old, const Tensor& lp, const Tensor& a
   require_f32_like(ent, lp, "entropy");
   require_f32_like(ref, lp, "ref_log_prob");
   require_mask(mask, lp);
+  require_f32_like(aux, lp, "token_aux");
+  TORCH_CHECK_VALUE(has(aux) == is_cov_loss(c.loss_mode), "siirl_amd: token_aux goes with the kl_cov and clip_cov losses");
   const int64_t B = lp.size(0), L = lp.size(1);
   DeviceGuard guard(lp.device());
+  if (has(aux)) {
+    check_rc(siirl_actor_loss_cov_fwd(ptr<float>(old), ptr<float>(lp), ptr<float>(adv), ptr(mask), mask_code(mask),
+                                      ptr<float>(isw), ptr<float>(ent), ptr<float>(ref), ptr<float>(aux), B, L,
+                                      (int)c.loss_mode, (float)c.clip_low, (float)c.clip_high, (int)c.agg_mode,
+                                      (float)c.entropy_coeff, (int)c.kl_mode, (int)c.kl_st, (float)c.kl_coef,
+                                      (float)c.drift_coef, (float)c.scale, out16, row_msum, ws, nws, stream_of(lp)),
+             "siirl_actor_loss_cov_fwd");
+    return;
+  }
   check_rc(siirl_actor_loss_fwd(ptr<float>(old), ptr<float>(lp), ptr<float>(adv), ptr(mask), mask_code(mask),
                                 ptr<float>(isw), ptr<float>(ent), ptr<float>(ref), B, L, (int)c.loss_mode,
                                 (float)c.clip_low, (float)c.clip_high, (float)c.clip_c, (float)c.log_ratio_clamp,
@@ -656,13 +670,13 @@ void policy_loss_fwd_launch(const Tensor& old, const Tensor& lp, const Tensor& a
 std::tuple<Tensor, Tensor, Tensor> policy_loss_fwd_impl(const Tensor& old, const Tensor& lp, const Tensor& adv,
                                                         const Tensor& mask, const optional<Tensor>& isw,
                                                         const optional<Tensor>& ent, const optional<Tensor>& ref,
-                                                        const LossCfg& c) {
+                                                        const optional<Tensor>& aux, const LossCfg& c) {
   TORCH_CHECK_VALUE(lp.dim() == 2, "log_prob must be [B, L]");
   const int64_t B = lp.size(0), L = lp.size(1);
   Tensor out16 = empty_f32({16}, lp), row_msum = empty_f32({B}, lp), row_s = empty_f32({B}, lp);
   size_t nws;
   Tensor ws = loss_workspace(B, L, lp, &nws);
-  policy_loss_fwd_launch(old, lp, adv, mask, isw, ent, ref, c, ptr<float>(out16), ptr<float>(row_msum),
+  policy_loss_fwd_launch(old, lp, adv, mask, isw, ent, ref, aux, c, ptr<float>(out16), ptr<float>(row_msum),
                          ptr<float>(row_s), ptr(ws), nws);
   return {out16, row_msum, row_s};
 }
@@ -670,8 +684,8 @@ std::tuple<Tensor, Tensor, Tensor> policy_loss_fwd_impl(const Tensor& old, const
 std::tuple<Tensor, Tensor> policy_loss_bwd_impl(const Tensor& g, const Tensor& old, const Tensor& lp, const Tensor& adv,
                                                 const Tensor& mask, const optional<Tensor>& isw,
                                                 const optional<Tensor>& ent, const optional<Tensor>& ref,
-                                                const LossCfg& c, const Tensor& out16, const Tensor& row_msum,
-                                                const Tensor& row_s) {
+                                                const optional<Tensor>& aux, const LossCfg& c, const Tensor& out16,
+                                                const Tensor& row_msum, const Tensor& row_s) {
   require_f32c(lp, "log_prob");
   require_f32c(g, "g_loss");
   require_f32c(old, "old_log_prob");
@@ -691,10 +705,23 @@ std::tuple<Tensor, Tensor> policy_loss_bwd_impl(const Tensor& g, const Tensor& o
   require_f32_n(out16, 16, lp, "out16");
   require_f32_n(row_msum, B, lp, "row_msum");
   require_f32_n(row_s, B, lp, "row_s");
+  require_f32_like(aux, lp, "token_aux");
+  TORCH_CHECK_VALUE(has(aux) == is_cov_loss(c.loss_mode), "siirl_amd: token_aux goes with the kl_cov and clip_cov losses");
   Tensor d_lp = empty_f32({B, L}, lp);
   const std::vector<int64_t> full{B, L}, none{0};
   Tensor d_ent = empty_f32(has(ent) ? at::IntArrayRef(full) : at::IntArrayRef(none), lp);
   DeviceGuard guard(lp.device());
+  if (has(aux)) {
+    check_rc(siirl_actor_loss_cov_bwd(ptr<float>(g), ptr<float>(old), ptr<float>(lp), ptr<float>(adv), ptr(mask),
+                                      mask_code(mask), ptr<float>(isw), ptr<float>(ent), ptr<float>(ref),
+                                      ptr<float>(aux), B, L, (int)c.loss_mode, (float)c.clip_low, (float)c.clip_high,
+                                      (int)c.agg_mode, (float)c.entropy_coeff, (int)c.kl_mode, (int)c.kl_st,
+                                      (float)c.kl_coef, (float)c.drift_coef, (float)c.scale, ptr<float>(out16),
+                                      ptr<float>(row_msum), ptr<float>(d_lp), has(ent) ? ptr<float>(d_ent) : nullptr,
+                                      stream_of(lp)),
+             "siirl_actor_loss_cov_bwd");
+    return {d_lp, d_ent};
+  }
   check_rc(siirl_actor_loss_bwd(ptr<float>(g), ptr<float>(old), ptr<float>(lp), ptr<float>(adv), ptr(mask),
                                 mask_code(mask), ptr<float>(isw), ptr<float>(ent), ptr<float>(ref), B, L,
                                 (int)c.loss_mode, (float)c.clip_low, (float)c.clip_high, (float)c.clip_c,
@@ -712,8 +739,8 @@ std::tuple<Tensor, Tensor, Tensor> policy_loss_fwd(const Tensor& old, const Tens
                                                    int64_t loss_mode, double clip_low, double clip_high, double clip_c,
                                                    double log_ratio_clamp, int64_t agg_mode, double entropy_coeff,
                                                    int64_t kl_mode, bool kl_st, double kl_coef, double drift_coef,
-                                                   double scale) {
-  return policy_loss_fwd_impl(old, lp, adv, mask, isw, ent, ref,
+                                                   double scale, const optional<Tensor>& aux) {
+  return policy_loss_fwd_impl(old, lp, adv, mask, isw, ent, ref, aux,
                               LossCfg{loss_mode, agg_mode, kl_mode, clip_low, clip_high, clip_c, log_ratio_clamp,
                                       entropy_coeff, kl_coef, drift_coef, scale, kl_st});
 }
@@ -724,11 +751,34 @@ std::tuple<Tensor, Tensor> policy_loss_bwd(const Tensor& g, const Tensor& old, c
                                            double clip_high, double clip_c, double log_ratio_clamp, int64_t agg_mode,
                                            double entropy_coeff, int64_t kl_mode, bool kl_st, double kl_coef,
                                            double drift_coef, double scale, const Tensor& out16, const Tensor& row_msum,
-                                           const Tensor& row_s) {
-  return policy_loss_bwd_impl(g, old, lp, adv, mask, isw, ent, ref,
+                                           const Tensor& row_s, const optional<Tensor>& aux) {
+  return policy_loss_bwd_impl(g, old, lp, adv, mask, isw, ent, ref, aux,
                               LossCfg{loss_mode, agg_mode, kl_mode, clip_low, clip_high, clip_c, log_ratio_clamp,
                                       entropy_coeff, kl_coef, drift_coef, scale, kl_st},
                               out16, row_msum, row_s);
+}
+
+// Scores that the covariance losses pick their tokens from: (cov [B, L], stats {count of mask > 0, sum of the mask,
+// mean advantage, mean log-prob}).  No gradient: the pick is a set of indices.
+std::tuple<Tensor, Tensor> cov_scores(const optional<Tensor>& old, const Tensor& lp, const Tensor& adv, const Tensor& mask,
+                                      int64_t loss_mode, double clip_low, double clip_high) {
+  require_f32c(lp, "log_prob");
+  TORCH_CHECK_VALUE(lp.dim() == 2, "log_prob must be [B, L]");
+  require_f32_like(adv, lp, "advantages");
+  require_f32_like(old, lp, "old_log_prob");
+  require_mask(mask, lp);
+  TORCH_CHECK_VALUE(is_cov_loss(loss_mode), "siirl_amd: covariance scores belong to the kl_cov and clip_cov losses");
+  TORCH_CHECK_VALUE(loss_mode != SIIRL_LOSS_CLIP_COV || has(old), "siirl_amd: clip_cov needs old_log_prob");
+  const int64_t B = lp.size(0), L = lp.size(1);
+  Tensor cov = at::empty_like(lp), stats = empty_f32({4}, lp);
+  const size_t nws = siirl_cov_workspace_bytes();
+  Tensor ws = at::empty({(int64_t)nws}, lp.options().dtype(at::kByte));
+  DeviceGuard guard(lp.device());
+  check_rc(siirl_cov_scores(ptr<float>(old), ptr<float>(lp), ptr<float>(adv), ptr(mask), mask_code(mask), B, L,
+                            (int)loss_mode, (float)clip_low, (float)clip_high, ptr<float>(cov), ptr<float>(stats),
+                            ptr(ws), nws, stream_of(lp)),
+           "siirl_cov_scores");
+  return {cov, stats};
 }
 
 constexpr int kActorOuts = 13;  // SIIRL_OUT_LOSS .. SIIRL_OUT_DRIFT_LOSS
@@ -742,7 +792,8 @@ struct ActorLossFn : public torch::autograd::Function<ActorLossFn> {
                                const optional<Tensor>& is_weights, const optional<Tensor>& ref_log_prob,
                                int64_t loss_mode, double clip_low, double clip_high, double clip_c,
                                double log_ratio_clamp, int64_t agg_mode, double entropy_coeff, int64_t kl_mode,
-                               bool kl_st, double kl_coef, double drift_coef, double scale, bool policy_only) {
+                               bool kl_st, double kl_coef, double drift_coef, double scale, bool policy_only,
+                               const optional<Tensor>& token_aux) {
     at::AutoDispatchBelowADInplaceOrView below;
     require_gpu(log_prob, "log_prob");
     const auto dev = log_prob.device();
@@ -750,10 +801,11 @@ struct ActorLossFn : public torch::autograd::Function<ActorLossFn> {
     const auto shape = lp.sizes();
     Tensor old = as_2d(f32c(old_log_prob, dev)), adv = as_2d(f32c(advantages, dev));
     Tensor m = as_2d(mask_arg(response_mask, dev));
-    optional<Tensor> isw, ent, ref;
+    optional<Tensor> isw, ent, ref, aux;
     if (has(is_weights)) isw = as_2d(f32c(*is_weights, dev));
     if (has(entropy)) ent = as_2d(f32c(*entropy, dev));
     if (has(ref_log_prob)) ref = as_2d(f32c(*ref_log_prob, dev));
+    if (has(token_aux)) aux = as_2d(f32c(*token_aux, dev));
     auto same = [&](const Tensor& t, const char* name) {
       TORCH_CHECK_VALUE(t.sizes() == shape, name, " has shape ", t.sizes(), ", expected ", shape);
     };
@@ -763,6 +815,7 @@ struct ActorLossFn : public torch::autograd::Function<ActorLossFn> {
     if (isw) same(*isw, "rollout_is_weights");
     if (ent) same(*ent, "entropy");
     if (ref) same(*ref, "ref_log_prob");
+    if (aux) same(*aux, "token_aux");
     const LossCfg c{loss_mode, agg_mode, kl_mode, clip_low, clip_high, clip_c, log_ratio_clamp, entropy_coeff,
                     kl_coef, drift_coef, scale, kl_st};
     // one allocation for the result block, the two per-row vectors kept for the backward, and the scratch
@@ -773,10 +826,10 @@ struct ActorLossFn : public torch::autograd::Function<ActorLossFn> {
     const int64_t head = (64 + 2 * B + 63) / 64 * 64;  // floats before the workspace
     Tensor buf = empty_f32({head + (int64_t)((nws + 3) / 4)}, lp);
     Tensor out16 = buf.narrow(0, 0, 16), row_msum = buf.narrow(0, 64, B), row_s = buf.narrow(0, 64 + B, B);
-    policy_loss_fwd_launch(old, lp, adv, m, isw, ent, ref, c, ptr<float>(out16), ptr<float>(row_msum),
+    policy_loss_fwd_launch(old, lp, adv, m, isw, ent, ref, aux, c, ptr<float>(out16), ptr<float>(row_msum),
                            ptr<float>(row_s), ptr<float>(buf) + head, nws);
     ctx->save_for_backward({lp, old, adv, m, out16, row_msum, row_s, isw ? *isw : Tensor(), ent ? *ent : Tensor(),
-                            ref ? *ref : Tensor()});
+                            ref ? *ref : Tensor(), aux ? *aux : Tensor()});
     ctx->saved_data["i"] = std::vector<int64_t>{loss_mode, agg_mode, kl_mode, (int64_t)kl_st, (int64_t)policy_only,
                                                 (int64_t)log_prob.scalar_type(),
                                                 has(entropy) ? (int64_t)entropy->scalar_type() : -1};
@@ -800,17 +853,18 @@ struct ActorLossFn : public torch::autograd::Function<ActorLossFn> {
     const auto dv = ctx->saved_data["d"].toDoubleVector();
     const bool policy_only = iv[4] != 0;
     const Tensor& g_in = grads[policy_only ? SIIRL_OUT_PG_LOSS : SIIRL_OUT_LOSS];
-    variable_list none(20);
+    variable_list none(21);
     if (!g_in.defined()) return none;
     const auto s = ctx->get_saved_variables();
     at::AutoDispatchBelowADInplaceOrView below;
     const LossCfg c{iv[0], iv[1], iv[2], dv[0], dv[1], dv[2], dv[3], dv[4], dv[5], dv[6], dv[7], iv[3] != 0};
-    optional<Tensor> isw, ent, ref;
+    optional<Tensor> isw, ent, ref, aux;
     if (s[7].defined()) isw = s[7];
     if (s[8].defined()) ent = s[8];
     if (s[9].defined()) ref = s[9];
-    auto [d_lp, d_ent] = policy_loss_bwd_impl(scalar_grad(g_in), s[1], s[0], s[2], s[3], isw, ent, ref, c, s[4], s[5],
-                                              s[6]);
+    if (s[10].defined()) aux = s[10];
+    auto [d_lp, d_ent] = policy_loss_bwd_impl(scalar_grad(g_in), s[1], s[0], s[2], s[3], isw, ent, ref, aux, c, s[4],
+                                              s[5], s[6]);
     d_lp = d_lp.reshape(ctx->saved_data["lp_shape"].toIntVector());
     if ((at::ScalarType)iv[5] != at::kFloat) d_lp = d_lp.to((at::ScalarType)iv[5]);
     none[0] = d_lp;
@@ -828,10 +882,11 @@ std::vector<Tensor> actor_loss(const Tensor& log_prob, const optional<Tensor>& e
                                const optional<Tensor>& is_weights, const optional<Tensor>& ref_log_prob,
                                int64_t loss_mode, double clip_low, double clip_high, double clip_c,
                                double log_ratio_clamp, int64_t agg_mode, double entropy_coeff, int64_t kl_mode,
-                               bool kl_st, double kl_coef, double drift_coef, double scale, bool policy_only) {
+                               bool kl_st, double kl_coef, double drift_coef, double scale, bool policy_only,
+                               const optional<Tensor>& token_aux) {
   return ActorLossFn::apply(log_prob, entropy, old_log_prob, advantages, response_mask, is_weights, ref_log_prob,
                             loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff, kl_mode,
-                            kl_st, kl_coef, drift_coef, scale, policy_only);
+                            kl_st, kl_coef, drift_coef, scale, policy_only, token_aux);
 }
 
 // ------------------------------------------------------------------ value loss
@@ -1120,12 +1175,14 @@ TORCH_LIBRARY(siirl_hip, m) {
   m.def("policy_loss_fwd(Tensor old_log_prob, Tensor log_prob, Tensor advantages, Tensor mask, Tensor? is_weights, "
         "Tensor? entropy, Tensor? ref_log_prob, int loss_mode, float clip_low, float clip_high, float clip_c, "
         "float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode, bool kl_straight_through, "
-        "float kl_coef, float policy_drift_coeff, float loss_scale) -> (Tensor, Tensor, Tensor)");
+        "float kl_coef, float policy_drift_coeff, float loss_scale, Tensor? token_aux=None) -> (Tensor, Tensor, Tensor)");
   m.def("policy_loss_bwd(Tensor g_loss, Tensor old_log_prob, Tensor log_prob, Tensor advantages, Tensor mask, "
         "Tensor? is_weights, Tensor? entropy, Tensor? ref_log_prob, int loss_mode, float clip_low, float clip_high, "
         "float clip_c, float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode, "
         "bool kl_straight_through, float kl_coef, float policy_drift_coeff, float loss_scale, Tensor out16, "
-        "Tensor row_msum, Tensor row_s) -> (Tensor, Tensor)");
+        "Tensor row_msum, Tensor row_s, Tensor? token_aux=None) -> (Tensor, Tensor)");
+  m.def("cov_scores(Tensor? old_log_prob, Tensor log_prob, Tensor advantages, Tensor mask, int loss_mode, "
+        "float clip_low, float clip_high) -> (Tensor, Tensor)");
   m.def("kl_penalty_fwd(Tensor log_prob, Tensor ref_log_prob, int kl_mode) -> Tensor");
   m.def("kl_penalty_bwd(Tensor g, Tensor log_prob, Tensor ref_log_prob, int kl_mode, bool straight_through, "
         "bool need_log_prob, bool need_ref) -> (Tensor, Tensor)");
@@ -1142,7 +1199,8 @@ TORCH_LIBRARY(siirl_hip, m) {
   m.def("actor_loss(Tensor log_prob, Tensor? entropy, Tensor old_log_prob, Tensor advantages, Tensor response_mask, "
         "Tensor? is_weights, Tensor? ref_log_prob, int loss_mode, float clip_low, float clip_high, float clip_c, "
         "float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode, bool kl_straight_through, "
-        "float kl_coef, float policy_drift_coeff, float loss_scale, bool policy_only) -> Tensor[]", &actor_loss);
+        "float kl_coef, float policy_drift_coeff, float loss_scale, bool policy_only, Tensor? token_aux=None) -> Tensor[]",
+        &actor_loss);
   m.def("agg_loss(Tensor loss_mat, Tensor loss_mask, int agg_mode) -> Tensor", &agg_loss);
   m.def("masked_reduce(Tensor values, Tensor mask, int[] axes, bool want_mean) -> Tensor", &masked_reduce);
   m.def("value_loss(Tensor vpreds, Tensor returns, Tensor values, Tensor response_mask, float cliprange_value, "
@@ -1164,6 +1222,7 @@ TORCH_LIBRARY_IMPL(siirl_hip, CUDA, m) {
   m.impl("masked_reduce_bwd", &masked_reduce_bwd);
   m.impl("policy_loss_fwd", &policy_loss_fwd);
   m.impl("policy_loss_bwd", &policy_loss_bwd);
+  m.impl("cov_scores", &cov_scores);
   m.impl("kl_penalty_fwd", &kl_penalty_fwd);
   m.impl("kl_penalty_bwd", &kl_penalty_bwd);
   m.impl("fused_linear_logprob_entropy_fwd", &fused_linear_fwd);

@@ -122,7 +122,7 @@ def _(g, mask, per_row, mask_sums):
 @_fake(f"{_NS}::policy_loss_fwd")
 def _(old_log_prob, log_prob, advantages, mask, is_weights, entropy, ref_log_prob, loss_mode, clip_low, clip_high,
       clip_c, log_ratio_clamp, agg_mode, entropy_coeff, kl_mode, kl_straight_through, kl_coef, policy_drift_coeff,
-      loss_scale):
+      loss_scale, token_aux=None):
     B = log_prob.shape[0]
     mk = lambda n: log_prob.new_empty(n, dtype=torch.float32)  # noqa: E731
     return mk(16), mk(B), mk(B)
@@ -131,9 +131,14 @@ def _(old_log_prob, log_prob, advantages, mask, is_weights, entropy, ref_log_pro
 @_fake(f"{_NS}::policy_loss_bwd")
 def _(g_loss, old_log_prob, log_prob, advantages, mask, is_weights, entropy, ref_log_prob, loss_mode, clip_low,
       clip_high, clip_c, log_ratio_clamp, agg_mode, entropy_coeff, kl_mode, kl_straight_through, kl_coef,
-      policy_drift_coeff, loss_scale, out16, row_msum, row_s):
+      policy_drift_coeff, loss_scale, out16, row_msum, row_s, token_aux=None):
     return (log_prob.new_empty(log_prob.shape, dtype=torch.float32),
             log_prob.new_empty(log_prob.shape if entropy is not None else (0,), dtype=torch.float32))
+
+
+@_fake(f"{_NS}::cov_scores")
+def _(old_log_prob, log_prob, advantages, mask, loss_mode, clip_low, clip_high):
+    return log_prob.new_empty(log_prob.shape, dtype=torch.float32), log_prob.new_empty(4, dtype=torch.float32)
 
 
 @_fake(f"{_NS}::kl_penalty_fwd")

@@ -47,7 +47,7 @@ def test_every_entry_point_cites_the_reference():
             assert "no counterpart in the reference" in text[text.rfind("/*", 0, pos):pos]
             continue
         if n in ("siirl_hip_abi_version", "siirl_hip_last_error", "siirl_agg_loss_bwd", "siirl_actor_loss_bwd",
-                 "siirl_kl_penalty_bwd", "siirl_masked_reduce_bwd") or n.endswith("_workspace_bytes") or n.endswith("_logits_bytes"):
+                 "siirl_kl_penalty_bwd", "siirl_masked_reduce_bwd", "siirl_actor_loss_cov_bwd") or n.endswith("_workspace_bytes") or n.endswith("_logits_bytes"):
             continue  # utilities and backward halves documented with their forward
         pos = text.index(n + "(")
         comment = text[text.rfind("/*", 0, pos):pos]
@@ -85,6 +85,23 @@ def test_argument_validation_without_gpu():
     assert h.siirl_actor_loss_fwd_static(p, p, p, p, L.F32, None, None, None, 1 << 20, 4096, 0, 0.2, 0.2, 3.0, 20.0, 0,
                                          0.0, 0, 0, 0.0, 0.0, 1.0, p, p, p, None) == -4
     assert b"static buffer" in h.siirl_hip_last_error()
+    # the covariance losses: their two modes go through their own entry points and nowhere else
+    assert h.siirl_actor_loss_fwd(p, p, p, p, L.F32, None, None, None, 2, 4, 5, 0.2, 0.2, 3.0, 20.0, 0, 0.0, 0, 0, 0.0,
+                                  0.0, 1.0, p, p, p, p, 1 << 20, None) == -1
+    assert b"Unsupported loss mode" in h.siirl_hip_last_error()
+    assert h.siirl_actor_loss_cov_fwd(p, p, p, p, L.F32, None, None, None, p, 2, 4, 0, 0.2, 0.2, 0, 0.0, 0, 0, 0.0, 0.0,
+                                      1.0, p, p, p, 1 << 20, None) == -1
+    assert b"per-token selection" in h.siirl_hip_last_error()
+    assert h.siirl_actor_loss_cov_fwd(p, p, p, p, L.F32, None, None, None, None, 2, 4, 5, 0.2, 0.2, 0, 0.0, 0, 0, 0.0,
+                                      0.0, 1.0, p, p, p, 1 << 20, None) == -1
+    assert b"token_aux" in h.siirl_hip_last_error()
+    assert h.siirl_actor_loss_cov_bwd(p, p, p, p, p, L.F32, None, None, None, p, 2, 4, 6, 0.2, 0.2, 9, 0.0, 0, 0, 0.0,
+                                      0.0, 1.0, p, p, p, None, None) == -1
+    assert h.siirl_cov_scores(p, p, p, p, L.F32, 2, 4, 0, 0.2, 0.2, p, p, p, 1 << 20, None) == -1
+    assert b"kl_cov and clip_cov" in h.siirl_hip_last_error()
+    assert h.siirl_cov_scores(None, p, p, p, L.F32, 2, 4, 6, 0.2, 0.2, p, p, p, 1 << 20, None) == -1  # clip_cov: old
+    assert h.siirl_cov_scores(p, p, p, p, L.F32, 2, 4, 6, 0.2, 0.2, p, p, p, 8, None) == -4
+    assert h.siirl_cov_workspace_bytes() > 0
     assert h.siirl_value_loss_fwd(p, p, p, p, L.F32, 2, 4, 0.5, 7, p, p, p, 1 << 20, None) == -1
     assert h.siirl_gae_advantage_return(p, p, p, L.F32, 2, 4, 1.0, 1.0, p, p, p, p, 8, 0, None) == -1  # adv == returns
     q2 = ctypes.c_void_p(p.value + 64)

@@ -6,7 +6,8 @@ import torch
 import siirl_amd.ops  # noqa: F401  (registers the ops)
 
 OPS = ("logprob_entropy_fwd", "logprob_entropy_bwd", "logprob_entropy_bwd_", "grpo_advantage", "group_keep_mask",
-       "agg_loss_fwd", "agg_loss_bwd", "masked_reduce_fwd", "masked_reduce_bwd", "policy_loss_fwd", "policy_loss_bwd", "kl_penalty_fwd", "kl_penalty_bwd",
+       "agg_loss_fwd", "agg_loss_bwd", "masked_reduce_fwd", "masked_reduce_bwd", "policy_loss_fwd", "policy_loss_bwd",
+       "cov_scores", "kl_penalty_fwd", "kl_penalty_bwd",
        "fused_linear_logprob_entropy_fwd", "fused_linear_logprob_entropy_bwd")
 
 
@@ -61,6 +62,13 @@ def test_fake_kernels_give_shapes_without_a_gpu(with_optional):
         r, ms = ns.masked_reduce_fwd(mk((B, L), torch.float32), mk((B, L), torch.int64), False, False)
         assert r.shape == (2,) and ms.shape == (1,)
         assert ns.masked_reduce_bwd(mk((B,), torch.float32), mk((B, L), torch.bool), True, None).shape == (B, L)
+        cov, stats = ns.cov_scores(mk((B, L), torch.float32), mk((B, L), torch.float32), mk((B, L), torch.float32),
+                                   mk((B, L), torch.int64), 6, 0.2, 0.28)
+        assert cov.shape == (B, L) and stats.shape == (4,) and cov.dtype == torch.float32
+        a5 = list(_loss_args(mk, B, L, with_optional))
+        a5[7] = 5
+        o5, _, _ = ns.policy_loss_fwd(*a5, mk((B, L), torch.float32))
+        assert o5.shape == (16,)
         assert ns.kl_penalty_fwd(mk((B, L), torch.float32), mk((B, L), torch.float32), 3).shape == (B, L)
         d1, d2 = ns.kl_penalty_bwd(mk((B, L), torch.float32), mk((B, L), torch.float32), mk((B, L), torch.float32), 3,
                                    False, True, False)
@@ -98,6 +106,13 @@ def test_opcheck_on_the_gpu():
     torch.library.opcheck(ns.policy_loss_bwd, (torch.ones(1, device=dev), *args, out16, row_msum, row_s), test_utils=checks)
     lm, m = mk((B, L), torch.float32), torch.ones(B, L, dtype=torch.bool, device=dev)
     torch.library.opcheck(ns.agg_loss_fwd, (lm, m, 2), test_utils=checks)
+    torch.library.opcheck(ns.cov_scores, (lm, mk((B, L), torch.float32), mk((B, L), torch.float32), m, 6, 0.2, 0.28),
+                          test_utils=checks)
+    torch.library.opcheck(ns.cov_scores, (None, mk((B, L), torch.float32), mk((B, L), torch.float32), m, 5, 0.0, 0.0),
+                          test_utils=checks)
+    cov_args = list(args)
+    cov_args[7] = 5
+    torch.library.opcheck(ns.policy_loss_fwd, (*cov_args, mk((B, L), torch.float32)), test_utils=checks)
     torch.library.opcheck(ns.kl_penalty_fwd, (lm, mk((B, L), torch.float32), 3), test_utils=checks)
     torch.library.opcheck(ns.masked_reduce_fwd, (lm, m, True, True), test_utils=checks)
     torch.library.opcheck(ns.masked_reduce_fwd, (lm, m, False, True), test_utils=checks)

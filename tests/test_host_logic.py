@@ -11,9 +11,10 @@ import torch
 def test_registries_mirror_the_reference():
     import siirl_amd.core_algos as CA
 
-    assert set(CA.POLICY_LOSS_REGISTRY) >= {"vanilla", "gspo"}
-    with pytest.raises(ValueError, match=r"Unsupported loss mode: kl_cov. Supported modes are: \["):
-        CA.get_policy_loss_fn("kl_cov")
+    # every name the reference registers (core_algos.py:572,710,795,865,898,998,1074)
+    assert set(CA.POLICY_LOSS_REGISTRY) == {"vanilla", "gspo", "cpgd", "gpg", "clip_cov", "kl_cov", "geo_mean"}
+    with pytest.raises(ValueError, match=r"Unsupported loss mode: reinforce. Supported modes are: \["):
+        CA.get_policy_loss_fn("reinforce")
 
     @CA.register_policy_loss("mine")
     def mine(*a, **k):

@@ -341,9 +341,11 @@ def kl_cov_selection(log_prob, advantages, response_mask, kl_cov_ratio):
 
 
 def compute_policy_loss_kl_cov(old_log_prob, log_prob, advantages, response_mask, loss_agg_mode="token-mean",
-                               config=None, rollout_is_weights=None):
+                               config=None, rollout_is_weights=None, chosen=None):
     """KL-Cov (reference ``core_algos.py:998-1071``): the unclipped surrogate ``-A * ratio``; the tokens selected by
-    ``kl_cov_selection`` additionally pay ``ppo_kl_coef * |lp - old|``.  Returns ``(pg_loss, 0, masked_mean(|lp - old|), 0)``."""
+    ``kl_cov_selection`` additionally pay ``ppo_kl_coef * |lp - old|``.  Returns ``(pg_loss, 0, masked_mean(|lp - old|), 0)``.
+    ``chosen`` (flat indices) overrides the selection: for checks of the arithmetic in another precision than the
+    one the selection was made in (two tokens of equal covariance sort differently in float32 and float64)."""
     assert config is not None and config.policy_loss is not None
     pl = config.policy_loss
     kl_cov_ratio = pl.kl_cov_ratio if pl.kl_cov_ratio is not None else 0.0002
@@ -356,7 +358,8 @@ def compute_policy_loss_kl_cov(old_log_prob, log_prob, advantages, response_mask
     ppo_kl_abs = masked_mean(abs_kl, response_mask)
     plain = -advantages * ratio
     with_kl = -advantages * ratio + coef * abs_kl
-    chosen, _ = kl_cov_selection(log_prob, advantages, response_mask, kl_cov_ratio)
+    if chosen is None:
+        chosen, _ = kl_cov_selection(log_prob, advantages, response_mask, kl_cov_ratio)
     pick = torch.zeros(advantages.numel(), dtype=torch.bool)
     pick[chosen] = True
     tok = torch.where(pick.reshape(advantages.shape), with_kl, plain)

@@ -32,8 +32,8 @@ def _case(seed, B, L, mask_dtype=torch.int64, spread=0.05):
     return old, lp, A, m.to(mask_dtype), w
 
 
-def _close(a, b, rtol=1e-5, atol=1e-6):
-    assert abs(float(a) - float(b)) <= atol + rtol * abs(float(b)), (float(a), float(b))
+def _close(a, b, rtol=1e-5, atol=1e-6, what=None):
+    assert abs(float(a) - float(b)) <= atol + rtol * abs(float(b)), (float(a), float(b), what)
 
 
 @pytest.mark.parametrize("agg", O.AGG_MODES)
@@ -53,7 +53,8 @@ def test_kl_cov_matches_oracle(agg, B, L, mask_dtype, with_w):
     assert torch.all(aux.reshape(-1)[got_idx.to(DEV)] == 0.8)
 
     lp64 = lp.double().requires_grad_(True)
-    want = O.compute_policy_loss_kl_cov(old.double(), lp64, A.double(), mf, agg, cfg, w.double() if with_w else None)
+    want = O.compute_policy_loss_kl_cov(old.double(), lp64, A.double(), mf, agg, cfg, w.double() if with_w else None,
+                                        chosen=want_idx)
     (gwant,) = torch.autograd.grad(want[0], lp64)
     lpd = lp.to(DEV).requires_grad_(True)
     got = CA.compute_policy_loss_kl_cov(old.to(DEV), lpd, A.to(DEV), m.to(DEV), agg, cfg, w.to(DEV) if with_w else None)
@@ -183,6 +184,8 @@ def test_actor_loss_with_covariance_losses(mode):
     kw = {}
     if mode == "clip_cov":
         _, kw["dropped"] = _oracle_dropped(old, lp, A, m, cfg, 0.2, 0.28, seed=21)
+    else:
+        kw["chosen"], _ = O.kl_cov_selection(lp, A, m.to(torch.float32), 0.03)
     fn = O.compute_policy_loss_clip_cov if mode == "clip_cov" else O.compute_policy_loss_kl_cov
     pg, frac, kl, _ = fn(old.double(), lp64, A.double(), m.double(), cfg.loss_agg_mode, cfg, w.double(), **kw)
     total = (pg - 0.01 * O.agg_loss(ent64, m.double(), cfg.loss_agg_mode)
@@ -248,3 +251,74 @@ def test_cpgd_outcome_advantage(mode, on_host):
     assert torch.allclose(got.cpu().double(), want, rtol=1e-5, atol=1e-6)
     with pytest.raises(NotImplementedError):
         CA.compute_cpgd_outcome_advantage(r, mk, uid, weight_factor_in_cpgd="other")
+
+
+def test_sweep_covariance_losses():
+    """Seeded random shapes, mask dtypes (weighted float masks included), aggregation modes, bounds and quotas through
+    both losses; the picks must equal the float32 oracle's, loss and gradient the float64 oracle's.
+    ``SIIRL_TEST_SEED=<int>`` shifts the seeds."""
+    import os
+    import random
+
+    import siirl_amd.core_algos as CA
+
+    shift = 100003 * int(os.environ.get("SIIRL_TEST_SEED", "0"))
+    for case in range(60):
+        rnd = random.Random(7000 + case + shift)
+        B, L = rnd.randint(1, 24), rnd.choice((1, 3, 4, 17, 64, 129, 256, 2049))
+        mdt = rnd.choice((torch.int64, torch.bool, torch.int32, torch.float32, torch.bfloat16))
+        old, lp, A, m, w = _case(9000 + case + shift, B, L, torch.float32, spread=rnd.choice((0.02, 0.1, 0.3)))
+        if mdt in (torch.float32, torch.bfloat16) and case % 2:
+            m = m * torch.tensor([0.5, 1.0, 2.0])[torch.randint(0, 3, m.shape, generator=torch.Generator().manual_seed(case))]
+        m = m.to(mdt)
+        agg = rnd.choice(O.AGG_MODES)
+        with_w = rnd.random() < 0.5
+        mf = m.to(torch.float64)
+        # KL-Cov
+        ratio, coef = rnd.choice((0.0002, 0.01, 0.2)), rnd.choice((1.0, 0.3))
+        cfg = _cfg(kl_cov_ratio=ratio, ppo_kl_coef=coef)
+        want_idx, cov32 = O.kl_cov_selection(lp, A, m.to(torch.float32), ratio)
+        aux = CA._kl_cov_weights(lp.to(DEV), A.to(DEV), m.to(DEV), ratio, coef)
+        got_idx = sorted(torch.nonzero(aux.reshape(-1)).reshape(-1).tolist())
+        if sorted(want_idx.tolist()) != got_idx:
+            # allowed only when the cut falls between two covariances that float32 rounding cannot tell apart
+            k = len(want_idx)
+            top = torch.sort(cov32, descending=True).values
+            assert k < len(top) and abs(float(top[k - 1] - top[k])) <= 1e-6 * max(1.0, abs(float(top[k]))), (case, B, L)
+            want_idx = torch.tensor(got_idx)  # the device's side of the tie, for the arithmetic below
+        lp64 = lp.double().requires_grad_(True)
+        want = O.compute_policy_loss_kl_cov(old.double(), lp64, A.double(), mf, agg, cfg, w.double() if with_w else None,
+                                            chosen=want_idx)
+        lpd = lp.to(DEV).requires_grad_(True)
+        got = CA.compute_policy_loss_kl_cov(old.to(DEV), lpd, A.to(DEV), m.to(DEV), agg, cfg, w.to(DEV) if with_w else None)
+        if torch.isnan(want[0]):  # seq-mean-token-mean with an empty row
+            assert torch.isnan(got[0]), (case, agg)
+        else:
+            (gwant,) = torch.autograd.grad(want[0], lp64)
+            got[0].backward()
+            info = (case, B, L, str(mdt), agg, with_w, ratio, coef)
+            _close(got[0], want[0], what=info)
+            _close(got[2], want[2], what=info)
+            assert torch.allclose(lpd.grad.cpu().double(), gwant, rtol=1e-5, atol=1e-7), (case, "kl_cov grad")
+        # Clip-Cov
+        pl = dict(clip_cov_ratio=rnd.choice((0.0002, 0.05, 1.0)), clip_cov_lb=rnd.choice((0.1, 1.0)), clip_cov_ub=rnd.choice((2.0, 5.0)))
+        cfg = _cfg(**pl)
+        cov_d, _ = torch.ops.siirl_hip.cov_scores(old.to(DEV), lp.to(DEV), A.to(DEV), m.to(DEV), CA.LOSS_CLIP_COV, 0.2, 0.28)
+        cand_d = torch.nonzero((cov_d < pl["clip_cov_ub"]) & (cov_d > pl["clip_cov_lb"]) & (m.to(DEV) > 0)).cpu()
+        cand, dropped = _oracle_dropped(old, lp, A, m.to(torch.float32), cfg, 0.2, 0.28, seed=case)
+        if not torch.equal(cand, cand_d):
+            continue  # a covariance within rounding of a bound: the two candidate lists differ, so would the draw
+        torch.manual_seed(case)
+        lpd = lp.to(DEV).requires_grad_(True)
+        got = CA.compute_policy_loss_clip_cov(old.to(DEV), lpd, A.to(DEV), m.to(DEV), agg, cfg, w.to(DEV) if with_w else None)
+        lp64 = lp.double().requires_grad_(True)
+        want = O.compute_policy_loss_clip_cov(old.double(), lp64, A.double(), mf, agg, cfg,
+                                              w.double() if with_w else None, dropped=dropped)
+        if torch.isnan(want[0]):
+            assert torch.isnan(got[0]), (case, agg)
+            continue
+        (gwant,) = torch.autograd.grad(want[0], lp64)
+        got[0].backward()
+        for a, b in zip(got, want):
+            _close(a, b, what=(case, B, L, str(mdt), agg, with_w, pl))
+        assert torch.allclose(lpd.grad.cpu().double(), gwant, rtol=1e-5, atol=1e-7), (case, "clip_cov grad")

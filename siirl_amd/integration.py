@@ -8,22 +8,28 @@ tensors of the actor's micro-batch:
 
 * ``logprobs_from_logits``, ``entropy_from_logits``, ``entropy_from_logits_with_chunking``
   (``siirl/engine/actor/dp_actor.py:75-84,179-195,254-260``);
-* ``agg_loss``, ``kl_penalty``, ``compute_policy_loss``, ``compute_policy_loss_vanilla``,
-  ``compute_policy_loss_gspo`` and the two registry entries (``dp_actor.py:453-486``);
+* ``agg_loss``, ``kl_penalty``, ``compute_policy_loss`` and the seven registered policy losses
+  (``compute_policy_loss_vanilla`` / ``_gspo`` / ``_cpgd`` / ``_gpg`` / ``_clip_cov`` / ``_kl_cov`` / ``_geo_mean``) with
+  their registry entries (``dp_actor.py:453-486``).  Three of the reference's own (``clip_cov``, ``kl_cov``,
+  ``geo_mean``) refuse the stock actors' config class (``core_algos.py:940,1031,1104``); the replacements read the
+  same attributes from any config object and have no such check;
 * ``compute_grpo_outcome_advantage`` and ``apply_kl_penalty``, which the reference runs on host tensors
   (``siirl/dag_worker/dagworker.py:542-560``): the replacements stage host inputs to the GPU and return host results.
 
 Deliberately NOT replaced: ``masked_sum`` / ``masked_mean`` / ``masked_var`` / ``masked_whiten``.  The reference's own
-``compute_gae_advantage_return``, ``clip_cov`` and ``kl_cov`` resolve those globals and call them on host tensors,
-where this package's versions raise (no CPU path); import them from ``siirl_amd.torch_functional`` explicitly where the
-tensors are on the GPU.
+``compute_gae_advantage_return`` resolves those globals and calls them on host tensors, where this package's versions
+raise (no CPU path); import them from ``siirl_amd.torch_functional`` explicitly where the tensors are on the GPU.
 """
 
 from __future__ import annotations
 
 TORCH_FUNCTIONAL_NAMES = ("logprobs_from_logits", "entropy_from_logits", "entropy_from_logits_with_chunking")
-CORE_ALGOS_NAMES = ("agg_loss", "kl_penalty", "compute_policy_loss", "compute_policy_loss_vanilla",
-                    "compute_policy_loss_gspo", "compute_grpo_outcome_advantage", "apply_kl_penalty")
+POLICY_LOSSES = {"vanilla": "compute_policy_loss_vanilla", "gspo": "compute_policy_loss_gspo",
+                 "cpgd": "compute_policy_loss_cpgd", "gpg": "compute_policy_loss_gpg",
+                 "clip_cov": "compute_policy_loss_clip_cov", "kl_cov": "compute_policy_loss_kl_cov",
+                 "geo_mean": "compute_policy_loss_geo_mean"}
+CORE_ALGOS_NAMES = ("agg_loss", "kl_penalty", "compute_policy_loss", *POLICY_LOSSES.values(),
+                    "compute_grpo_outcome_advantage", "apply_kl_penalty")
 
 
 def patch_reference(ref_torch_functional, ref_core_algos) -> dict:
@@ -40,7 +46,7 @@ def patch_reference(ref_torch_functional, ref_core_algos) -> dict:
         setattr(ref_core_algos, name, getattr(A, name))
     losses = getattr(ref_core_algos, "POLICY_LOSS_REGISTRY", None)
     if losses is not None:
-        losses.update(vanilla=A.compute_policy_loss_vanilla, gspo=A.compute_policy_loss_gspo)
+        losses.update({mode: getattr(A, fn) for mode, fn in POLICY_LOSSES.items()})
     estimators = getattr(ref_core_algos, "ADV_ESTIMATOR_REGISTRY", None)
     if estimators is not None:
         estimators["grpo"] = A.compute_grpo_outcome_advantage

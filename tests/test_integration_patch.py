@@ -1,6 +1,6 @@
 """The start-up patch of ``siirl_amd.integration``, applied to stand-ins for the reference's two modules (CPU only):
-the actor-side functions and registry entries are replaced, the masked reductions that the reference also calls on
-host tensors (compute_gae_advantage_return -> masked_whiten -> masked_mean, clip_cov, kl_cov) are left alone."""
+the actor-side functions and all seven policy-loss registry entries are replaced, the masked reductions that the
+reference also calls on host tensors (compute_gae_advantage_return -> masked_whiten -> masked_mean) are left alone."""
 import types
 
 import torch
@@ -19,11 +19,12 @@ def _stub_modules():
     for name in ("logprobs_from_logits", "entropy_from_logits", "entropy_from_logits_with_chunking", "masked_sum"):
         setattr(F, name, lambda *a, **k: "reference")
     F.masked_mean, F.masked_whiten = masked_mean, masked_whiten
-    for name in ("agg_loss", "kl_penalty", "compute_policy_loss", "compute_policy_loss_vanilla",
-                 "compute_policy_loss_gspo", "compute_grpo_outcome_advantage", "apply_kl_penalty", "compute_policy_loss_gpg"):
+    modes = ("vanilla", "gspo", "cpgd", "gpg", "clip_cov", "kl_cov", "geo_mean")
+    for name in ("agg_loss", "kl_penalty", "compute_policy_loss", "compute_grpo_outcome_advantage", "apply_kl_penalty",
+                 "compute_value_loss", *(f"compute_policy_loss_{m}" for m in modes)):
         setattr(A, name, lambda *a, **k: "reference")
-    A.POLICY_LOSS_REGISTRY = {"vanilla": A.compute_policy_loss_vanilla, "gspo": A.compute_policy_loss_gspo,
-                              "gpg": A.compute_policy_loss_gpg}
+    A.POLICY_LOSS_REGISTRY = {m: getattr(A, f"compute_policy_loss_{m}") for m in modes}
+    A.POLICY_LOSS_REGISTRY["users_own"] = A.compute_value_loss
     A.ADV_ESTIMATOR_REGISTRY = {"grpo": A.compute_grpo_outcome_advantage, "gae": object()}
     return F, A
 
@@ -34,15 +35,15 @@ def test_patch_replaces_the_actor_side_and_leaves_host_side_reductions():
     from siirl_amd.integration import CORE_ALGOS_NAMES, TORCH_FUNCTIONAL_NAMES, patch_reference
 
     F, A = _stub_modules()
-    gae_before, gpg_before, masked_sum_before = A.ADV_ESTIMATOR_REGISTRY["gae"], A.compute_policy_loss_gpg, F.masked_sum
+    gae_before, own_before, masked_sum_before = A.ADV_ESTIMATOR_REGISTRY["gae"], A.POLICY_LOSS_REGISTRY["users_own"], F.masked_sum
     undo = patch_reference(F, A)
     for name in TORCH_FUNCTIONAL_NAMES:
         assert getattr(F, name) is getattr(SF, name)
     for name in CORE_ALGOS_NAMES:
         assert getattr(A, name) is getattr(CA, name)
-    assert A.POLICY_LOSS_REGISTRY["vanilla"] is CA.compute_policy_loss_vanilla
-    assert A.POLICY_LOSS_REGISTRY["gspo"] is CA.compute_policy_loss_gspo
-    assert A.POLICY_LOSS_REGISTRY["gpg"] is gpg_before
+    for mode in ("vanilla", "gspo", "cpgd", "gpg", "clip_cov", "kl_cov", "geo_mean"):
+        assert A.POLICY_LOSS_REGISTRY[mode] is CA.POLICY_LOSS_REGISTRY[mode] is getattr(CA, f"compute_policy_loss_{mode}")
+    assert A.POLICY_LOSS_REGISTRY["users_own"] is own_before and A.compute_value_loss is own_before
     assert A.ADV_ESTIMATOR_REGISTRY["grpo"] is CA.compute_grpo_outcome_advantage
     assert A.ADV_ESTIMATOR_REGISTRY["gae"] is gae_before
     assert len(undo) == len(TORCH_FUNCTIONAL_NAMES) + len(CORE_ALGOS_NAMES)

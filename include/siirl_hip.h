@@ -289,6 +289,19 @@ int siirl_cov_scores(const float* old_log_prob, const float* log_prob, const flo
                      float* stats, void* workspace, size_t workspace_bytes, siirl_stream_t stream);
 
 /*
+ * marks[i] = value for the k largest of scores[0..n) and 0 for the rest: the selection step of KL-Cov (the
+ * max(1, int(n_valid * kl_cov_ratio)) tokens of largest covariance get the coefficient of their KL term), in place of
+ * torch.topk followed by an indexed assignment.  Radix select over three streaming passes; entries equal to the k-th
+ * largest are taken lowest index first until k are marked; NaN ranks above every number (as for torch.topk), -0 and
+ * +0 are one value.  Deterministic (no atomics on memory).  n < 2^32, 0 <= k <= n; scores and marks must not
+ * overlap.  workspace: siirl_topk_mark_workspace_bytes(), 16-byte aligned.
+ * Replaces: siirl/dag_worker/core_algos.py:1055-1063 (torch.topk(cov, k).indices and the assignment through them).
+ */
+size_t siirl_topk_mark_workspace_bytes(void);
+int siirl_topk_mark(const float* scores, int64_t n, int64_t k, float value, float* marks, void* workspace,
+                    size_t workspace_bytes, siirl_stream_t stream);
+
+/*
  * siirl_actor_loss_fwd for the two covariance losses: the same composition (entropy, KL and drift terms, ratio
  * statistics, loss_scale) around a policy term that takes one more [B, L] fp32 operand, token_aux:
  *   SIIRL_LOSS_KL_COV:   tok = -A * ratio + token_aux * |log_prob - old_log_prob|  (token_aux = ppo_kl_coef on the

@@ -40,6 +40,8 @@ SIGNATURES = {
                                     _i32, _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _p, _p, _p]),
     "siirl_cov_workspace_bytes": (_sz, []),
     "siirl_cov_scores": (_i32, [_p, _p, _p, _p, _i32, _i64, _i64, _i32, _f32, _f32, _p, _p, _p, _sz, _p]),
+    "siirl_topk_mark_workspace_bytes": (_sz, []),
+    "siirl_topk_mark": (_i32, [_p, _i64, _i64, _f32, _p, _p, _sz, _p]),
     "siirl_actor_loss_cov_fwd": (_i32, [_p, _p, _p, _p, _i32, _p, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _i32, _f32,
                                         _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _sz, _p]),
     "siirl_actor_loss_cov_bwd": (_i32, [_p, _p, _p, _p, _p, _i32, _p, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _i32,

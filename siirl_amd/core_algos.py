@@ -559,15 +559,13 @@ def _kl_cov_weights(log_prob, advantages, response_mask, kl_cov_ratio: float, pp
     count ``n``), as the reference's ``len(all_valid_adv)``."""
     dev, _, lp, adv, m = _cov_operands(None, log_prob, advantages, response_mask)
     cov, stats = _OPS.cov_scores(None, lp, adv, m, LOSS_KL_COV, 0.0, 0.0)
-    aux = torch.zeros_like(cov)
     n = int(stats[0].item())
+    k = 0
     if min(kl_cov_ratio, n) != 0:  # reference :1052-1054
         k = max(1, int(n * kl_cov_ratio))
         if k > n:
             raise RuntimeError(f"kl_cov_ratio {kl_cov_ratio} selects {k} of {n} valid tokens")  # torch.topk: k out of range
-        idx = torch.topk(cov.reshape(-1), k, largest=True).indices
-        aux.reshape(-1)[idx] = float(ppo_kl_coef)
-    return aux
+    return _OPS.topk_mark(cov, k, float(ppo_kl_coef))
 
 
 def _clip_cov_dropped(old_log_prob, log_prob, advantages, response_mask, lo, hi, clip_cov_ratio, lb, ub) -> torch.Tensor:
@@ -644,8 +642,9 @@ def compute_policy_loss_kl_cov(old_log_prob: torch.Tensor, log_prob: torch.Tenso
     """KL-Cov (reference ``core_algos.py:998-1071``): the unclipped surrogate ``-A * ratio``; the
     ``max(1, int(n * kl_cov_ratio))`` valid tokens of largest covariance between advantage and log-prob additionally
     pay ``ppo_kl_coef * |log_prob - old_log_prob|``.  ``config.policy_loss`` carries ``kl_cov_ratio`` (0.0002) and
-    ``ppo_kl_coef`` (1.0).  Returns ``(pg_loss, 0, masked_mean(|log_prob - old_log_prob|), 0)``.  Tokens whose
-    covariances are equal at the cut are taken in the order ``torch.topk`` yields on the device."""
+    ``ppo_kl_coef`` (1.0).  Returns ``(pg_loss, 0, masked_mean(|log_prob - old_log_prob|), 0)``.  Of tokens whose
+    covariances are equal at the cut the ones with the lowest flat index are taken (``torch.topk`` promises no order
+    there)."""
     ratio, coef = _kl_cov_params(config)
     agg_code = _agg_code(loss_agg_mode)
     aux = _kl_cov_weights(log_prob, advantages, response_mask, ratio, coef)

@@ -139,7 +139,7 @@ __global__ __launch_bounds__(kStream) void loss_partials_kernel(LossArgs a, cons
     const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
     const Quad ent4 = a.ent ? load_quad(a.ent, idx0, vec, nv, 0.f) : const_quad(0.f);
     const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
-    const Quad aux4 = (KIND < 0 && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
+    const Quad aux4 = ((KIND < 0 || KIND >= KIND_KL_COV) && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (e >= nv) break;
@@ -405,7 +405,7 @@ __global__ __launch_bounds__(kStream) void loss_bwd_kernel(LossArgs a, const flo
     const Quad adv4 = load_quad(a.adv, idx0, vec, nv, 0.f);
     const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
     const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
-    const Quad aux4 = (KIND < 0 && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
+    const Quad aux4 = ((KIND < 0 || KIND >= KIND_KL_COV) && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float m = m4.v[e], lp = lp4.v[e];
@@ -438,6 +438,8 @@ int launch_loss_bwd(const LossArgs& a, const float* g_out, const float* saved_ou
     case KIND_GSPO: loss_bwd_kernel<KIND_GSPO><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
     case KIND_AGG: loss_bwd_kernel<KIND_AGG><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
     case KIND_VALUE: loss_bwd_kernel<KIND_VALUE><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
+    case KIND_KL_COV: loss_bwd_kernel<KIND_KL_COV><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
+    case KIND_CLIP_COV: loss_bwd_kernel<KIND_CLIP_COV><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent); break;
     default: loss_bwd_kernel<-1><<<grid, block, 0, st>>>(a, g_out, saved_out, row_msum, row_s, d_lp, d_ent);
   }
   SIIRL_LAUNCH_CHECK("loss_bwd_kernel");
@@ -643,16 +645,25 @@ __global__ __launch_bounds__(kThreads) void mean_rows_kernel(const float* __rest
 constexpr int kCovGrid = 1024;
 constexpr int kCovSums = 6;
 __global__ __launch_bounds__(kThreads) void cov_sums_kernel(const float* __restrict__ lp, const float* __restrict__ adv,
-                                                            const void* mask, int mask_dtype, int64_t n,
+                                                            const void* mask, int mask_dtype, int64_t n, int vec,
                                                             double* __restrict__ part) {
   float s[kCovSums] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
-    const float m = load_mask(mask, mask_dtype, i);
-    const float a = adv[i], l = lp[i];
-    if (m > 0.f) { s[0] += 1.f; s[1] += a; s[2] += l; }
-    s[3] += m;
-    s[4] += contrib_where(a, m);  // masked_mean: where(mask, v, 0) * mask
-    s[5] += contrib_where(l, m);
+  const int64_t nq = (n + 3) / 4;  // four tokens per thread and access
+  for (int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x; q < nq; q += (int64_t)gridDim.x * kThreads) {
+    const int64_t i = 4 * q;
+    const int nv = (int)((n - i) < 4 ? (n - i) : 4);
+    const bool v = vec != 0 && nv == 4;
+    const Quad m4 = load_mask_quad(mask, mask_dtype, i, v, nv);
+    const Quad a4 = load_quad(adv, i, v, nv, 0.f), l4 = load_quad(lp, i, v, nv, 0.f);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (e >= nv) break;
+      const float m = m4.v[e], a = a4.v[e], l = l4.v[e];
+      if (m > 0.f) { s[0] += 1.f; s[1] += a; s[2] += l; }
+      s[3] += m;
+      s[4] += contrib_where(a, m);  // masked_mean: where(mask, v, 0) * mask
+      s[5] += contrib_where(l, m);
+    }
   }
   __shared__ double sh[kThreads / kWave + 1];
   for (int k = 0; k < kCovSums; ++k) {
@@ -688,21 +699,33 @@ __global__ __launch_bounds__(kThreads) void cov_stats_kernel(const double* __res
 // excluded) and, for clip_cov, where the PPO clip already bites (l2 > l1 under a positive mask)
 __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __restrict__ old_lp, const float* __restrict__ lp,
                                                               const float* __restrict__ adv, const void* mask,
-                                                              int mask_dtype, int64_t n, int clip_mode, float lo, float hi,
-                                                              const float* __restrict__ stats, float* __restrict__ cov) {
+                                                              int mask_dtype, int64_t n, int vec, int clip_mode, float lo,
+                                                              float hi, const float* __restrict__ stats,
+                                                              float* __restrict__ cov) {
   const float ma = stats[2], ml = stats[3];
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
-    const float m = load_mask(mask, mask_dtype, i);
-    const float a = adv[i], l = lp[i];
-    float c = (a - ma) * (l - ml);
-    if (clip_mode) {
-      const float r = expf(l - old_lp[i]);
-      const float l1 = -a * r, l2 = -a * clampf(r, lo, hi);
-      if (m == 0.f || (l2 > l1 && m > 0.f)) c = -__builtin_inff();
-    } else if (!(m > 0.f)) {
-      c = -__builtin_inff();
+  const int64_t nq = (n + 3) / 4;
+  for (int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x; q < nq; q += (int64_t)gridDim.x * kThreads) {
+    const int64_t i = 4 * q;
+    const int nv = (int)((n - i) < 4 ? (n - i) : 4);
+    const bool v = vec != 0 && nv == 4;
+    const Quad m4 = load_mask_quad(mask, mask_dtype, i, v, nv);
+    const Quad a4 = load_quad(adv, i, v, nv, 0.f), l4 = load_quad(lp, i, v, nv, 0.f);
+    const Quad o4 = clip_mode ? load_quad(old_lp, i, v, nv, 0.f) : const_quad(0.f);
+    Quad c4;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float m = m4.v[e], a = a4.v[e], l = l4.v[e];
+      float c = (a - ma) * (l - ml);
+      if (clip_mode) {
+        const float r = expf(l - o4.v[e]);
+        const float l1 = -a * r, l2 = -a * clampf(r, lo, hi);
+        if (m == 0.f || (l2 > l1 && m > 0.f)) c = -__builtin_inff();
+      } else if (!(m > 0.f)) {
+        c = -__builtin_inff();
+      }
+      c4.v[e] = c;
     }
-    cov[i] = c;
+    store_quad(cov, i, v, nv, c4);
   }
 }
 
@@ -751,6 +774,8 @@ int launch_loss_partials(const LossArgs& a, const float* row_s, float* partials,
     case KIND_GSPO: loss_partials_kernel<KIND_GSPO><<<grid, block, 0, st>>>(a, row_s, partials); break;
     case KIND_AGG: loss_partials_kernel<KIND_AGG><<<grid, block, 0, st>>>(a, row_s, partials); break;
     case KIND_VALUE: loss_partials_kernel<KIND_VALUE><<<grid, block, 0, st>>>(a, row_s, partials); break;
+    case KIND_KL_COV: loss_partials_kernel<KIND_KL_COV><<<grid, block, 0, st>>>(a, row_s, partials); break;
+    case KIND_CLIP_COV: loss_partials_kernel<KIND_CLIP_COV><<<grid, block, 0, st>>>(a, row_s, partials); break;
     default: loss_partials_kernel<-1><<<grid, block, 0, st>>>(a, row_s, partials);
   }
   SIIRL_LAUNCH_CHECK("loss_partials_kernel");
@@ -1000,16 +1025,22 @@ extern "C" int siirl_cov_scores(const float* old_log_prob, const float* log_prob
   hipStream_t st = (hipStream_t)stream;
   const int64_t n = B * L;
   const int clip_mode = loss_mode == SIIRL_LOSS_CLIP_COV;
-  const int grid = (int)(n == 0 ? 1 : ((n + kThreads - 1) / kThreads < kCovGrid ? (n + kThreads - 1) / kThreads : kCovGrid));
+  const int64_t wgs = ((n + 3) / 4 + kThreads - 1) / kThreads;
+  const int grid = (int)(wgs < 1 ? 1 : (wgs < kCovGrid ? wgs : kCovGrid));
   double* part = (double*)workspace;
-  cov_sums_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(log_prob, advantages, mask, mask_dtype, n, part);
+  // four tokens per access when every operand starts on a 16-byte boundary (the mask: four of its elements)
+  auto ok16 = [](const void* p) { return p == nullptr || ((uintptr_t)p & 15) == 0; };
+  const size_t msz = dtype_size(mask_dtype);
+  const int vec = ok16(old_log_prob) && ok16(log_prob) && ok16(advantages) && ok16(cov) &&
+                  ((uintptr_t)mask & (msz * 4 > 16 ? 15 : msz * 4 - 1)) == 0;
+  cov_sums_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(log_prob, advantages, mask, mask_dtype, n, vec, part);
   SIIRL_LAUNCH_CHECK("cov_sums_kernel");
   cov_stats_kernel<<<1, dim3(kThreads), 0, st>>>(part, grid, clip_mode, stats);
   SIIRL_LAUNCH_CHECK("cov_stats_kernel");
   if (n == 0) return SIIRL_OK;
   cov_scores_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(old_log_prob, log_prob, advantages, mask, mask_dtype,
-                                                                    n, clip_mode, 1.f - clip_low, 1.f + clip_high, stats,
-                                                                    cov);
+                                                                    n, vec, clip_mode, 1.f - clip_low, 1.f + clip_high,
+                                                                    stats, cov);
   SIIRL_LAUNCH_CHECK("cov_scores_kernel");
   return SIIRL_OK;
 }

@@ -781,6 +781,20 @@ std::tuple<Tensor, Tensor> cov_scores(const optional<Tensor>& old, const Tensor&
   return {cov, stats};
 }
 
+// marks (shaped like scores): `value` at the k largest scores, 0 elsewhere
+Tensor topk_mark(const Tensor& scores, int64_t k, double value) {
+  require_f32c(scores, "scores");
+  const int64_t n = scores.numel();
+  TORCH_CHECK(k >= 0 && k <= n, "siirl_amd: k=", k, " is out of range for ", n, " scores");  // torch.topk: RuntimeError
+  Tensor marks = at::empty_like(scores);
+  const size_t nws = siirl_topk_mark_workspace_bytes();
+  Tensor ws = at::empty({(int64_t)nws}, scores.options().dtype(at::kByte));
+  DeviceGuard guard(scores.device());
+  check_rc(siirl_topk_mark(ptr<float>(scores), n, k, (float)value, ptr<float>(marks), ptr(ws), nws, stream_of(scores)),
+           "siirl_topk_mark");
+  return marks;
+}
+
 constexpr int kActorOuts = 13;  // SIIRL_OUT_LOSS .. SIIRL_OUT_DRIFT_LOSS
 
 // One fused forward (partials + finish) and one elementwise backward for the whole micro-batch loss.  The 13 scalars
@@ -1183,6 +1197,7 @@ TORCH_LIBRARY(siirl_hip, m) {
         "Tensor row_msum, Tensor row_s, Tensor? token_aux=None) -> (Tensor, Tensor)");
   m.def("cov_scores(Tensor? old_log_prob, Tensor log_prob, Tensor advantages, Tensor mask, int loss_mode, "
         "float clip_low, float clip_high) -> (Tensor, Tensor)");
+  m.def("topk_mark(Tensor scores, int k, float value) -> Tensor");
   m.def("kl_penalty_fwd(Tensor log_prob, Tensor ref_log_prob, int kl_mode) -> Tensor");
   m.def("kl_penalty_bwd(Tensor g, Tensor log_prob, Tensor ref_log_prob, int kl_mode, bool straight_through, "
         "bool need_log_prob, bool need_ref) -> (Tensor, Tensor)");
@@ -1223,6 +1238,7 @@ TORCH_LIBRARY_IMPL(siirl_hip, CUDA, m) {
   m.impl("policy_loss_fwd", &policy_loss_fwd);
   m.impl("policy_loss_bwd", &policy_loss_bwd);
   m.impl("cov_scores", &cov_scores);
+  m.impl("topk_mark", &topk_mark);
   m.impl("kl_penalty_fwd", &kl_penalty_fwd);
   m.impl("kl_penalty_bwd", &kl_penalty_bwd);
   m.impl("fused_linear_logprob_entropy_fwd", &fused_linear_fwd);

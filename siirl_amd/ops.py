@@ -141,6 +141,11 @@ def _(old_log_prob, log_prob, advantages, mask, loss_mode, clip_low, clip_high):
     return log_prob.new_empty(log_prob.shape, dtype=torch.float32), log_prob.new_empty(4, dtype=torch.float32)
 
 
+@_fake(f"{_NS}::topk_mark")
+def _(scores, k, value):
+    return scores.new_empty(scores.shape, dtype=torch.float32)
+
+
 @_fake(f"{_NS}::kl_penalty_fwd")
 def _(log_prob, ref_log_prob, kl_mode):
     return log_prob.new_empty(log_prob.shape, dtype=torch.float32)

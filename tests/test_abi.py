@@ -102,6 +102,12 @@ def test_argument_validation_without_gpu():
     assert h.siirl_cov_scores(None, p, p, p, L.F32, 2, 4, 6, 0.2, 0.2, p, p, p, 1 << 20, None) == -1  # clip_cov: old
     assert h.siirl_cov_scores(p, p, p, p, L.F32, 2, 4, 6, 0.2, 0.2, p, p, p, 8, None) == -4
     assert h.siirl_cov_workspace_bytes() > 0
+    q2 = ctypes.c_void_p(p.value + 64)
+    assert h.siirl_topk_mark(p, 8, 9, 1.0, q2, p, 1 << 20, None) == -1  # k > n
+    assert h.siirl_topk_mark(p, 8, 2, 1.0, p, p, 1 << 20, None) == -1  # marks alias scores
+    assert h.siirl_topk_mark(p, 8, 2, 1.0, q2, p, 8, None) == -4
+    assert h.siirl_topk_mark(p, 0, 0, 1.0, q2, None, 0, None) == 0  # nothing to mark: no workspace, no launch
+    assert h.siirl_topk_mark_workspace_bytes() > 0
     assert h.siirl_value_loss_fwd(p, p, p, p, L.F32, 2, 4, 0.5, 7, p, p, p, 1 << 20, None) == -1
     assert h.siirl_gae_advantage_return(p, p, p, L.F32, 2, 4, 1.0, 1.0, p, p, p, p, 8, 0, None) == -1  # adv == returns
     q2 = ctypes.c_void_p(p.value + 64)

@@ -210,7 +210,7 @@ def test_policy_loss_errors(dev):
     with pytest.raises(ValueError, match="Invalid loss_agg_mode"):
         CA.compute_policy_loss_vanilla(*args, loss_agg_mode="bogus", config=_cfg())
     with pytest.raises(ValueError, match="Unsupported loss mode"):
-        CA.get_policy_loss_fn("clip_cov")
+        CA.get_policy_loss_fn("clip_higher")
     assert CA.get_policy_loss_fn("vanilla") is CA.compute_policy_loss_vanilla
     assert CA.get_policy_loss_fn("gspo") is CA.compute_policy_loss_gspo
     with pytest.raises(RuntimeError, match="GPU only"):

@@ -187,7 +187,21 @@ def bench_config3(args, dev):
         CA.agg_loss(lm, mk, "seq-mean-token-mean").backward()
         lm.grad = None
 
+    adv_b, _ = CA.compute_grpo_outcome_advantage(rk, mk, uk)
+    cov_cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=10.0,
+                              policy_loss=SimpleNamespace(kl_cov_ratio=0.0002, ppo_kl_coef=1.0, clip_cov_ratio=0.0002,
+                                                          clip_cov_lb=1.0, clip_cov_ub=5.0))
+
+    def kl_cov_fb():
+        CA.compute_policy_loss_kl_cov(old, x, adv_b, mk, "token-mean", cov_cfg)[0].backward()
+        x.grad = None
+
+    cov_scores, cov_stats = torch.ops.siirl_hip.cov_scores(None, lpd, adv_b, mk, CA.LOSS_KL_COV, 0.0, 0.0)
+    k_cov = max(1, int(int(cov_stats[0]) * 0.0002))
     blocks = {
+        "kl_cov policy loss forward + backward: scores, top-k pick, loss, gradient (108 B/token)": (kl_cov_fb, 108),
+        f"siirl_topk_mark: the {k_cov} largest of the covariance scores marked (20 B/token: four reads, one write)":
+            (lambda: torch.ops.siirl_hip.topk_mark(cov_scores, k_cov, 1.0), 20),
         "masked_mean(values, mask) -> scalar (12 B/token)": (lambda: SF.masked_mean(lpd, mk), 12),
         "masked_mean(values, mask, axis=-1) -> [B] (12 B/token)": (lambda: SF.masked_mean(lpd, mk, axis=-1), 12),
         "kl_penalty low_var_kl forward (12 B/token)": (lambda: CA.kl_penalty(lpd, ref, "low_var_kl"), 12),

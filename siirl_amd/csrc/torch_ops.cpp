@@ -598,8 +598,15 @@ Tensor masked_reduce(const Tensor& values, const Tensor& mask, at::IntArrayRef a
       v = v.reshape({0, 1});
       m = m.reshape({0, 1});
     } else {
-      v = v.reshape({1, -1});
-      m = m.reshape({1, -1});
+      // rows for the kernels' two-level fold: the tensor's own last axis, or a power of two that divides the count
+      // (one row of millions of tokens would leave the fold of its segments to a single thread)
+      const int64_t n = v.numel();
+      int64_t cols = nd >= 2 && v.size(-1) >= 256 ? v.size(-1) : n;
+      if (cols == n && n > (1 << 16))
+        for (int64_t c = 8192; c >= 256; c >>= 1)
+          if (n % c == 0) { cols = c; break; }
+      v = v.reshape({n / cols, cols});
+      m = m.reshape({n / cols, cols});
     }
   } else {
     std::vector<int64_t> perm;

@@ -197,7 +197,7 @@ def bench_config3(args, dev):
         x.grad = None
 
     cov_scores, cov_stats = torch.ops.siirl_hip.cov_scores(None, lpd, adv_b, mk, CA.LOSS_KL_COV, 0.0, 0.0)
-    k_cov = max(1, int(int(cov_stats[0]) * 0.0002))
+    k_cov = max(1, int(int(float(cov_stats[0]) + float(cov_stats[4])) * 0.0002))
     blocks = {
         "kl_cov policy loss forward + backward: scores, top-k pick, loss, gradient (108 B/token)": (kl_cov_fb, 108),
         f"siirl_topk_mark: the {k_cov} largest of the covariance scores marked (20 B/token: four reads, one write)":

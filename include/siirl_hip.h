@@ -279,7 +279,8 @@ int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const f
  * max(1, int(n * kl_cov_ratio)) largest); SIIRL_LOSS_CLIP_COV: masked means sum(v * m) / (sum(m) + 1e-8), cov = -inf
  * where mask == 0 and where the PPO clip already bites (-A * clamp(ratio, 1 - clip_low, 1 + clip_high) > -A * ratio,
  * ratio = exp(log_prob - old_log_prob)); the caller draws its tokens among clip_cov_lb < cov < clip_cov_ub.
- * stats[4] (device) receives {count of mask > 0, sum of the mask, mean A, mean log_prob}.  old_log_prob may be NULL
+ * stats[6] (device) receives {count of mask > 0, sum of the mask, mean A, mean log_prob, and the float32 rounding
+ * residues of the first two: count = stats[0] + stats[4] and mask sum = stats[1] + stats[5] exactly}.  old_log_prob may be NULL
  * for SIIRL_LOSS_KL_COV.  workspace: siirl_cov_workspace_bytes(), 8-byte aligned.
  * Replaces: siirl/dag_worker/core_algos.py:952-971 (clip_cov) and :1047-1055 (kl_cov).
  */

@@ -559,7 +559,8 @@ def _kl_cov_weights(log_prob, advantages, response_mask, kl_cov_ratio: float, pp
     count ``n``), as the reference's ``len(all_valid_adv)``."""
     dev, _, lp, adv, m = _cov_operands(None, log_prob, advantages, response_mask)
     cov, stats = _OPS.cov_scores(None, lp, adv, m, LOSS_KL_COV, 0.0, 0.0)
-    n = int(stats[0].item())
+    st = stats.tolist()  # one host sync, as the reference's len(all_valid_adv)
+    n = int(st[0] + st[4])  # exact beyond 2^24 tokens: the count and what float32 rounding took from it
     k = 0
     if min(kl_cov_ratio, n) != 0:  # reference :1052-1054
         k = max(1, int(n * kl_cov_ratio))
@@ -575,7 +576,8 @@ def _clip_cov_dropped(old_log_prob, log_prob, advantages, response_mask, lo, hi,
     reference's own draw.  Two host syncs (mask sum, candidate count), as there."""
     dev, old, lp, adv, m = _cov_operands(old_log_prob, log_prob, advantages, response_mask)
     cov, stats = _OPS.cov_scores(old, lp, adv, m, LOSS_CLIP_COV, lo, hi)
-    clip_num = max(int(clip_cov_ratio * stats[1].item()), 1)
+    st = stats.tolist()
+    clip_num = max(int(clip_cov_ratio * (st[1] + st[5])), 1)  # the mask sum, exact in double
     cand = torch.nonzero((cov < ub) & (cov > lb) & (m > 0))
     aux = torch.zeros_like(cov)
     if len(cand) > 0:

@@ -671,8 +671,9 @@ __global__ __launch_bounds__(kThreads) void cov_sums_kernel(const float* __restr
     if (threadIdx.x == 0) part[(int64_t)blockIdx.x * kCovSums + k] = t;
   }
 }
-// stats[0..3] = {count of m > 0, sum of the mask, mean A, mean lp}; plain means over m > 0 (kl_cov, core_algos.py:1055)
-// or masked means sum(v * m) / (sum(m) + 1e-8) in fp32 (clip_cov, :967-969)
+// stats[0..5] = {count of m > 0, sum of the mask, mean A, mean lp, and what the first two lost to float32 rounding
+// (count = stats[0] + stats[4], mask sum = stats[1] + stats[5], exact in double)}; plain means over m > 0 (kl_cov,
+// core_algos.py:1055) or masked means sum(v * m) / (sum(m) + 1e-8) in fp32 (clip_cov, :967-969)
 __global__ __launch_bounds__(kThreads) void cov_stats_kernel(const double* __restrict__ part, int nparts, int masked_means,
                                                              float* __restrict__ stats) {
   __shared__ double sh[kThreads / kWave + 1];
@@ -685,6 +686,8 @@ __global__ __launch_bounds__(kThreads) void cov_stats_kernel(const double* __res
   if (threadIdx.x == 0) {
     stats[0] = (float)t[0];
     stats[1] = (float)t[3];
+    stats[4] = (float)(t[0] - (double)stats[0]);
+    stats[5] = (float)(t[3] - (double)stats[1]);
     if (masked_means) {
       const float den = (float)t[3] + 1e-8f;
       stats[2] = (float)t[4] / den;

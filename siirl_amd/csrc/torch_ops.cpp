@@ -766,7 +766,7 @@ std::tuple<Tensor, Tensor> policy_loss_bwd(const Tensor& g, const Tensor& old, c
 }
 
 // Scores that the covariance losses pick their tokens from: (cov [B, L], stats {count of mask > 0, sum of the mask,
-// mean advantage, mean log-prob}).  No gradient: the pick is a set of indices.
+// mean advantage, mean log-prob, float32 residues of the first two}).  No gradient: the pick is a set of indices.
 std::tuple<Tensor, Tensor> cov_scores(const optional<Tensor>& old, const Tensor& lp, const Tensor& adv, const Tensor& mask,
                                       int64_t loss_mode, double clip_low, double clip_high) {
   require_f32c(lp, "log_prob");
@@ -777,7 +777,7 @@ std::tuple<Tensor, Tensor> cov_scores(const optional<Tensor>& old, const Tensor&
   TORCH_CHECK_VALUE(is_cov_loss(loss_mode), "siirl_amd: covariance scores belong to the kl_cov and clip_cov losses");
   TORCH_CHECK_VALUE(loss_mode != SIIRL_LOSS_CLIP_COV || has(old), "siirl_amd: clip_cov needs old_log_prob");
   const int64_t B = lp.size(0), L = lp.size(1);
-  Tensor cov = at::empty_like(lp), stats = empty_f32({4}, lp);
+  Tensor cov = at::empty_like(lp), stats = empty_f32({6}, lp);
   const size_t nws = siirl_cov_workspace_bytes();
   Tensor ws = at::empty({(int64_t)nws}, lp.options().dtype(at::kByte));
   DeviceGuard guard(lp.device());

@@ -138,7 +138,7 @@ def _(g_loss, old_log_prob, log_prob, advantages, mask, is_weights, entropy, ref
 
 @_fake(f"{_NS}::cov_scores")
 def _(old_log_prob, log_prob, advantages, mask, loss_mode, clip_low, clip_high):
-    return log_prob.new_empty(log_prob.shape, dtype=torch.float32), log_prob.new_empty(4, dtype=torch.float32)
+    return log_prob.new_empty(log_prob.shape, dtype=torch.float32), log_prob.new_empty(6, dtype=torch.float32)
 
 
 @_fake(f"{_NS}::topk_mark")

@@ -64,7 +64,7 @@ def test_fake_kernels_give_shapes_without_a_gpu(with_optional):
         assert ns.masked_reduce_bwd(mk((B,), torch.float32), mk((B, L), torch.bool), True, None).shape == (B, L)
         cov, stats = ns.cov_scores(mk((B, L), torch.float32), mk((B, L), torch.float32), mk((B, L), torch.float32),
                                    mk((B, L), torch.int64), 6, 0.2, 0.28)
-        assert cov.shape == (B, L) and stats.shape == (4,) and cov.dtype == torch.float32
+        assert cov.shape == (B, L) and stats.shape == (6,) and cov.dtype == torch.float32
         a5 = list(_loss_args(mk, B, L, with_optional))
         a5[7] = 5
         o5, _, _ = ns.policy_loss_fwd(*a5, mk((B, L), torch.float32))

@@ -216,6 +216,9 @@ def test_cov_selection_at_batch_scale():
     aux = CA._kl_cov_weights(lp, A, m, 0.0002, 1.0)
     k = max(1, int(n * 0.0002))
     assert int((aux != 0).sum()) == k
+    _, st = torch.ops.siirl_hip.cov_scores(None, lp, A, m, CA.LOSS_KL_COV, 0.0, 0.0)
+    st = st.double().cpu()
+    assert int(st[0] + st[4]) == n and int(st[1] + st[5]) == n
     cov, _ = torch.ops.siirl_hip.cov_scores(None, lp, A, m, CA.LOSS_KL_COV, 0.0, 0.0)
     assert float(cov[aux != 0].min()) >= float(cov[aux == 0].max())
     assert bool((m[aux != 0] > 0).all())

@@ -111,7 +111,16 @@ def test_sweep_grpo_advantage_random_groups(dev):
                                                      uid, norm_adv_by_std_in_grpo=norm)
         assert got is ret or torch.equal(got, ret)
         err = (got.cpu().double() - want.double()).abs()
-        assert bool((err <= 1e-6 + 1e-5 * want.double().abs()).all()), (case, B, L, norm, err.max().item())
+        tol = 1e-6 + 1e-5 * want.double().abs()
+        if not bool((err <= tol).all()):
+            # a group of nearly equal scores divides float32 rounding by a tiny std: the reference's own float32
+            # arithmetic is then off by far more than the tolerance; there the result must be no farther from the
+            # float64 value than the reference's is
+            exact, _ = OC.compute_grpo_outcome_advantage(torch.from_numpy(rewards).double(), torch.from_numpy(mask).double(),
+                                                         uid, norm_adv_by_std_in_grpo=norm)
+            ref_err = (want.double() - exact).abs()
+            ok = (err <= tol) | ((got.cpu().double() - exact).abs() <= ref_err + tol)
+            assert bool(ok.all()), (case, B, L, norm, err.max().item())
         assert bool((got.cpu()[mask == 0] == 0).all()), case
 
 

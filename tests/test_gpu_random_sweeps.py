@@ -112,15 +112,20 @@ def test_sweep_grpo_advantage_random_groups(dev):
         assert got is ret or torch.equal(got, ret)
         err = (got.cpu().double() - want.double()).abs()
         tol = 1e-6 + 1e-5 * want.double().abs()
-        if not bool((err <= tol).all()):
-            # a group of nearly equal scores divides float32 rounding by a tiny std: the reference's own float32
-            # arithmetic is then off by far more than the tolerance; there the result must be no farther from the
-            # float64 value than the reference's is
-            exact, _ = OC.compute_grpo_outcome_advantage(torch.from_numpy(rewards).double(), torch.from_numpy(mask).double(),
-                                                         uid, norm_adv_by_std_in_grpo=norm)
-            ref_err = (want.double() - exact).abs()
-            ok = (err <= tol) | ((got.cpu().double() - exact).abs() <= ref_err + tol)
-            assert bool(ok.all()), (case, B, L, norm, err.max().item())
+        if norm:
+            # Conditioning: the reference takes mean and std in float32 (torch's two-pass std around its own float32
+            # mean, whose summation order depends on the host's vector width), so a group whose spread is within a few
+            # float32 ulps of its scores' magnitude gets an advantage that is off by ulp(|s|) / (std + eps) -- per cent,
+            # not 1e-5 -- and not the same on every host.  The kernel takes the statistics in double; the two are
+            # compared at four such units.
+            amp = np.zeros(B)
+            for u in np.unique(uid):
+                rows = np.nonzero(uid == u)[0]
+                if rows.size > 1:
+                    sc = score[rows].astype(np.float64)
+                    amp[rows] = np.spacing(np.float32(np.abs(sc).max())) / (sc.std(ddof=1) + 1e-6)
+            tol = tol + torch.from_numpy(4.0 * amp)[:, None]
+        assert bool((err <= tol).all()), (case, B, L, norm, err.max().item())
         assert bool((got.cpu()[mask == 0] == 0).all()), case
 
 

@@ -387,7 +387,7 @@ def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_i
     """Dispatcher (reference ``core_algos.py:1400-1492``).  The GAE (``:1424-1439``, without the PF-PPO
     reweighting) and GRPO (``:1440-1471``) branches are built; MARFT raises ``NotImplementedError`` here, and
     the CPGD branch fails with the reference's own ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a
-    keyword it does not take, ``:1475-1480``)."""
+    keyword it does not take, ``:1475-1480``); ``compute_cpgd_outcome_advantage`` is there to be called directly."""
     if "response_mask" not in data.keys():
         _td_set(data, "response_mask", compute_response_mask(data))
     est = adv_estimator.value if isinstance(adv_estimator, Enum) else adv_estimator

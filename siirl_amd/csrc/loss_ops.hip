@@ -191,6 +191,60 @@ __global__ __launch_bounds__(kStream) void loss_partials_kernel(LossArgs a, cons
   }
 }
 
+// ---------------------------------------------------------------------------- very long rows
+
+// The finish kernels give a row to one thread, which walks the row's segments.  A row of more than kFoldAbove
+// segments (half a million tokens) first has its segment partials folded 64 to 1, one wave per group of 64, sums in
+// double, as often as it takes; rows of ordinary length never come here, so their results do not depend on it.
+constexpr int kFoldAbove = 256, kFoldBy = 64;
+__global__ __launch_bounds__(kThreads) void fold_segments_kernel(const float* __restrict__ in, int64_t B, int nseg,
+                                                                 int nseg2, float* __restrict__ out) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t g = (int64_t)blockIdx.x * (kThreads / kWave) + threadIdx.x / kWave;  // (row, group of segments)
+  if (g >= B * nseg2) return;
+  const int64_t b = g / nseg2;
+  const int s2 = (int)(g - b * nseg2), s = s2 * kFoldBy + lane;
+  const bool have = s < nseg;
+  const float* p = in + (b * nseg + (have ? s : 0)) * kNP;
+  float res = 0.f;
+#pragma unroll
+  for (int k = 0; k < kNP; ++k) {
+    float r;
+    if (k == P_RMIN) {
+      float v = have ? p[k] : __builtin_inff();
+#pragma unroll
+      for (int o = kWave / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
+      r = v;
+    } else if (k == P_RMAX) {
+      float v = have ? p[k] : -__builtin_inff();
+#pragma unroll
+      for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+      r = v;
+    } else {
+      r = (float)wave_sum(have ? (double)p[k] : 0.0);
+    }
+    if (lane == k) res = r;
+  }
+  if (lane < kNP) out[g * kNP + lane] = res;
+}
+
+// Folds `partials` ([B][nseg][kNP]) until a row has at most kFoldAbove segments, alternating between `spare` and
+// `partials`; returns where the result lies and updates nseg.
+int fold_long_rows(const float*& cur, float* partials, float* spare, int64_t B, int& nseg, hipStream_t st) {
+  float* dst = spare;
+  while (nseg > kFoldAbove) {
+    const int nseg2 = (nseg + kFoldBy - 1) / kFoldBy;
+    const int64_t groups = B * nseg2;
+    fold_segments_kernel<<<dim3((unsigned)((groups + kThreads / kWave - 1) / (kThreads / kWave))), dim3(kThreads), 0, st>>>(
+        cur, B, nseg, nseg2, dst);
+    SIIRL_LAUNCH_CHECK("fold_segments_kernel");
+    cur = dst;
+    dst = dst == spare ? partials : spare;
+    nseg = nseg2;
+  }
+  return SIIRL_OK;
+}
+
 // ---------------------------------------------------------------------------- finish
 
 __device__ __forceinline__ double block_sum_d(double v, double* sh) { return block_sum(v, sh); }
@@ -810,14 +864,16 @@ int run_forward(LossArgs& a, float* out16, float* row_msum, float* row_s, void* 
     SIIRL_LAUNCH_CHECK("row_finish_kernel");
   }
   if (int rc = launch_loss_partials(a, row_s, partials, st)) return rc;
+  const size_t used = ((size_t)a.B * a.nseg * (kNP + kNPre) * sizeof(float) + 255) / 256 * 256;
+  const float* folded = partials;  // the pre-pass sums are spent by now: their room serves the folding of long rows
+  if (int rc = fold_long_rows(folded, partials, pre, a.B, a.nseg, st)) return rc;
   if (a.B <= kTwoLevelRows) {
-    loss_finish_kernel<<<1, block, 0, st>>>(a, partials, row_s, out16, row_msum);
+    loss_finish_kernel<<<1, block, 0, st>>>(a, folded, row_s, out16, row_msum);
     SIIRL_LAUNCH_CHECK("loss_finish_kernel");
   } else {
-    const size_t used = ((size_t)a.B * a.nseg * (kNP + kNPre) * sizeof(float) + 255) / 256 * 256;
     double* rec = reinterpret_cast<double*>((char*)ws + used);
     const int nrec = (int)((a.B + kThreads - 1) / kThreads);
-    loss_rows_kernel<<<dim3((unsigned)nrec), block, 0, st>>>(a, partials, row_s, row_msum, rec);
+    loss_rows_kernel<<<dim3((unsigned)nrec), block, 0, st>>>(a, folded, row_s, row_msum, rec);
     SIIRL_LAUNCH_CHECK("loss_rows_kernel");
     loss_finish2_kernel<<<1, block, 0, st>>>(a, rec, nrec, out16);
     SIIRL_LAUNCH_CHECK("loss_finish2_kernel");
@@ -1180,16 +1236,18 @@ extern "C" int siirl_masked_reduce(const float* values, const void* mask, int ma
   float* partials = (float*)workspace;
   set_vec(a);
   if (int rc = launch_loss_partials(a, nullptr, partials, st)) return rc;
+  const size_t used = ((size_t)B * a.nseg * (kNP + kNPre) * sizeof(float) + 255) / 256 * 256;
+  const float* folded = partials;
+  if (int rc = fold_long_rows(folded, partials, partials + (size_t)B * a.nseg * kNP, B, a.nseg, st)) return rc;
   if (B <= kTwoLevelRows) {
-    masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, total2, row_msum,
+    masked_finish_kernel<<<1, dim3(kThreads), 0, st>>>(folded, a.nseg, B, row_sum, row_mean, total2, row_msum,
                                                        mask_total);
     SIIRL_LAUNCH_CHECK("masked_finish_kernel");
     return SIIRL_OK;
   }
-  const size_t used = ((size_t)B * a.nseg * (kNP + kNPre) * sizeof(float) + 255) / 256 * 256;
   double* rec = reinterpret_cast<double*>((char*)workspace + used);  // room for kFinRec >= 2 doubles per workgroup
   const int nrec = (int)((B + kThreads - 1) / kThreads);
-  masked_rows_kernel<<<dim3((unsigned)nrec), dim3(kThreads), 0, st>>>(partials, a.nseg, B, row_sum, row_mean, row_msum,
+  masked_rows_kernel<<<dim3((unsigned)nrec), dim3(kThreads), 0, st>>>(folded, a.nseg, B, row_sum, row_mean, row_msum,
                                                                       rec);
   SIIRL_LAUNCH_CHECK("masked_rows_kernel");
   if (total2 || mask_total) {

@@ -464,3 +464,42 @@ def test_kl_penalty_lengths_and_alignment(dev, n, offset):
         for got, ref64 in ((x.grad, x64.grad), (r.grad, r64.grad)):
             ok, err = _grad_close(got.cpu(), ref64)
             assert ok, (kind, err)
+
+
+@pytest.mark.parametrize("B,L", [(2, 2048 * 300 + 5), (1, 2048 * 20000 + 12)])
+def test_very_long_rows(dev, B, L):
+    """Rows of more than 256 segments (half a million tokens) have their segment partials folded before the finish:
+    one level at 300 segments, two at 20000.  Same values as the float64 oracle; the forward must not be slower than a
+    few passes over the data (a single thread used to walk all segments of a row)."""
+    import time
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.torch_functional as SF
+
+    g = torch.Generator(device=dev).manual_seed(L % 1000)
+    x = torch.randn(B, L, device=dev, generator=g)
+    m = (torch.rand(B, L, device=dev, generator=g) < 0.7)
+    for mode in ("token-mean", "seq-mean-token-sum", "seq-mean-token-mean", "seq-mean-token-sum-norm"):
+        want = OC.agg_loss(x.double().cpu(), m.double().cpu(), mode)
+        got = CA.agg_loss(x, m, mode)
+        assert abs(float(got) - float(want)) <= 1e-6 + 2e-5 * abs(float(want)), (mode, float(got), float(want))
+    want = (x.double() * m).sum(-1) / (m.double().sum(-1) + 1e-8)
+    got = SF.masked_mean(x, m, axis=-1)
+    assert torch.allclose(got.double(), want, rtol=2e-5, atol=1e-7)
+    if B == 2:
+        old = x * 0.1 - 1.0
+        lp = (old + 0.05 * torch.randn(B, L, device=dev, generator=g)).requires_grad_(True)
+        adv = torch.randn(B, L, device=dev, generator=g)
+        got = CA.compute_policy_loss_vanilla(old, lp, adv, m, "seq-mean-token-mean", _cfg())
+        lp64 = lp.detach().double().cpu().requires_grad_(True)
+        want = OC.compute_policy_loss_vanilla(old.double().cpu(), lp64, adv.double().cpu(), m.double().cpu(),
+                                              "seq-mean-token-mean", _cfg())
+        for a, b in zip(got, want):
+            assert abs(float(a) - float(b)) <= 1e-6 + 2e-5 * abs(float(b))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        CA.agg_loss(x, m, "token-mean")
+    torch.cuda.synchronize()
+    per_call = (time.perf_counter() - t0) / 3
+    assert per_call < 1.5e-3, per_call  # 0.2 GB of operands at most: well under a millisecond of streaming

@@ -62,6 +62,16 @@ def test_heavy_ties_and_special_values():
     assert np.array_equal(_run(z, k), _expected(z.numpy().reshape(-1), k))
 
 
+def test_ties_across_several_tiles_of_a_chunk():
+    """3 M scores of seven distinct values: a workgroup's chunk spans three tiles, so the rank of an entry at the cut
+    runs over tiles and chunks."""
+    g = torch.Generator().manual_seed(6)
+    n = 3_000_000 + 3
+    x = torch.randint(-3, 4, (n,), generator=g).float()
+    for k in (5, 430_000, 1_500_000, n - 2):
+        assert np.array_equal(_run(x, k), _expected(x.numpy(), k)), k
+
+
 def test_unaligned_and_refusals():
     g = torch.Generator().manual_seed(9)
     base = torch.randn(10_001, generator=g).to(DEV)

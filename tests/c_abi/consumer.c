@@ -1,6 +1,6 @@
 /* A host program in plain C that uses libsiirl_hip.so through include/siirl_hip.h alone -- no Python, no torch:
  * device buffers from the HIP runtime, log-prob / entropy forward and backward of fp32 logits [T, V], checked
- * against a double-precision loop written here.  Exit status 0 and a line starting with "OK" on success. */
+ * against a double-precision loop written here, and the top-k pick of the KL-Cov loss over the same values.  Exit status 0 and a line starting with "OK" on success. */
 #include <hip/hip_runtime_api.h>
 #include <math.h>
 #include <stdint.h>
@@ -100,8 +100,38 @@ int main(void) {
       e_dx = fmax(e_dx, fabs((double)dx[(size_t)t * V + v] - want));
     }
   }
-  const int ok = e_lp < 1e-4 && e_ent < 1e-4 && e_dx < 1e-6;
-  printf("%s C ABI consumer: T=%d V=%d max |err| logprob %.2e entropy %.2e dlogits %.2e\n", ok ? "OK" : "FAIL", T, V,
-         e_lp, e_ent, e_dx);
+  /* the k largest of the T * V logits, marked by the selection step of the KL-Cov loss: exactly k marks, none of
+   * them below an unmarked value */
+  enum { K = 777 };
+  float* d_marks;
+  void* d_ws;
+  const size_t ws_bytes = siirl_topk_mark_workspace_bytes();
+  CK(hipMalloc((void**)&d_marks, sizeof(float) * T * V));
+  CK(hipMalloc(&d_ws, ws_bytes));
+  CALL(siirl_topk_mark(d_x, (int64_t)T * V, K, 1.0f, d_marks, d_ws, ws_bytes, stream));
+  CK(hipStreamSynchronize(stream));
+  if (siirl_topk_mark(d_x, (int64_t)T * V, (int64_t)T * V + 1, 1.0f, d_marks, d_ws, ws_bytes, stream) !=
+      SIIRL_ERR_INVALID_ARGUMENT) {
+    printf("FAIL k > n was accepted\n");
+    return 6;
+  }
+  float* marks = (float*)malloc(sizeof(float) * T * V);
+  CK(hipMemcpy(marks, d_marks, sizeof(float) * T * V, hipMemcpyDeviceToHost));
+  int n_marked = 0;
+  float lowest_marked = INFINITY, highest_unmarked = -INFINITY;
+  for (int i = 0; i < T * V; ++i) {
+    if (marks[i] != 0.0f) {
+      ++n_marked;
+      lowest_marked = fminf(lowest_marked, x[i]);
+    } else {
+      highest_unmarked = fmaxf(highest_unmarked, x[i]);
+    }
+  }
+  const int ok_sel = n_marked == K && lowest_marked >= highest_unmarked;
+
+  const int ok = e_lp < 1e-4 && e_ent < 1e-4 && e_dx < 1e-6 && ok_sel;
+  printf("%s C ABI consumer: T=%d V=%d max |err| logprob %.2e entropy %.2e dlogits %.2e; top-%d pick: %d marked, "
+         "lowest marked %.6f, highest unmarked %.6f\n", ok ? "OK" : "FAIL", T, V, e_lp, e_ent, e_dx, K, n_marked,
+         (double)lowest_marked, (double)highest_unmarked);
   return ok ? 0 : 1;
 }

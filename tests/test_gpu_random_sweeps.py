@@ -400,7 +400,13 @@ def test_sweep_loss_functions_over_shapes_dtypes_and_layouts(dev):
         want.backward()
         # a 16-bit log-prob makes kl_penalty return 16-bit values (as the reference's arithmetic would): bf16 accuracy
         vtol = 2.0 ** -7 if (lp_dtype == torch.bfloat16 and which == 1) else 1e-5
-        assert abs(total.item() - want.item()) < 1e-6 + vtol * abs(want.item()), (case, which, agg, total.item(), want.item())
+        tol = 1e-6 + vtol * abs(want.item())
+        if which == 0:
+            # the policy loss sums terms of both signs: float32 accumulation is accurate relative to the sum of their
+            # magnitudes (|tok| <= |A| * ratio, ratio < 2 here), not relative to what is left after they cancel
+            mag = OC.agg_loss(2.0 * adv.double().abs().reshape(-1, L), m64, agg).item()
+            tol += 2.0 ** -24 * mag / 8
+        assert abs(total.item() - want.item()) < tol, (case, which, agg, total.item(), want.item())
         gw = (x32.grad.double() if which == 0 else x64.grad).reshape(shape)
         rel = 2.0 ** -6 if lp_dtype == torch.bfloat16 else 1e-5
         err = (lp.grad.cpu().double() - gw).abs()

@@ -94,3 +94,31 @@ def test_at_batch_scale_against_torch_topk():
     want = torch.zeros_like(x)
     want[torch.topk(x, k).indices] = 1.0
     assert int(marks.sum()) == k and torch.equal(marks, want)
+
+
+def test_sweep_random_selections():
+    """Seeded random sizes, value distributions (continuous, a handful of distinct values, masked -inf stretches, NaN
+    sprinkled in) and k; ``SIIRL_TEST_SEED=<int>`` shifts the seeds."""
+    import os
+
+    shift = 100003 * int(os.environ.get("SIIRL_TEST_SEED", "0"))
+    rng = np.random.default_rng(4242 + shift)
+    for case in range(80):
+        n = int(rng.choice([1, 2, 7, 64, 65, 4095, 4096, 4097, 20_000, 70_001, 300_000]))
+        kind = case % 5
+        if kind == 0:
+            x = rng.standard_normal(n).astype(np.float32) * np.float32(10.0 ** rng.integers(-3, 4))
+        elif kind == 1:
+            x = rng.integers(-2, 3, n).astype(np.float32)
+        elif kind == 2:
+            x = rng.standard_normal(n).astype(np.float32)
+            x[rng.random(n) < rng.random()] = -np.inf
+        elif kind == 3:
+            x = rng.standard_normal(n).astype(np.float32)
+            x[rng.random(n) < 0.01] = np.nan
+            x[rng.random(n) < 0.01] = np.inf
+        else:
+            x = np.full(n, np.float32(rng.standard_normal()), dtype=np.float32)
+        k = int(rng.integers(0, n + 1)) if case % 3 else int(min(n, max(1, n // 5000)))
+        got = _run(torch.from_numpy(x), k)
+        assert np.array_equal(got, _expected(x, k)), (case, n, kind, k)

@@ -36,6 +36,13 @@ def _close(a, b, rtol=1e-5, atol=1e-6, what=None):
     assert abs(float(a) - float(b)) <= atol + rtol * abs(float(b)), (float(a), float(b), what)
 
 
+def _cancel_slack(A, m, agg, w=None):
+    """Float32 accumulation of a policy loss is accurate relative to the sum of the magnitudes of its signed terms
+    (|tok| <= |A| * ratio * weight, ratio < 3 in these cases), not relative to what cancellation leaves of them."""
+    mag = 3.0 * A.double().abs() * (w.double() if w is not None else 1.0)
+    return 2.0 ** -24 / 8 * float(O.agg_loss(mag, m.double(), agg))
+
+
 @pytest.mark.parametrize("agg", O.AGG_MODES)
 @pytest.mark.parametrize("B,L,mask_dtype,with_w", [(6, 64, torch.int64, False), (5, 37, torch.bool, True),
                                                    (33, 2052, torch.float32, True), (1, 5, torch.int64, False)])
@@ -300,7 +307,7 @@ def test_sweep_covariance_losses():
             (gwant,) = torch.autograd.grad(want[0], lp64)
             got[0].backward()
             info = (case, B, L, str(mdt), agg, with_w, ratio, coef)
-            _close(got[0], want[0], what=info)
+            _close(got[0], want[0], atol=1e-6 + _cancel_slack(A, m, agg, w if with_w else None), what=info)
             _close(got[2], want[2], what=info)
             assert torch.allclose(lpd.grad.cpu().double(), gwant, rtol=1e-5, atol=1e-7), (case, "kl_cov grad")
         # Clip-Cov
@@ -322,6 +329,8 @@ def test_sweep_covariance_losses():
             continue
         (gwant,) = torch.autograd.grad(want[0], lp64)
         got[0].backward()
-        for a, b in zip(got, want):
+        _close(got[0], want[0], atol=1e-6 + _cancel_slack(A, m, agg, w if with_w else None),
+               what=(case, B, L, str(mdt), agg, with_w, pl))
+        for a, b in zip(got[1:], want[1:]):
             _close(a, b, what=(case, B, L, str(mdt), agg, with_w, pl))
         assert torch.allclose(lpd.grad.cpu().double(), gwant, rtol=1e-5, atol=1e-7), (case, "clip_cov grad")

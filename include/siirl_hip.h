@@ -75,7 +75,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1004
+#define SIIRL_HIP_ABI_VERSION 1005
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -277,7 +277,7 @@ int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const f
  *   cov[b, t] = (A - mean A) * (log_prob - mean log_prob),
  * SIIRL_LOSS_KL_COV: plain means over the tokens with mask > 0, cov = -inf where mask <= 0 (the caller takes the
  * max(1, int(n * kl_cov_ratio)) largest); SIIRL_LOSS_CLIP_COV: masked means sum(v * m) / (sum(m) + 1e-8), cov = -inf
- * where mask == 0 and where the PPO clip already bites (-A * clamp(ratio, 1 - clip_low, 1 + clip_high) > -A * ratio,
+ * where mask <= 0 (no candidate there) and where the PPO clip already bites (-A * clamp(ratio, 1 - clip_low, 1 + clip_high) > -A * ratio,
  * ratio = exp(log_prob - old_log_prob)); the caller draws its tokens among clip_cov_lb < cov < clip_cov_ub.
  * stats[6] (device) receives {count of mask > 0, sum of the mask, mean A, mean log_prob, and the float32 rounding
  * residues of the first two: count = stats[0] + stats[4] and mask sum = stats[1] + stats[5] exactly}.  old_log_prob may be NULL
@@ -301,6 +301,22 @@ int siirl_cov_scores(const float* old_log_prob, const float* log_prob, const flo
 size_t siirl_topk_mark_workspace_bytes(void);
 int siirl_topk_mark(const float* scores, int64_t n, int64_t k, float value, float* marks, void* workspace,
                     size_t workspace_bytes, siirl_stream_t stream);
+
+/*
+ * Flat indices, ascending, of the entries with lower_open < scores[i] < upper_open: Clip-Cov's candidate list (the
+ * tokens whose covariance lies inside (clip_cov_lb, clip_cov_ub); masked and already-clipped tokens carry -inf and
+ * stay out), in place of three comparisons, two logical ands and torch.nonzero.  Two steps, because the caller sizes
+ * the list: siirl_range_select_count leaves the number of such entries in *count (a device uint32) and the per-chunk
+ * counts in the workspace; after reading the count the caller passes the same scores and workspace, untouched, to
+ * siirl_range_select_write together with a list of `capacity` >= count entries (nothing is written beyond capacity).
+ * n < 2^32.  workspace: siirl_range_select_workspace_bytes(), 4-byte aligned.
+ * Replaces: siirl/dag_worker/core_algos.py:974-975.
+ */
+size_t siirl_range_select_workspace_bytes(void);
+int siirl_range_select_count(const float* scores, int64_t n, float lower_open, float upper_open, uint32_t* count,
+                             void* workspace, size_t workspace_bytes, siirl_stream_t stream);
+int siirl_range_select_write(const float* scores, int64_t n, float lower_open, float upper_open, const void* workspace,
+                             int64_t* indices, int64_t capacity, siirl_stream_t stream);
 
 /*
  * siirl_actor_loss_fwd for the two covariance losses: the same composition (entropy, KL and drift terms, ratio

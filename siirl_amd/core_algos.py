@@ -578,12 +578,11 @@ def _clip_cov_dropped(old_log_prob, log_prob, advantages, response_mask, lo, hi,
     cov, stats = _OPS.cov_scores(old, lp, adv, m, LOSS_CLIP_COV, lo, hi)
     st = stats.tolist()
     clip_num = max(int(clip_cov_ratio * (st[1] + st[5])), 1)  # the mask sum, exact in double
-    cand = torch.nonzero((cov < ub) & (cov > lb) & (m > 0))
+    cand = _OPS.range_indices(cov, lb, ub)  # flat indices, ascending = row-major order; the second host sync
     aux = torch.zeros_like(cov)
     if len(cand) > 0:
         perm = torch.randperm(len(cand))
-        chosen = cand[perm[: min(clip_num, len(cand))].to(dev)]
-        aux[chosen[:, 0], chosen[:, 1]] = 1.0
+        aux.reshape(-1)[cand[perm[: min(clip_num, len(cand))].to(dev)]] = 1.0
     return aux
 
 

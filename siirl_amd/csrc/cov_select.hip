@@ -274,6 +274,86 @@ __global__ __launch_bounds__(kSelThreads) void select_mark_kernel(const float* _
   }
 }
 
+// ------------------------------------------------------------------------------ entries inside an open interval
+
+// Clip-Cov's candidate list (siirl/dag_worker/core_algos.py:974-975: nonzero of lb < cov < ub): first the number of
+// such entries per chunk, then their flat indices in ascending order, each chunk writing behind the chunks before it
+// and ranking its own entries tile by tile with a scan.
+__global__ __launch_bounds__(kSelThreads) void range_count_kernel(const float* __restrict__ x, int64_t n, int64_t per, int vec,
+                                                                  float lo_open, float hi_open,
+                                                                  uint32_t* __restrict__ counts) {
+  __shared__ double sh[kSelThreads / kWave + 1];
+  int64_t lo, hi;
+  chunk_of(n, per, lo, hi);
+  uint32_t c = 0;
+  for (int64_t i = lo + 4 * (int64_t)threadIdx.x; i < hi; i += kTile) {
+    float v[4];
+    const int m = load4(x, i, hi, vec != 0, v);
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (e < m) c += (v[e] > lo_open && v[e] < hi_open) ? 1u : 0u;
+  }
+  const double total = block_sum((double)c, sh);
+  if (threadIdx.x == 0) counts[blockIdx.x] = (uint32_t)total;
+}
+// counts[grid] = the sum of the chunk counts (one workgroup)
+__global__ __launch_bounds__(kSelGrid) void range_total_kernel(uint32_t* __restrict__ counts, int grid,
+                                                               uint32_t* __restrict__ total) {
+  __shared__ double sh[kSelGrid / kWave + 1];
+  const double t = block_sum(threadIdx.x < (unsigned)grid ? (double)counts[threadIdx.x] : 0.0, sh);
+  if (threadIdx.x == 0) {
+    counts[grid] = (uint32_t)t;
+    *total = (uint32_t)t;
+  }
+}
+__global__ __launch_bounds__(kSelThreads) void range_write_kernel(const float* __restrict__ x, int64_t n, int64_t per, int vec,
+                                                                  float lo_open, float hi_open,
+                                                                  const uint32_t* __restrict__ counts,
+                                                                  int64_t* __restrict__ indices, int64_t capacity) {
+  __shared__ uint32_t wsum[kSelThreads / kWave];
+  __shared__ uint32_t run;
+  uint32_t base = 0;
+  for (int b = 0; b < (int)blockIdx.x; ++b) base += counts[b];
+  if (threadIdx.x == 0) run = base;
+  __syncthreads();
+  int64_t lo, hi;
+  chunk_of(n, per, lo, hi);
+  const int lane = threadIdx.x & (kWave - 1), w = threadIdx.x / kWave;
+  for (int64_t t0 = lo; t0 < hi; t0 += kTile) {  // every thread runs every tile: the barriers are uniform
+    const int64_t i = t0 + 4 * (int64_t)threadIdx.x;
+    float v[4];
+    const int m = i < hi ? load4(x, i, hi, vec != 0, v) : 0;
+    bool in[4];
+    uint32_t mine = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      in[e] = e < m && v[e] > lo_open && v[e] < hi_open;
+      mine += in[e] ? 1u : 0u;
+    }
+    uint32_t incl = mine;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+      const uint32_t dn = __shfl_up(incl, o, kWave);
+      if (lane >= o) incl += dn;
+    }
+    if (lane == kWave - 1) wsum[w] = incl;
+    __syncthreads();
+    uint32_t r = run + incl - mine;
+    for (int q = 0; q < w; ++q) r += wsum[q];
+    uint32_t tile_total = 0;
+    for (int q = 0; q < kSelThreads / kWave; ++q) tile_total += wsum[q];
+    __syncthreads();
+    if (threadIdx.x == 0) run += tile_total;
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (in[e]) {
+        if ((int64_t)r < capacity) indices[r] = i + e;  // (the scores changed since they were counted: no write past the end)
+        ++r;
+      }
+  }
+}
+
 struct SelWs {
   size_t part, state, ties, total;
 };
@@ -290,6 +370,54 @@ SelWs sel_ws() {
 }  // namespace siirl
 
 using namespace siirl;
+
+// chunk layout shared by the interval pair: `per` entries per workgroup, `grid` workgroups
+static void range_chunks(int64_t n, int64_t& per, int& grid) {
+  per = ((n + kSelGrid - 1) / kSelGrid + kTile - 1) / kTile * kTile;
+  grid = (int)((n + per - 1) / per);
+}
+
+extern "C" size_t siirl_range_select_workspace_bytes(void) { return (size_t)(kSelGrid + 1) * sizeof(uint32_t); }
+
+extern "C" int siirl_range_select_count(const float* scores, int64_t n, float lower_open, float upper_open,
+                                        uint32_t* count, void* workspace, size_t workspace_bytes, siirl_stream_t stream) {
+  SIIRL_REQUIRE(n >= 0 && n < (1LL << 32), "n=%lld out of range (below 2^32)", (long long)n);
+  SIIRL_REQUIRE(count != nullptr && (n == 0 || scores != nullptr), "NULL operand");
+  if (workspace == nullptr || workspace_bytes < siirl_range_select_workspace_bytes())
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes,
+                siirl_range_select_workspace_bytes());
+  SIIRL_REQUIRE(((uintptr_t)workspace & 3) == 0 && ((uintptr_t)count & 3) == 0, "workspace and count must be 4-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  uint32_t* counts = (uint32_t*)workspace;
+  int64_t per = kTile;
+  int grid = 0;
+  if (n > 0) {
+    range_chunks(n, per, grid);
+    const int vec = ((uintptr_t)scores & 15) == 0;
+    range_count_kernel<<<dim3((unsigned)grid), dim3(kSelThreads), 0, st>>>(scores, n, per, vec, lower_open, upper_open, counts);
+    SIIRL_LAUNCH_CHECK("range_count_kernel");
+  }
+  range_total_kernel<<<1, dim3(kSelGrid), 0, st>>>(counts, grid, count);
+  SIIRL_LAUNCH_CHECK("range_total_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_range_select_write(const float* scores, int64_t n, float lower_open, float upper_open,
+                                        const void* workspace, int64_t* indices, int64_t capacity,
+                                        siirl_stream_t stream) {
+  SIIRL_REQUIRE(n >= 0 && n < (1LL << 32) && capacity >= 0, "n=%lld (below 2^32) or capacity=%lld out of range",
+                (long long)n, (long long)capacity);
+  if (n == 0 || capacity == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(scores && workspace && indices, "NULL operand");
+  int64_t per;
+  int grid;
+  range_chunks(n, per, grid);
+  const int vec = ((uintptr_t)scores & 15) == 0;
+  range_write_kernel<<<dim3((unsigned)grid), dim3(kSelThreads), 0, (hipStream_t)stream>>>(
+      scores, n, per, vec, lower_open, upper_open, (const uint32_t*)workspace, indices, capacity);
+  SIIRL_LAUNCH_CHECK("range_write_kernel");
+  return SIIRL_OK;
+}
 
 extern "C" size_t siirl_topk_mark_workspace_bytes(void) { return sel_ws().total; }
 

@@ -752,8 +752,8 @@ __global__ __launch_bounds__(kThreads) void cov_stats_kernel(const double* __res
     }
   }
 }
-// cov[b, t] = (A - mean A) * (lp - mean lp), minus infinity where m <= 0 (kl_cov: m > 0 selects; clip_cov: m == 0 is
-// excluded) and, for clip_cov, where the PPO clip already bites (l2 > l1 under a positive mask)
+// cov[b, t] = (A - mean A) * (lp - mean lp), minus infinity where the mask is not positive (neither loss ever picks
+// such a token) and, for clip_cov, where the PPO clip already bites (l2 > l1)
 __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __restrict__ old_lp, const float* __restrict__ lp,
                                                               const float* __restrict__ adv, const void* mask,
                                                               int mask_dtype, int64_t n, int vec, int clip_mode, float lo,
@@ -776,7 +776,7 @@ __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __res
       if (clip_mode) {
         const float r = expf(l - o4.v[e]);
         const float l1 = -a * r, l2 = -a * clampf(r, lo, hi);
-        if (m == 0.f || (l2 > l1 && m > 0.f)) c = -__builtin_inff();
+        if (!(m > 0.f) || l2 > l1) c = -__builtin_inff();
       } else if (!(m > 0.f)) {
         c = -__builtin_inff();
       }

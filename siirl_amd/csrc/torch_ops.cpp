@@ -802,6 +802,26 @@ Tensor topk_mark(const Tensor& scores, int64_t k, double value) {
   return marks;
 }
 
+// int64 flat indices, ascending, of the scores inside the open interval (lower, upper).  One host sync: the length
+// of the list, as torch.nonzero has.
+Tensor range_indices(const Tensor& scores, double lower, double upper) {
+  require_f32c(scores, "scores");
+  const int64_t n = scores.numel();
+  const size_t nws = siirl_range_select_workspace_bytes();
+  Tensor ws = at::empty({(int64_t)nws + 4}, scores.options().dtype(at::kByte));  // chunk counts, then the total
+  uint32_t* count = reinterpret_cast<uint32_t*>(ptr<char>(ws) + nws);
+  DeviceGuard guard(scores.device());
+  siirl_stream_t st = stream_of(scores);
+  check_rc(siirl_range_select_count(ptr<float>(scores), n, (float)lower, (float)upper, count, ptr(ws), nws, st),
+           "siirl_range_select_count");
+  const int64_t total = (int64_t)ws.narrow(0, (int64_t)nws, 4).view(at::kInt).item<int32_t>() & 0xffffffffLL;
+  Tensor idx = at::empty({total}, scores.options().dtype(at::kLong));
+  check_rc(siirl_range_select_write(ptr<float>(scores), n, (float)lower, (float)upper, ptr(ws), ptr<int64_t>(idx),
+                                    total, st),
+           "siirl_range_select_write");
+  return idx;
+}
+
 constexpr int kActorOuts = 13;  // SIIRL_OUT_LOSS .. SIIRL_OUT_DRIFT_LOSS
 
 // One fused forward (partials + finish) and one elementwise backward for the whole micro-batch loss.  The 13 scalars
@@ -1205,6 +1225,7 @@ TORCH_LIBRARY(siirl_hip, m) {
   m.def("cov_scores(Tensor? old_log_prob, Tensor log_prob, Tensor advantages, Tensor mask, int loss_mode, "
         "float clip_low, float clip_high) -> (Tensor, Tensor)");
   m.def("topk_mark(Tensor scores, int k, float value) -> Tensor");
+  m.def("range_indices(Tensor scores, float lower, float upper) -> Tensor");
   m.def("kl_penalty_fwd(Tensor log_prob, Tensor ref_log_prob, int kl_mode) -> Tensor");
   m.def("kl_penalty_bwd(Tensor g, Tensor log_prob, Tensor ref_log_prob, int kl_mode, bool straight_through, "
         "bool need_log_prob, bool need_ref) -> (Tensor, Tensor)");
@@ -1246,6 +1267,7 @@ TORCH_LIBRARY_IMPL(siirl_hip, CUDA, m) {
   m.impl("policy_loss_bwd", &policy_loss_bwd);
   m.impl("cov_scores", &cov_scores);
   m.impl("topk_mark", &topk_mark);
+  m.impl("range_indices", &range_indices);
   m.impl("kl_penalty_fwd", &kl_penalty_fwd);
   m.impl("kl_penalty_bwd", &kl_penalty_bwd);
   m.impl("fused_linear_logprob_entropy_fwd", &fused_linear_fwd);

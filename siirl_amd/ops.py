@@ -146,6 +146,12 @@ def _(scores, k, value):
     return scores.new_empty(scores.shape, dtype=torch.float32)
 
 
+@_fake(f"{_NS}::range_indices")
+def _(scores, lower, upper):
+    # the length of the list depends on the data: an unbacked size, as for torch.nonzero
+    return scores.new_empty(torch.library.get_ctx().new_dynamic_size(), dtype=torch.int64)
+
+
 @_fake(f"{_NS}::kl_penalty_fwd")
 def _(log_prob, ref_log_prob, kl_mode):
     return log_prob.new_empty(log_prob.shape, dtype=torch.float32)

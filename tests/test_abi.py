@@ -47,7 +47,8 @@ def test_every_entry_point_cites_the_reference():
             assert "no counterpart in the reference" in text[text.rfind("/*", 0, pos):pos]
             continue
         if n in ("siirl_hip_abi_version", "siirl_hip_last_error", "siirl_agg_loss_bwd", "siirl_actor_loss_bwd",
-                 "siirl_kl_penalty_bwd", "siirl_masked_reduce_bwd", "siirl_actor_loss_cov_bwd") or n.endswith("_workspace_bytes") or n.endswith("_logits_bytes"):
+                 "siirl_kl_penalty_bwd", "siirl_masked_reduce_bwd", "siirl_actor_loss_cov_bwd",
+                 "siirl_range_select_write") or n.endswith("_workspace_bytes") or n.endswith("_logits_bytes"):
             continue  # utilities and backward halves documented with their forward
         pos = text.index(n + "(")
         comment = text[text.rfind("/*", 0, pos):pos]
@@ -108,6 +109,11 @@ def test_argument_validation_without_gpu():
     assert h.siirl_topk_mark(p, 8, 2, 1.0, q2, p, 8, None) == -4
     assert h.siirl_topk_mark(p, 0, 0, 1.0, q2, None, 0, None) == 0  # nothing to mark: no workspace, no launch
     assert h.siirl_topk_mark_workspace_bytes() > 0
+    assert h.siirl_range_select_count(p, 8, 0.0, 1.0, None, p, 1 << 20, None) == -1  # no place for the count
+    assert h.siirl_range_select_count(p, 8, 0.0, 1.0, p, p, 8, None) == -4
+    assert h.siirl_range_select_write(p, 8, 0.0, 1.0, p, None, 4, None) == -1
+    assert h.siirl_range_select_write(p, 8, 0.0, 1.0, p, None, 0, None) == 0  # an empty list: nothing to write
+    assert h.siirl_range_select_workspace_bytes() > 0
     assert h.siirl_value_loss_fwd(p, p, p, p, L.F32, 2, 4, 0.5, 7, p, p, p, 1 << 20, None) == -1
     assert h.siirl_gae_advantage_return(p, p, p, L.F32, 2, 4, 1.0, 1.0, p, p, p, p, 8, 0, None) == -1  # adv == returns
     q2 = ctypes.c_void_p(p.value + 64)

@@ -7,7 +7,7 @@ import siirl_amd.ops  # noqa: F401  (registers the ops)
 
 OPS = ("logprob_entropy_fwd", "logprob_entropy_bwd", "logprob_entropy_bwd_", "grpo_advantage", "group_keep_mask",
        "agg_loss_fwd", "agg_loss_bwd", "masked_reduce_fwd", "masked_reduce_bwd", "policy_loss_fwd", "policy_loss_bwd",
-       "cov_scores", "topk_mark", "kl_penalty_fwd", "kl_penalty_bwd",
+       "cov_scores", "topk_mark", "range_indices", "kl_penalty_fwd", "kl_penalty_bwd",
        "fused_linear_logprob_entropy_fwd", "fused_linear_logprob_entropy_bwd")
 
 

@@ -122,3 +122,25 @@ def test_sweep_random_selections():
         k = int(rng.integers(0, n + 1)) if case % 3 else int(min(n, max(1, n // 5000)))
         got = _run(torch.from_numpy(x), k)
         assert np.array_equal(got, _expected(x, k)), (case, n, kind, k)
+
+
+# ------------------------------------------------------------------------------------------ entries inside an interval
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 4096, 4097, 250_001, 3_000_003])
+def test_range_indices_equals_nonzero(n):
+    """``range_indices`` (Clip-Cov's candidate list, reference ``core_algos.py:974-975``) against torch.nonzero of the
+    same two comparisons: same indices in the same (ascending) order, bit-exact."""
+    g = torch.Generator().manual_seed(n + 1)
+    x = torch.randn(n, generator=g) * 2
+    if n > 10:
+        x[torch.rand(n, generator=g) < 0.3] = float("-inf")
+        x[3], x[7] = float("nan"), float("inf")
+    xd = x.to(DEV)
+    for lo, hi in ((1.0, 5.0), (-0.5, 0.5), (10.0, 20.0), (float("-inf"), float("inf")), (0.0, 0.0)):
+        got = torch.ops.siirl_hip.range_indices(xd, lo, hi)
+        want = torch.nonzero((x < hi) & (x > lo)).reshape(-1)
+        assert got.dtype == torch.int64 and torch.equal(got.cpu(), want), (n, lo, hi, got.numel(), want.numel())
+    m = torch.randn(37, 129, generator=g).to(DEV)  # a matrix: flat, row-major indices
+    got = torch.ops.siirl_hip.range_indices(m, 0.2, 1.1)
+    assert torch.equal(got.cpu(), torch.nonzero(((m < 1.1) & (m > 0.2)).reshape(-1).cpu()).reshape(-1))

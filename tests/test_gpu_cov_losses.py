@@ -334,3 +334,42 @@ def test_sweep_covariance_losses():
         for a, b in zip(got[1:], want[1:]):
             _close(a, b, what=(case, B, L, str(mdt), agg, with_w, pl))
         assert torch.allclose(lpd.grad.cpu().double(), gwant, rtol=1e-5, atol=1e-7), (case, "clip_cov grad")
+
+
+@pytest.mark.parametrize("mode", ["kl_cov", "clip_cov"])
+def test_cov_losses_accept_other_ranks_and_dtypes(mode):
+    """1-D and 3-D operands, a bf16 log-prob (its gradient comes back in bf16), a bool mask that is a non-contiguous
+    view: same value as the 2-D float32 call on the same numbers."""
+    import siirl_amd.core_algos as CA
+
+    old, lp, A, m, w = _case(91, 6, 40, torch.bool, spread=0.2)
+    lp = lp.to(torch.bfloat16).float()  # representable in bf16, so both calls see the same numbers
+    cfg = _cfg(kl_cov_ratio=0.05, ppo_kl_coef=0.5, clip_cov_ratio=0.03, clip_cov_lb=0.2, clip_cov_ub=4.0)
+    fn = CA.compute_policy_loss_kl_cov if mode == "kl_cov" else CA.compute_policy_loss_clip_cov
+
+    def call(o, l, a, k):
+        torch.manual_seed(13)
+        l = l.clone().requires_grad_(True)
+        out = fn(o, l, a, k, "token-mean", cfg)
+        out[0].backward()
+        return [float(v) for v in out], l.grad
+
+    base, g2 = call(old.to(DEV), lp.to(DEV), A.to(DEV), m.to(DEV))
+    # 3-D: [2, 3, 40] is the same six rows
+    v3, g3 = call(old.reshape(2, 3, 40).to(DEV), lp.reshape(2, 3, 40).to(DEV), A.reshape(2, 3, 40).to(DEV),
+                  m.reshape(2, 3, 40).to(DEV))
+    assert v3 == base and g3.shape == (2, 3, 40) and torch.equal(g3.reshape(6, 40), g2)
+    # bf16 log-prob
+    vb, gb = call(old.to(DEV), lp.to(DEV).to(torch.bfloat16), A.to(DEV), m.to(DEV))
+    assert vb == base and gb.dtype == torch.bfloat16
+    assert torch.allclose(gb.float(), g2, rtol=2 ** -7, atol=1e-9)
+    # the mask as a non-contiguous view
+    wide = torch.zeros(6, 80, dtype=torch.bool, device=DEV)
+    wide[:, ::2] = m.to(DEV)
+    vn, gn = call(old.to(DEV), lp.to(DEV), A.to(DEV), wide[:, ::2])
+    assert vn == base and torch.equal(gn, g2)
+    # one row (token-mean does not care how the tokens are cut into rows... but the covariance means do not either)
+    v1, g1 = call(old.reshape(-1).to(DEV), lp.reshape(-1).to(DEV), A.reshape(-1).to(DEV), m.reshape(-1).to(DEV))
+    assert g1.shape == (240,)
+    for a, b in zip(v1, base):
+        assert abs(a - b) <= 1e-6 + 1e-5 * abs(b)

@@ -125,21 +125,21 @@ __global__ __launch_bounds__(kStream) void loss_partials_kernel(LossArgs a, cons
   acc[P_RMAX] = -__builtin_inff();
   const float seq_s = (kind == KIND_GSPO) ? row_s[b] : 0.f;
 
-  const bool vec = a.vec != 0;
+  const bool vec = a.vec != 0, nt = a.nt != 0;
   for (int gq = threadIdx.x; gq < kSeg / 4; gq += kStream) {
     const int64_t t = t0 + 4 * gq;
     if (t >= a.L) break;
     const int nv = (int)((a.L - t) < 4 ? (a.L - t) : 4);
     const int64_t idx0 = b * a.L + t;
-    const Quad m4 = load_mask_quad(a.mask, a.mask_dtype, idx0, vec, nv);
-    const Quad lp4 = load_quad(a.lp, idx0, vec, nv, 0.f);
+    const Quad m4 = load_mask_quad(a.mask, a.mask_dtype, idx0, vec, nv, nt);
+    const Quad lp4 = load_quad(a.lp, idx0, vec, nv, 0.f, nt);
     const bool agg_only = kind == KIND_AGG;
-    const Quad old4 = agg_only ? const_quad(0.f) : load_quad(a.old_lp, idx0, vec, nv, 0.f);
-    const Quad adv4 = agg_only ? const_quad(0.f) : load_quad(a.adv, idx0, vec, nv, 0.f);
-    const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
-    const Quad ent4 = a.ent ? load_quad(a.ent, idx0, vec, nv, 0.f) : const_quad(0.f);
-    const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
-    const Quad aux4 = ((KIND < 0 || KIND >= KIND_KL_COV) && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
+    const Quad old4 = agg_only ? const_quad(0.f) : load_quad(a.old_lp, idx0, vec, nv, 0.f, nt);
+    const Quad adv4 = agg_only ? const_quad(0.f) : load_quad(a.adv, idx0, vec, nv, 0.f, nt);
+    const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f, nt) : const_quad(1.f);
+    const Quad ent4 = a.ent ? load_quad(a.ent, idx0, vec, nv, 0.f, nt) : const_quad(0.f);
+    const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f, nt) : const_quad(0.f);
+    const Quad aux4 = ((KIND < 0 || KIND >= KIND_KL_COV) && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f, nt) : const_quad(0.f);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (e >= nv) break;
@@ -435,7 +435,7 @@ __global__ __launch_bounds__(kStream) void loss_bwd_kernel(LossArgs a, const flo
   const float mtotal = saved_out[O_MTOTAL];
   const float mrow = row_msum[b];
   const float seq_s = (kind == KIND_GSPO || kind == KIND_GEO) ? row_s[b] : 0.f;
-  const bool vec = a.vec != 0;
+  const bool vec = a.vec != 0, nt = a.nt != 0;
   const bool agg_only = kind == KIND_AGG;
   // aggregation weights are m * c with c fixed for the row: one division per thread instead of up to three per token
   const AggCoef w_pg = agg_coef(a.agg_mode, mtotal, mrow, a.B, a.L);
@@ -446,20 +446,20 @@ __global__ __launch_bounds__(kStream) void loss_bwd_kernel(LossArgs a, const flo
     if (t >= a.L) break;
     const int nv = (int)((a.L - t) < 4 ? (a.L - t) : 4);
     const int64_t idx0 = b * a.L + t;
-    const Quad m4 = load_mask_quad(a.mask, a.mask_dtype, idx0, vec, nv);
+    const Quad m4 = load_mask_quad(a.mask, a.mask_dtype, idx0, vec, nv, nt);
     Quad dlp, dent;
     if (agg_only) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) dlp.v[e] = g * w_pg(m4.v[e]);
-      store_quad(d_lp, idx0, vec, nv, dlp);
+      store_quad(d_lp, idx0, vec, nv, dlp, nt);
       continue;
     }
-    const Quad lp4 = load_quad(a.lp, idx0, vec, nv, 0.f);
-    const Quad old4 = load_quad(a.old_lp, idx0, vec, nv, 0.f);
-    const Quad adv4 = load_quad(a.adv, idx0, vec, nv, 0.f);
-    const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f) : const_quad(1.f);
-    const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f) : const_quad(0.f);
-    const Quad aux4 = ((KIND < 0 || KIND >= KIND_KL_COV) && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f) : const_quad(0.f);
+    const Quad lp4 = load_quad(a.lp, idx0, vec, nv, 0.f, nt);
+    const Quad old4 = load_quad(a.old_lp, idx0, vec, nv, 0.f, nt);
+    const Quad adv4 = load_quad(a.adv, idx0, vec, nv, 0.f, nt);
+    const Quad isw4 = a.isw ? load_quad(a.isw, idx0, vec, nv, 1.f, nt) : const_quad(1.f);
+    const Quad ref4 = a.ref ? load_quad(a.ref, idx0, vec, nv, 0.f, nt) : const_quad(0.f);
+    const Quad aux4 = ((KIND < 0 || KIND >= KIND_KL_COV) && a.aux) ? load_quad(a.aux, idx0, vec, nv, 0.f, nt) : const_quad(0.f);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float m = m4.v[e], lp = lp4.v[e];
@@ -479,8 +479,8 @@ __global__ __launch_bounds__(kStream) void loss_bwd_kernel(LossArgs a, const flo
       }
       dlp.v[e] = g * d;
     }
-    store_quad(d_lp, idx0, vec, nv, dlp);
-    if (a.ent && d_ent) store_quad(d_ent, idx0, vec, nv, dent);
+    store_quad(d_lp, idx0, vec, nv, dlp, nt);
+    if (a.ent && d_ent) store_quad(d_ent, idx0, vec, nv, dent, nt);
   }
 }
 
@@ -797,6 +797,10 @@ void set_vec(LossArgs& a, const void* o1 = nullptr, const void* o2 = nullptr) {
   const bool mask_ok = ((uintptr_t)a.mask & (msz * 4 > 16 ? 15 : msz * 4 - 1)) == 0;
   a.vec = (a.L % 4 == 0) && mask_ok && ok16(a.old_lp) && ok16(a.lp) && ok16(a.adv) && ok16(a.isw) && ok16(a.ent) &&
           ok16(a.ref) && ok16(a.aux) && ok16(o1) && ok16(o2);
+  // bytes one pass reads: ordinary accesses while they fit the memory-side cache, non-temporal ones beyond
+  const int n_f32 = (a.old_lp != nullptr) + (a.lp != nullptr) + (a.adv != nullptr) + (a.isw != nullptr) + (a.ent != nullptr) +
+                    (a.ref != nullptr) + (a.aux != nullptr);
+  a.nt = streams_past_cache((double)a.B * (double)a.L * (double)(4 * n_f32 + (a.mask ? msz : 0)));
 }
 
 size_t ws_bytes_of(int64_t B, int64_t L) {

@@ -11,6 +11,11 @@
 
 // Cache hints of the [B, L] streaming kernels.  Measured at [5488, 8192] fp32 with an int64 mask (actor loss forward +
 // backward): non-temporal loads 0.467 -> 0.428 ms, non-temporal stores of the gradient a further 0.428 -> 0.420 ms.
+// That is for operands several times the part's 256 MB memory-side cache.  A pass that reads less than
+// kCacheResidentBytes uses ordinary accesses instead (`nt` of the helpers below, decided on the host per launch):
+// what the forward has read is then still cached when the backward reads it again -- forward + backward at
+// [1024, 8192] (192 MiB per pass) 99.8 -> 90.3 us, at [512, 8192] 55.3 -> 50.8 us; at [2048, 8192] (384 MiB) the
+// non-temporal accesses are the faster ones again (166 against 183 us).
 #ifndef SIIRL_LOSS_NT_STORE
 #define SIIRL_LOSS_NT_STORE 1
 #endif
@@ -20,6 +25,9 @@
 
 namespace siirl {
 namespace tok {
+
+constexpr double kCacheResidentBytes = 300.0 * 1048576.0;
+inline bool streams_past_cache(double bytes_per_pass) { return bytes_per_pass > kCacheResidentBytes; }
 
 struct LossArgs {
   const float* old_lp;   // [B,L] or null (kind == KIND_AGG)
@@ -42,6 +50,7 @@ struct LossArgs {
   int64_t B, L;
   int nseg;
   int vec;  // L % 4 == 0 and every operand 16-byte aligned: tokens are moved four at a time
+  int nt;   // the operands of a pass exceed the memory-side cache: non-temporal loads and stores
 };
 enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6,
        KIND_KL_COV = 7, KIND_CLIP_COV = 8 };
@@ -63,16 +72,17 @@ __device__ __forceinline__ float contrib(float v, float m, int agg) {
 struct Quad {
   float v[4];
 };
-__device__ __forceinline__ Quad load_quad(const float* __restrict__ p, int64_t idx, bool vec, int nv, float fill) {
+__device__ __forceinline__ Quad load_quad(const float* __restrict__ p, int64_t idx, bool vec, int nv, float fill,
+                                          bool nt = SIIRL_LOSS_NT_LOAD != 0) {
   Quad q;
   if (vec) {
-#if SIIRL_LOSS_NT_LOAD
-    const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + idx));
-    q.v[0] = u2f(t.x); q.v[1] = u2f(t.y); q.v[2] = u2f(t.z); q.v[3] = u2f(t.w);
-#else
-    const float4 t = *reinterpret_cast<const float4*>(p + idx);
-    q.v[0] = t.x; q.v[1] = t.y; q.v[2] = t.z; q.v[3] = t.w;
-#endif
+    if (SIIRL_LOSS_NT_LOAD && nt) {
+      const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p + idx));
+      q.v[0] = u2f(t.x); q.v[1] = u2f(t.y); q.v[2] = u2f(t.z); q.v[3] = u2f(t.w);
+    } else {
+      const float4 t = *reinterpret_cast<const float4*>(p + idx);
+      q.v[0] = t.x; q.v[1] = t.y; q.v[2] = t.z; q.v[3] = t.w;
+    }
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? p[idx + e] : fill;
@@ -80,19 +90,20 @@ __device__ __forceinline__ Quad load_quad(const float* __restrict__ p, int64_t i
   return q;
 }
 __device__ __forceinline__ Quad const_quad(float c) { return Quad{{c, c, c, c}}; }
-__device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t idx, bool vec, int nv) {
+__device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t idx, bool vec, int nv,
+                                               bool nt = SIIRL_LOSS_NT_LOAD != 0) {
   Quad q;
   if (vec && dt == SIIRL_I64) {
-#if SIIRL_LOSS_NT_LOAD
-    const u32x4 ra = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const int64_t*)p + idx));
-    const u32x4 rb = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const int64_t*)p + idx) + 1);
     longlong2 a, b;
-    a.x = (int64_t)(((uint64_t)ra.y << 32) | ra.x); a.y = (int64_t)(((uint64_t)ra.w << 32) | ra.z);
-    b.x = (int64_t)(((uint64_t)rb.y << 32) | rb.x); b.y = (int64_t)(((uint64_t)rb.w << 32) | rb.z);
-#else
-    const longlong2 a = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[0];
-    const longlong2 b = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[1];
-#endif
+    if (SIIRL_LOSS_NT_LOAD && nt) {
+      const u32x4 ra = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const int64_t*)p + idx));
+      const u32x4 rb = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>((const int64_t*)p + idx) + 1);
+      a.x = (int64_t)(((uint64_t)ra.y << 32) | ra.x); a.y = (int64_t)(((uint64_t)ra.w << 32) | ra.z);
+      b.x = (int64_t)(((uint64_t)rb.y << 32) | rb.x); b.y = (int64_t)(((uint64_t)rb.w << 32) | rb.z);
+    } else {
+      a = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[0];
+      b = reinterpret_cast<const longlong2*>((const int64_t*)p + idx)[1];
+    }
     // masks hold small integers: when every value in the wave fits 32 bits, one v_cvt_f32_i32 each replaces the
     // 64-bit conversion sequence (the wave-uniform test keeps the general path out of the way, not out of the code)
     const int32_t l0 = (int32_t)a.x, l1 = (int32_t)a.y, l2 = (int32_t)b.x, l3 = (int32_t)b.y;
@@ -107,20 +118,20 @@ __device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t id
     q.v[0] = (float)(u & 0xffu); q.v[1] = (float)((u >> 8) & 0xffu); q.v[2] = (float)((u >> 16) & 0xffu);
     q.v[3] = (float)(u >> 24);
   } else if (vec && dt == SIIRL_F32) {
-    q = load_quad((const float*)p, idx, true, 4, 0.f);
+    q = load_quad((const float*)p, idx, true, 4, 0.f, nt);
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e) q.v[e] = e < nv ? load_mask(p, dt, idx + e) : 0.f;
   }
   return q;
 }
-__device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q) {
+__device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q,
+                                           bool nt = SIIRL_LOSS_NT_STORE != 0) {
   if (vec) {
-#if SIIRL_LOSS_NT_STORE
-    __builtin_nontemporal_store(u32x4{f2u(q.v[0]), f2u(q.v[1]), f2u(q.v[2]), f2u(q.v[3])}, reinterpret_cast<u32x4*>(p + idx));
-#else
-    *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
-#endif
+    if (SIIRL_LOSS_NT_STORE && nt)
+      __builtin_nontemporal_store(u32x4{f2u(q.v[0]), f2u(q.v[1]), f2u(q.v[2]), f2u(q.v[3])}, reinterpret_cast<u32x4*>(p + idx));
+    else
+      *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e)

@@ -15,6 +15,13 @@ constexpr int kWave = 64;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+// The part has a 256 MB memory-side cache in front of the HBM.  A tensor that a later launch reads again is read
+// and written with ordinary accesses while one pass over it moves no more than this many bytes (the cache and a
+// little more: the measured break-even lies between 260 and 375 MiB), and with non-temporal ones beyond, where
+// ordinary accesses would only evict each other.
+constexpr double kCacheResidentBytes = 300.0 * 1048576.0;
+inline bool streams_past_cache(double bytes_per_pass) { return bytes_per_pass > kCacheResidentBytes; }
+
 // ---------------------------------------------------------------------------------- host side
 
 // Records a message for siirl_hip_last_error() on this thread and returns `code`.

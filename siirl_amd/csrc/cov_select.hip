@@ -42,10 +42,20 @@ __device__ __forceinline__ void chunk_of(int64_t n, int64_t per, int64_t& lo, in
   if (lo > n) lo = n;
 }
 
+// Access mode of a launch: bit 0 = 16-byte accesses (aligned operands), bit 1 = non-temporal loads.  The passes of
+// one call read the same vector up to five times: one that fits the memory-side cache is read with ordinary loads
+// so that the later passes find it there (three histogram passes over 180 MB: 94.5 -> 89.6 us), a larger one
+// streams past the caches.  The marks are always stored non-temporally: ordinary stores made this kernel 9 us
+// faster and the loss kernel that runs next 33 us slower (it then shares the memory with their write-back).
+constexpr int kVec = 1, kNt = 2;
+__device__ __forceinline__ u32x4 load16(const float* __restrict__ p, bool nt) {
+  return nt ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)) : *reinterpret_cast<const u32x4*>(p);
+}
+
 // four consecutive scores from index i (a multiple of 4 when vec); entries at or beyond hi are reported as absent
-__device__ __forceinline__ int load4(const float* __restrict__ x, int64_t i, int64_t hi, bool vec, float (&v)[4]) {
-  if (i + 4 <= hi && vec) {
-    const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + i));
+__device__ __forceinline__ int load4(const float* __restrict__ x, int64_t i, int64_t hi, int mode, float (&v)[4]) {
+  if (i + 4 <= hi && (mode & kVec)) {
+    const u32x4 t = load16(x + i, (mode & kNt) != 0);
     v[0] = u2f(t.x); v[1] = u2f(t.y); v[2] = u2f(t.z); v[3] = u2f(t.w);
     return 4;
   }
@@ -63,7 +73,7 @@ __device__ __forceinline__ int load4(const float* __restrict__ x, int64_t i, int
 // 9..0 of the keys whose top 22 bits do.
 template <int PASS>
 __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const float* __restrict__ x, int64_t n, int64_t per,
-                                                                  int vec, const SelState* __restrict__ st,
+                                                                  int mode, const SelState* __restrict__ st,
                                                                   uint32_t* __restrict__ ghist) {
   __shared__ uint32_t hist[kCopies][kBins];
   for (int i = threadIdx.x; i < kCopies * kBins; i += kSelThreads) (&hist[0][0])[i] = 0u;
@@ -100,12 +110,12 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const float* _
   // whole tiles, four 16-byte loads in flight per thread; then what is left, one (possibly partial) vector at a time
   constexpr int kInFlight = 4;
   int64_t i = lo + 4 * (int64_t)threadIdx.x;
-  if (vec) {
+  if (mode & kVec) {
+    const bool nt = (mode & kNt) != 0;
     for (; i + (int64_t)(kInFlight - 1) * kTile + 4 <= hi; i += (int64_t)kInFlight * kTile) {
       u32x4 t[kInFlight];
 #pragma unroll
-      for (int u = 0; u < kInFlight; ++u)
-        t[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(x + i + (int64_t)u * kTile));
+      for (int u = 0; u < kInFlight; ++u) t[u] = load16(x + i + (int64_t)u * kTile, nt);
 #pragma unroll
       for (int u = 0; u < kInFlight; ++u) {
         count(u2f(t[u].x));
@@ -117,7 +127,7 @@ __global__ __launch_bounds__(kSelThreads) void select_hist_kernel(const float* _
   }
   for (; i < hi; i += kTile) {
     float v[4];
-    const int c = load4(x, i, hi, vec != 0, v);
+    const int c = load4(x, i, hi, mode, v);
     if (c > 0) count(v[0]);
     if (c > 1) count(v[1]);
     if (c > 2) count(v[2]);
@@ -177,7 +187,7 @@ __global__ __launch_bounds__(kSelThreads) void select_scan_kernel(const uint32_t
 
 // per chunk: entries equal to the cut.  Skipped (zeros) when every such entry is taken anyway.
 __global__ __launch_bounds__(kSelThreads) void select_count_ties_kernel(const float* __restrict__ x, int64_t n, int64_t per,
-                                                                        int vec, const SelState* __restrict__ st,
+                                                                        int mode, const SelState* __restrict__ st,
                                                                         uint32_t* __restrict__ ties) {
   __shared__ double sh[kSelThreads / kWave + 1];
   uint32_t c = 0;
@@ -187,7 +197,7 @@ __global__ __launch_bounds__(kSelThreads) void select_count_ties_kernel(const fl
     chunk_of(n, per, lo, hi);
     for (int64_t i = lo + 4 * (int64_t)threadIdx.x; i < hi; i += kTile) {
       float v[4];
-      const int m = load4(x, i, hi, vec != 0, v);
+      const int m = load4(x, i, hi, mode, v);
 #pragma unroll
       for (int e = 0; e < 4; ++e)
         if (e < m) c += key_of(v[e]) == cut ? 1u : 0u;
@@ -205,7 +215,7 @@ __global__ __launch_bounds__(kSelThreads) void select_init_kernel(uint32_t* __re
 }
 
 // aux[i] = coef where the entry is taken, 0 elsewhere
-__global__ __launch_bounds__(kSelThreads) void select_mark_kernel(const float* __restrict__ x, int64_t n, int64_t per, int vec,
+__global__ __launch_bounds__(kSelThreads) void select_mark_kernel(const float* __restrict__ x, int64_t n, int64_t per, int mode,
                                                                   const SelState* __restrict__ st,
                                                                   const uint32_t* __restrict__ ties, float coef,
                                                                   float* __restrict__ aux) {
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(kSelThreads) void select_mark_kernel(const float* _
   for (int64_t t0 = lo; t0 < hi; t0 += kTile) {  // every thread runs every tile: the barriers below are uniform
     const int64_t i = t0 + 4 * (int64_t)threadIdx.x;
     float v[4];
-    const int m = i < hi ? load4(x, i, hi, vec != 0, v) : 0;
+    const int m = i < hi ? load4(x, i, hi, mode, v) : 0;
     uint32_t key[4] = {0u, 0u, 0u, 0u};
     uint32_t mine = 0;
 #pragma unroll
@@ -263,9 +273,9 @@ __global__ __launch_bounds__(kSelThreads) void select_mark_kernel(const float* _
       }
       out[e] = take ? coef : 0.f;
     }
-    if (m == 4 && vec) {
-      __builtin_nontemporal_store(u32x4{f2u(out[0]), f2u(out[1]), f2u(out[2]), f2u(out[3])},
-                                  reinterpret_cast<u32x4*>(aux + i));
+    if (m == 4 && (mode & kVec)) {
+      const u32x4 o{f2u(out[0]), f2u(out[1]), f2u(out[2]), f2u(out[3])};
+      __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(aux + i));  // (see kNt: stores always)
     } else {
 #pragma unroll
       for (int e = 0; e < 4; ++e)
@@ -279,7 +289,7 @@ __global__ __launch_bounds__(kSelThreads) void select_mark_kernel(const float* _
 // Clip-Cov's candidate list (siirl/dag_worker/core_algos.py:974-975: nonzero of lb < cov < ub): first the number of
 // such entries per chunk, then their flat indices in ascending order, each chunk writing behind the chunks before it
 // and ranking its own entries tile by tile with a scan.
-__global__ __launch_bounds__(kSelThreads) void range_count_kernel(const float* __restrict__ x, int64_t n, int64_t per, int vec,
+__global__ __launch_bounds__(kSelThreads) void range_count_kernel(const float* __restrict__ x, int64_t n, int64_t per, int mode,
                                                                   float lo_open, float hi_open,
                                                                   uint32_t* __restrict__ counts) {
   __shared__ double sh[kSelThreads / kWave + 1];
@@ -288,7 +298,7 @@ __global__ __launch_bounds__(kSelThreads) void range_count_kernel(const float* _
   uint32_t c = 0;
   for (int64_t i = lo + 4 * (int64_t)threadIdx.x; i < hi; i += kTile) {
     float v[4];
-    const int m = load4(x, i, hi, vec != 0, v);
+    const int m = load4(x, i, hi, mode, v);
 #pragma unroll
     for (int e = 0; e < 4; ++e)
       if (e < m) c += (v[e] > lo_open && v[e] < hi_open) ? 1u : 0u;
@@ -306,7 +316,7 @@ __global__ __launch_bounds__(kSelGrid) void range_total_kernel(uint32_t* __restr
     *total = (uint32_t)t;
   }
 }
-__global__ __launch_bounds__(kSelThreads) void range_write_kernel(const float* __restrict__ x, int64_t n, int64_t per, int vec,
+__global__ __launch_bounds__(kSelThreads) void range_write_kernel(const float* __restrict__ x, int64_t n, int64_t per, int mode,
                                                                   float lo_open, float hi_open,
                                                                   const uint32_t* __restrict__ counts,
                                                                   int64_t* __restrict__ indices, int64_t capacity) {
@@ -322,7 +332,7 @@ __global__ __launch_bounds__(kSelThreads) void range_write_kernel(const float* _
   for (int64_t t0 = lo; t0 < hi; t0 += kTile) {  // every thread runs every tile: the barriers are uniform
     const int64_t i = t0 + 4 * (int64_t)threadIdx.x;
     float v[4];
-    const int m = i < hi ? load4(x, i, hi, vec != 0, v) : 0;
+    const int m = i < hi ? load4(x, i, hi, mode, v) : 0;
     bool in[4];
     uint32_t mine = 0;
 #pragma unroll
@@ -352,6 +362,10 @@ __global__ __launch_bounds__(kSelThreads) void range_write_kernel(const float* _
         ++r;
       }
   }
+}
+
+int access_mode(bool aligned, int64_t n) {
+  return (aligned ? kVec : 0) | (streams_past_cache(4.0 * (double)n) ? kNt : 0);
 }
 
 struct SelWs {
@@ -393,8 +407,8 @@ extern "C" int siirl_range_select_count(const float* scores, int64_t n, float lo
   int grid = 0;
   if (n > 0) {
     range_chunks(n, per, grid);
-    const int vec = ((uintptr_t)scores & 15) == 0;
-    range_count_kernel<<<dim3((unsigned)grid), dim3(kSelThreads), 0, st>>>(scores, n, per, vec, lower_open, upper_open, counts);
+    const int mode = access_mode(((uintptr_t)scores & 15) == 0, n);
+    range_count_kernel<<<dim3((unsigned)grid), dim3(kSelThreads), 0, st>>>(scores, n, per, mode, lower_open, upper_open, counts);
     SIIRL_LAUNCH_CHECK("range_count_kernel");
   }
   range_total_kernel<<<1, dim3(kSelGrid), 0, st>>>(counts, grid, count);
@@ -412,9 +426,9 @@ extern "C" int siirl_range_select_write(const float* scores, int64_t n, float lo
   int64_t per;
   int grid;
   range_chunks(n, per, grid);
-  const int vec = ((uintptr_t)scores & 15) == 0;
+  const int mode = access_mode(((uintptr_t)scores & 15) == 0, n);
   range_write_kernel<<<dim3((unsigned)grid), dim3(kSelThreads), 0, (hipStream_t)stream>>>(
-      scores, n, per, vec, lower_open, upper_open, (const uint32_t*)workspace, indices, capacity);
+      scores, n, per, mode, lower_open, upper_open, (const uint32_t*)workspace, indices, capacity);
   SIIRL_LAUNCH_CHECK("range_write_kernel");
   return SIIRL_OK;
 }
@@ -437,7 +451,7 @@ extern "C" int siirl_topk_mark(const float* scores, int64_t n, int64_t k, float 
   uint32_t* part = (uint32_t*)(base + ws.part);
   SelState* state = (SelState*)(base + ws.state);
   uint32_t* ties = (uint32_t*)(base + ws.ties);
-  const int vec = (((uintptr_t)scores | (uintptr_t)marks) & 15) == 0;
+  const int mode = access_mode((((uintptr_t)scores | (uintptr_t)marks) & 15) == 0, n);
   const int64_t per = ((n + kSelGrid - 1) / kSelGrid + kTile - 1) / kTile * kTile;
   const int grid = (int)((n + per - 1) / per);  // <= kSelGrid; chunks beyond n do not exist
   const dim3 g((unsigned)grid), b(kSelThreads);
@@ -449,21 +463,21 @@ extern "C" int siirl_topk_mark(const float* scores, int64_t n, int64_t k, float 
   static_assert(3 * kBins % kSelThreads == 0, "the histograms are cleared by whole workgroups");
   select_init_kernel<<<dim3(3 * kBins / kSelThreads), b, 0, st>>>(part);
   SIIRL_LAUNCH_CHECK("select_init_kernel");
-  select_hist_kernel<0><<<g, b, 0, st>>>(scores, n, per, vec, state, part);
+  select_hist_kernel<0><<<g, b, 0, st>>>(scores, n, per, mode, state, part);
   SIIRL_LAUNCH_CHECK("select_hist_kernel<0>");
   select_scan_kernel<0><<<1, b, 0, st>>>(part, (uint32_t)k, state);
   SIIRL_LAUNCH_CHECK("select_scan_kernel<0>");
-  select_hist_kernel<1><<<g, b, 0, st>>>(scores, n, per, vec, state, part);
+  select_hist_kernel<1><<<g, b, 0, st>>>(scores, n, per, mode, state, part);
   SIIRL_LAUNCH_CHECK("select_hist_kernel<1>");
   select_scan_kernel<1><<<1, b, 0, st>>>(part, 0u, state);
   SIIRL_LAUNCH_CHECK("select_scan_kernel<1>");
-  select_hist_kernel<2><<<g, b, 0, st>>>(scores, n, per, vec, state, part);
+  select_hist_kernel<2><<<g, b, 0, st>>>(scores, n, per, mode, state, part);
   SIIRL_LAUNCH_CHECK("select_hist_kernel<2>");
   select_scan_kernel<2><<<1, b, 0, st>>>(part, 0u, state);
   SIIRL_LAUNCH_CHECK("select_scan_kernel<2>");
-  select_count_ties_kernel<<<g, b, 0, st>>>(scores, n, per, vec, state, ties);
+  select_count_ties_kernel<<<g, b, 0, st>>>(scores, n, per, mode, state, ties);
   SIIRL_LAUNCH_CHECK("select_count_ties_kernel");
-  select_mark_kernel<<<g, b, 0, st>>>(scores, n, per, vec, state, ties, value, marks);
+  select_mark_kernel<<<g, b, 0, st>>>(scores, n, per, mode, state, ties, value, marks);
   SIIRL_LAUNCH_CHECK("select_mark_kernel");
   return SIIRL_OK;
 }

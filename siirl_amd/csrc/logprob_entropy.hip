@@ -679,12 +679,11 @@ int launch_fwd(const void* logits, int64_t T, int V, int64_t row_stride, const i
                float* logprob, float* entropy, float* lse, float* ex, hipStream_t st) {
   using elem_t = typename E::elem_t;
   dim3 grid((unsigned)T), block(kFwdThreads);
-  // Logits of up to kCacheResident bytes (the part's 256 MB memory-side cache and a little more) are read with
+  // Logits of up to kCacheResidentBytes (the part's 256 MB memory-side cache and a little more) are read with
   // ordinary loads, so that the backward pass that follows finds them cached: measured on [2048, 32000] fp32
   // (250 MiB) forward + backward 128 -> 117 us, [768, 152064] bf16 (223 MiB) 114 -> 103 us, the forward alone
   // unchanged; from 375 MiB upwards the non-temporal loads win (forward alone 60 against 70 us at that size).
-  constexpr int64_t kCacheResident = 300LL << 20;
-  const bool nt = SIIRL_LPE_FWD_NT_LOAD && T * (int64_t)V * (int64_t)sizeof(elem_t) > kCacheResident;
+  const bool nt = SIIRL_LPE_FWD_NT_LOAD && streams_past_cache((double)T * (double)V * (double)sizeof(elem_t));
   auto go = [&](auto ent_tag, auto nt_tag) {
     lpe_fwd_kernel<E, decltype(ent_tag)::value, decltype(nt_tag)::value><<<grid, block, 0, st>>>(
         (const elem_t*)logits, row_stride, V, labels, inv_T, logprob, decltype(ent_tag)::value ? entropy : nullptr, lse,

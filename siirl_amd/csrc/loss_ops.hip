@@ -700,15 +700,15 @@ constexpr int kCovGrid = 1024;
 constexpr int kCovSums = 6;
 __global__ __launch_bounds__(kThreads) void cov_sums_kernel(const float* __restrict__ lp, const float* __restrict__ adv,
                                                             const void* mask, int mask_dtype, int64_t n, int vec,
-                                                            double* __restrict__ part) {
+                                                            int nt_in, double* __restrict__ part) {
   float s[kCovSums] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int64_t nq = (n + 3) / 4;  // four tokens per thread and access
   for (int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x; q < nq; q += (int64_t)gridDim.x * kThreads) {
     const int64_t i = 4 * q;
     const int nv = (int)((n - i) < 4 ? (n - i) : 4);
     const bool v = vec != 0 && nv == 4;
-    const Quad m4 = load_mask_quad(mask, mask_dtype, i, v, nv);
-    const Quad a4 = load_quad(adv, i, v, nv, 0.f), l4 = load_quad(lp, i, v, nv, 0.f);
+    const Quad m4 = load_mask_quad(mask, mask_dtype, i, v, nv, nt_in != 0);
+    const Quad a4 = load_quad(adv, i, v, nv, 0.f, nt_in != 0), l4 = load_quad(lp, i, v, nv, 0.f, nt_in != 0);
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       if (e >= nv) break;
@@ -756,8 +756,9 @@ __global__ __launch_bounds__(kThreads) void cov_stats_kernel(const double* __res
 // such a token) and, for clip_cov, where the PPO clip already bites (l2 > l1)
 __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __restrict__ old_lp, const float* __restrict__ lp,
                                                               const float* __restrict__ adv, const void* mask,
-                                                              int mask_dtype, int64_t n, int vec, int clip_mode, float lo,
-                                                              float hi, const float* __restrict__ stats,
+                                                              int mask_dtype, int64_t n, int vec, int nt_in, int nt_out,
+                                                              int clip_mode, float lo, float hi,
+                                                              const float* __restrict__ stats,
                                                               float* __restrict__ cov) {
   const float ma = stats[2], ml = stats[3];
   const int64_t nq = (n + 3) / 4;
@@ -765,9 +766,9 @@ __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __res
     const int64_t i = 4 * q;
     const int nv = (int)((n - i) < 4 ? (n - i) : 4);
     const bool v = vec != 0 && nv == 4;
-    const Quad m4 = load_mask_quad(mask, mask_dtype, i, v, nv);
-    const Quad a4 = load_quad(adv, i, v, nv, 0.f), l4 = load_quad(lp, i, v, nv, 0.f);
-    const Quad o4 = clip_mode ? load_quad(old_lp, i, v, nv, 0.f) : const_quad(0.f);
+    const Quad m4 = load_mask_quad(mask, mask_dtype, i, v, nv, nt_in != 0);
+    const Quad a4 = load_quad(adv, i, v, nv, 0.f, nt_in != 0), l4 = load_quad(lp, i, v, nv, 0.f, nt_in != 0);
+    const Quad o4 = clip_mode ? load_quad(old_lp, i, v, nv, 0.f, nt_in != 0) : const_quad(0.f);
     Quad c4;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
@@ -782,7 +783,7 @@ __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __res
       }
       c4.v[e] = c;
     }
-    store_quad(cov, i, v, nv, c4);
+    store_quad(cov, i, v, nv, c4, nt_out != 0);
   }
 }
 
@@ -1096,14 +1097,18 @@ extern "C" int siirl_cov_scores(const float* old_log_prob, const float* log_prob
   const size_t msz = dtype_size(mask_dtype);
   const int vec = ok16(old_log_prob) && ok16(log_prob) && ok16(advantages) && ok16(cov) &&
                   ((uintptr_t)mask & (msz * 4 > 16 ? 15 : msz * 4 - 1)) == 0;
-  cov_sums_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(log_prob, advantages, mask, mask_dtype, n, vec, part);
+  // the operands are read twice here and again by the loss; the scores are read by the selection that follows
+  const int nt_in = streams_past_cache((double)n * (double)(8 + msz + (clip_mode ? 4 : 0)));
+  const int nt_out = 1;  // (ordinary stores of the scores: this launch 8 us slower, the selection's first pass no faster)
+  cov_sums_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(log_prob, advantages, mask, mask_dtype, n, vec, nt_in,
+                                                                  part);
   SIIRL_LAUNCH_CHECK("cov_sums_kernel");
   cov_stats_kernel<<<1, dim3(kThreads), 0, st>>>(part, grid, clip_mode, stats);
   SIIRL_LAUNCH_CHECK("cov_stats_kernel");
   if (n == 0) return SIIRL_OK;
   cov_scores_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(old_log_prob, log_prob, advantages, mask, mask_dtype,
-                                                                    n, vec, clip_mode, 1.f - clip_low, 1.f + clip_high,
-                                                                    stats, cov);
+                                                                    n, vec, nt_in, nt_out, clip_mode, 1.f - clip_low,
+                                                                    1.f + clip_high, stats, cov);
   SIIRL_LAUNCH_CHECK("cov_scores_kernel");
   return SIIRL_OK;
 }

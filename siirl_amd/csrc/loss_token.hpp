@@ -12,7 +12,7 @@
 // Cache hints of the [B, L] streaming kernels.  Measured at [5488, 8192] fp32 with an int64 mask (actor loss forward +
 // backward): non-temporal loads 0.467 -> 0.428 ms, non-temporal stores of the gradient a further 0.428 -> 0.420 ms.
 // That is for operands several times the part's 256 MB memory-side cache.  A pass that reads less than
-// kCacheResidentBytes uses ordinary accesses instead (`nt` of the helpers below, decided on the host per launch):
+// kCacheResidentBytes (common.hpp) uses ordinary accesses instead (`nt` of the helpers below, decided on the host per launch):
 // what the forward has read is then still cached when the backward reads it again -- forward + backward at
 // [1024, 8192] (192 MiB per pass) 99.8 -> 90.3 us, at [512, 8192] 55.3 -> 50.8 us; at [2048, 8192] (384 MiB) the
 // non-temporal accesses are the faster ones again (166 against 183 us).
@@ -25,9 +25,6 @@
 
 namespace siirl {
 namespace tok {
-
-constexpr double kCacheResidentBytes = 300.0 * 1048576.0;
-inline bool streams_past_cache(double bytes_per_pass) { return bytes_per_pass > kCacheResidentBytes; }
 
 struct LossArgs {
   const float* old_lp;   // [B,L] or null (kind == KIND_AGG)

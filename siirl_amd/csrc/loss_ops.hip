@@ -451,7 +451,7 @@ __global__ __launch_bounds__(kStream) void loss_bwd_kernel(LossArgs a, const flo
     if (agg_only) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) dlp.v[e] = g * w_pg(m4.v[e]);
-      store_quad(d_lp, idx0, vec, nv, dlp, nt);
+      store_quad(d_lp, idx0, vec, nv, dlp);
       continue;
     }
     const Quad lp4 = load_quad(a.lp, idx0, vec, nv, 0.f, nt);
@@ -479,8 +479,8 @@ __global__ __launch_bounds__(kStream) void loss_bwd_kernel(LossArgs a, const flo
       }
       dlp.v[e] = g * d;
     }
-    store_quad(d_lp, idx0, vec, nv, dlp, nt);
-    if (a.ent && d_ent) store_quad(d_ent, idx0, vec, nv, dent, nt);
+    store_quad(d_lp, idx0, vec, nv, dlp);
+    if (a.ent && d_ent) store_quad(d_ent, idx0, vec, nv, dent);
   }
 }
 
@@ -756,7 +756,7 @@ __global__ __launch_bounds__(kThreads) void cov_stats_kernel(const double* __res
 // such a token) and, for clip_cov, where the PPO clip already bites (l2 > l1)
 __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __restrict__ old_lp, const float* __restrict__ lp,
                                                               const float* __restrict__ adv, const void* mask,
-                                                              int mask_dtype, int64_t n, int vec, int nt_in, int nt_out,
+                                                              int mask_dtype, int64_t n, int vec, int nt_in,
                                                               int clip_mode, float lo, float hi,
                                                               const float* __restrict__ stats,
                                                               float* __restrict__ cov) {
@@ -783,7 +783,7 @@ __global__ __launch_bounds__(kThreads) void cov_scores_kernel(const float* __res
       }
       c4.v[e] = c;
     }
-    store_quad(cov, i, v, nv, c4, nt_out != 0);
+    store_quad(cov, i, v, nv, c4);
   }
 }
 
@@ -798,7 +798,7 @@ void set_vec(LossArgs& a, const void* o1 = nullptr, const void* o2 = nullptr) {
   const bool mask_ok = ((uintptr_t)a.mask & (msz * 4 > 16 ? 15 : msz * 4 - 1)) == 0;
   a.vec = (a.L % 4 == 0) && mask_ok && ok16(a.old_lp) && ok16(a.lp) && ok16(a.adv) && ok16(a.isw) && ok16(a.ent) &&
           ok16(a.ref) && ok16(a.aux) && ok16(o1) && ok16(o2);
-  // bytes one pass reads: ordinary accesses while they fit the memory-side cache, non-temporal ones beyond
+  // bytes one pass reads: ordinary loads while they fit the memory-side cache, non-temporal ones beyond
   const int n_f32 = (a.old_lp != nullptr) + (a.lp != nullptr) + (a.adv != nullptr) + (a.isw != nullptr) + (a.ent != nullptr) +
                     (a.ref != nullptr) + (a.aux != nullptr);
   a.nt = streams_past_cache((double)a.B * (double)a.L * (double)(4 * n_f32 + (a.mask ? msz : 0)));
@@ -1097,9 +1097,8 @@ extern "C" int siirl_cov_scores(const float* old_log_prob, const float* log_prob
   const size_t msz = dtype_size(mask_dtype);
   const int vec = ok16(old_log_prob) && ok16(log_prob) && ok16(advantages) && ok16(cov) &&
                   ((uintptr_t)mask & (msz * 4 > 16 ? 15 : msz * 4 - 1)) == 0;
-  // the operands are read twice here and again by the loss; the scores are read by the selection that follows
+  // the operands are read twice here and again by the loss
   const int nt_in = streams_past_cache((double)n * (double)(8 + msz + (clip_mode ? 4 : 0)));
-  const int nt_out = 1;  // (ordinary stores of the scores: this launch 8 us slower, the selection's first pass no faster)
   cov_sums_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(log_prob, advantages, mask, mask_dtype, n, vec, nt_in,
                                                                   part);
   SIIRL_LAUNCH_CHECK("cov_sums_kernel");
@@ -1107,7 +1106,7 @@ extern "C" int siirl_cov_scores(const float* old_log_prob, const float* log_prob
   SIIRL_LAUNCH_CHECK("cov_stats_kernel");
   if (n == 0) return SIIRL_OK;
   cov_scores_kernel<<<dim3((unsigned)grid), dim3(kThreads), 0, st>>>(old_log_prob, log_prob, advantages, mask, mask_dtype,
-                                                                    n, vec, nt_in, nt_out, clip_mode, 1.f - clip_low,
+                                                                    n, vec, nt_in, clip_mode, 1.f - clip_low,
                                                                     1.f + clip_high, stats, cov);
   SIIRL_LAUNCH_CHECK("cov_scores_kernel");
   return SIIRL_OK;

@@ -12,10 +12,11 @@
 // Cache hints of the [B, L] streaming kernels.  Measured at [5488, 8192] fp32 with an int64 mask (actor loss forward +
 // backward): non-temporal loads 0.467 -> 0.428 ms, non-temporal stores of the gradient a further 0.428 -> 0.420 ms.
 // That is for operands several times the part's 256 MB memory-side cache.  A pass that reads less than
-// kCacheResidentBytes (common.hpp) uses ordinary accesses instead (`nt` of the helpers below, decided on the host per launch):
-// what the forward has read is then still cached when the backward reads it again -- forward + backward at
-// [1024, 8192] (192 MiB per pass) 99.8 -> 90.3 us, at [512, 8192] 55.3 -> 50.8 us; at [2048, 8192] (384 MiB) the
-// non-temporal accesses are the faster ones again (166 against 183 us).
+// kCacheResidentBytes (common.hpp) uses ordinary loads instead (`nt` of the load helpers below, decided on the host
+// per launch): what the forward has read is then still cached when the backward reads it again -- forward + backward
+// at [1024, 8192] (192 MiB per pass) 99.8 -> 94 us, at [512, 8192] 55.3 -> 51 us; at [2048, 8192] (384 MiB) the
+// non-temporal loads are the faster ones again (166 against 183 us).  Stores are non-temporal at every size: ordinary
+// ones gain nothing there (51.8 against 51.1 us, 94.9 against 94.4 us) and their write-back delays the next kernel.
 #ifndef SIIRL_LOSS_NT_STORE
 #define SIIRL_LOSS_NT_STORE 1
 #endif
@@ -47,7 +48,7 @@ struct LossArgs {
   int64_t B, L;
   int nseg;
   int vec;  // L % 4 == 0 and every operand 16-byte aligned: tokens are moved four at a time
-  int nt;   // the operands of a pass exceed the memory-side cache: non-temporal loads and stores
+  int nt;   // the operands of a pass exceed the memory-side cache: non-temporal loads
 };
 enum { KIND_AGG = 0, KIND_VANILLA = 1, KIND_GSPO = 2, KIND_CPGD = 3, KIND_GPG = 4, KIND_GEO = 5, KIND_VALUE = 6,
        KIND_KL_COV = 7, KIND_CLIP_COV = 8 };
@@ -122,13 +123,13 @@ __device__ __forceinline__ Quad load_mask_quad(const void* p, int dt, int64_t id
   }
   return q;
 }
-__device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q,
-                                           bool nt = SIIRL_LOSS_NT_STORE != 0) {
+__device__ __forceinline__ void store_quad(float* __restrict__ p, int64_t idx, bool vec, int nv, const Quad& q) {
   if (vec) {
-    if (SIIRL_LOSS_NT_STORE && nt)
-      __builtin_nontemporal_store(u32x4{f2u(q.v[0]), f2u(q.v[1]), f2u(q.v[2]), f2u(q.v[3])}, reinterpret_cast<u32x4*>(p + idx));
-    else
-      *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
+#if SIIRL_LOSS_NT_STORE
+    __builtin_nontemporal_store(u32x4{f2u(q.v[0]), f2u(q.v[1]), f2u(q.v[2]), f2u(q.v[3])}, reinterpret_cast<u32x4*>(p + idx));
+#else
+    *reinterpret_cast<float4*>(p + idx) = make_float4(q.v[0], q.v[1], q.v[2], q.v[3]);
+#endif
   } else {
 #pragma unroll
     for (int e = 0; e < 4; ++e)

@@ -311,6 +311,14 @@ def bench_config5(args, dev):
     FL.set_saved_logits_limit(0)
     saved_gb = FL._saved_logits_bytes(T, V) / 1e9
     gemm = 2.0 * T * H * V
+    # the same tensors as a packed batch of 8 sequences of 2048 tokens whose first 512 are prompt tokens: their rows
+    # arrive with zero gradients and the backward leaves them out of its GEMMs
+    live = (torch.arange(T, device=dev) % 2048 >= 512).float()
+    dense_g = (g_lp, g_h)
+    g_lp, g_h = dense_g[0] * live, dense_g[1] * live
+    r_wall, r_fwd_ms, r_bwd_ms = timed()
+    g_lp, g_h = dense_g
+    n_live = int(live.sum().item())
     tf_step = 3 * gemm / (wall / steps) / 1e12
 
     # the same forward launch on quiet operands (all zeros): identical instruction stream, fewer wires toggling.
@@ -350,6 +358,11 @@ def bench_config5(args, dev):
                            "forward_ms": p_fwd_ms, "backward_ms": p_bwd_ms,
                            "algorithmic_TFLOP/s": 3 * gemm / (p_wall / steps) / 1e12,
                            "frac_of_peak": 3 * gemm / (p_wall / steps) / 1e12 / 2500.0},
+        "response_rows_variant": {"what": "8 packed sequences of 2048 tokens, the first 512 of each prompt tokens with "
+                                          "zero upstream gradients: the backward runs its GEMMs over the "
+                                          f"{n_live} response rows only (set_skip_zero_rows, on by default)",
+                                  "ms_per_step": r_wall * 1e3 / steps, "tokens_per_s": T * steps / r_wall,
+                                  "forward_ms": r_fwd_ms, "backward_ms": r_bwd_ms, "rows_with_gradient": n_live},
         "power_limit_probe": {"what": "the forward alone (no grad) on the configuration's random operands and on "
                                       "all-zero operands: same instructions, quieter data",
                               "forward_ms_random_operands": fwd_random_ms, "TFLOP/s_random": gemm / fwd_random_ms / 1e9,

@@ -75,7 +75,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1005
+#define SIIRL_HIP_ABI_VERSION 1006
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -612,6 +612,28 @@ int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const void* weigh
                                            const float* ex, const float* saved_logits, const float* g_logprob,
                                            const float* g_entropy, void* d_hidden, void* d_weight, void* workspace,
                                            size_t workspace_bytes, siirl_stream_t stream);
+
+/*
+ * The same backward restricted to the n_rows token rows listed in rows[] (distinct indices into [0, T), any
+ * order): the rows whose upstream gradients are not both zero.  The actor takes the log-probs of every packed token
+ * but only the response slice reaches the loss, so the rows of prompt tokens arrive with zero gradients; they
+ * contribute nothing to either result and are left out of all three GEMMs here.  Rows not listed get zeros in
+ * d_hidden; d_weight sums over the listed rows only.  The results are those of
+ * siirl_fused_linear_logprob_entropy_bwd on the gathered operands, bit for bit (against the full call d_weight
+ * differs by the rounding order of its sum over tokens).  n_rows == 0 writes zeros.  The logits are always
+ * recomputed on this route.  workspace: siirl_fused_linear_bwd_rows_workspace_bytes(n_rows, ...) bytes, 256-byte
+ * aligned.
+ * Replaces: FusedLinearForPPO.backward siirl/utils/experimental/torch_functional.py:35-67,135-188 as reached from
+ *           siirl/engine/actor/dp_actor.py:170-172 (log-probs of all packed tokens) and :228-231 (only the
+ *           response slice [:, -response_length - 1 : -1] is used).
+ */
+size_t siirl_fused_linear_bwd_rows_workspace_bytes(int64_t n_rows, int64_t H, int64_t V, int want_d_hidden,
+                                                   int want_d_weight);
+int siirl_fused_linear_logprob_entropy_bwd_rows(const void* hidden, const void* weight, int dtype, const int64_t* labels,
+                                                int64_t T, int64_t H, int64_t V, float inv_temperature, const float* lse,
+                                                const float* ex, const float* g_logprob, const float* g_entropy,
+                                                const int64_t* rows, int64_t n_rows, void* d_hidden, void* d_weight,
+                                                void* workspace, size_t workspace_bytes, siirl_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -768,6 +768,52 @@ int pack_hidden(const uint16_t* h, int64_t T, int64_t H, u32x4* out, hipStream_t
   return SIIRL_OK;
 }
 
+// The per-token operands of the backward for the listed token rows only (a row index outside [0, T) yields zero
+// gradients: the row then contributes nothing).
+__global__ __launch_bounds__(256) void gather_token_operands_kernel(const int64_t* __restrict__ rows, int64_t n, int64_t T,
+                                                                    const int64_t* __restrict__ labels,
+                                                                    const float* __restrict__ lse,
+                                                                    const float* __restrict__ ex,
+                                                                    const float* __restrict__ g_lp,
+                                                                    const float* __restrict__ g_ent,
+                                                                    int64_t* __restrict__ labels_c, float* __restrict__ lse_c,
+                                                                    float* __restrict__ ex_c, float* __restrict__ g_lp_c,
+                                                                    float* __restrict__ g_ent_c) {
+  const int64_t j = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (j >= n) return;
+  const int64_t r = rows[j];
+  const bool ok = r >= 0 && r < T;
+  labels_c[j] = ok && labels ? labels[r] : -1;
+  lse_c[j] = ok ? lse[r] : 0.f;
+  ex_c[j] = ok && ex ? ex[r] : 0.f;
+  g_lp_c[j] = ok && g_lp ? g_lp[r] : 0.f;
+  g_ent_c[j] = ok && g_ent ? g_ent[r] : 0.f;
+}
+
+struct RowsWs {
+  size_t hidden, labels, lse, ex, g_lp, g_ent, dh, inner, inner_bytes, total;
+};
+RowsWs rows_ws(int64_t n, int64_t H, int64_t V, bool want_dh, bool want_dw) {
+  RowsWs w;
+  size_t off = 0;
+  auto take = [&off](size_t bytes) {
+    const size_t at = off;
+    off += round_up(bytes, 256);
+    return at;
+  };
+  w.hidden = take((size_t)n * H * 2);
+  w.labels = take((size_t)n * 8);
+  w.lse = take((size_t)n * 4);
+  w.ex = take((size_t)n * 4);
+  w.g_lp = take((size_t)n * 4);
+  w.g_ent = take((size_t)n * 4);
+  w.dh = take(want_dh ? (size_t)n * H * 2 : 0);
+  w.inner = off;
+  w.inner_bytes = n > 0 ? bwd_ws(n, H, V, want_dh, want_dw).total : 0;
+  w.total = off + w.inner_bytes;
+  return w;
+}
+
 }  // namespace
 }  // namespace siirl
 
@@ -919,5 +965,61 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
                                                            (uint16_t*)d_hidden, n);
     SIIRL_LAUNCH_CHECK("f32_to_bf16_kernel");
   }
+  return SIIRL_OK;
+}
+
+extern "C" size_t siirl_fused_linear_bwd_rows_workspace_bytes(int64_t n_rows, int64_t H, int64_t V, int want_d_hidden,
+                                                              int want_d_weight) {
+  if (n_rows < 0 || H <= 0 || V <= 0) return 0;
+  return rows_ws(n_rows, H, V, want_d_hidden != 0, want_d_weight != 0).total;
+}
+
+extern "C" int siirl_fused_linear_logprob_entropy_bwd_rows(const void* hidden, const void* weight, int dtype,
+                                                           const int64_t* labels, int64_t T, int64_t H, int64_t V,
+                                                           float inv_temperature, const float* lse, const float* ex,
+                                                           const float* g_logprob, const float* g_entropy,
+                                                           const int64_t* rows, int64_t n_rows, void* d_hidden,
+                                                           void* d_weight, void* workspace, size_t workspace_bytes,
+                                                           siirl_stream_t stream) {
+  if (int rc = check_fused(hidden, weight, T, H, V, inv_temperature, dtype)) return rc;
+  SIIRL_REQUIRE(n_rows >= 0 && n_rows <= T, "n_rows=%lld must lie in [0, T=%lld]", (long long)n_rows, (long long)T);
+  SIIRL_REQUIRE(n_rows == 0 || rows != nullptr, "rows is NULL");
+  SIIRL_REQUIRE(lse != nullptr, "lse is NULL");
+  SIIRL_REQUIRE(g_logprob != nullptr || g_entropy != nullptr, "no upstream gradient given");
+  SIIRL_REQUIRE(g_logprob == nullptr || labels != nullptr, "labels is required with g_logprob");
+  SIIRL_REQUIRE(g_entropy == nullptr || ex != nullptr, "ex is required with g_entropy");
+  SIIRL_REQUIRE(d_hidden != nullptr || d_weight != nullptr, "neither d_hidden nor d_weight requested");
+  const bool want_dh = d_hidden != nullptr, want_dw = d_weight != nullptr;
+  if (n_rows == 0) {  // no row carries a gradient: both results are zero
+    if (want_dh)
+      if (int rc = siirl_scatter_rows(nullptr, nullptr, 0, H * 2, T, d_hidden, stream)) return rc;
+    if (want_dw)
+      if (int rc = siirl_scatter_rows(nullptr, nullptr, 0, H * 2, V, d_weight, stream)) return rc;
+    return SIIRL_OK;
+  }
+  const RowsWs ws = rows_ws(n_rows, H, V, want_dh, want_dw);
+  if (workspace == nullptr || workspace_bytes < ws.total)
+    return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, ws.total);
+  if (int rc = check_ws_align(workspace)) return rc;
+  hipStream_t st = (hipStream_t)stream;
+  char* base = (char*)workspace;
+  void* hidden_c = base + ws.hidden;
+  int64_t* labels_c = (int64_t*)(base + ws.labels);
+  float* lse_c = (float*)(base + ws.lse);
+  float* ex_c = (float*)(base + ws.ex);
+  float* g_lp_c = (float*)(base + ws.g_lp);
+  float* g_ent_c = (float*)(base + ws.g_ent);
+  void* dh_c = base + ws.dh;
+  if (int rc = siirl_gather_rows(hidden, rows, n_rows, H * 2, T, hidden_c, stream)) return rc;
+  gather_token_operands_kernel<<<dim3((unsigned)((n_rows + 255) / 256)), dim3(256), 0, st>>>(
+      rows, n_rows, T, labels, lse, ex, g_logprob, g_entropy, labels_c, lse_c, ex_c, g_lp_c, g_ent_c);
+  SIIRL_LAUNCH_CHECK("gather_token_operands_kernel");
+  if (int rc = siirl_fused_linear_logprob_entropy_bwd(hidden_c, weight, dtype, labels_c, n_rows, H, V, inv_temperature,
+                                                      lse_c, ex_c, nullptr, g_logprob ? g_lp_c : nullptr,
+                                                      g_entropy ? g_ent_c : nullptr, want_dh ? dh_c : nullptr, d_weight,
+                                                      base + ws.inner, ws.inner_bytes, stream))
+    return rc;
+  if (want_dh)
+    if (int rc = siirl_scatter_rows(dh_c, rows, n_rows, H * 2, T, d_hidden, stream)) return rc;
   return SIIRL_OK;
 }

@@ -17,6 +17,7 @@
 #include <ATen/ATen.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <c10/hip/HIPGraphsC10Utils.h>
 #include <torch/csrc/autograd/custom_function.h>
 #include <torch/library.h>
 
@@ -1110,7 +1111,8 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> fused_linear_fwd(const Tensor
 std::tuple<Tensor, Tensor> fused_linear_bwd(const Tensor& hidden, const Tensor& weight, const Tensor& labels,
                                             double inv_temperature, const Tensor& lse, const Tensor& ex,
                                             const optional<Tensor>& g_lp, const optional<Tensor>& g_ent,
-                                            bool need_hidden, bool need_weight, const optional<Tensor>& saved_in) {
+                                            bool need_hidden, bool need_weight, const optional<Tensor>& saved_in,
+                                            bool skip_zero_rows) {
   require_bf16_2d(hidden, "hidden");
   require_bf16_2d(weight, "weight");
   require_f32c(g_lp, "g_logprob");
@@ -1135,10 +1137,30 @@ std::tuple<Tensor, Tensor> fused_linear_bwd(const Tensor& hidden, const Tensor& 
                           (size_t)saved->numel() * 4 == siirl_fused_linear_saved_logits_bytes(T, V),
                       "saved is not the buffer the forward op returned for these shapes");
   }
-  const size_t nws = siirl_fused_linear_bwd_workspace_bytes(T, H, V, (int)need_hidden, (int)need_weight);
-  Tensor ws = at::empty({(int64_t)std::max<size_t>(nws, 256)}, hidden.options().dtype(at::kByte));
   Tensor y = labels.contiguous();
   DeviceGuard guard(hidden.device());
+  // Token rows whose upstream gradients are both zero (the prompt tokens of a packed batch: only the response slice
+  // of the log-probs reaches the loss) drop out of all three GEMMs.  Finding them costs one host synchronisation,
+  // so not under stream capture; parked logits are indexed by the forward's token tiles, so not with them either.
+  if (skip_zero_rows && !has(saved) && T > 0 && (has(g_lp) || has(g_ent)) &&
+      c10::hip::currentStreamCaptureStatusMayInitCtx() == c10::hip::CaptureStatus::None) {
+    Tensor live = has(g_lp) ? g_lp->ne(0) : g_ent->ne(0);
+    if (has(g_lp) && has(g_ent)) live = live.logical_or(g_ent->ne(0));
+    Tensor rows = at::nonzero(live).reshape({-1});
+    const int64_t n = rows.size(0);
+    if (n < T) {
+      const size_t nws = siirl_fused_linear_bwd_rows_workspace_bytes(n, H, V, (int)need_hidden, (int)need_weight);
+      Tensor ws = at::empty({(int64_t)std::max<size_t>(nws, 256)}, hidden.options().dtype(at::kByte));
+      check_rc(siirl_fused_linear_logprob_entropy_bwd_rows(
+                   ptr(hidden), ptr(weight), SIIRL_BF16, ptr<int64_t>(y), T, H, V, (float)inv_temperature, ptr<float>(lse),
+                   ptr<float>(ex), ptr<float>(g_lp), ptr<float>(g_ent), ptr<int64_t>(rows), n,
+                   need_hidden ? ptr(d_h) : nullptr, need_weight ? ptr(d_w) : nullptr, ptr(ws), nws, stream_of(hidden)),
+               "siirl_fused_linear_logprob_entropy_bwd_rows");
+      return {d_h, d_w};
+    }
+  }
+  const size_t nws = siirl_fused_linear_bwd_workspace_bytes(T, H, V, (int)need_hidden, (int)need_weight);
+  Tensor ws = at::empty({(int64_t)std::max<size_t>(nws, 256)}, hidden.options().dtype(at::kByte));
   check_rc(siirl_fused_linear_logprob_entropy_bwd(ptr(hidden), ptr(weight), SIIRL_BF16, ptr<int64_t>(y), T, H, V,
                                                   (float)inv_temperature, ptr<float>(lse), ptr<float>(ex),
                                                   ptr<float>(saved), ptr<float>(g_lp), ptr<float>(g_ent),
@@ -1150,7 +1172,7 @@ std::tuple<Tensor, Tensor> fused_linear_bwd(const Tensor& hidden, const Tensor& 
 
 struct FusedLinearFn : public torch::autograd::Function<FusedLinearFn> {
   static variable_list forward(AutogradContext* ctx, const Tensor& hidden, const Tensor& weight, const Tensor& labels,
-                               double inv_temperature, bool save_logits) {
+                               double inv_temperature, bool save_logits, bool skip_zero_rows) {
     at::AutoDispatchBelowADInplaceOrView below;
     require_gpu(hidden, "hidden");
     require_gpu(weight, "weight");
@@ -1166,12 +1188,13 @@ struct FusedLinearFn : public torch::autograd::Function<FusedLinearFn> {
     auto [lp, ent, lse, ex, saved] = fused_linear_fwd(h, w, y, inv_temperature, save_logits);
     ctx->save_for_backward({h, w, y, lse, ex, saved});
     ctx->saved_data["inv_t"] = inv_temperature;
+    ctx->saved_data["skip_zero_rows"] = skip_zero_rows;
     ctx->set_materialize_grads(false);
     return {lp, ent};
   }
   static variable_list backward(AutogradContext* ctx, variable_list grads) {
     const bool need_h = ctx->needs_input_grad(0), need_w = ctx->needs_input_grad(1);
-    variable_list out(5);
+    variable_list out(6);
     if ((!grads[0].defined() && !grads[1].defined()) || !(need_h || need_w)) return out;
     const auto s = ctx->get_saved_variables();
     at::AutoDispatchBelowADInplaceOrView below;
@@ -1179,7 +1202,7 @@ struct FusedLinearFn : public torch::autograd::Function<FusedLinearFn> {
     if (grads[0].defined()) g_lp = f32c(grads[0], s[0].device());
     if (grads[1].defined()) g_ent = f32c(grads[1], s[0].device());
     auto [d_h, d_w] = fused_linear_bwd(s[0], s[1], s[2], ctx->saved_data["inv_t"].toDouble(), s[3], s[4], g_lp, g_ent,
-                                       need_h, need_w, s[5]);
+                                       need_h, need_w, s[5], ctx->saved_data["skip_zero_rows"].toBool());
     if (need_h) out[0] = d_h;
     if (need_w) out[1] = d_w;
     return out;
@@ -1188,12 +1211,13 @@ struct FusedLinearFn : public torch::autograd::Function<FusedLinearFn> {
 
 // `save_limit_bytes`: largest fp32 logit buffer the forward may park for the backward (0: never park).
 std::tuple<Tensor, Tensor> fused_linear_logprob_entropy(const Tensor& hidden, const Tensor& weight, const Tensor& labels,
-                                                        double inv_temperature, int64_t save_limit_bytes) {
+                                                        double inv_temperature, int64_t save_limit_bytes,
+                                                        bool skip_zero_rows) {
   bool save = false;
   if (save_limit_bytes > 0 && at::GradMode::is_enabled() && (hidden.requires_grad() || weight.requires_grad()) &&
       hidden.dim() == 2 && weight.dim() == 2)
     save = (int64_t)siirl_fused_linear_saved_logits_bytes(hidden.size(0), weight.size(0)) <= save_limit_bytes;
-  auto out = FusedLinearFn::apply(hidden, weight, labels, inv_temperature, save);
+  auto out = FusedLinearFn::apply(hidden, weight, labels, inv_temperature, save, skip_zero_rows);
   return {out[0], out[1]};
 }
 
@@ -1233,7 +1257,7 @@ TORCH_LIBRARY(siirl_hip, m) {
         "bool save_logits=False) -> (Tensor, Tensor, Tensor, Tensor, Tensor)");
   m.def("fused_linear_logprob_entropy_bwd(Tensor hidden, Tensor weight, Tensor labels, float inv_temperature, "
         "Tensor lse, Tensor ex, Tensor? g_logprob, Tensor? g_entropy, bool need_hidden, bool need_weight, "
-        "Tensor? saved=None) -> (Tensor, Tensor)");
+        "Tensor? saved=None, bool skip_zero_rows=False) -> (Tensor, Tensor)");
   // how the log-prob operators cut a (..., V) view into launches; no device work (used by the host-side tests)
   m.def("row_blocks(Tensor x) -> int[]", &row_blocks_op);
   // differentiable operators (autograd nodes in C++; eager use only)
@@ -1250,7 +1274,7 @@ TORCH_LIBRARY(siirl_hip, m) {
         "int agg_mode) -> (Tensor, Tensor)", &value_loss);
   m.def("kl_penalty(Tensor logprob, Tensor ref_logprob, int kl_mode, bool straight_through) -> Tensor", &kl_penalty);
   m.def("fused_linear_logprob_entropy(Tensor hidden, Tensor weight, Tensor labels, float inv_temperature, "
-        "int save_limit_bytes) -> (Tensor, Tensor)", &fused_linear_logprob_entropy);
+        "int save_limit_bytes, bool skip_zero_rows=False) -> (Tensor, Tensor)", &fused_linear_logprob_entropy);
 }
 
 TORCH_LIBRARY_IMPL(siirl_hip, CUDA, m) {

@@ -40,6 +40,20 @@ def set_saved_logits_limit(nbytes: int) -> None:
     _SAVED_LOGITS_LIMIT = int(nbytes)
 
 
+_SKIP_ZERO_ROWS = True
+
+
+def set_skip_zero_rows(flag: bool) -> None:
+    """Backward leaves token rows whose upstream gradients are both zero out of its three GEMMs (the prompt tokens
+    of a packed batch: the actor keeps only the response slice of the log-probs, reference
+    ``siirl/engine/actor/dp_actor.py:170-172,228-231``).  On by default.  Costs one host synchronisation per backward
+    (the count of such rows), so it is skipped under stream capture and when the logits were parked; ``d_hidden``
+    of a skipped row is zero even where its hidden state holds NaN or Inf; ``d_weight`` is summed over the remaining
+    rows, which changes its rounding order, not its value."""
+    global _SKIP_ZERO_ROWS
+    _SKIP_ZERO_ROWS = bool(flag)
+
+
 def _saved_logits_bytes(T: int, V: int) -> int:
     return ((V + 255) // 256) * ((T + 255) // 256) * (256 * 256 * 4)
 
@@ -48,7 +62,7 @@ def _apply(hidden2d, weight, labels1d, temperature):
     if not hidden2d.is_cuda or not weight.is_cuda:
         raise RuntimeError("siirl_amd: the fused lm_head path runs on the GPU only (no CPU fallback)")
     return torch.ops.siirl_hip.fused_linear_logprob_entropy(hidden2d, weight, labels1d, 1.0 / float(temperature),
-                                                            _SAVED_LOGITS_LIMIT)
+                                                            _SAVED_LOGITS_LIMIT, _SKIP_ZERO_ROWS)
 
 
 def fused_linear_logprob_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor,

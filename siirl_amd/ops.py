@@ -172,6 +172,7 @@ def _(hidden, weight, labels, inv_temperature, save_logits=False):
 
 
 @_fake(f"{_NS}::fused_linear_logprob_entropy_bwd")
-def _(hidden, weight, labels, inv_temperature, lse, ex, g_logprob, g_entropy, need_hidden, need_weight, saved=None):
+def _(hidden, weight, labels, inv_temperature, lse, ex, g_logprob, g_entropy, need_hidden, need_weight, saved=None,
+      skip_zero_rows=False):
     return (hidden.new_empty(hidden.shape if need_hidden else (0,)),
             weight.new_empty(weight.shape if need_weight else (0,)))

@@ -153,4 +153,9 @@ def test_size_queries_agree_with_the_host_side():
     both = h.siirl_fused_linear_bwd_workspace_bytes(512, 128, 4096, 1, 1)
     assert both > h.siirl_fused_linear_bwd_workspace_bytes(512, 128, 4096, 1, 0) > 0
     assert both > h.siirl_fused_linear_bwd_workspace_bytes(512, 128, 4096, 0, 1) > 0
+    # the row-subset backward: the dense workspace for its rows plus the gathered operands
+    rows = h.siirl_fused_linear_bwd_rows_workspace_bytes(100, 128, 4096, 1, 1)
+    assert rows > h.siirl_fused_linear_bwd_workspace_bytes(100, 128, 4096, 1, 1)
+    assert h.siirl_fused_linear_bwd_rows_workspace_bytes(0, 128, 4096, 1, 1) < 4096
+    assert h.siirl_fused_linear_bwd_rows_workspace_bytes(-1, 128, 4096, 1, 1) == 0
     assert h.siirl_fused_linear_fwd_workspace_bytes(512, 128, 4096) > 512 * 128 * 2

@@ -232,3 +232,137 @@ def test_parked_logits_allocation_failure_falls_back_to_recompute(dev):
         torch.cuda.empty_cache()
     for a, b in zip(got, want):
         assert torch.equal(a, b)
+
+
+def _live_rows(T, pattern, seed):
+    g = torch.Generator().manual_seed(seed)
+    if pattern == "packed":  # sequences of prompt + response tokens: only the response rows carry a gradient
+        live = torch.zeros(T, dtype=torch.bool)
+        t = 0
+        while t < T:
+            n = int(torch.randint(3, 40, (1,), generator=g))
+            p = int(torch.randint(1, n, (1,), generator=g))
+            live[t + p:t + n] = True
+            t += n
+        return live
+    if pattern == "random":
+        return torch.rand(T, generator=g) < 0.4
+    if pattern == "one":
+        live = torch.zeros(T, dtype=torch.bool)
+        live[T // 2] = True
+        return live
+    if pattern == "none":
+        return torch.zeros(T, dtype=torch.bool)
+    return torch.ones(T, dtype=torch.bool)
+
+
+@pytest.mark.parametrize("T,H,V", [(7, 64, 50), (300, 128, 1000), (513, 256, 8200), (1000, 192, 40000)])
+@pytest.mark.parametrize("pattern", ["packed", "random", "one", "none", "all"])
+def test_zero_gradient_rows_left_out_of_backward(dev, T, H, V, pattern):
+    """Token rows whose two upstream gradients are zero are left out of the backward's GEMMs: d_hidden is exactly
+    zero there (also where the hidden state holds NaN), both gradients match the oracle's, and they are, bit for
+    bit, what the plain backward gives on the gathered rows."""
+    import siirl_amd.fused_linear as FL
+
+    h, w, y, g_lp, g_h = _inputs(T, H, V, seed=3 * T + V)
+    live = _live_rows(T, pattern, seed=T + V)
+    g_lp, g_h = g_lp * live, g_h * live
+    if pattern == "packed":
+        g_h = g_h * (torch.arange(T) % 3 != 0)  # rows with a log-prob gradient only
+    rows = torch.nonzero((g_lp != 0) | (g_h != 0)).reshape(-1)
+    dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp, g_h, h, w, y, 0.9, dtype=torch.float64)
+    out = {}
+    for skip in (True, False):
+        FL.set_skip_zero_rows(skip)
+        try:
+            hd, wd = h.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+            lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y.to(dev), 0.9)
+            torch.autograd.backward([lp, ent], [g_lp.to(dev), g_h.to(dev)])
+        finally:
+            FL.set_skip_zero_rows(True)
+        _check_grad(hd.grad, dh64, f"d_hidden skip={skip}")
+        _check_grad(wd.grad, dw64, f"d_weight skip={skip}")
+        out[skip] = (hd.grad, wd.grad)
+    dead = ~live
+    assert not out[True][0][dead.to(dev)].any()
+    assert torch.equal(out[True][0], out[False][0])  # a row of d_hidden does not depend on the other rows
+    if len(rows) == T:
+        assert torch.equal(out[True][1], out[False][1])
+    elif len(rows):
+        # the plain backward on the gathered operands
+        ns = torch.ops.siirl_hip
+        hc, yc = h[rows].to(dev), y[rows].to(dev)
+        _, _, lse, ex, _ = ns.fused_linear_logprob_entropy_fwd(hc, w.to(dev), yc, 1 / 0.9, False)
+        d_hc, d_w = ns.fused_linear_logprob_entropy_bwd(hc, w.to(dev), yc, 1 / 0.9, lse, ex, g_lp[rows].to(dev),
+                                                        g_h[rows].to(dev), True, True)
+        assert torch.equal(out[True][1], d_w)
+        assert torch.equal(out[True][0][rows.to(dev)], d_hc)
+    else:
+        assert not out[True][1].any()
+
+
+def test_zero_gradient_rows_hide_nan_hidden_states(dev):
+    import siirl_amd.fused_linear as FL
+
+    T, H, V = 200, 64, 700
+    h, w, y, g_lp, g_h = _inputs(T, H, V, seed=11)
+    live = torch.arange(T) >= 60
+    h[:60] = float("nan")
+    hd, wd = h.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y.to(dev), 1.0)
+    torch.autograd.backward([lp, ent], [(g_lp * live).to(dev), (g_h * live).to(dev)])
+    assert torch.isfinite(hd.grad).all() and torch.isfinite(wd.grad).all()
+    assert not hd.grad[:60].any()
+    dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp[60:], g_h[60:], h[60:], w, y[60:], 1.0, dtype=torch.float64)
+    _check_grad(hd.grad[60:], dh64, "d_hidden")
+    _check_grad(wd.grad, dw64, "d_weight")
+
+
+def test_backward_rows_through_the_c_abi(dev):
+    """siirl_fused_linear_logprob_entropy_bwd_rows called directly: rows in any order, an index outside [0, T)
+    contributes nothing, a short workspace and a bad count are refused."""
+    import ctypes as C
+
+    from siirl_amd import _lib
+
+    T, H, V = 260, 64, 900
+    h, w, y, g_lp, g_h = _inputs(T, H, V, seed=5)
+    hd, wd, yd = h.to(dev), w.to(dev), y.to(dev)
+    ns = torch.ops.siirl_hip
+    _, _, lse, ex, _ = ns.fused_linear_logprob_entropy_fwd(hd, wd, yd, 1.0, False)
+    lib = _lib.lib()
+    st = _lib.current_stream(dev)
+
+    def call(rows, n=None, ws_short=0):
+        rows_d = torch.tensor(rows, dtype=torch.int64, device=dev)
+        n = len(rows) if n is None else n
+        nws = lib.siirl_fused_linear_bwd_rows_workspace_bytes(max(n, 0), H, V, 1, 1)
+        ws = torch.empty(max(nws - ws_short, 256), dtype=torch.uint8, device=dev)
+        d_h = torch.full((T, H), 7.0, dtype=torch.bfloat16, device=dev)
+        d_w = torch.full((V, H), 7.0, dtype=torch.bfloat16, device=dev)
+        glp_d, gh_d = g_lp.to(dev), g_h.to(dev)
+        rc = lib.siirl_fused_linear_logprob_entropy_bwd_rows(
+            _lib.ptr(hd), _lib.ptr(wd), _lib.BF16, _lib.ptr(yd), T, H, V, 1.0, _lib.ptr(lse), _lib.ptr(ex),
+            _lib.ptr(glp_d), _lib.ptr(gh_d), _lib.ptr(rows_d), n, _lib.ptr(d_h), _lib.ptr(d_w), _lib.ptr(ws),
+            C.c_size_t(nws - ws_short), st)
+        torch.cuda.synchronize()
+        return rc, d_h, d_w
+
+    picked = [259, 3, 100, 17, 256, 4]
+    rc, d_h, d_w = call(picked)
+    assert rc == 0
+    sel = torch.zeros(T, dtype=torch.bool)
+    sel[picked] = True
+    dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp * sel, g_h * sel, h, w, y, 1.0, dtype=torch.float64)
+    _check_grad(d_h, dh64, "d_hidden")
+    _check_grad(d_w, dw64, "d_weight")
+    assert not d_h[(~sel).to(dev)].any()
+    rc, d_h2, d_w2 = call(picked + [T + 5, -1])
+    assert rc == 0
+    assert torch.equal(d_h2, d_h)
+    _check_grad(d_w2, dw64, "d_weight with two rows outside the batch")
+    rc, d_h0, d_w0 = call([])
+    assert rc == 0 and not d_h0.any() and not d_w0.any()
+    assert call(picked, ws_short=512)[0] == -4
+    assert call(picked, n=T + 1)[0] == -1
+    assert call(picked, n=-1)[0] == -1

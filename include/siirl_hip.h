@@ -75,7 +75,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1006
+#define SIIRL_HIP_ABI_VERSION 1007
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -569,6 +569,41 @@ int siirl_grpo_outcome_advantage(const float* token_level_rewards, const void* m
  */
 int siirl_group_keep_mask(const void* metric, int metric_dtype, const int64_t* uid, int64_t B, uint8_t* keep,
                           int32_t* group_size, siirl_stream_t stream);
+
+/* ------------------------------------------------------------------- multi-agent GAE (MARFT) */
+
+#define SIIRL_MARFT_MAX_AGENTS 16
+
+/* What the reference's assignment into a tensor of the mask's dtype keeps of each float32 result. */
+typedef enum siirl_marft_store {
+  SIIRL_MARFT_STORE_FLOAT = 0,     /* the value itself */
+  SIIRL_MARFT_STORE_TRUNCATED = 1, /* its integer part (the reference's outputs take the integer mask's dtype) */
+  SIIRL_MARFT_STORE_NONZERO = 2    /* 1 where it is not zero (bool masks) */
+} siirl_marft_store;
+
+/*
+ * GAE over the trajectories of multi-agent requests, before whitening.  The batch of B rows holds each request as
+ * chain_len[c] consecutive rows from chain_start[c] (its steps, last step first); agent g (0 .. n_agents - 1, the
+ * last one being the batch's own response) has fp32 rewards / values [B, widths[g]] and an integer mask
+ * [B, widths[g]] whose row sum is the number of generated tokens, which sit at the front of the row.  One
+ * accumulator runs over a request: rows in order, agents from last to first, tokens from the last generated one to
+ * the first;  delta = gamma * V[t+1] - V[t] inside an agent's tokens and rew + gamma * V_next - V at its last token,
+ * where V_next is the first value of the next agent in the row, or for the last agent the first agent's first value
+ * in the row before (nothing in a request's first row);  gae = delta + gamma_lam * gae;  advantages[g][row, t] = gae,
+ * returns[g][row, t] = gae + V[t]; every other element of the outputs is zero.  float32 operation order of the
+ * reference: bit-identical results.  gamma_lam is the product as the caller's arithmetic yields it (the
+ * reference multiplies two Python floats in double and rounds the product once).
+ * token_level_rewards / values / masks / advantages / returns / widths: HOST arrays of n_agents device pointers
+ * (row lengths); chain_start / chain_len: device int64[n_chains]; status: device int32, 0 on success, 1 when a mask
+ * row summed to more than its length (clamped; the reference raises IndexError), 2 when a request's rows leave the
+ * batch (that request is skipped).
+ * Replaces: compute_marft_gae_advantage_return siirl/dag_worker/core_algos.py:351-450 (the whitening of :451 is
+ *           siirl_masked_whiten per agent).
+ */
+int siirl_marft_gae(const float* const* token_level_rewards, const float* const* values, const void* const* masks,
+                    int mask_dtype, const int64_t* widths, int n_agents, int64_t B, const int64_t* chain_start,
+                    const int64_t* chain_len, int64_t n_chains, float gamma, float gamma_lam, int store_mode,
+                    float* const* advantages, float* const* returns, int32_t* status, siirl_stream_t stream);
 
 /* ------------------------------------------------- lm_head projection fused with log-prob / entropy */
 

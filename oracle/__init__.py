@@ -38,6 +38,10 @@ compute_gae_advantage_return           gamma = lam = 1 -> reward-to-go minus val
                                        selection has mean 0 / unbiased variance 1 (numpy)
 masked_var / masked_whiten             numpy mean / var(ddof) of the selected elements; the two
                                        ValueErrors
+marft_gae_unwhitened /                 a two-agent, two-step request worked by hand (float and
+compute_marft_gae_advantage_return     truncated outputs); single agent == the GAE scan above;
+                                       gamma = lam = 1 -> rewards met so far minus value; keys
+                                       written, id list growth, dtypes and the four errors
 compute_value_loss                     hand-computed cases either side of the clip range; zero
                                        gradient where clipped
 compute_policy_loss_cpgd / drift       hand-computed tokens with log(1 +- eps) bounds; gradient

@@ -107,6 +107,78 @@ def compute_gae_advantage_return(token_level_rewards, values, response_mask, gam
     return masked_whiten(adv, response_mask), returns
 
 
+def marft_gae_unwhitened(rewards, values, masks, chains, gamma, lam, out_dtype=None):
+    """The token walk of the reference's multi-agent GAE (``core_algos.py:400-448``) on explicit operands:
+    ``rewards`` / ``values`` / ``masks`` are lists over the agents (the batch's own response last) of ``[B, L_a]``
+    tensors, ``chains`` a list of ``(first_row, n_rows)`` per request (rows = trajectory steps, last step first).
+    One accumulator runs through a request: rows in order, agents from last to first, tokens from the last
+    generated one (``mask row sum - 1``) down to 0.  Inside an agent ``delta = gamma * V[t + 1] - V[t]``; at its
+    last token ``delta = rew + gamma * V_next - V`` with ``V_next`` the next agent's first value in the row, or, for
+    the last agent, the first agent's first value in the row before (0 in the request's first row).  The outputs
+    take the masks' dtype, as the reference's ``zeros_like(response_mask)`` does (``:386-392``): an integer mask
+    truncates every stored advantage and return (``out_dtype`` overrides that, to see the values before the
+    truncation).  Arithmetic is that of 0-d tensors and Python floats, as there.
+    Returns ``(advantages, returns)``, lists over the agents."""
+    adv = [torch.zeros_like(m, dtype=out_dtype) for m in masks]
+    ret = [torch.zeros_like(a) for a in adv]
+    last = len(masks) - 1
+    for first_row, n_rows in chains:
+        gae = 0
+        for step in range(n_rows):
+            row = first_row + step
+            for agent in range(last, -1, -1):
+                gen = masks[agent][row].sum()
+                for t in reversed(range(gen)):
+                    v = values[agent][row, t]
+                    if t == gen - 1:
+                        if agent == last:
+                            v_next = 0 if step == 0 else values[0][row - 1, 0]
+                        else:
+                            v_next = values[agent + 1][row, 0]
+                        delta = rewards[agent][row, t] + gamma * v_next - v
+                    else:
+                        delta = gamma * values[agent][row, t + 1] - v
+                    gae = delta + gamma * lam * gae
+                    adv[agent][row, t] = gae
+                    ret[agent][row, t] = gae + v
+    return adv, ret
+
+
+def compute_marft_gae_advantage_return(data, pre_agent_group_ids, gamma, lam):
+    """``siirl/dag_worker/core_algos.py:351-458``.  ``data.batch`` holds ``agent_group_<id>_token_level_rewards`` /
+    ``_values`` / ``_response_mask`` for every id of ``pre_agent_group_ids`` and the unprefixed three for the last
+    agent; ``data.non_tensor_batch`` holds ``request_id`` (rows of one request are consecutive; the first row of each
+    distinct id starts a request) and ``traj_len`` (read at that first row).  As in the reference: the id list is
+    indexed by its own values (so it must be 0 .. n - 1) and grows by one id per call (``:395``); every agent's
+    advantages are whitened over its mask (``:451``) but the results of all the earlier agents are stored under the
+    LAST of the given ids, each overwriting the one before (``:452-454`` use the loop variable left over from
+    ``:379``), so only that id's two keys and ``advantages`` / ``returns`` appear in ``data.batch``."""
+    prefix = "agent_group_"
+    names = [prefix + str(g) + "_" for g in pre_agent_group_ids] + [""]
+    rewards = [data.batch[n + "token_level_rewards"] for n in names]
+    values = [data.batch[n + "values"] for n in names]
+    masks = [data.batch[n + "response_mask"] for n in names]
+    last_given = pre_agent_group_ids[-1]
+    pre_agent_group_ids.append(last_given + 1)
+    seen, chains = set(), []
+    for row, rid in enumerate(data.non_tensor_batch["request_id"]):
+        if rid not in seen:
+            seen.add(rid)
+            chains.append((row, int(data.non_tensor_batch["traj_len"][row])))
+    with torch.no_grad():
+        order = list(pre_agent_group_ids)
+        adv, ret = marft_gae_unwhitened([rewards[g] for g in order], [values[g] for g in order],
+                                        [masks[g] for g in order], chains, gamma, lam)
+        for g in order:
+            white = masked_whiten(adv[g], masks[g])
+            if g != order[-1]:
+                data.batch[prefix + str(last_given) + "_advantages"] = white
+                data.batch[prefix + str(last_given) + "_returns"] = ret[g]
+            else:
+                data.batch["advantages"] = white
+                data.batch["returns"] = ret[g]
+
+
 # --------------------------------------------------------------------------- aggregation
 
 

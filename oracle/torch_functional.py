@@ -124,7 +124,7 @@ def logprob_entropy_backward_autograd(logits, labels, g_logprob, g_entropy, temp
 def masked_sum(values, mask, axis=None):
     """``sum(where(mask, v, 0) * mask)`` (reference ``torch_functional.py:146-151``): values outside
     the mask, NaN included, do not contribute."""
-    kept = torch.where(mask.bool(), values, torch.zeros((), dtype=values.dtype))
+    kept = torch.where(mask.bool(), values, 0.0)  # (integer values become float32 here, as in the reference)
     return (kept * mask).sum(axis)
 
 

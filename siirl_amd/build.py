@@ -26,9 +26,9 @@ ARCH = "gfx950"
 # -packed-fp32-ops: keep the compiler from forming v_pk_{add,mul,fma}_f32 out of scalar float code.
 CXXFLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
             "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-fno-gpu-rdc"]
-# per-file additions: the numpy-emulating group statistics and the GAE recurrence must not be contracted into FMAs
+# per-file additions: the numpy-emulating group statistics and the GAE recurrences must not be contracted into FMAs
 EXTRA = {"group_ops.hip": ["-ffp-contract=off"], "gae.hip": ["-ffp-contract=off"],
-         "reward.hip": ["-ffp-contract=off"]}
+         "reward.hip": ["-ffp-contract=off"], "marft_gae.hip": ["-ffp-contract=off"]}
 
 
 def sources():

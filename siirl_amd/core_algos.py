@@ -335,6 +335,122 @@ def compute_cpgd_outcome_advantage(token_level_rewards: torch.Tensor, response_m
     return adv, adv
 
 
+_MARFT_INT_MASKS = (torch.bool, torch.uint8, torch.int32, torch.int64)
+
+
+def marft_gae_unwhitened(rewards, values, masks, chains, gamma, lam, out_dtype=None):
+    """The token walk of the reference's multi-agent GAE (``core_algos.py:400-448``) for explicit operands: lists
+    over the agents (the batch's own response last) of ``[B, L_a]`` tensors, ``chains`` = ``(first_row, n_rows)`` per
+    request.  Returns ``(advantages, returns)``, lists of tensors of ``out_dtype`` (default: each mask's dtype, what
+    the reference's ``zeros_like(response_mask)`` gives: integer masks keep the integer part of every result)."""
+    n_agents = len(masks)
+    if not (len(rewards) == len(values) == n_agents) or n_agents < 1:
+        raise ValueError("rewards, values and masks must list the same agents")
+    if n_agents > _lib.MARFT_MAX_AGENTS:
+        raise NotImplementedError(f"siirl_amd: at most {_lib.MARFT_MAX_AGENTS} agents, got {n_agents}")
+    dev, back = _staging_device(*rewards, *values, *masks)
+    B = masks[0].shape[0]
+    mdt = masks[0].dtype
+    for r, v, m in zip(rewards, values, masks):
+        if m.dim() != 2 or m.shape[0] != B or r.shape != m.shape or v.shape != m.shape:
+            raise ValueError(f"every agent needs [B, L] rewards, values and mask with B = {B}; got {tuple(r.shape)}, "
+                             f"{tuple(v.shape)}, {tuple(m.shape)}")
+        if m.shape[1] < 1:
+            raise IndexError("index 0 is out of bounds for dimension 1 with size 0")
+        if m.dtype != mdt:
+            raise NotImplementedError("siirl_amd: the agents' masks must share one dtype")
+    chains = [(int(s), int(n)) for s, n in chains]
+    walked = [c for c in chains if c[1] > 0]
+    if walked and mdt not in _MARFT_INT_MASKS:
+        # the reference's range(mask row sum) (:410-412)
+        raise TypeError("only integer tensors of a single element can be converted to an index")
+    for first, n in walked:
+        if first < 0 or first + n > B:
+            raise IndexError(f"index {first + n - 1} is out of bounds for dimension 0 with size {B}")
+    out_dtypes = [out_dtype or m.dtype for m in masks]
+    if any(d != out_dtypes[0] for d in out_dtypes):
+        raise NotImplementedError("siirl_amd: the agents' outputs must share one dtype")
+    if out_dtypes[0].is_floating_point:
+        mode = _lib.MARFT_STORE_FLOAT
+    else:
+        mode = _lib.MARFT_STORE_NONZERO if out_dtypes[0] == torch.bool else _lib.MARFT_STORE_TRUNCATED
+    r32 = [_f32(t, dev) for t in rewards]
+    v32 = [_f32(t, dev) for t in values]
+    m_dev = [m.detach().to(dev).contiguous() for m in masks]
+    if mdt not in _MARFT_INT_MASKS:  # no request is walked: the masks are never read
+        m_dev = [torch.zeros(m.shape, dtype=torch.int64, device=dev) for m in masks]
+    mcode = _lib.dtype_code(m_dev[0].dtype)
+    adv = [torch.empty(m.shape, dtype=torch.float32, device=dev) for m in masks]
+    ret = [torch.empty(m.shape, dtype=torch.float32, device=dev) for m in masks]
+    status = torch.empty(1, dtype=torch.int32, device=dev)
+    starts = torch.tensor([c[0] for c in walked], dtype=torch.int64).to(dev)
+    lens = torch.tensor([c[1] for c in walked], dtype=torch.int64).to(dev)
+    ptrs = lambda ts: (C.c_void_p * n_agents)(*[t.data_ptr() for t in ts])  # noqa: E731
+    widths = (C.c_int64 * n_agents)(*[m.shape[1] for m in masks])
+    # gamma * lam as the reference forms it: the product of two Python floats, rounded to float32 once; of two
+    # tensors, their float32 product
+    if isinstance(gamma, torch.Tensor) or isinstance(lam, torch.Tensor):
+        g32 = float(torch.as_tensor(gamma, dtype=torch.float32))
+        gl32 = float(torch.as_tensor(gamma, dtype=torch.float32) * torch.as_tensor(lam, dtype=torch.float32))
+    else:
+        g32, gl32 = float(gamma), float(gamma) * float(lam)
+    with torch.cuda.device(dev):
+        rc = _lib.lib().siirl_marft_gae(ptrs(r32), ptrs(v32), ptrs(m_dev), mcode, widths, n_agents, B, _lib.ptr(starts),
+                                        _lib.ptr(lens), len(walked), g32, gl32, mode, ptrs(adv), ptrs(ret),
+                                        _lib.ptr(status), _lib.current_stream(dev))
+    _lib.check(rc, "siirl_marft_gae")
+    if int(status.item()) == 1:
+        raise IndexError("a response_mask row sums to more than its length: the token walk would leave the row")
+    adv = [a.to(d) for a, d in zip(adv, out_dtypes)]
+    ret = [a.to(d) for a, d in zip(ret, out_dtypes)]
+    if back:
+        adv = [a.to(m.device) for a, m in zip(adv, masks)]
+        ret = [a.to(m.device) for a, m in zip(ret, masks)]
+    return adv, ret
+
+
+def compute_marft_gae_advantage_return(data, pre_agent_group_ids, gamma, lam):
+    """Multi-agent GAE over reversed trajectories (reference ``core_algos.py:351-458``).  ``data.batch`` holds
+    ``agent_group_<id>_token_level_rewards`` / ``_values`` / ``_response_mask`` for every id of
+    ``pre_agent_group_ids`` plus the unprefixed three of the last agent; ``data.non_tensor_batch`` holds
+    ``request_id`` (the first row of each distinct id starts a request) and ``traj_len`` (read at that row).
+    Writes ``advantages`` / ``returns`` and returns ``None``.  Kept from the reference, because callers see them:
+    the id list grows by one id per call (``:395``); the ids index the agent list, so they must be ``0 .. n - 1``;
+    every agent's advantages are whitened over its own mask (``:451``, with ``masked_var``'s two ``ValueError``s),
+    but the results of all the earlier agents go to the keys of the LAST given id, each overwriting the one
+    before (``:452-454``); outputs before whitening take the mask's dtype (``:386-392``), so with the integer masks
+    the token walk requires every stored advantage and return is truncated to its integer part."""
+    batch, extra = data.batch, data.non_tensor_batch
+    prefix = "agent_group_"
+    names = [prefix + str(g) + "_" for g in pre_agent_group_ids] + [""]
+    rewards = [batch[n + "token_level_rewards"] for n in names]
+    values = [batch[n + "values"] for n in names]
+    masks = [batch[n + "response_mask"] for n in names]
+    last_given = pre_agent_group_ids[-1]  # IndexError for an empty list, as in the reference
+    pre_agent_group_ids.append(last_given + 1)
+    if list(pre_agent_group_ids) != list(range(len(pre_agent_group_ids))):
+        raise NotImplementedError("siirl_amd: agent group ids must be 0 .. n - 1 (the reference indexes its agent list "
+                                  f"with them), got {pre_agent_group_ids[:-1]}")
+    seen, chains = set(), []
+    for row, rid in enumerate(extra["request_id"]):
+        if rid not in seen:
+            seen.add(rid)
+            chains.append((row, int(extra["traj_len"][row])))
+    adv, ret = marft_gae_unwhitened(rewards, values, masks, chains, gamma, lam)
+    for g, (a, r, m) in enumerate(zip(adv, ret, masks)):
+        if a.is_cuda:
+            white = siirl_F.masked_whiten(a, m)
+        else:
+            dev, _ = _staging_device(a)
+            white = siirl_F.masked_whiten(a.to(dev), m.to(dev)).to(a.device)
+        if g != len(adv) - 1:
+            _td_set(data, prefix + str(last_given) + "_advantages", white)
+            _td_set(data, prefix + str(last_given) + "_returns", r)
+        else:
+            _td_set(data, "advantages", white)
+            _td_set(data, "returns", r)
+
+
 def compute_rewards(token_level_scores, old_log_prob, ref_log_prob, kl_ratio):
     """reference ``core_algos.py:520-533``: ``scores - (old - ref) * kl_ratio`` (k1 estimator, no mask)."""
     dev = _gpu_of(token_level_scores, old_log_prob, ref_log_prob)
@@ -385,8 +501,8 @@ def apply_kl_penalty(data, kl_ctrl, kl_penalty="kl", multi_turn=False):
 def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_in_grpo=True,
                       weight_factor_in_cpgd="STD_weight", **kwargs):
     """Dispatcher (reference ``core_algos.py:1400-1492``).  The GAE (``:1424-1439``, without the PF-PPO
-    reweighting) and GRPO (``:1440-1471``) branches are built; MARFT raises ``NotImplementedError`` here, and
-    the CPGD branch fails with the reference's own ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a
+    reweighting), GRPO (``:1440-1471``) and multi-agent GAE (``:1483-1489``, ``data`` then needs ``.batch`` and
+    ``.non_tensor_batch``) branches are built; the CPGD branch fails with the reference's own ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a
     keyword it does not take, ``:1475-1480``); ``compute_cpgd_outcome_advantage`` is there to be called directly."""
     if "response_mask" not in data.keys():
         _td_set(data, "response_mask", compute_response_mask(data))
@@ -420,7 +536,10 @@ def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_i
         compute_grpo_outcome_advantage(token_level_rewards=data["token_level_rewards"],
                                        response_mask=data["response_mask"], index=data["uid"],
                                        weight_factor_in_cpgd=weight_factor_in_cpgd)
-    raise NotImplementedError(f"advantage estimator {est!r} is outside this build (GAE and GRPO only)")
+    if est == "gae_marft":
+        compute_marft_gae_advantage_return(data, pre_agent_group_ids=kwargs["agent_group_ids"], gamma=gamma, lam=lam)
+        return data
+    raise NotImplementedError
 
 
 # ------------------------------------------------------------------------------------ aggregation

@@ -13,8 +13,10 @@ tensors of the actor's micro-batch:
   their registry entries (``dp_actor.py:453-486``).  Three of the reference's own (``clip_cov``, ``kl_cov``,
   ``geo_mean``) refuse the stock actors' config class (``core_algos.py:940,1031,1104``); the replacements read the
   same attributes from any config object and have no such check;
-* ``compute_grpo_outcome_advantage`` and ``apply_kl_penalty``, which the reference runs on host tensors
-  (``siirl/dag_worker/dagworker.py:542-560``): the replacements stage host inputs to the GPU and return host results.
+* ``compute_grpo_outcome_advantage``, ``compute_marft_gae_advantage_return`` and ``apply_kl_penalty``, which the
+  reference runs on host tensors (``siirl/dag_worker/dagworker.py:542-560,585-630``): the replacements stage host inputs
+  to the GPU and return host results.  (The multi-agent GAE is a Python loop over every token in the reference,
+  ``core_algos.py:400-448``.)
 
 Deliberately NOT replaced: ``masked_sum`` / ``masked_mean`` / ``masked_var`` / ``masked_whiten``.  The reference's own
 ``compute_gae_advantage_return`` resolves those globals and calls them on host tensors, where this package's versions
@@ -29,7 +31,7 @@ POLICY_LOSSES = {"vanilla": "compute_policy_loss_vanilla", "gspo": "compute_poli
                  "clip_cov": "compute_policy_loss_clip_cov", "kl_cov": "compute_policy_loss_kl_cov",
                  "geo_mean": "compute_policy_loss_geo_mean"}
 CORE_ALGOS_NAMES = ("agg_loss", "kl_penalty", "compute_policy_loss", *POLICY_LOSSES.values(),
-                    "compute_grpo_outcome_advantage", "apply_kl_penalty")
+                    "compute_grpo_outcome_advantage", "compute_marft_gae_advantage_return", "apply_kl_penalty")
 
 
 def patch_reference(ref_torch_functional, ref_core_algos) -> dict:

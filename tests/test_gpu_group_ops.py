@@ -143,8 +143,10 @@ def test_compute_advantage_dispatch(dev):
         CA.get_adv_estimator_fn("gae_marft")
     with pytest.raises(TypeError):  # the reference's CPGD branch passes a keyword GRPO does not take
         CA.compute_advantage(dict(data), "cpgd")
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(KeyError):  # the multi-agent estimator reads its agent list from the keyword arguments
         CA.compute_advantage(dict(data), "gae_marft")
+    with pytest.raises(NotImplementedError):
+        CA.compute_advantage(dict(data), "reinforce_plus_plus")
 
 
 # ------------------------------------------------------------------------------------ DAPO keep mask

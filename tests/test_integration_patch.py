@@ -21,7 +21,7 @@ def _stub_modules():
     F.masked_mean, F.masked_whiten = masked_mean, masked_whiten
     modes = ("vanilla", "gspo", "cpgd", "gpg", "clip_cov", "kl_cov", "geo_mean")
     for name in ("agg_loss", "kl_penalty", "compute_policy_loss", "compute_grpo_outcome_advantage", "apply_kl_penalty",
-                 "compute_value_loss", *(f"compute_policy_loss_{m}" for m in modes)):
+                 "compute_marft_gae_advantage_return", "compute_value_loss", *(f"compute_policy_loss_{m}" for m in modes)):
         setattr(A, name, lambda *a, **k: "reference")
     A.POLICY_LOSS_REGISTRY = {m: getattr(A, f"compute_policy_loss_{m}") for m in modes}
     A.POLICY_LOSS_REGISTRY["users_own"] = A.compute_value_loss

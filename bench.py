@@ -681,6 +681,25 @@ def bench_critic(args, dev):
         gae_chunked_ms = g0.elapsed_time(g1) / steps
     finally:
         CA.set_gae_scan_order("exact")
+    # multi-agent GAE: 128 requests of 4 trajectory steps, 3 agents answering with 1024-2048 tokens each; one call
+    # of the token walk (the reference's per-token Python loop), operands on the GPU
+    m_req, m_steps, m_w = 128, 4, 2048
+    m_rows = m_req * m_steps
+    m_vals = [torch.randn(m_rows, m_w, device=dev, generator=gen) for _ in range(3)]
+    m_rews = [torch.randn(m_rows, m_w, device=dev, generator=gen) for _ in range(3)]
+    m_masks = [(torch.arange(m_w, device=dev)[None] <
+                torch.randint(m_w // 2, m_w + 1, (m_rows, 1), device=dev, generator=gen)).long() for _ in range(3)]
+    m_chains = [(i * m_steps, m_steps) for i in range(m_req)]
+    m_tokens = sum(int(m.sum()) for m in m_masks)
+    for _ in range(warm):
+        CA.marft_gae_unwhitened(m_rews, m_vals, m_masks, m_chains, 0.99, 0.95)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    for _ in range(steps):
+        CA.marft_gae_unwhitened(m_rews, m_vals, m_masks, m_chains, 0.99, 0.95)
+    torch.cuda.synchronize()
+    marft_ms = (time.perf_counter() - t1) * 1e3 / steps
+    marft = {"ms": marft_ms, "tokens_walked": m_tokens, "tokens_per_s": m_tokens / marft_ms * 1e3}
     # GAE + whitening: the scan reads rewards, values, mask and writes advantages, returns (24 B + 8 B mask), the
     # whitening apply reads and writes the advantages once more
     gae_bytes = tokens * (4 + 4 + 8 + 4 + 4 + 4 + 4)
@@ -692,7 +711,9 @@ def bench_critic(args, dev):
         "config": {"workload": f"critic: {B} trajectories, prompt {P} + response {L}, gamma 1.0, lam 0.95, "
                                f"cliprange_value 0.5, overlong buffer 1024", "seed": SEED},
         "kernels": {**{name: {"ms": t} for name, t in zip(ops, ms)},
-                    "GAE + whitening, chunked scan order (not in the step above)": {"ms": gae_chunked_ms}},
+                    "GAE + whitening, chunked scan order (not in the step above)": {"ms": gae_chunked_ms},
+                    f"multi-agent GAE token walk, {m_req} requests x {m_steps} steps x 3 agents x <= {m_w} tokens "
+                    "(not in the step above)": marft},
         "roofline": {"bound": "hbm", "kernel": "gae_scan_vec_kernel + whiten_apply_kernel", "achieved": gae_bytes / ms[1] / 1e6,
                      "peak": 8000.0, "unit": "GB/s", "frac": gae_bytes / ms[1] / 1e6 / 8000.0, "traffic": None,
                      "note": "the scan is a sequential recurrence per row: its duration is the latency of 8192 dependent "
@@ -725,6 +746,13 @@ def bench_critic(args, dev):
         out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(),
                                "kind": "port", "sample": f"first {n_s} of {B} trajectories x {L} tokens; median of 2 "
                                                          f"passes ({med:.2f} s each)"}
+        # the oracle's multi-agent walk (the reference's loop over every token): two requests of the batch above
+        cut = 2 * m_steps
+        t1 = time.perf_counter()
+        OC.marft_gae_unwhitened([t[:cut].cpu() for t in m_rews], [t[:cut].cpu() for t in m_vals],
+                                [t[:cut].cpu() for t in m_masks], m_chains[:2], 0.99, 0.95)
+        dt = time.perf_counter() - t1
+        marft["cpu_oracle_tokens_per_s"] = sum(int(m[:cut].sum()) for m in m_masks) / dt
     print(json.dumps(out), flush=True)
 
 

@@ -366,3 +366,26 @@ def test_backward_rows_through_the_c_abi(dev):
     assert call(picked, ws_short=512)[0] == -4
     assert call(picked, n=T + 1)[0] == -1
     assert call(picked, n=-1)[0] == -1
+
+
+@pytest.mark.parametrize("wrt", ["hidden", "weight"])
+def test_zero_gradient_rows_with_one_gradient_requested(dev, wrt):
+    """The row-subset backward when only d_hidden or only d_weight is asked for."""
+    import siirl_amd.fused_linear as FL
+
+    T, H, V = 300, 128, 1000
+    h, w, y, g_lp, g_h = _inputs(T, H, V, seed=77)
+    live = _live_rows(T, "packed", seed=77)
+    g_lp, g_h = g_lp * live, g_h * live
+    dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp, g_h, h, w, y, 1.0, dtype=torch.float64)
+    hd = h.to(dev).requires_grad_(wrt == "hidden")
+    wd = w.to(dev).requires_grad_(wrt == "weight")
+    lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y.to(dev), 1.0)
+    torch.autograd.backward([lp, ent], [g_lp.to(dev), g_h.to(dev)])
+    if wrt == "hidden":
+        assert wd.grad is None
+        _check_grad(hd.grad, dh64, "d_hidden")
+        assert not hd.grad[(~live).to(dev)].any()
+    else:
+        assert hd.grad is None
+        _check_grad(wd.grad, dw64, "d_weight")

@@ -38,6 +38,9 @@ compute_gae_advantage_return           gamma = lam = 1 -> reward-to-go minus val
                                        selection has mean 0 / unbiased variance 1 (numpy)
 masked_var / masked_whiten             numpy mean / var(ddof) of the selected elements; the two
                                        ValueErrors
+pf_ppo_weights /                       the three weightings by hand (|s|^p, 1 at max and min,
+compute_pf_ppo_reweight_data           0.4 / 0.1); one draw indexes tensors, arrays, lists and
+                                       meta lists alike; the input is left alone
 marft_gae_unwhitened /                 a two-agent, two-step request worked by hand (float and
 compute_marft_gae_advantage_return     truncated outputs); single agent == the GAE scan above;
                                        gamma = lam = 1 -> rewards met so far minus value; keys

@@ -179,6 +179,40 @@ def compute_marft_gae_advantage_return(data, pre_agent_group_ids, gamma, lam):
                 data.batch["returns"] = ret[g]
 
 
+def pf_ppo_weights(scores, reweight_method: str, weight_pow: float):
+    """Resampling weights of PF-PPO from per-sequence scores (reference ``core_algos.py:1296-1327``), with the
+    ``+ 1e-8`` floor of ``:1329``."""
+    if reweight_method == "pow":
+        w = scores.abs() ** weight_pow
+    elif reweight_method == "max_min":
+        w = ((scores == scores.max()) | (scores == scores.min())).to(torch.float32)
+    elif reweight_method == "max_random":
+        w = torch.full_like(scores, 0.1)
+        w[scores == scores.max()] = 0.4
+    else:
+        raise ValueError(f"Unsupported reweight_method: {reweight_method}")
+    return torch.clamp(w + 1e-8, min=1e-8)
+
+
+def compute_pf_ppo_reweight_data(data, reweight_method: str = "pow", weight_pow: float = 2.0):
+    """``siirl/dag_worker/core_algos.py:1279-1355``: ``batch_size`` rows drawn with replacement (``torch.multinomial``
+    on the host generator) with the weights above; tensors, per-row arrays / lists and ``batch_size``-long meta
+    lists are indexed with the draw; the input is left alone and a copy returned."""
+    import copy
+
+    scores = data.batch["token_level_scores"].sum(dim=-1)
+    n = scores.shape[0]
+    picks = torch.multinomial(pf_ppo_weights(scores, reweight_method, weight_pow), n, replacement=True)
+    out = copy.deepcopy(data)
+    out.batch = type(data.batch)({k: t[picks] for k, t in data.batch.items()})
+    idx = picks.numpy()
+    out.non_tensor_batch = {k: (a[idx] if isinstance(a, np.ndarray) else [a[i] for i in idx])
+                            for k, a in data.non_tensor_batch.items()}
+    out.meta_info = {k: ([v[i] for i in idx] if isinstance(v, list) and len(v) == n else v)
+                     for k, v in data.meta_info.items()}
+    return out
+
+
 # --------------------------------------------------------------------------- aggregation
 
 

@@ -477,6 +477,57 @@ def _kl_in_reward(scores, old, ref, mask, kl_type, beta, dev):
     return rewards.reshape(scores.shape), cur
 
 
+def _resample_rows(t: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+    """``t[idx]`` along the first axis; tensors on the GPU whose rows are whole 4-byte words go through the row
+    gather of the un-padding path."""
+    if t.is_cuda and t.dim() >= 1 and t.shape[0] and (t[0].numel() * t.element_size()) % 4 == 0 \
+            and t[0].numel() * t.element_size() >= 4 and not t.requires_grad:
+        from . import padding as _padding
+
+        return _padding.index_first_axis(t, idx.to(t.device))
+    return t[idx.to(t.device)]
+
+
+def compute_pf_ppo_reweight_data(data, reweight_method: str = "pow", weight_pow: float = 2.0):
+    """PF-PPO resampling of a batch by its scores (reference ``core_algos.py:1279-1355``): per-sequence score =
+    ``token_level_scores.sum(-1)``; weight ``|score| ** weight_pow`` ("pow"), 1 at the batch's maximum and minimum
+    score and 0 elsewhere ("max_min"), or 0.4 at the maximum and 0.1 elsewhere ("max_random"), ``+ 1e-8``;
+    ``batch_size`` indices are drawn with replacement by ``torch.multinomial`` on the scores' device (the reference's
+    batch lives on the host, so the same seed gives the same draw) and every tensor of ``data.batch``, every array or
+    list of ``data.non_tensor_batch`` and every ``batch_size``-long list of ``data.meta_info`` is indexed with them.
+    Returns a deep copy of ``data`` holding the resampled parts; ``data`` itself is left alone."""
+    from copy import deepcopy
+
+    with torch.no_grad():
+        scores = data.batch["token_level_scores"].sum(dim=-1)
+        if reweight_method == "pow":
+            weights = torch.pow(torch.abs(scores), weight_pow)
+        elif reweight_method == "max_min":
+            weights = torch.where((scores == torch.max(scores)) | (scores == torch.min(scores)), 1.0, 0.0)
+        elif reweight_method == "max_random":
+            weights = torch.where(scores == torch.max(scores), 0.4, 0.1)
+        else:
+            raise ValueError(f"Unsupported reweight_method: {reweight_method}")
+        weights = torch.clamp(weights + 1e-8, min=1e-8)
+        batch_size = scores.shape[0]
+        picks = torch.multinomial(weights, batch_size, replacement=True)
+        resampled = {key: _resample_rows(t, picks) for key, t in data.batch.items()}
+    picks_np = picks.cpu().numpy()
+    extra = {}
+    for key, arr in data.non_tensor_batch.items():
+        extra[key] = arr[picks_np] if isinstance(arr, np.ndarray) else [arr[i] for i in picks_np]
+    meta = {}
+    for key, val in data.meta_info.items():
+        meta[key] = [val[i] for i in picks_np] if isinstance(val, list) and len(val) == batch_size else val
+    out = deepcopy(data)
+    out.batch = type(data.batch)(resampled)
+    if hasattr(data.batch, "batch_size"):
+        out.batch.batch_size = data.batch.batch_size
+    out.non_tensor_batch = extra
+    out.meta_info = meta
+    return out
+
+
 def _td_set(data, key, value):
     target = data.batch if hasattr(data, "batch") and not callable(getattr(data, "batch")) else data
     target[key] = value
@@ -508,13 +559,14 @@ def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_i
         _td_set(data, "response_mask", compute_response_mask(data))
     est = adv_estimator.value if isinstance(adv_estimator, Enum) else adv_estimator
     if est == "gae":
-        if kwargs.get("use_pf_ppo", False):
-            raise NotImplementedError("PF-PPO reweighting is outside this build")
         advantages, returns = compute_gae_advantage_return(
             token_level_rewards=data["token_level_rewards"], values=data["values"],
             response_mask=data["response_mask"], gamma=gamma, lam=lam)
         data["advantages"] = advantages
         data["returns"] = returns
+        if kwargs.get("use_pf_ppo", False):
+            data = compute_pf_ppo_reweight_data(data, kwargs.get("pf_ppo_reweight_method", "pow"),
+                                                kwargs.get("pf_ppo_weight_pow", 2.0))
         return data
     if est == "grpo":
         if "finish_step" in data.keys() and data["responses"].ndim == 3:

@@ -239,3 +239,64 @@ def test_geo_mean_importance_weights_enter_as_their_geometric_mean():
     w = torch.tensor([[4.0, 1.0]], dtype=torch.float64)
     loss, *_ = O.compute_policy_loss_geo_mean(old, lp, A, torch.ones(1, 2), "token-mean", cfg, w)
     assert abs(float(loss) - (-1.0 * math.exp(0.0) * 2.0)) < 1e-6
+
+
+# ------------------------------------------------------------------------------------ PF-PPO resampling
+
+
+def test_pf_ppo_weights_by_hand():
+    import math
+
+    import torch
+
+    from oracle import core_algos as OC
+
+    s = torch.tensor([2.0, -3.0, 0.0, 2.0, 0.5])
+    w = OC.pf_ppo_weights(s, "pow", 2.0)
+    assert w.tolist() == pytest.approx([4.0, 9.0, 1e-8, 4.0, 0.25], rel=1e-6)
+    w = OC.pf_ppo_weights(s, "pow", 0.5)
+    assert w.tolist() == pytest.approx([math.sqrt(2), math.sqrt(3), 1e-8, math.sqrt(2), math.sqrt(0.5)], rel=1e-6)
+    w = OC.pf_ppo_weights(s, "max_min", 2.0)  # both sequences at the maximum, the one at the minimum
+    assert w.tolist() == pytest.approx([1.0, 1.0, 1e-8, 1.0, 1e-8], rel=1e-6)
+    w = OC.pf_ppo_weights(s, "max_random", 2.0)
+    assert w.tolist() == pytest.approx([0.4, 0.1, 0.1, 0.4, 0.1], rel=1e-6)
+    with pytest.raises(ValueError, match="Unsupported reweight_method"):
+        OC.pf_ppo_weights(s, "median", 2.0)
+
+
+def _pf_ppo_batch(B=12, L=5, seed=0):
+    from types import SimpleNamespace
+
+    import numpy as np
+    import torch
+
+    g = torch.Generator().manual_seed(seed)
+    batch = {"token_level_scores": torch.randn(B, L, generator=g), "responses": torch.randint(0, 99, (B, L), generator=g),
+             "advantages": torch.randn(B, L, generator=g), "flag": torch.arange(B, dtype=torch.uint8)}
+    extra = {"uid": np.array([f"u{i}" for i in range(B)], dtype=object), "names": [f"n{i}" for i in range(B)]}
+    meta = {"per_row": list(range(B)), "temperature": 0.7, "short_list": [1, 2]}
+    return SimpleNamespace(batch=batch, non_tensor_batch=extra, meta_info=meta)
+
+
+def test_pf_ppo_resampling_is_one_draw_applied_everywhere():
+    import torch
+
+    from oracle import core_algos as OC
+
+    data = _pf_ppo_batch()
+    before = {k: v.clone() for k, v in data.batch.items()}
+    torch.manual_seed(5)
+    out = OC.compute_pf_ppo_reweight_data(data, "pow", 2.0)
+    # the draw: torch.multinomial on the global host generator, from the hand-checked weights
+    torch.manual_seed(5)
+    picks = torch.multinomial(OC.pf_ppo_weights(before["token_level_scores"].sum(-1), "pow", 2.0), 12, replacement=True)
+    for k, v in before.items():
+        assert torch.equal(out.batch[k], v[picks]) and torch.equal(data.batch[k], v)  # the input is left alone
+    assert list(out.non_tensor_batch["uid"]) == [f"u{i}" for i in picks.tolist()]
+    assert out.non_tensor_batch["names"] == [f"n{i}" for i in picks.tolist()]
+    assert out.meta_info == {"per_row": picks.tolist(), "temperature": 0.7, "short_list": [1, 2]}
+    # "max_min": only the best and the worst sequence are ever drawn (their weight is 1 against 1e-8)
+    torch.manual_seed(1)
+    out = OC.compute_pf_ppo_reweight_data(data, "max_min")
+    s = before["token_level_scores"].sum(-1)
+    assert set(out.meta_info["per_row"]) <= {int(s.argmax()), int(s.argmin())}

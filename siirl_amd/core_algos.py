@@ -342,7 +342,18 @@ def marft_gae_unwhitened(rewards, values, masks, chains, gamma, lam, out_dtype=N
     """The token walk of the reference's multi-agent GAE (``core_algos.py:400-448``) for explicit operands: lists
     over the agents (the batch's own response last) of ``[B, L_a]`` tensors, ``chains`` = ``(first_row, n_rows)`` per
     request.  Returns ``(advantages, returns)``, lists of tensors of ``out_dtype`` (default: each mask's dtype, what
-    the reference's ``zeros_like(response_mask)`` gives: integer masks keep the integer part of every result)."""
+    the reference's ``zeros_like(response_mask)`` gives: integer masks keep the integer part of every result), on the
+    device of the inputs (host inputs are staged to the GPU and the results copied back)."""
+    adv, ret, _, back = _marft_walk(rewards, values, masks, chains, gamma, lam, out_dtype)
+    if back:
+        adv = [a.to(m.device) for a, m in zip(adv, masks)]
+        ret = [a.to(m.device) for a, m in zip(ret, masks)]
+    return adv, ret
+
+
+def _marft_walk(rewards, values, masks, chains, gamma, lam, out_dtype=None):
+    """``marft_gae_unwhitened`` with the results left on the GPU: ``(advantages, returns, masks on the GPU, whether
+    the inputs were on the host)``."""
     n_agents = len(masks)
     if not (len(rewards) == len(values) == n_agents) or n_agents < 1:
         raise ValueError("rewards, values and masks must list the same agents")
@@ -403,10 +414,7 @@ def marft_gae_unwhitened(rewards, values, masks, chains, gamma, lam, out_dtype=N
         raise IndexError("a response_mask row sums to more than its length: the token walk would leave the row")
     adv = [a.to(d) for a, d in zip(adv, out_dtypes)]
     ret = [a.to(d) for a, d in zip(ret, out_dtypes)]
-    if back:
-        adv = [a.to(m.device) for a, m in zip(adv, masks)]
-        ret = [a.to(m.device) for a, m in zip(ret, masks)]
-    return adv, ret
+    return adv, ret, [m.detach().to(dev) for m in masks], back
 
 
 def compute_marft_gae_advantage_return(data, pre_agent_group_ids, gamma, lam):
@@ -436,13 +444,11 @@ def compute_marft_gae_advantage_return(data, pre_agent_group_ids, gamma, lam):
         if rid not in seen:
             seen.add(rid)
             chains.append((row, int(extra["traj_len"][row])))
-    adv, ret = marft_gae_unwhitened(rewards, values, masks, chains, gamma, lam)
-    for g, (a, r, m) in enumerate(zip(adv, ret, masks)):
-        if a.is_cuda:
-            white = siirl_F.masked_whiten(a, m)
-        else:
-            dev, _ = _staging_device(a)
-            white = siirl_F.masked_whiten(a.to(dev), m.to(dev)).to(a.device)
+    adv, ret, masks_dev, back = _marft_walk(rewards, values, masks, chains, gamma, lam)
+    for g, (a, r, m, m_src) in enumerate(zip(adv, ret, masks_dev, masks)):
+        white = siirl_F.masked_whiten(a, m)
+        if back:
+            white, r = white.to(m_src.device), r.to(m_src.device)
         if g != len(adv) - 1:
             _td_set(data, prefix + str(last_given) + "_advantages", white)
             _td_set(data, prefix + str(last_given) + "_returns", r)

@@ -368,6 +368,27 @@ def test_backward_rows_through_the_c_abi(dev):
     assert call(picked, n=-1)[0] == -1
 
 
+def test_zero_gradient_rows_sweep(dev):
+    """Seeded random shapes and row patterns (``SIIRL_TEST_SEED`` shifts the seed): the backward that leaves rows out
+    against the oracle, and zero rows of d_hidden exactly zero."""
+    import siirl_amd.fused_linear as FL
+
+    rng = np.random.default_rng(4242 + 100003 * int(os.environ.get("SIIRL_TEST_SEED", "0")))
+    for case in range(10):
+        T, H, V = int(rng.integers(1, 600)), 64 * int(rng.integers(1, 4)), int(rng.integers(2, 9000))
+        h, w, y, g_lp, g_h = _inputs(T, H, V, seed=int(rng.integers(1 << 30)))
+        live = torch.from_numpy(rng.random(T) < rng.random())
+        g_lp, g_h = g_lp * live, g_h * (live & torch.from_numpy(rng.random(T) < 0.7))
+        temperature = float(rng.choice([1.0, 0.6, 1.3]))
+        dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp, g_h, h, w, y, temperature, dtype=torch.float64)
+        hd, wd = h.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+        lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y.to(dev), temperature)
+        torch.autograd.backward([lp, ent], [g_lp.to(dev), g_h.to(dev)])
+        _check_grad(hd.grad, dh64, f"d_hidden case {case} {(T, H, V)}")
+        _check_grad(wd.grad, dw64, f"d_weight case {case} {(T, H, V)}")
+        assert not hd.grad[(~live).to(dev)].any(), (case, T, H, V)
+
+
 @pytest.mark.parametrize("wrt", ["hidden", "weight"])
 def test_zero_gradient_rows_with_one_gradient_requested(dev, wrt):
     """The row-subset backward when only d_hidden or only d_weight is asked for."""

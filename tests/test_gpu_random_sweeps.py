@@ -411,3 +411,32 @@ def test_sweep_loss_functions_over_shapes_dtypes_and_layouts(dev):
         rel = 2.0 ** -6 if lp_dtype == torch.bfloat16 else 1e-5
         err = (lp.grad.cpu().double() - gw).abs()
         assert bool((err <= rel * gw.abs() + 1e-7).all()), (case, which, agg, lp_dtype, tuple(shape), err.max().item())
+
+
+def test_sweep_marft_gae(dev):
+    """Random requests, agents, row lengths, token counts (zero included) and mask dtypes: the multi-agent token walk
+    equals the oracle's bit for bit, in float and in the mask's dtype."""
+    import siirl_amd.core_algos as CA
+
+    rng = np.random.default_rng(110 + _SEED)
+    for case in range(40):
+        n_agents = int(rng.integers(1, 6))
+        lens = rng.integers(1, 5, size=int(rng.integers(1, 6))).tolist()
+        B = int(sum(lens))
+        widths = rng.integers(1, 140, size=n_agents).tolist()
+        mdt = [torch.int64, torch.int32, torch.uint8, torch.bool][case % 4]
+        rews = [torch.from_numpy(rng.standard_normal((B, w)).astype(np.float32) * 4) for w in widths]
+        vals = [torch.from_numpy(rng.standard_normal((B, w)).astype(np.float32) * 4) for w in widths]
+        masks = [torch.from_numpy((np.arange(w)[None] < rng.integers(0, w + 1, (B, 1))).astype(np.int64)).to(mdt)
+                 for w in widths]
+        chains, row = [], 0
+        for n in lens:
+            chains.append((row, int(n)))
+            row += int(n)
+        gamma, lam = float(rng.choice([1.0, 0.99, 0.9])), float(rng.choice([1.0, 0.95, 0.5]))
+        out_dtype = torch.float32 if case % 2 else None
+        want_a, want_r = OC.marft_gae_unwhitened(rews, vals, masks, chains, gamma, lam, out_dtype=out_dtype)
+        got_a, got_r = CA.marft_gae_unwhitened([t.to(dev) for t in rews], [t.to(dev) for t in vals],
+                                               [t.to(dev) for t in masks], chains, gamma, lam, out_dtype=out_dtype)
+        for a in range(n_agents):
+            assert torch.equal(got_a[a].cpu(), want_a[a]) and torch.equal(got_r[a].cpu(), want_r[a]), (case, a, widths, lens)

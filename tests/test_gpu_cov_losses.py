@@ -331,9 +331,19 @@ def test_sweep_covariance_losses():
         got[0].backward()
         _close(got[0], want[0], atol=1e-6 + _cancel_slack(A, m, agg, w if with_w else None),
                what=(case, B, L, str(mdt), agg, with_w, pl))
-        for a, b in zip(got[1:], want[1:]):
-            _close(a, b, what=(case, B, L, str(mdt), agg, with_w, pl))
-        assert torch.allclose(lpd.grad.cpu().double(), gwant, rtol=1e-5, atol=1e-7), (case, "clip_cov grad")
+        # What hangs on a strict comparison of float32 numbers -- the clip fractions, the side of `maximum` a token's
+        # gradient takes when its ratio rounds onto a clip bound (a tie in float32, none in float64) -- may instead
+        # agree with the oracle run in float32, the reference's own dtype.
+        lp32 = lp.clone().requires_grad_(True)
+        want32 = O.compute_policy_loss_clip_cov(old, lp32, A, m.to(torch.float32), agg, cfg, w if with_w else None,
+                                                dropped=dropped)
+        (gwant32,) = torch.autograd.grad(want32[0], lp32)
+        for a, b, b32 in zip(got[1:], want[1:], want32[1:]):
+            if abs(float(a) - float(b32)) > 1e-6 + 1e-5 * abs(float(b32)):
+                _close(a, b, what=(case, B, L, str(mdt), agg, with_w, pl))
+        g = lpd.grad.cpu().double()
+        ok = torch.isclose(g, gwant, rtol=1e-5, atol=1e-7) | torch.isclose(g, gwant32.double(), rtol=1e-5, atol=1e-7)
+        assert bool(ok.all()), (case, "clip_cov grad", torch.nonzero(~ok).tolist()[:5])
 
 
 @pytest.mark.parametrize("mode", ["kl_cov", "clip_cov"])

@@ -1032,8 +1032,26 @@ def main():
         skip_wall = time.perf_counter() - t1
         SF.set_skip_zero_rows(False)
         n_valid = int(mask.sum().item())
-        row_skip = {"tokens_per_s": T * args.steps / skip_wall, "valid_tokens": n_valid,
-                    "algorithmic_bytes": es * V * (3 * n_valid + (T - n_valid))}
+        # forward reads every row; backward reads the valid rows and writes every row
+        row_skip = {"tokens_per_s": T * args.steps / skip_wall, "ms_per_step": skip_wall * 1e3 / args.steps,
+                    "valid_tokens": n_valid, "algorithmic_bytes": es * V * (2 * T + n_valid)}
+        # and with the rows outside the mask labelled LABEL_SKIP_ROW, so that the forward does not read them either
+        from siirl_amd.padding import LABEL_SKIP_ROW
+
+        dense_labels = labels
+        labels = torch.where(mask > 0, labels, torch.full_like(labels, LABEL_SKIP_ROW))
+        for _ in range(2):
+            step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        label_wall = time.perf_counter() - t1
+        labels = dense_labels
+        row_skip["labelled_rows_skipped_in_both_passes"] = {
+            "tokens_per_s": T * args.steps / label_wall, "ms_per_step": label_wall * 1e3 / args.steps,
+            "algorithmic_bytes": es * V * (T + 2 * n_valid)}  # both passes read the valid rows only
 
     # the same micro-batch as ONE launch from logits to dlogits (PPO clip loss, entropy bonus, low-variance KL loss
     # evaluated in-kernel from each row's log-prob and entropy); reported beside the headline, never as `value`

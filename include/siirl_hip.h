@@ -75,7 +75,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1007
+#define SIIRL_HIP_ABI_VERSION 1008
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -83,6 +83,12 @@ int siirl_hip_abi_version(void);
 const char* siirl_hip_last_error(void);
 
 /* ---------------------------------------------------------- log-prob and entropy from logits */
+
+/* A label with this value marks a row nothing is wanted of (a prompt token of a packed batch, see
+ * siirl_mark_rows_outside_response): siirl_logprob_entropy_fwd writes 0 to all of the row's outputs without reading
+ * its logits, siirl_logprob_entropy_bwd writes a zero gradient whatever the upstream gradients hold.  The fused
+ * step and lm_head entry points treat it as an ignored label (log-prob 0) and still read the row. */
+#define SIIRL_LABEL_SKIP_ROW (-101)
 
 /*
  * Forward: one streaming pass over logits[T, V] (row r starts at logits + r * row_stride elements).
@@ -92,6 +98,7 @@ const char* siirl_hip_last_error(void);
  *     logprob[r] = z[labels[r]] - lse[r]          (0 when labels[r] == -100, the ignore_index of flash-attn's
  *                                                  cross_entropy_loss; NaN for any other label outside [0, V))
  *     entropy[r] = lse[r] - ex[r]
+ * A row whose label is SIIRL_LABEL_SKIP_ROW is not read: its four outputs are 0.
  * Outputs are fp32.  labels and logprob may both be NULL (entropy only); entropy may be NULL;
  * lse is required; ex is required when entropy is requested and may be NULL otherwise.
  * logits_dtype: SIIRL_F32, SIIRL_BF16 or SIIRL_F16.  Accumulation is fp32.
@@ -436,6 +443,17 @@ int siirl_scatter_rows(const void* src, const int64_t* indices, int64_t n, int64
  */
 int siirl_unpad_ids_labels(const int64_t* input_ids, int64_t n_ids, const int64_t* indices, int64_t nnz,
                            int64_t* ids_rmpad, int64_t* labels_rolled, siirl_stream_t stream);
+
+/*
+ * labels[j] = SIIRL_LABEL_SKIP_ROW for every packed token j whose position in its sequence,
+ * indices[j] mod S, lies outside [S - L - 1, S - 2]: the rows of the packed logits whose log-prob and entropy the
+ * response window does not keep.  The log-prob entry points then neither read those rows nor send a gradient into
+ * them.  Other labels are left as they are.
+ * Replaces: the work the reference spends on rows it then drops with the slice
+ *           full_log_probs.squeeze(-1)[:, -response_length - 1 : -1]  siirl/engine/actor/dp_actor.py:214-231.
+ */
+int siirl_mark_rows_outside_response(const int64_t* indices, int64_t nnz, int64_t S, int64_t L, int64_t* labels,
+                                     siirl_stream_t stream);
 
 /*
  * pad_input followed by the response window: out[b, t] = full[b, S - L - 1 + t], t in [0, L), where full is the

@@ -13,9 +13,10 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libsiirl_hip.so"
 # dtype codes of siirl_dtype
 F32, BF16, F16, F64, I64, I32, U8 = range(7)
 MARFT_MAX_AGENTS = 16  # SIIRL_MARFT_MAX_AGENTS
+LABEL_SKIP_ROW = -101  # SIIRL_LABEL_SKIP_ROW
 MARFT_STORE_FLOAT, MARFT_STORE_TRUNCATED, MARFT_STORE_NONZERO = range(3)  # siirl_marft_store
 MAX_EOS_TOKENS = 16  # SIIRL_MAX_EOS_TOKENS
-ABI_VERSION = 1007  # SIIRL_HIP_ABI_VERSION of include/siirl_hip.h that SIGNATURES below transcribes
+ABI_VERSION = 1008  # SIIRL_HIP_ABI_VERSION of include/siirl_hip.h that SIGNATURES below transcribes
 BWD_SKIP_ZERO_ROWS = 1
 
 _p, _i64, _i32, _f32, _u32, _sz, _f64 = (C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint32, C.c_size_t,
@@ -57,6 +58,7 @@ SIGNATURES = {
     "siirl_gather_rows": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
     "siirl_scatter_rows": (_i32, [_p, _p, _i64, _i64, _i64, _p, _p]),
     "siirl_unpad_ids_labels": (_i32, [_p, _i64, _p, _i64, _p, _p, _p]),
+    "siirl_mark_rows_outside_response": (_i32, [_p, _i64, _i64, _i64, _p, _p]),
     "siirl_response_scatter": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p]),
     "siirl_response_gather": (_i32, [_p, _p, _i64, _i64, _i64, _i64, _p, _p]),
     "siirl_eos_response_mask": (_i32, [_p, _i32, _i64, _i64, _p, _i32, _p, _i32, _p]),

@@ -22,6 +22,10 @@ namespace {
 // flash-attn's cross_entropy_loss, which the reference's logprobs_from_logits dispatches to when flash-attn is
 // installed (siirl/utils/model_utils/torch_functional.py:73-90).  Any other label outside [0, V) yields NaN.
 constexpr int64_t kIgnoreIndex = -100;
+// A label equal to this value says that nothing of the row is wanted (a prompt token of a packed batch: the actor
+// keeps the response slice of the log-probs only, siirl/engine/actor/dp_actor.py:228-231): the forward writes zeros
+// for the row without reading it, the backward writes a zero gradient whatever the upstream gradients hold.
+constexpr int64_t kSkipRow = SIIRL_LABEL_SKIP_ROW;
 
 // Tuning knobs.  Measured on MI355X at T=32768, V=152064, bf16: non-temporal loads are worth 12% on the
 // forward (a pure read stream); on the backward (read + write) the hints are within run-to-run noise;
@@ -198,6 +202,17 @@ __global__ __launch_bounds__(kFwdThreads) void lpe_fwd_kernel(const typename E::
   const int64_t row = blockIdx.x;
   const elem_t* __restrict__ x = logits + row * row_stride;
   const int tid = threadIdx.x;
+  if (labels != nullptr && labels[row] == kSkipRow) {  // (uniform over the workgroup: no barrier is left behind)
+    if (tid == 0) {
+      lse_out[row] = 0.f;
+      if (ENT) {
+        ex_out[row] = 0.f;
+        entropy[row] = 0.f;
+      }
+      if (logprob != nullptr) logprob[row] = 0.f;
+    }
+    return;
+  }
   const float k = inv_T * kLog2e;
   const RowSplit<E> sp(x, nullptr, V);
 
@@ -283,12 +298,13 @@ __global__ __launch_bounds__(kBwdThreads) void lpe_bwd_kernel(const typename E::
   const int tid = threadIdx.x;
   const RowSplit<E> sp(x, d, V);
 
+  const bool skipped = labels != nullptr && labels[row] == kSkipRow;
   const float g1 = (g_lp && labels[row] != kIgnoreIndex) ? g_lp[row] : 0.f;
   const float g2 = HAS_ENT ? g_ent[row] : 0.f;
   const u32x4* xv = reinterpret_cast<const u32x4*>(x + sp.head);
   u32x4* dv = reinterpret_cast<u32x4*>(d + sp.head);
 
-  if ((flags & SIIRL_BWD_SKIP_ZERO_ROWS) && g1 == 0.f && g2 == 0.f) {
+  if (skipped || ((flags & SIIRL_BWD_SKIP_ZERO_ROWS) && g1 == 0.f && g2 == 0.f)) {
     for (int i = tid; i < sp.head; i += kBwdThreads) E::store1(d + i, 0.f);
     for (int i = sp.tail0 + tid; i < V; i += kBwdThreads) E::store1(d + i, 0.f);
     const u32x4 z = u32x4{0u, 0u, 0u, 0u};
@@ -398,7 +414,8 @@ __global__ __launch_bounds__(kBwdThreads) void lpe_bwd_flat_kernel(const typenam
     if (row < T) {
       const float g1 = (g_lp && labels[row] != kIgnoreIndex) ? g_lp[row] : 0.f;
       const float g2 = HAS_ENT ? g_ent[row] : 0.f;
-      rc[q].zero = (flags & SIIRL_BWD_SKIP_ZERO_ROWS) && g1 == 0.f && g2 == 0.f;
+      rc[q].zero = (labels != nullptr && labels[row] == kSkipRow) ||
+                   ((flags & SIIRL_BWD_SKIP_ZERO_ROWS) && g1 == 0.f && g2 == 0.f);
       rc[q].nl = -lse[row] * kLog2e;
       rc[q].c0 = inv_T * ((HAS_ENT ? g2 * ex[row] : 0.f) - g1);
       rc[q].c1 = -g2 * inv_T * inv_T;
@@ -572,7 +589,7 @@ __global__ __launch_bounds__(kFusedThreads) void lpe_fused_kernel(const typename
   {
     const int64_t yl = labels ? labels[row] : -1;
     if (yl >= 0 && yl < (int64_t)V) y = (int)yl;
-    ignored = labels && yl == kIgnoreIndex;
+    ignored = labels && (yl == kIgnoreIndex || yl == kSkipRow);
   }
   if (tid == 0) {
     for (int w = 1; w < kFusedThreads / kWave; ++w) merge(st, sm[w * 3], sm[w * 3 + 1], sm[w * 3 + 2], k);

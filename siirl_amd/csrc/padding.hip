@@ -133,6 +133,18 @@ __global__ __launch_bounds__(kThreads) void unpad_ids_kernel(const int64_t* __re
   }
 }
 
+// labels[j] = SIIRL_LABEL_SKIP_ROW for the packed tokens whose log-prob the response window [S - L - 1, S - 2] of
+// their sequence does not keep
+__global__ __launch_bounds__(kThreads) void mark_outside_response_kernel(const int64_t* __restrict__ indices, int64_t nnz,
+                                                                         int64_t S, int64_t L,
+                                                                         int64_t* __restrict__ labels) {
+  for (int64_t j = (int64_t)blockIdx.x * kThreads + threadIdx.x; j < nnz; j += (int64_t)gridDim.x * kThreads) {
+    const int64_t r = indices[j];
+    const int64_t s = r >= 0 ? r % S : -1;
+    if (s < S - L - 1 || s > S - 2) labels[j] = SIIRL_LABEL_SKIP_ROW;
+  }
+}
+
 // out[b, t] = values[j] for the j with indices[j] == b * S + (S - L - 1 + t); positions nobody writes stay 0
 __global__ __launch_bounds__(kThreads) void response_scatter_kernel(const float* __restrict__ values,
                                                                     const int64_t* __restrict__ indices, int64_t nnz,
@@ -311,5 +323,17 @@ extern "C" int siirl_eos_response_mask(const void* response_id, int id_dtype, in
   eos_mask_kernel<<<dim3((unsigned)((B + rows_per_wg - 1) / rows_per_wg)), dim3(kThreads), 0, (hipStream_t)stream>>>(
       response_id, id_dtype, B, L, eos, mask, mask_dtype);
   SIIRL_LAUNCH_CHECK("eos_mask_kernel");
+  return SIIRL_OK;
+}
+
+extern "C" int siirl_mark_rows_outside_response(const int64_t* indices, int64_t nnz, int64_t S, int64_t L,
+                                                int64_t* labels, siirl_stream_t stream) {
+  SIIRL_REQUIRE(nnz >= 0 && S >= 1 && L >= 0 && L < S, "nnz=%lld S=%lld response_length=%lld out of range (0 <= L < S)",
+                (long long)nnz, (long long)S, (long long)L);
+  if (nnz == 0) return SIIRL_OK;
+  SIIRL_REQUIRE(indices && labels, "NULL operand");
+  mark_outside_response_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, (hipStream_t)stream>>>(indices, nnz, S, L,
+                                                                                                 labels);
+  SIIRL_LAUNCH_CHECK("mark_outside_response_kernel");
   return SIIRL_OK;
 }

@@ -325,7 +325,7 @@ void lpe_bwd_launch(const Tensor& logits, const optional<Tensor>& labels_in, dou
     const auto& b = in_blocks[i];
     if (b.rows == 0) continue;
     int rc = siirl_logprob_entropy_bwd(ptr<char>(logits) + b.off * es, code, b.rows, V, b.stride,
-                                       has(g_lp) ? ptr<int64_t>(labels) + done : nullptr, (float)inv_temperature,
+                                       labels.defined() ? ptr<int64_t>(labels) + done : nullptr, (float)inv_temperature,
                                        ptr<float>(lse) + done, has(g_ent) ? ptr<float>(ex) + done : nullptr,
                                        has(g_lp) ? ptr<float>(g_lp) + done : nullptr,
                                        has(g_ent) ? ptr<float>(g_ent) + done : nullptr,
@@ -390,7 +390,8 @@ struct LogprobEntropyFn : public torch::autograd::Function<LogprobEntropyFn> {
     auto it = ctx->saved_data.find("defer");
     if (inplace && it != ctx->saved_data.end() && it->second.toTensor().item<int>() != 0) inplace = false;
     at::AutoDispatchBelowADInplaceOrView below;
-    const optional<Tensor> lab = has(g_lp) ? optional<Tensor>(labels) : c10::nullopt;
+    // (the labels go along without a log-prob gradient too: they mark the rows the forward skipped)
+    const optional<Tensor> lab = labels.defined() ? optional<Tensor>(labels) : c10::nullopt;
     const optional<Tensor> exo = has(g_ent) ? optional<Tensor>(ex) : c10::nullopt;
     if (inplace) {
       lpe_bwd_inplace(logits, lab, inv_t, lse, exo, g_lp, g_ent, skip);

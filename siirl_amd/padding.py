@@ -15,6 +15,9 @@ from . import _lib
 __all__ = ["unpad_input", "index_first_axis", "pad_input", "unpad_ids_and_labels", "pad_and_slice_response"]
 
 
+LABEL_SKIP_ROW = _lib.LABEL_SKIP_ROW  # label of a packed row that the log-prob kernels skip
+
+
 def _need_gpu(t: torch.Tensor, name: str):
     if not t.is_cuda:
         raise RuntimeError(f"siirl_amd: `{name}` is on {t.device}; these ops run on the GPU only (no CPU fallback)")
@@ -121,9 +124,14 @@ def pad_input(hidden_states: torch.Tensor, indices: torch.Tensor, batch: int, se
     return out.reshape((batch, seqlen) + tuple(hidden_states.shape[1:]))
 
 
-def unpad_ids_and_labels(input_ids: torch.Tensor, attention_mask: torch.Tensor):
+def unpad_ids_and_labels(input_ids: torch.Tensor, attention_mask: torch.Tensor, response_length: int = None):
     """``(input_ids_rmpad [1, nnz], input_ids_rmpad_rolled [nnz], indices, cu_seqlens, max_seqlen)``: the packed ids
-    and ``torch.roll(input_ids_rmpad, -1)`` of reference ``dp_actor.py:112-127`` from one kernel."""
+    and ``torch.roll(input_ids_rmpad, -1)`` of reference ``dp_actor.py:112-127`` from one kernel.
+
+    With ``response_length`` the rolled labels of the packed tokens outside each sequence's response window (the
+    positions the slice ``[:, -response_length - 1 : -1]`` of ``dp_actor.py:228-231`` drops) are set to
+    ``LABEL_SKIP_ROW``: ``logprobs_from_logits`` / ``entropy_from_logits`` then neither read those rows of the
+    packed logits nor send a gradient into them, and return 0 there; what the window keeps is unchanged."""
     _need_gpu(input_ids, "input_ids")
     indices, cu, max_seqlen, _ = _unpad_indices(attention_mask)
     ids = input_ids.to(torch.int64).contiguous()
@@ -134,6 +142,12 @@ def unpad_ids_and_labels(input_ids: torch.Tensor, attention_mask: torch.Tensor):
         rc = _lib.lib().siirl_unpad_ids_labels(_lib.ptr(ids), ids.numel(), _lib.ptr(indices), nnz, _lib.ptr(rm),
                                                _lib.ptr(rolled), _lib.current_stream(ids.device))
     _lib.check(rc, "siirl_unpad_ids_labels")
+    if response_length is not None:
+        S = attention_mask.shape[1]
+        with torch.cuda.device(ids.device):
+            rc = _lib.lib().siirl_mark_rows_outside_response(_lib.ptr(indices), nnz, S, int(response_length),
+                                                             _lib.ptr(rolled), _lib.current_stream(ids.device))
+        _lib.check(rc, "siirl_mark_rows_outside_response")
     return rm.unsqueeze(0), rolled, indices, cu, max_seqlen
 
 

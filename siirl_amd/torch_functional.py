@@ -12,6 +12,9 @@ Differences a caller can observe, all deliberate:
   returned log-probs, so that the ``entropy_from_logits(logits)`` call that the actor issues next on the same
   tensor (``siirl/engine/actor/dp_actor.py:179-195,254-260``) costs no second pass and both gradients are written
   by one backward kernel.  ``set_pairing(False)`` turns this off;
+* a label of ``-101`` (``siirl_amd.padding.LABEL_SKIP_ROW``, set by ``unpad_ids_and_labels(..., response_length=L)``
+  on the packed tokens outside the response window) makes both passes skip the row: log-prob and entropy 0, zero
+  gradient, the logits of the row are never read;
 * the backward writes zeros, without reading the row, where both upstream gradients of a row are zero
   (``set_skip_zero_rows``): a NaN or Inf in a padded row's logits therefore does not reach ``dlogits`` as it would
   through the reference's autograd.
@@ -71,7 +74,7 @@ class _LogprobEntropy(torch.autograd.Function):
             g_ent = None
         if g_lp is None and g_ent is None:
             return None, None, None, None, None
-        args = (logits, labels if g_lp is not None else None, ctx.inv_temperature, lse,
+        args = (logits, labels, ctx.inv_temperature, lse,  # (labels also mark the rows the forward skipped)
                 ex if g_ent is not None else None, g_lp, g_ent, _SKIP_ZERO_ROWS)
         if ctx.inplace:
             _bwd_(*args)

@@ -514,3 +514,88 @@ def test_ops_run_on_the_current_stream(dev):
     side.synchronize()
     for i, (a, b) in enumerate(zip(got, want)):
         assert torch.equal(a, b), i
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("inplace", [False, True])
+@pytest.mark.parametrize("skip_zero_rows", [True, False])
+def test_packed_rows_outside_the_response_window_are_skipped(dev, dtype, inplace, skip_zero_rows):
+    """``unpad_ids_and_labels(..., response_length=L)`` labels the packed tokens the response slice drops with
+    ``LABEL_SKIP_ROW``.  The remove-padding actor flow (reference ``dp_actor.py:112-127,170-231``) then gives, bit for
+    bit, the log-probs, entropies and logits gradient of the unmarked flow on the rows the window keeps, zeros
+    elsewhere, and never looks at the other rows: NaN logits there change nothing."""
+    import siirl_amd.padding as PD
+    import siirl_amd.torch_functional as TF
+
+    B, S, L, V = 5, 40, 12, 1003
+    g = torch.Generator().manual_seed(17)
+    am = torch.ones(B, S, dtype=torch.long)
+    for b, (left, right) in enumerate([(0, 0), (7, 0), (3, 4), (20, 9), (0, 11)]):  # left and right padding
+        am[b, :left] = 0
+        if right:
+            am[b, S - right:] = 0
+    ids = torch.randint(0, V, (B, S), generator=g)
+    nnz = int(am.sum())
+    logits = (torch.randn(nnz, V, generator=g) * 2).to(dtype)
+    g_lp, g_ent = torch.randn(B, L, generator=g), torch.randn(B, L, generator=g)
+
+    def flow(response_length, poison):
+        _, labels, indices, _, _ = PD.unpad_ids_and_labels(ids.to(dev), am.to(dev), response_length=response_length)
+        x = logits.to(dev).clone()
+        if poison is not None:
+            x[poison] = float("nan")
+        x.requires_grad_(True)
+        lp = TF.logprobs_from_logits(x, labels, inplace_backward=inplace)
+        ent = TF.entropy_from_logits(x)
+        lp_w = PD.pad_and_slice_response(lp, indices, B, S, L)
+        ent_w = PD.pad_and_slice_response(ent, indices, B, S, L)
+        (dx,) = torch.autograd.grad([lp_w, ent_w], [x], [g_lp.to(dev), g_ent.to(dev)])
+        return labels, lp.detach(), ent.detach(), lp_w.detach(), ent_w.detach(), dx
+
+    TF.set_skip_zero_rows(skip_zero_rows)
+    try:
+        labels0, lp0, ent0, lpw0, entw0, dx0 = flow(None, None)
+        labels1, _, _, _, _, _ = flow(L, None)
+        skipped = labels1 == PD.LABEL_SKIP_ROW
+        assert 0 < int(skipped.sum()) < nnz and torch.equal(labels1[~skipped], labels0[~skipped])
+        # the marked rows are exactly those whose position is outside [S - L - 1, S - 2]
+        pos = torch.nonzero(am.flatten()).flatten() % S
+        assert torch.equal(skipped.cpu(), (pos < S - L - 1) | (pos > S - 2))
+        labels1, lp1, ent1, lpw1, entw1, dx1 = flow(L, skipped)
+    finally:
+        TF.set_skip_zero_rows(True)
+    assert torch.equal(lpw1, lpw0) and torch.equal(entw1, entw0)
+    assert torch.equal(lp1[~skipped], lp0[~skipped]) and torch.equal(ent1[~skipped], ent0[~skipped])
+    assert not lp1[skipped].any() and not ent1[skipped].any()
+    assert torch.equal(dx1[~skipped], dx0[~skipped])
+    assert not dx1[skipped].any() and not dx0[skipped].any()
+
+
+def test_skip_row_label_through_the_plain_operators(dev):
+    """The label alone decides: with a non-zero upstream gradient on a skipped row, and with the entropy gradient
+    only (no log-prob gradient), the row's gradient is zero and finite."""
+    from siirl_amd import _lib
+
+    ns = torch.ops.siirl_hip
+    T, V = 9, 300
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, V, generator=g).to(dev)
+    x[4] = 1e30  # exp() of this row overflows: reading it would show
+    y = torch.randint(0, V, (T,), generator=g).to(dev)
+    y[4] = _lib.LABEL_SKIP_ROW
+    y[6] = -100
+    lp, ent, lse, ex = ns.logprob_entropy_fwd(x, y, 1.0, True)
+    assert lp[4] == 0 and ent[4] == 0 and lse[4] == 0 and ex[4] == 0
+    assert lp[6] == 0 and ent[6] > 0  # an ignored label still has an entropy
+    ones = torch.ones(T, device=dev)
+    for skip_zero in (False, True):
+        d = ns.logprob_entropy_bwd(x, y, 1.0, lse, ex, ones, ones, skip_zero)
+        assert not d[4].any() and torch.isfinite(d).all() and d[3].any()
+        d = ns.logprob_entropy_bwd(x, y, 1.0, lse, ex, None, ones, skip_zero)
+        assert not d[4].any() and torch.isfinite(d).all() and d[6].any()
+    # a strided view takes the row-per-workgroup kernels
+    xs = torch.randn(T, 2 * V, generator=g).to(dev)[:, :V]
+    xs[4] = 1e30
+    lp, ent, lse, ex = ns.logprob_entropy_fwd(xs, y, 1.0, True)
+    d = ns.logprob_entropy_bwd(xs, y, 1.0, lse, ex, ones, ones, False)
+    assert lp[4] == 0 and not d[4].any() and torch.isfinite(d).all()

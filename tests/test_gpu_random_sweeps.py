@@ -181,9 +181,14 @@ def test_sweep_policy_loss(dev, loss):
         # loss and KL are continuous in the inputs: against the float64 value.  The clip fractions and the branch a
         # token's gradient takes are comparisons of float32 quantities (a ratio that rounds onto `1 - eps` is a tie in
         # float32 and not in float64): against the oracle run in the reference's own dtype.
+        # Float32 accumulation is accurate relative to the sum of the magnitudes of the signed terms it adds
+        # (|token loss| <= |A| * ratio * weight, ratio < 3 here), not relative to what cancellation leaves of them:
+        # 2^-27 of that sum on top of the bar (a row-sum mode at L in the hundreds adds up to ~1e-5).
+        mag = 3.0 * adv.double().abs() * (isw.double() if isw is not None else 1.0)
+        slack = 2.0 ** -27 * float(OC.agg_loss(mag, mask.double(), mode if loss == "vanilla" else "seq-mean-token-mean"))
         for k in (0, 2):
             a, b = float(got[k].detach()), float(want[k].detach())
-            assert abs(a - b) <= 2e-5 + 1e-5 * abs(b), (case, loss, mode, k, a, b)
+            assert abs(a - b) <= 2e-5 + 1e-5 * abs(b) + (slack if k == 0 else 0.0), (case, loss, mode, k, a, b, slack)
         for k in (1, 3):
             a, b = float(got[k]), float(want32[k])
             assert abs(a - b) <= 1e-6, (case, loss, mode, k, a, b)

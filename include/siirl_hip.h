@@ -86,8 +86,10 @@ const char* siirl_hip_last_error(void);
 
 /* A label with this value marks a row nothing is wanted of (a prompt token of a packed batch, see
  * siirl_mark_rows_outside_response): siirl_logprob_entropy_fwd writes 0 to all of the row's outputs without reading
- * its logits, siirl_logprob_entropy_bwd writes a zero gradient whatever the upstream gradients hold.  The fused
- * step and lm_head entry points treat it as an ignored label (log-prob 0) and still read the row. */
+ * its logits, siirl_logprob_entropy_bwd writes a zero gradient whatever the upstream gradients hold.  The
+ * single-launch step entry points (siirl_logprob_entropy_fwd_bwd, siirl_actor_step_fused) treat it as an ignored
+ * label (log-prob 0, no log-prob gradient) and still read the row; the lm_head entry points know no special labels
+ * (any label outside [0, V) gives NaN there). */
 #define SIIRL_LABEL_SKIP_ROW (-101)
 
 /*

@@ -10,7 +10,7 @@ batch is then index-selected in ascending order of the kept positions.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List
 
 import numpy as np
 import torch

@@ -86,7 +86,9 @@ const char* siirl_hip_last_error(void);
 
 /* A label with this value marks a row nothing is wanted of (a prompt token of a packed batch, see
  * siirl_mark_rows_outside_response): siirl_logprob_entropy_fwd writes 0 to all of the row's outputs without reading
- * its logits, siirl_logprob_entropy_bwd writes a zero gradient whatever the upstream gradients hold.  The
+ * its logits, siirl_logprob_entropy_bwd counts both upstream gradients of the row as zero: with
+ * SIIRL_BWD_SKIP_ZERO_ROWS the row's gradient is written as zeros unread; without that flag it is zero as well unless
+ * the row holds +inf or NaN logits (contiguous rows are then still read, with their probabilities forced to 0).  The
  * single-launch step entry points (siirl_logprob_entropy_fwd_bwd, siirl_actor_step_fused) treat it as an ignored
  * label (log-prob 0, no log-prob gradient) and still read the row; the lm_head entry points know no special labels
  * (any label outside [0, V) gives NaN there). */

@@ -523,7 +523,8 @@ def test_packed_rows_outside_the_response_window_are_skipped(dev, dtype, inplace
     """``unpad_ids_and_labels(..., response_length=L)`` labels the packed tokens the response slice drops with
     ``LABEL_SKIP_ROW``.  The remove-padding actor flow (reference ``dp_actor.py:112-127,170-231``) then gives, bit for
     bit, the log-probs, entropies and logits gradient of the unmarked flow on the rows the window keeps, zeros
-    elsewhere, and never looks at the other rows: NaN logits there change nothing."""
+    elsewhere, and never looks at the other rows: NaN logits there change nothing (huge finite ones when the backward
+    has been told to read every row)."""
     import siirl_amd.padding as PD
     import siirl_amd.torch_functional as TF
 
@@ -542,8 +543,8 @@ def test_packed_rows_outside_the_response_window_are_skipped(dev, dtype, inplace
     def flow(response_length, poison):
         _, labels, indices, _, _ = PD.unpad_ids_and_labels(ids.to(dev), am.to(dev), response_length=response_length)
         x = logits.to(dev).clone()
-        if poison is not None:
-            x[poison] = float("nan")
+        if poison is not None:  # the backward is NaN-proof on such rows when it may skip rows; else for finite logits
+            x[poison] = float("nan") if skip_zero_rows else 3e38
         x.requires_grad_(True)
         lp = TF.logprobs_from_logits(x, labels, inplace_backward=inplace)
         ent = TF.entropy_from_logits(x)

@@ -826,6 +826,95 @@ def bench_glue(args, dev):
     print(json.dumps(out), flush=True)
 
 
+def bench_actor(args, dev):
+    """One remove-padding micro-batch of the actor end to end (reference siirl/engine/actor/dp_actor.py:112-127,
+    170-231,455-501 with the drop-in functions): 8 sequences of 1024 prompt + 3072 response tokens, right padded
+    responses, bf16 logits [nnz, 152064].  Packed ids and rolled labels from the attention mask -> log-prob + entropy of
+    the packed logits -> response windows [8, 3072] -> clipped loss - entropy bonus + low-variance KL -> backward to
+    the logits.  Timed twice: as the reference composes it (every packed row goes through the log-prob kernels), and
+    with the rolled labels of the rows outside the response window marked so that the kernels skip them.  Not the
+    headline."""
+    import torch
+    from types import SimpleNamespace
+
+    import siirl_amd.core_algos as CA
+    import siirl_amd.padding as PD
+    import siirl_amd.torch_functional as SF
+
+    B, P, L, V = 8, 1024, 3072, VOCAB
+    S = P + L
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    lens = torch.randint(L // 4, L + 1, (B,), device=dev, generator=gen)
+    am = torch.ones(B, S, dtype=torch.long, device=dev)
+    am[:, P:] = (torch.arange(L, device=dev)[None] < lens[:, None]).long()
+    ids = torch.randint(0, V, (B, S), device=dev, generator=gen)
+    nnz = int(am.sum())
+    logits = torch.empty(nnz, V, dtype=torch.bfloat16, device=dev)
+    for lo in range(0, nnz, 2048):
+        n = min(2048, nnz - lo)
+        logits[lo:lo + n] = (torch.randn(n, V, device=dev, generator=gen) * 3.0).to(torch.bfloat16)
+    logits.requires_grad_(True)
+    mask = am[:, P:].contiguous()
+    adv = torch.randn(B, 1, device=dev, generator=gen).expand(B, L).contiguous()
+    cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=3.0, entropy_coeff=0.001,
+                          use_kl_loss=True, kl_loss_coef=0.001, kl_loss_type="low_var_kl", loss_agg_mode="token-mean",
+                          policy_loss=SimpleNamespace(loss_mode="vanilla"))
+
+    def windows(response_length):
+        _, labels, indices, _, _ = PD.unpad_ids_and_labels(ids, am, response_length=response_length)
+        lp, ent = SF.logprobs_and_entropy_from_logits(logits, labels, temperature=1.0, inplace_backward=False)
+        return (PD.pad_and_slice_response(lp, indices, B, S, L), PD.pad_and_slice_response(ent, indices, B, S, L))
+
+    with torch.no_grad():
+        lp0, _ = windows(None)
+    old = (lp0 + 0.05 * torch.randn(B, L, device=dev, generator=gen)) * mask
+    ref = (lp0 + 0.1 * torch.randn(B, L, device=dev, generator=gen)) * mask
+
+    def step(response_length):
+        lp_w, ent_w = windows(response_length)
+        out = CA.actor_loss(old, lp_w, adv, mask, cfg, entropy=ent_w, ref_log_prob=ref)
+        out.loss.backward()
+        g = logits.grad
+        logits.grad = None
+        return out.loss.detach(), g
+
+    steps, warm = min(args.steps, 20), min(args.warmup, 3)
+    res = {}
+    for name, rl in (("every packed row", None), ("rows outside the response window skipped", L)):
+        for _ in range(warm):
+            step(rl)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss, g = step(rl)
+        torch.cuda.synchronize()
+        res[name] = ((time.perf_counter() - t0) / steps, float(loss), g)
+    (t_all, loss_all, g_all), (t_skip, loss_skip, g_skip) = res.values()
+    n_resp = int(mask.sum())
+    es = logits.element_size()
+    out = {
+        "metric": "remove-padding actor micro-batch (unpad -> log-prob + entropy -> response windows -> clipped loss + "
+                  "entropy + KL -> backward to the logits) tokens/sec @vocab152k bf16",
+        "value": nnz / t_all, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
+        "ms_per_step": t_all * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"actor: {B} sequences x ({P} prompt + <= {L} response), {nnz} packed tokens of which "
+                               f"{n_resp} response tokens, V = {V}", "seed": SEED},
+        "response_rows_only": {"what": "unpad_ids_and_labels(..., response_length=L): the packed rows the response "
+                                       "window drops are labelled SIIRL_LABEL_SKIP_ROW and read by the log-prob kernels "
+                                       "in neither pass (their gradient rows are zero-filled)",
+                               "ms_per_step": t_skip * 1e3, "tokens_per_s": nnz / t_skip,
+                               "same_loss": loss_all == loss_skip, "same_gradient": bool(torch.equal(g_all, g_skip))},
+        # the default flow reads every packed row once in the forward; its backward reads the rows with a gradient
+        # and writes every row (zero rows unread, the library's default)
+        "roofline": {"bound": "hbm", "kernel": "lpe_fwd_kernel + lpe_bwd_flat_kernel",
+                     "achieved": es * V * (2 * nnz + n_resp) / t_all / 1e9, "peak": 8000.0, "unit": "GB/s",
+                     "frac": es * V * (2 * nnz + n_resp) / t_all / 1e9 / 8000.0, "traffic": None},
+        "cpu_baseline": None,
+    }
+    print(json.dumps(out), flush=True)
+
+
 def bench_host(args, dev):
     """Host time per call of the drop-in functions (the cost of the boundary itself): operands small enough that
     the GPU is never the bottleneck, the host clock read before any synchronisation.  One line of JSON: microseconds
@@ -939,11 +1028,12 @@ def main():
                     help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 2 GiB device copy (for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "critic", "glue", "host"],
+    ap.add_argument("--workload", default="config2", choices=["config1", "config2", "config3", "config4", "config5", "critic", "glue", "host", "actor"],
                     help="config2 (default): the headline logprob+entropy fwd+bwd; config1: fp32 GRPO step at V = 32000; "
                          "config4: GSPO long-context sequence; config3: DAPO [B, L] loss path; "
                          "config5: fused lm_head variant; critic: reward placement + GAE + value loss + metrics; "
-                         "glue: remove-padding bookkeeping")
+                         "glue: remove-padding bookkeeping; actor: one remove-padding micro-batch end to end; "
+                         "host: host time per call")
     ap.add_argument("--seqs", type=int, default=SEQS, help="sequences of 4096 tokens (8 = the baseline's config)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -981,6 +1071,8 @@ def main():
         return bench_glue(args, dev)
     if args.workload == "host":
         return bench_host(args, dev)
+    if args.workload == "actor":
+        return bench_actor(args, dev)
     SF.set_skip_zero_rows(False)  # dense: every row is read and written, as the algorithmic byte count assumes
 
     logits, labels, g_lp, g_ent, mask = make_workload(dev, seqs=args.seqs)

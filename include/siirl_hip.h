@@ -123,8 +123,10 @@ int siirl_logprob_entropy_fwd(const void* logits, int logits_dtype, int64_t T, i
  *     dlogits[r, v] = inv_T * ( g_logprob[r] * (1[v == labels[r]] - p) - g_entropy[r] * p * (z - ex[r]) ),
  *     p = exp(z - lse[r]),  z = x * inv_T,
  * in the dtype of the logits (round to nearest even).  g_logprob or g_entropy may be NULL (that
- * branch contributes nothing); labels is required iff g_logprob is given; ex iff g_entropy is.
- * A row whose label is -100 (ignored) takes no gradient from g_logprob.
+ * branch contributes nothing); labels is required when g_logprob is given and may be given without it; ex is
+ * required iff g_entropy is.
+ * A row whose label is -100 (ignored) takes no gradient from g_logprob; a row whose label is SIIRL_LABEL_SKIP_ROW
+ * takes none at all (see there).
  * dlogits may be the logits buffer itself (in-place backward, same stride), otherwise the two must
  * not overlap.  lse / ex are the forward's outputs for the same inv_temperature.
  *

@@ -130,7 +130,10 @@ def bench_config3(args, dev):
     lp = torch.randn(Bk, L, device=dev, generator=gen) - 1.5
     old = lp + 0.05 * torch.randn(Bk, L, device=dev, generator=gen)
     ref = lp + 0.1 * torch.randn(Bk, L, device=dev, generator=gen)
-    mk, rk, uk = mask[kept].contiguous(), rewards[kept].contiguous(), uid[kept].contiguous()
+    # the filter's index select of the kept trajectories (reference data_coordinator/sample.py:242-322)
+    kept_list = kept.tolist()
+    sel = DF.filter_tensordict({"response_mask": mask, "token_level_rewards": rewards, "uid": uid}, kept_list)
+    mk, rk, uk = sel["response_mask"], sel["token_level_rewards"], sel["uid"]
     cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=10.0,
                           entropy_coeff=0.0, use_kl_loss=True, kl_loss_coef=0.001, kl_loss_type="low_var_kl",
                           loss_agg_mode="token-mean", loss_mode="vanilla")
@@ -208,6 +211,9 @@ def bench_config3(args, dev):
         "apply_kl_penalty: rewards = scores - beta * kl * mask, batch KL, one host sync (24 B/token)":
             (lambda: CA.apply_kl_penalty(td, kl_ctrl, "low_var_kl"), 24),
         "agg_loss seq-mean-token-mean forward + backward (28 B/token)": (agg_fb, 28),
+        # per kept token: the int64 mask and the fp32 rewards, read and written once each (the uids are B values)
+        "filter_tensordict: the kept trajectories of response_mask, token_level_rewards and uid selected (24 B/token)":
+            (lambda: DF.filter_tensordict({"response_mask": mask, "token_level_rewards": rewards, "uid": uid}, kept_list), 24),
     }
     block_ms = {}
     for name, (fn, bpt) in blocks.items():

@@ -484,14 +484,10 @@ def _kl_in_reward(scores, old, ref, mask, kl_type, beta, dev):
 
 
 def _resample_rows(t: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
-    """``t[idx]`` along the first axis; tensors on the GPU whose rows are whole 4-byte words go through the row
-    gather of the un-padding path."""
-    if t.is_cuda and t.dim() >= 1 and t.shape[0] and (t[0].numel() * t.element_size()) % 4 == 0 \
-            and t[0].numel() * t.element_size() >= 4 and not t.requires_grad:
-        from . import padding as _padding
+    """``t[idx]`` along the first axis (GPU tensors through the row gather of the un-padding path)."""
+    from .dapo_filter import _select_rows
 
-        return _padding.index_first_axis(t, idx.to(t.device))
-    return t[idx.to(t.device)]
+    return _select_rows(t, idx)
 
 
 def compute_pf_ppo_reweight_data(data, reweight_method: str = "pow", weight_pow: float = 2.0):

@@ -101,24 +101,50 @@ __global__ __launch_bounds__(kThreads) void indices_kernel(const void* mask, int
   }
 }
 
-// dst[j] = src[indices[j]] (GATHER) or dst[indices[j]] = src[j] (scatter), rows of `words` 4-byte words
-template <bool GATHER>
-__global__ __launch_bounds__(kThreads) void move_rows_kernel(const uint32_t* __restrict__ src,
+// dst[j] = src[indices[j]] (GATHER) or dst[indices[j]] = src[j] (scatter), rows of `units` elements of U (16 bytes
+// when the rows allow it, else 4).  Workgroups are laid out as (piece of a row, row): a row's index is read once per
+// workgroup and no address needs a division; every row is moved by 16-byte accesses that bypass the caches (each
+// byte is touched once).
+template <bool GATHER, typename U>
+__global__ __launch_bounds__(kThreads) void move_rows_kernel(const U* __restrict__ src,
                                                              const int64_t* __restrict__ indices, int64_t n,
-                                                             int64_t words, int64_t indexed_rows,
-                                                             uint32_t* __restrict__ dst) {
-  const int64_t total = n * words;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
-    const int64_t j = i / words, w = i - j * words;
+                                                             int64_t units, int64_t indexed_rows,
+                                                             U* __restrict__ dst) {
+  for (int64_t j = blockIdx.y; j < n; j += gridDim.y) {
     const int64_t r = indices[j];
     const bool ok = r >= 0 && r < indexed_rows;  // an index outside the indexed tensor never touches memory
-    if (GATHER) dst[i] = ok ? src[r * words + w] : 0u;
-    else if (ok) dst[r * words + w] = src[i];
+    const U* __restrict__ from = GATHER ? src + r * units : src + j * units;
+    U* __restrict__ to = GATHER ? dst + j * units : dst + r * units;
+    if (!ok && !GATHER) continue;
+    for (int64_t u = (int64_t)blockIdx.x * kThreads + threadIdx.x; u < units; u += (int64_t)gridDim.x * kThreads) {
+      if (ok)
+        __builtin_nontemporal_store(__builtin_nontemporal_load(from + u), to + u);
+      else
+        __builtin_nontemporal_store(U{}, to + u);
+    }
   }
 }
 
-__global__ __launch_bounds__(kThreads) void fill_zero_kernel(uint32_t* __restrict__ p, int64_t words) {
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < words; i += (int64_t)gridDim.x * kThreads) p[i] = 0u;
+// The same for short rows (a workgroup would be mostly idle on one of them): elements of all rows in one flat range.
+template <bool GATHER, typename U>
+__global__ __launch_bounds__(kThreads) void move_short_rows_kernel(const U* __restrict__ src,
+                                                                   const int64_t* __restrict__ indices, int64_t n,
+                                                                   int units, int64_t indexed_rows, U* __restrict__ dst) {
+  const int64_t total = n * units;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kThreads) {
+    const int64_t j = i / units;
+    const int u = (int)(i - j * units);
+    const int64_t r = indices[j];
+    const bool ok = r >= 0 && r < indexed_rows;
+    if (GATHER) dst[i] = ok ? src[r * units + u] : U{};
+    else if (ok) dst[r * units + u] = src[i];
+  }
+}
+
+template <typename U>
+__global__ __launch_bounds__(kThreads) void fill_zero_kernel(U* __restrict__ p, int64_t units) {
+  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < units; i += (int64_t)gridDim.x * kThreads)
+    __builtin_nontemporal_store(U{}, p + i);
 }
 
 // ids_rmpad[j] = input_ids[indices[j]],  labels[j] = input_ids[indices[(j + 1) % nnz]]  (torch.roll(..., -1))
@@ -211,6 +237,44 @@ unsigned blocks_for(int64_t n) {
   return (unsigned)(b < 1 ? 1 : (b > 16384 ? 16384 : b));
 }
 
+// rows of `row_bytes` move as 16-byte units when both tensors allow it, else as 4-byte words
+bool rows_by_16(const void* a, const void* b, int64_t row_bytes) {
+  return row_bytes % 16 == 0 && (((uintptr_t)a | (uintptr_t)b) & 15) == 0;
+}
+// (pieces of a row, rows): enough workgroups to fill the part, at most 65535 rows in flight
+dim3 rows_grid(int64_t n, int64_t units) {
+  const int64_t per_row = (units + kThreads - 1) / kThreads;
+  const int64_t gx = per_row < 1 ? 1 : (per_row > 32 ? 32 : per_row);
+  return dim3((unsigned)gx, (unsigned)(n > 65535 ? 65535 : n));
+}
+template <bool GATHER>
+void launch_move_rows(const void* src, const int64_t* indices, int64_t n, int64_t row_bytes, int64_t indexed_rows, void* dst,
+                      hipStream_t st) {
+  const bool by16 = rows_by_16(src, dst, row_bytes);
+  const int64_t units = by16 ? row_bytes / 16 : row_bytes / 4;
+  if (units < kThreads / 2) {  // short rows: several per workgroup
+    const dim3 grid(blocks_for(n * units));
+    if (by16)
+      move_short_rows_kernel<GATHER, u32x4><<<grid, dim3(kThreads), 0, st>>>((const u32x4*)src, indices, n, (int)units,
+                                                                             indexed_rows, (u32x4*)dst);
+    else
+      move_short_rows_kernel<GATHER, uint32_t><<<grid, dim3(kThreads), 0, st>>>((const uint32_t*)src, indices, n, (int)units,
+                                                                                indexed_rows, (uint32_t*)dst);
+  } else if (by16) {
+    move_rows_kernel<GATHER, u32x4><<<rows_grid(n, units), dim3(kThreads), 0, st>>>((const u32x4*)src, indices, n, units,
+                                                                                    indexed_rows, (u32x4*)dst);
+  } else {
+    move_rows_kernel<GATHER, uint32_t><<<rows_grid(n, units), dim3(kThreads), 0, st>>>((const uint32_t*)src, indices, n, units,
+                                                                                       indexed_rows, (uint32_t*)dst);
+  }
+}
+void launch_fill_zero(void* p, int64_t bytes, hipStream_t st) {  // bytes: a multiple of 4
+  if (bytes % 16 == 0 && ((uintptr_t)p & 15) == 0)
+    fill_zero_kernel<u32x4><<<dim3(blocks_for(bytes / 16)), dim3(kThreads), 0, st>>>((u32x4*)p, bytes / 16);
+  else
+    fill_zero_kernel<uint32_t><<<dim3(blocks_for(bytes / 4)), dim3(kThreads), 0, st>>>((uint32_t*)p, bytes / 4);
+}
+
 int check_mask(int dt) {
   SIIRL_REQUIRE(dt == SIIRL_U8 || dt == SIIRL_I64 || dt == SIIRL_I32 || dt == SIIRL_F32 || dt == SIIRL_BF16 ||
                     dt == SIIRL_F16, "mask dtype %d not supported", dt);
@@ -246,8 +310,7 @@ extern "C" int siirl_gather_rows(const void* src, const int64_t* indices, int64_
                 (long long)row_bytes);
   if (n == 0) return SIIRL_OK;
   SIIRL_REQUIRE(src && indices && dst, "NULL operand");
-  move_rows_kernel<true><<<dim3(blocks_for(n * (row_bytes / 4))), dim3(kThreads), 0, (hipStream_t)stream>>>(
-      (const uint32_t*)src, indices, n, row_bytes / 4, src_rows, (uint32_t*)dst);
+  launch_move_rows<true>(src, indices, n, row_bytes, src_rows, dst, (hipStream_t)stream);
   SIIRL_LAUNCH_CHECK("move_rows_kernel<gather>");
   return SIIRL_OK;
 }
@@ -260,12 +323,10 @@ extern "C" int siirl_scatter_rows(const void* src, const int64_t* indices, int64
   if (total_rows == 0) return SIIRL_OK;
   SIIRL_REQUIRE(dst && (n == 0 || (src && indices)), "NULL operand");
   hipStream_t st = (hipStream_t)stream;
-  fill_zero_kernel<<<dim3(blocks_for(total_rows * (row_bytes / 4))), dim3(kThreads), 0, st>>>((uint32_t*)dst,
-                                                                                             total_rows * (row_bytes / 4));
+  launch_fill_zero(dst, total_rows * row_bytes, st);
   SIIRL_LAUNCH_CHECK("fill_zero_kernel");
   if (n == 0) return SIIRL_OK;
-  move_rows_kernel<false><<<dim3(blocks_for(n * (row_bytes / 4))), dim3(kThreads), 0, st>>>(
-      (const uint32_t*)src, indices, n, row_bytes / 4, total_rows, (uint32_t*)dst);
+  launch_move_rows<false>(src, indices, n, row_bytes, total_rows, dst, st);
   SIIRL_LAUNCH_CHECK("move_rows_kernel<scatter>");
   return SIIRL_OK;
 }
@@ -287,7 +348,7 @@ extern "C" int siirl_response_scatter(const float* values, const int64_t* indice
                 (long long)nnz, (long long)B, (long long)S, (long long)L);
   SIIRL_REQUIRE(out && (nnz == 0 || (values && indices)), "NULL operand");
   hipStream_t st = (hipStream_t)stream;
-  fill_zero_kernel<<<dim3(blocks_for(B * L)), dim3(kThreads), 0, st>>>((uint32_t*)out, B * L);
+  launch_fill_zero(out, B * L * 4, st);
   SIIRL_LAUNCH_CHECK("fill_zero_kernel");
   if (nnz == 0) return SIIRL_OK;
   response_scatter_kernel<<<dim3(blocks_for(nnz)), dim3(kThreads), 0, st>>>(values, indices, nnz, B, S, L, out);

@@ -634,11 +634,29 @@ __global__ __launch_bounds__(kThreads) void masked_finish2_kernel(const double* 
 }
 
 // backward of masked_sum / masked_mean: d[b, t] = g[b or 0] * m[b, t] (/ (mask sum of the reduced extent + 1e-8))
+// Four tokens per thread and access when rows allow it (`vec`: L % 4 == 0, 16-byte aligned operands): a quad then
+// lies inside one row.
 __global__ __launch_bounds__(kThreads) void masked_bwd_kernel(const float* __restrict__ g, const void* mask,
                                                               int mask_dtype, int64_t B, int64_t L, int per_row,
-                                                              const float* __restrict__ den, float* __restrict__ d) {
+                                                              const float* __restrict__ den, int vec, int nt,
+                                                              float* __restrict__ d) {
   const int64_t n = B * L;
   const float all = per_row ? 0.f : (den ? g[0] / (den[0] + 1e-8f) : g[0]);
+  if (vec) {
+    for (int64_t q = (int64_t)blockIdx.x * kThreads + threadIdx.x; q < n / 4; q += (int64_t)gridDim.x * kThreads) {
+      const int64_t i = 4 * q;
+      float w = all;
+      if (per_row) {
+        const int64_t b = i / L;
+        w = den ? g[b] / (den[b] + 1e-8f) : g[b];
+      }
+      Quad m4 = load_mask_quad(mask, mask_dtype, i, true, 4, nt != 0);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) m4.v[e] = w * m4.v[e];
+      store_quad(d, i, true, 4, m4);
+    }
+    return;
+  }
   for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += (int64_t)gridDim.x * kThreads) {
     float w = all;
     if (per_row) {
@@ -1271,10 +1289,16 @@ extern "C" int siirl_masked_reduce_bwd(const float* g, const void* mask, int mas
   if (int rc = check_mask_dtype(mask_dtype)) return rc;
   if (B == 0) return SIIRL_OK;
   SIIRL_REQUIRE(g && mask && d_values, "NULL operand");
-  const int64_t want = (B * L + kThreads - 1) / kThreads;
-  const unsigned blocks = (unsigned)(want < 16384 ? want : 16384);
+  LossArgs a{};  // only to decide whether rows can move as 16-byte quads
+  a.mask = mask;
+  a.mask_dtype = mask_dtype;
+  a.B = B;
+  a.L = L;
+  set_vec(a, d_values);
+  const int64_t want = (B * L / (a.vec ? 4 : 1) + kThreads - 1) / kThreads;
+  const unsigned blocks = (unsigned)(want < 16384 ? (want < 1 ? 1 : want) : 16384);
   masked_bwd_kernel<<<dim3(blocks), dim3(kThreads), 0, (hipStream_t)stream>>>(g, mask, mask_dtype, B, L, per_row,
-                                                                            mask_sums, d_values);
+                                                                            mask_sums, a.vec, a.nt, d_values);
   SIIRL_LAUNCH_CHECK("masked_bwd_kernel");
   return SIIRL_OK;
 }

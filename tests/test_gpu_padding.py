@@ -217,3 +217,52 @@ def test_response_logprobs_padded_and_packed(dev, B, S, L, V, dt):
         (got * w.to(dev)).sum().backward()
         # logprobs_from_logits defaults to the in-place backward: the gradient comes back in the logits' storage
         assert (p.grad.float().cpu() - po.grad).abs().max() < (1e-5 if dt == torch.float32 else 1e-2), route
+
+
+@pytest.mark.parametrize("cols,dtype", [(1, torch.float32), (3, torch.float32), (4, torch.float32), (2, torch.bfloat16),
+                                        (8, torch.bfloat16), (100, torch.float32), (511, torch.float32),
+                                        (512, torch.float32), (1000, torch.int64), (4100, torch.float32),
+                                        (8192, torch.bfloat16)])
+def test_row_moves_every_size_and_alignment(dev, cols, dtype):
+    """index_first_axis / pad_input over rows of 4 bytes to 32 KB: 4-byte and 16-byte units, short rows that share
+    workgroups and long rows cut into pieces, a source view that starts off a 16-byte boundary, repeated and unsorted
+    indices: equal to torch's own indexing, bit for bit."""
+    import siirl_amd.padding as PD
+
+    g = torch.Generator().manual_seed(cols)
+    n_src, n = 77, 50
+    x = (torch.randn(n_src + 1, cols, generator=g) * 100).to(dtype).to(dev)
+    idx = torch.randint(0, n_src, (n,), generator=g).to(dev)
+    assert torch.equal(PD.index_first_axis(x[:n_src], idx), x[:n_src][idx])
+    off = x.flatten()[1:1 + n_src * cols].view(n_src, cols)  # rows start 2 or 4 or 8 bytes off the allocation
+    if (off.data_ptr() % 4) == 0:
+        assert torch.equal(PD.index_first_axis(off, idx), off[idx])
+    # pad_input: distinct target rows, the others zero
+    rows = torch.randperm(n_src, generator=g)[:n].to(dev)
+    src = x[:n]
+    out = PD.pad_input(src, rows, 7, 11)  # 77 rows
+    want = torch.zeros(n_src, cols, dtype=dtype, device=dev)
+    want[rows] = src
+    assert torch.equal(out.reshape(n_src, cols), want)
+
+
+def test_row_moves_ignore_indices_outside_the_tensor(dev):
+    from siirl_amd import _lib
+
+    lib = _lib.lib()
+    for cols in (2, 64, 3000):
+        x = torch.randn(10, cols, device=dev)
+        idx = torch.tensor([3, -1, 9, 10, 0, 2 ** 40], device=dev)
+        out = torch.full((6, cols), 7.0, device=dev)
+        rc = lib.siirl_gather_rows(_lib.ptr(x), _lib.ptr(idx), 6, cols * 4, 10, _lib.ptr(out), _lib.current_stream(dev))
+        assert rc == 0
+        want = torch.stack([x[3], torch.zeros(cols, device=dev), x[9], torch.zeros(cols, device=dev), x[0],
+                            torch.zeros(cols, device=dev)])
+        assert torch.equal(out, want)
+        dst = torch.full((10, cols), 7.0, device=dev)
+        rc = lib.siirl_scatter_rows(_lib.ptr(x[:6].contiguous()), _lib.ptr(idx), 6, cols * 4, 10, _lib.ptr(dst),
+                                    _lib.current_stream(dev))
+        assert rc == 0
+        want = torch.zeros(10, cols, device=dev)
+        want[3], want[9], want[0] = x[0], x[2], x[4]
+        assert torch.equal(dst, want)

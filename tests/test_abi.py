@@ -159,3 +159,25 @@ def test_size_queries_agree_with_the_host_side():
     assert h.siirl_fused_linear_bwd_rows_workspace_bytes(0, 128, 4096, 1, 1) < 4096
     assert h.siirl_fused_linear_bwd_rows_workspace_bytes(-1, 128, 4096, 1, 1) == 0
     assert h.siirl_fused_linear_fwd_workspace_bytes(512, 128, 4096) > 512 * 128 * 2
+
+
+def test_python_constants_transcribe_the_header():
+    """The enum values and defines that the Python layer repeats by value are those of the header."""
+    L = _lib()
+    text = open(HEADER).read()
+
+    def enum_value(name):
+        m = re.search(rf"\b{name}\s*=\s*(-?\d+)", text)
+        assert m, name
+        return int(m.group(1))
+
+    assert re.search(r"#define SIIRL_LABEL_SKIP_ROW \((-?\d+)\)", text).group(1) == str(L.LABEL_SKIP_ROW)
+    assert re.search(r"#define SIIRL_MARFT_MAX_AGENTS (\d+)", text).group(1) == str(L.MARFT_MAX_AGENTS)
+    for name, value in (("SIIRL_MARFT_STORE_FLOAT", L.MARFT_STORE_FLOAT), ("SIIRL_MARFT_STORE_TRUNCATED", L.MARFT_STORE_TRUNCATED),
+                        ("SIIRL_MARFT_STORE_NONZERO", L.MARFT_STORE_NONZERO), ("SIIRL_F32", L.F32), ("SIIRL_BF16", L.BF16)):
+        assert enum_value(name) == value, name
+    import siirl_amd.core_algos as CA
+
+    for name, value in (("SIIRL_LOSS_VANILLA", CA.LOSS_VANILLA), ("SIIRL_LOSS_GSPO", CA.LOSS_GSPO),
+                        ("SIIRL_LOSS_KL_COV", CA.LOSS_KL_COV), ("SIIRL_LOSS_CLIP_COV", CA.LOSS_CLIP_COV)):
+        assert enum_value(name) == value, name

@@ -72,7 +72,7 @@ constexpr int kDhGroup = SIIRL_DH_GROUP;      // slabs of dlogits kept before d 
                                               // launch at 4 slabs), and 8 x 448 d-weight tiles fill 14 rounds of
                                               // the 256 CUs exactly; measured 4 / 8 / all 19 slabs of V = 152064:
                                               // 34.4 / 33.7 / 33.2 ms per backward
-constexpr int kLdPad = 64;                    // extra elements per row of D / Dt: keeps a tile's 256 rows off a
+constexpr int kLdPad = 64;                    // extra elements per row of D: keeps a tile's rows off a
                                               // power-of-two stride, which would put them all in one memory channel
 
 struct GemmArgs {
@@ -121,8 +121,9 @@ __device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (N
 // m0 (the DMA's LDS base) is a reserved register: naming it in a clobber list is right but draws a warning
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-template <class Epi>
+template <class Epi, bool AT = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void gemm_nt_kernel(GemmArgs g, Epi epi) {
+  static_assert(!AT || (BM == 256 && WN == 4), "the K-major-rows form of A is written for the 256-row tile and 8 waves");
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int wm = w / WN, wn = w % WN;
@@ -136,18 +137,31 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
   const int KT = (g.K / BK - kt_first < kt_per) ? g.K / BK - kt_first : kt_per;
 
   // A: global -> LDS by DMA (global_load_lds_dwordx4): wave instruction I = w * kDmaPerWave + i fills the 1 KB
-  // [I * 1024, I * 1024 + 1024) of the stage; 16-byte slot sl = I * 64 + lane holds row sl / 8, chunk
-  // (sl % 8) ^ ((row / 2) % 8).  Rows past the matrix edge are clamped to the last row.
+  // [I * 1024, I * 1024 + 1024) of the stage.
+  //   A[M][K] (AT = false): 16-byte slot sl = I * 64 + lane holds row sl / 8, chunk (sl % 8) ^ ((row / 2) % 8).  Rows
+  //     past the matrix edge are clamped to the last row.
+  //   A given as [K][M], M contiguous (AT = true): the stage is 64 K-rows of 512 bytes; slot sl holds K-row sl / 32,
+  //     chunk (sl % 32) ^ 2 * (row % 4), i.e. the 32-byte segments of a row are XOR-swizzled by the row so that the
+  //     four K-rows a transposing fragment read touches lie in different banks.  Columns past M are read as they are
+  //     (the row pitch covers whole tiles) and only reach output rows that the epilogue masks.
   const int wu = __builtin_amdgcn_readfirstlane(w);
-  const char* gA = reinterpret_cast<const char*>(g.A + (int64_t)m0 * g.lda + (int64_t)kt_first * BK);
+  const char* gA = AT ? reinterpret_cast<const char*>(g.A + (int64_t)kt_first * BK * g.lda + m0)
+                      : reinterpret_cast<const char*>(g.A + (int64_t)m0 * g.lda + (int64_t)kt_first * BK);
+  const int64_t a_step = AT ? (int64_t)BK * g.lda * 2 : (int64_t)BK * 2;  // bytes from one K-step to the next
   uint32_t offA[kDmaPerWave];
 #pragma unroll
   for (int i = 0; i < kDmaPerWave; ++i) {
     const int sl = (wu * kDmaPerWave + i) * 64 + lane;
-    int row = sl >> 3;
-    const int ch = (sl & 7) ^ ((row >> 1) & 7);
-    row = (m0 + row < g.M) ? row : g.M - 1 - m0;
-    offA[i] = (uint32_t)row * (uint32_t)g.lda * 2u + ch * 16;
+    if constexpr (AT) {
+      const int row = sl >> 5;
+      const int ch = (sl & 31) ^ ((row & 3) << 1);
+      offA[i] = (uint32_t)row * (uint32_t)g.lda * 2u + ch * 16;
+    } else {
+      int row = sl >> 3;
+      const int ch = (sl & 7) ^ ((row >> 1) & 7);
+      row = (m0 + row < g.M) ? row : g.M - 1 - m0;
+      offA[i] = (uint32_t)row * (uint32_t)g.lda * 2u + ch * 16;
+    }
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
   // B: fragment-packed, one 16-byte load per lane per MFMA operand, no LDS
@@ -167,7 +181,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
 
   u32x4 b0[NJ][BK / 16], b1[NJ][BK / 16];
   auto dma = [&](int stage, int kt, int i0 = 0, int i1 = kDmaPerWave) {
-    const char* base = gA + (int64_t)kt * (BK * 2);
+    const char* base = gA + (int64_t)kt * a_step;
 #pragma unroll
     for (int i = i0; i < i1; ++i) {
       const uint32_t dst = lds0 + stage * kStageBytes + (wu * kDmaPerWave + i) * 1024;
@@ -204,11 +218,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
   bwait(b0);
   __syncthreads();
 
+  // A fragments.  AT = false: lane (m = lane % 32, k-group lane / 32) reads its 8 consecutive K entries as one
+  // 16-byte chunk of row m.  AT = true: the stage holds K-rows, so the 8 entries come from two transposing reads
+  // (ds_read_b64_tr_b16): in each block of 16 lanes, lane 4 e + c addresses the 8 bytes of K-row e, M-chunk c, and
+  // receives the entries of K-rows 0..3 at M = its own index in the block.
   const int m31 = lane & 31, gsel = lane >> 5, sw = (m31 >> 1) & 7;
   const int frag_row = (wm * (MI * 32) + m31) * kRowBytes;
   int xk[BK / 16];
 #pragma unroll
   for (int kk = 0; kk < BK / 16; ++kk) xk[kk] = frag_row + (((kk * 2 + gsel) ^ sw) << 4);
+  const int tq = (lane & 15) >> 2, tmb = (lane >> 4) & 1;
+  const int xt0 = (gsel * 8 + tq) * 512 + wm * 256 + (lane & 3) * 8 + ((tmb ^ tq) << 5);  // M-tiles 0 and 2
+  const int xt1 = xt0 ^ 64;                                                                // M-tiles 1 and 3
 
   // step kt: stage kt % 4 is read; B(kt + 1) and DMA(kt + 3) are issued (K-steps past the end are clamped to the
   // last one: they land in stages that are not read again); the barrier at the end publishes stage
@@ -218,8 +239,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
   bf16x8 afa[MI], afb[MI];
   auto fread = [&](bf16x8 (&af)[MI], int stage, int kk) {
     const char* cur = smem + stage * kStageBytes;
+    if constexpr (AT) {
+      typedef short s16x4 __attribute__((ext_vector_type(4)));
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 #pragma unroll
-    for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + xk[kk] + i * 32 * kRowBytes);
+      for (int i = 0; i < MI; ++i) {
+        const char* at = cur + ((i & 1) ? xt1 : xt0) + kk * (16 * 512) + (i >> 1) * 128;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * 512));
+        af[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + xk[kk] + i * 32 * kRowBytes);
+    }
   };
   auto mma = [&](bf16x8 (&af)[MI], u32x4 (&bc)[NJ][BK / 16], int kk) {
 #pragma unroll
@@ -407,11 +441,10 @@ struct SoftmaxPartialsEpi {
 // ------------------------------------------------------------------------------ epilogue: dlogits
 
 // d raw_logit = inv_T * ( g_lp * (1[v == y] - p) - g_h * p * (z - ex) ),  p = exp(z - lse), z = acc * inv_T,
-// written as bf16 to D[token][v] (ld = ldd) and to Dt[v][token] (ld = ldt); v is slab-relative and is the M
-// dimension of this GEMM.  Rows v in [Vs, Vpad) are written as zeros: they are K-padding of the GEMM that
-// consumes D; likewise the token columns [T, ldt_k) of Dt.  A lane owns one token, so the per-token
-// coefficients are loaded once per lane and D gets 8-byte stores; the transposed copy goes through LDS and
-// leaves as whole 16-byte chunks of a row instead of 2-byte stores.
+// written as bf16 to D[token][v] (ld = ldd); v is slab-relative and is the M dimension of this GEMM.  Rows v in
+// [Vs, Vpad) are written as zeros: they are K-padding of the d-hidden GEMM that consumes D.  A lane owns one token,
+// so the per-token coefficients are loaded once per lane and D gets 8-byte stores.  This one token-major layout
+// serves both consumers: d hidden reads it as its A[M = token][K = vocabulary], d weight as A given by K-rows.
 struct DlogitsEpi {
   float inv_T;
   int T, Vs, Vpad;
@@ -423,34 +456,25 @@ struct DlogitsEpi {
   const int64_t* labels;
   uint16_t* D;
   int64_t ldd;
-  uint16_t* Dt;
-  int64_t ldt;
-  int64_t ldt_k;  // token columns of Dt that the consuming GEMM reads (a multiple of BK, >= T): [T, ldt_k) get zeros
-  // LDS image of the tile's Dt block: 256 vocabulary rows x 256 tokens of bf16, 512-byte rows, 16-byte chunks
-  // XOR-swizzled by the row so that the two lane halves (rows v and v + 4) and successive rows spread over the banks
-  static __device__ __forceinline__ int lds_at(int vrow, int tok_l) {
-    return vrow * (BN * 2) + ((((tok_l >> 3) ^ vrow) & 31) << 4) + ((tok_l & 7) << 1);
-  }
   // One lane's part of the tile.  With a = raw accumulator (z = a * inv_T) the gradient is
   //   d = p * (c0 + c1 * a) + [v == y] * cy,   p = exp2(a * ek + nl),
   // ek = inv_T * log2(e), nl = -lse * log2(e), c1 = -g_h * inv_T^2, c0 = inv_T * (g_h * ex - g_lp), cy = g_lp * inv_T:
-  // two fused multiply-adds, one exp2 and one multiply per logit.  A token past T has all coefficients zero (its
-  // accumulators are zero: p = 1, d = 0).  FULL: every vocabulary row of the tile is inside the slab.
+  // two fused multiply-adds, one exp2 and one multiply per logit.  FULL: every vocabulary row of the tile is inside
+  // the slab.
   template <bool FULL>
-  __device__ __forceinline__ void tile(floatx16 (&acc)[MI][NJ], int m0, int n0, int wm, int wn, int lane,
-                                       char* smem) const {
+  __device__ __forceinline__ void tile(floatx16 (&acc)[MI][NJ], int m0, int n0, int wm, int wn, int lane) const {
     const float ek = inv_T * kLog2e;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
-      const int tok_l = acc_col(wn, j, lane), tok = n0 + tok_l;
-      const bool live = tok < T;
-      const float g1 = (live && g_lp) ? g_lp[tok] : 0.f;
-      const float g2 = (live && g_h) ? g_h[tok] : 0.f;
-      const float nl = live ? -lse[tok] * kLog2e : 0.f;
-      const float exv = (live && g_h) ? ex[tok] : 0.f;
+      const int tok = n0 + acc_col(wn, j, lane);
+      if (tok >= T) continue;
+      const float g1 = g_lp ? g_lp[tok] : 0.f;
+      const float g2 = g_h ? g_h[tok] : 0.f;
+      const float nl = -lse[tok] * kLog2e;
+      const float exv = g_h ? ex[tok] : 0.f;
       const float c1 = -g2 * inv_T * inv_T, c0 = inv_T * (g2 * exv - g1), cy = g1 * inv_T;
       int y = -1;
-      if (live && g_lp) {
+      if (g_lp) {
         const int64_t yl = labels[tok] - v0;
         if (yl >= 0 && yl < Vs) y = (int)yl;
       }
@@ -459,8 +483,7 @@ struct DlogitsEpi {
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const int vl = acc_row(wm, i, q * 4, lane);  // 4 consecutive vocabulary rows of the tile
-          const int v = m0 + vl;
+          const int v = m0 + acc_row(wm, i, q * 4, lane);  // 4 consecutive vocabulary rows of the slab
           float d[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -470,33 +493,16 @@ struct DlogitsEpi {
             if (v + e == y) g += cy;
             d[e] = (FULL || v + e < Vs) ? g : 0.f;
           }
-          const uint32_t lo = pack_bf16(d[0], d[1]), hi = pack_bf16(d[2], d[3]);
-          if (live && v < Vpad) *reinterpret_cast<uint2*>(drow + v) = make_uint2(lo, hi);  // 8-byte aligned
-          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 0, tok_l)) = (uint16_t)(lo & 0xffffu);
-          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 1, tok_l)) = (uint16_t)(lo >> 16);
-          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 2, tok_l)) = (uint16_t)(hi & 0xffffu);
-          *reinterpret_cast<uint16_t*>(smem + lds_at(vl + 3, tok_l)) = (uint16_t)(hi >> 16);
+          if (FULL || v < Vpad) *reinterpret_cast<uint2*>(drow + v) = make_uint2(pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3]));
         }
     }
   }
   __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
                                              int lane, int tid, char* smem) const {
-    // the main loop's last barrier (and its vmcnt(0)) freed the ring: 256 x 512 B fit it exactly
     if (m0 + BM <= Vs)
-      tile<true>(acc, m0, n0, wm, wn, lane, smem);
+      tile<true>(acc, m0, n0, wm, wn, lane);
     else
-      tile<false>(acc, m0, n0, wm, wn, lane, smem);
-    __syncthreads();
-    // Dt[v][token]: rows leave the LDS as 16-byte chunks, 32 consecutive threads per 512-byte row
-#pragma unroll 4
-    for (int id = tid; id < BM * (BN / 8); id += kThreads) {
-      const int vrow = id >> 5, c = id & 31;
-      const int v = m0 + vrow, t0 = n0 + c * 8;
-      if (v < Vpad && t0 < ldt_k) {
-        const u32x4 val = *reinterpret_cast<const u32x4*>(smem + vrow * (BN * 2) + (((c ^ vrow) & 31) << 4));
-        *reinterpret_cast<u32x4*>(Dt + (int64_t)v * ldt + t0) = val;
-      }
-    }
+      tile<false>(acc, m0, n0, wm, wn, lane);
   }
 };
 
@@ -688,13 +694,15 @@ __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restric
 
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
-template <class Epi>
+// AT: A is given by its K-rows (A[K][M], M contiguous, row pitch lda >= tiles_m * BM, K readable rows)
+template <class Epi, bool AT = false>
 int launch_gemm(const uint16_t* A, int64_t lda, const u32x4* Bp, int64_t kb_total, int M, int N, int K, const Epi& epi,
                 hipStream_t st, const char* what, int splits = 1) {
-  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi>), kSmemBytes)) return rc;
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi, AT>), kSmemBytes)) return rc;
   GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN, splits};
+  if (AT && lda < (int64_t)g.tiles_m * BM) return fail(SIIRL_ERR_INVALID_ARGUMENT, "%s: row pitch %lld is shorter than %d tiles", what, (long long)lda, g.tiles_m);
   const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n * splits);
-  gemm_nt_kernel<Epi><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
+  gemm_nt_kernel<Epi, AT><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
   SIIRL_LAUNCH_CHECK(what);
   return SIIRL_OK;
 }
@@ -710,7 +718,7 @@ inline int pick_splits(int M, int N, int K) {
 
 int check_fused(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V, float inv_T, int dtype) {
   SIIRL_REQUIRE(dtype == SIIRL_BF16, "fused lm_head path takes bf16 operands (dtype %d given)", dtype);
-  // 32-bit byte offsets inside a 256-row tile bound the row pitch of every A operand (W: H, D: slab, Dt: T + pad)
+  // 32-bit byte offsets inside a 256-row tile bound the row pitch of every A operand (W: H, D: group of slabs + pad)
   SIIRL_REQUIRE(T >= 1 && T < (1LL << 22) && V >= 1 && V < (1LL << 30), "T=%lld (< 4194304) V=%lld out of range",
                 (long long)T, (long long)V);
   SIIRL_REQUIRE(H >= BK && H % BK == 0 && H < (1 << 22), "hidden size %lld must be a positive multiple of %d",
@@ -740,25 +748,27 @@ FwdWs fwd_ws(int64_t T, int64_t H, int64_t V) {
 }
 
 struct BwdWs {
-  size_t hp, wtp, htp, d, dt, dh32, total;
-  int64_t ldwt, ldt, hpad, ldd_row, ldt_row;  // ldt: token count padded to BK (a GEMM K); *_row: row strides
+  size_t hp, wtp, htp, d, dh32, total;
+  int64_t ldwt, ldt, hpad, ldd_row;  // ldt: token count padded to BK (the K of the d-weight GEMM); ldd_row: pitch of D
 };
 BwdWs bwd_ws(int64_t T, int64_t H, int64_t V, bool want_dh, bool want_dw) {
   BwdWs w;
   w.ldwt = round_up(V, BK);
   w.ldt = round_up(T, BK);
   w.ldd_row = (int64_t)kDhGroup * kSlab + kLdPad;
-  w.ldt_row = w.ldt + kLdPad;
   w.hpad = round_up(H, BN);
   size_t off = 0;
   w.hp = off; off += (size_t)round_up(T, BN) * H * 2;
   w.wtp = off; off += want_dh ? (size_t)w.hpad * w.ldwt * 2 : 0;
   w.htp = off; off += want_dw ? (size_t)w.hpad * w.ldt * 2 : 0;
-  w.d = off; off += round_up((size_t)T * w.ldd_row * 2, 256);
-  w.dt = off; off += round_up((size_t)kDhGroup * kSlab * w.ldt_row * 2, 256);
+  w.d = off; off += round_up((size_t)w.ldt * w.ldd_row * 2, 256);  // rows [T, ldt) are K-padding of d weight: zeros
   w.dh32 = off; off += want_dh ? 2 * round_up((size_t)T * H * 4, 256) : 0;  // one buffer per K run
   w.total = off;
   return w;
+}
+
+__global__ __launch_bounds__(256) void zero_fill_kernel(u32x4* __restrict__ p, int64_t n16) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (int64_t)gridDim.x * 256) p[i] = u32x4{0u, 0u, 0u, 0u};
 }
 
 int pack_hidden(const uint16_t* h, int64_t T, int64_t H, u32x4* out, hipStream_t st) {
@@ -893,8 +903,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
   u32x4* hp = (u32x4*)(base + ws.hp);          // packed hidden: B[n = token][k = H]
   u32x4* Wtp = (u32x4*)(base + ws.wtp);        // packed W^T:    B[n = H][k = vocabulary]
   u32x4* Htp = (u32x4*)(base + ws.htp);        // packed hidden^T: B[n = H][k = token]
-  uint16_t* D = (uint16_t*)(base + ws.d);      // [T][ldd_row]: kDhGroup slabs side by side
-  uint16_t* Dt = (uint16_t*)(base + ws.dt);    // [kDhGroup * kSlab][ldt_row]
+  uint16_t* D = (uint16_t*)(base + ws.d);      // [ldt][ldd_row]: kDhGroup slabs side by side
   float* dH32 = (float*)(base + ws.dh32);      // [T][H]
   const uint16_t* h = (const uint16_t*)hidden;
   const uint16_t* w = (const uint16_t*)weight;
@@ -911,6 +920,12 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
         h, H, (int)T, (int)H, Htp, ws.ldt / 16);
     SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(hidden)");
   }
+  if (want_dw && ws.ldt > T) {  // the token rows that only pad the K of the d-weight GEMM (ldd_row * 2 % 16 == 0)
+    const int64_t n16 = (ws.ldt - T) * ws.ldd_row * 2 / 16;
+    zero_fill_kernel<<<dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0, st>>>(
+        reinterpret_cast<u32x4*>(D + T * ws.ldd_row), n16);
+    SIIRL_LAUNCH_CHECK("zero_fill_kernel");
+  }
   int dh_splits = 1;
   const int64_t dh32_stride = (int64_t)(round_up((size_t)T * H * 4, 256) / 4);
   int slab_idx = 0;
@@ -921,14 +936,14 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
     const int gs = slab_idx % kDhGroup;  // position of this slab in its group of D columns
     if (!saved_logits) {
       DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
-                     D + (int64_t)gs * kSlab, ws.ldd_row, Dt + (int64_t)gs * kSlab * ws.ldt_row, ws.ldt_row, ws.ldt};
+                     D + (int64_t)gs * kSlab, ws.ldd_row};
       if (int rc = launch_gemm(w + v0 * H, H, hp, H / 16, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
     } else if (gs == 0) {
       // the whole group's dlogits in one pass over the tiles the forward parked
       const int64_t left = V - v0, cap = (int64_t)kDhGroup * kSlab;
       const int Ng = (int)(left < cap ? left : cap);
       DlogitsEpi epi{inv_temperature, (int)T, Ng, (int)round_up(Ng, BK), v0, lse, ex, g_logprob, g_entropy, labels,
-                     D, ws.ldd_row, Dt, ws.ldt_row, ws.ldt};
+                     D, ws.ldd_row};
       const void* fn = reinterpret_cast<const void*>(&replay_tiles_kernel<DlogitsEpi>);
       if (int rc = allow_dynamic_lds(fn, kSmemBytes)) return rc;
       const int64_t wgs = (int64_t)((Ng + BM - 1) / BM) * tiles_t;
@@ -950,11 +965,13 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
         return rc;
     }
     if (want_dw && (gs == kDhGroup - 1 || v0 + kSlab >= V)) {
-      // dW[g0 : g0 + M, H] = Dt[M, ldt] . Ht[H, ldt]^T over the group's vocabulary rows
+      // dW[g0 : g0 + M, H] = D[ldt, M]^T . Ht[H, ldt]^T over the group's vocabulary rows: D is the A operand given
+      // by its K-rows (tokens)
       const int64_t g0 = v0 - (int64_t)gs * kSlab;
       const int M = gs * kSlab + N;
       StoreBf16Epi sto{(uint16_t*)d_weight + g0 * H, H, M, (int)H};
-      if (int rc = launch_gemm(Dt, ws.ldt_row, Htp, ws.ldt / 16, M, (int)H, (int)ws.ldt, sto, st, "gemm_nt_kernel<StoreBf16Epi>"))
+      if (int rc = launch_gemm<StoreBf16Epi, true>(D, ws.ldd_row, Htp, ws.ldt / 16, M, (int)H, (int)ws.ldt, sto, st,
+                                                   "gemm_nt_kernel<StoreBf16Epi, A by K-rows>"))
         return rc;
     }
   }

@@ -2,8 +2,8 @@
 
 Tolerances: logprob / entropy within 1e-3 absolute of the fp32 oracle (exact products of the bf16 inputs);
 d_hidden / d_weight are bf16 outputs of fp32-accumulated GEMMs over bf16-rounded dlogits: compared with the fp64
-oracle within 2 % of the tensor's max magnitude per element (bf16 rounding of dlogits dominates) and 1e-2 relative
-in Frobenius norm."""
+oracle at the bar that those two roundings give (``tests/grad_bar.py``: 1 % of the tensor's largest magnitude per
+element, 5e-3 relative in Frobenius norm; the observed figures are printed)."""
 
 import os
 
@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 import torch
 
+from grad_bar import check_fused_grad
 from oracle import fused_linear as OFL
 
 pytestmark = pytest.mark.gpu
@@ -27,13 +28,7 @@ def _inputs(T, H, V, seed):
 
 
 def _check_grad(got, want64, name, floor=1e-7):
-    got = got.cpu().double()
-    scale = want64.abs().max().item()
-    err = (got - want64).abs().max().item()
-    assert err <= 0.02 * scale + floor, f"{name}: max err {err} vs scale {scale}"
-    if scale > 0:  # (a one-word vocabulary has an identically zero gradient)
-        rel_f = ((got - want64).norm() / want64.norm()).item()
-        assert rel_f < 1e-2, f"{name}: relative Frobenius error {rel_f}"
+    check_fused_grad(got, want64, name, floor)
 
 
 @pytest.mark.parametrize("T,H,V", [(1, 64, 1), (5, 64, 33), (256, 64, 256), (300, 128, 1000), (513, 256, 8200),

@@ -102,7 +102,7 @@ def cpu_baseline(logits, labels, g_lp, g_ent, rows=4096, iters=5):
                       f"median of {iters} fwd+bwd passes ({med:.2f} s each)"}
 
 
-def bench_config3(args, dev):
+def bench_config3(args, dev, quick=False):
     """DAPO [B, L] path at config 3: 512 prompts x 16 responses, L = 8192 fp32.  One step = dynamic-sampling keep
     mask over the 8192 trajectories, GRPO advantages on the kept ones, and the fused actor loss (asymmetric clip,
     low-variance KL term) forward + backward over the kept [~5.7k, 8192] tokens.  Not the headline."""
@@ -170,56 +170,59 @@ def bench_config3(args, dev):
     # the path's smaller building blocks on the same [kept, L] tensors, each timed alone (not part of the step)
     import siirl_amd.torch_functional as SF
 
-    def timed_ms(fn, iters=10):
-        fn()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(iters):
-            fn()
-        e1.record()
-        torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / iters
-
-    lpd = lp.detach()
-    kl_ctrl = CA.FixedKLController(0.001)
-    td = {"token_level_scores": rk, "old_log_probs": old, "ref_log_prob": ref, "response_mask": mk}
-    lm = torch.randn(Bk, L, device=dev, generator=gen).requires_grad_(True)
-
-    def agg_fb():
-        CA.agg_loss(lm, mk, "seq-mean-token-mean").backward()
-        lm.grad = None
-
-    adv_b, _ = CA.compute_grpo_outcome_advantage(rk, mk, uk)
-    cov_cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=10.0,
-                              policy_loss=SimpleNamespace(kl_cov_ratio=0.0002, ppo_kl_coef=1.0, clip_cov_ratio=0.0002,
-                                                          clip_cov_lb=1.0, clip_cov_ub=5.0))
-
-    def kl_cov_fb():
-        CA.compute_policy_loss_kl_cov(old, x, adv_b, mk, "token-mean", cov_cfg)[0].backward()
-        x.grad = None
-
-    cov_scores, cov_stats = torch.ops.siirl_hip.cov_scores(None, lpd, adv_b, mk, CA.LOSS_KL_COV, 0.0, 0.0)
-    k_cov = max(1, int(int(float(cov_stats[0]) + float(cov_stats[4])) * 0.0002))
-    blocks = {
-        "kl_cov policy loss forward + backward: scores, top-k pick, loss, gradient (108 B/token)": (kl_cov_fb, 108),
-        f"siirl_topk_mark: the {k_cov} largest of the covariance scores marked (20 B/token: four reads, one write)":
-            (lambda: torch.ops.siirl_hip.topk_mark(cov_scores, k_cov, 1.0), 20),
-        "masked_mean(values, mask) -> scalar (12 B/token)": (lambda: SF.masked_mean(lpd, mk), 12),
-        "masked_mean(values, mask, axis=-1) -> [B] (12 B/token)": (lambda: SF.masked_mean(lpd, mk, axis=-1), 12),
-        "kl_penalty low_var_kl forward (12 B/token)": (lambda: CA.kl_penalty(lpd, ref, "low_var_kl"), 12),
-        "apply_kl_penalty: rewards = scores - beta * kl * mask, batch KL, one host sync (24 B/token)":
-            (lambda: CA.apply_kl_penalty(td, kl_ctrl, "low_var_kl"), 24),
-        "agg_loss seq-mean-token-mean forward + backward (28 B/token)": (agg_fb, 28),
-        # per kept token: the int64 mask and the fp32 rewards, read and written once each (the uids are B values)
-        "filter_tensordict: the kept trajectories of response_mask, token_level_rewards and uid selected (24 B/token)":
-            (lambda: DF.filter_tensordict({"response_mask": mask, "token_level_rewards": rewards, "uid": uid}, kept_list), 24),
-    }
-    block_ms = {}
-    for name, (fn, bpt) in blocks.items():
-        ms = timed_ms(fn)
-        block_ms[name] = {"ms": ms, "GB/s": tokens * bpt / ms / 1e6}
+    block_ms = None
     gbs = loss_bytes / loss_ms / 1e6
+
+    if not quick:
+        def timed_ms(fn, iters=10):
+            fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / iters
+
+        lpd = lp.detach()
+        kl_ctrl = CA.FixedKLController(0.001)
+        td = {"token_level_scores": rk, "old_log_probs": old, "ref_log_prob": ref, "response_mask": mk}
+        lm = torch.randn(Bk, L, device=dev, generator=gen).requires_grad_(True)
+
+        def agg_fb():
+            CA.agg_loss(lm, mk, "seq-mean-token-mean").backward()
+            lm.grad = None
+
+        adv_b, _ = CA.compute_grpo_outcome_advantage(rk, mk, uk)
+        cov_cfg = SimpleNamespace(clip_ratio=0.2, clip_ratio_low=0.2, clip_ratio_high=0.28, clip_ratio_c=10.0,
+                                  policy_loss=SimpleNamespace(kl_cov_ratio=0.0002, ppo_kl_coef=1.0, clip_cov_ratio=0.0002,
+                                                              clip_cov_lb=1.0, clip_cov_ub=5.0))
+
+        def kl_cov_fb():
+            CA.compute_policy_loss_kl_cov(old, x, adv_b, mk, "token-mean", cov_cfg)[0].backward()
+            x.grad = None
+
+        cov_scores, cov_stats = torch.ops.siirl_hip.cov_scores(None, lpd, adv_b, mk, CA.LOSS_KL_COV, 0.0, 0.0)
+        k_cov = max(1, int(int(float(cov_stats[0]) + float(cov_stats[4])) * 0.0002))
+        blocks = {
+            "kl_cov policy loss forward + backward: scores, top-k pick, loss, gradient (108 B/token)": (kl_cov_fb, 108),
+            f"siirl_topk_mark: the {k_cov} largest of the covariance scores marked (20 B/token: four reads, one write)":
+                (lambda: torch.ops.siirl_hip.topk_mark(cov_scores, k_cov, 1.0), 20),
+            "masked_mean(values, mask) -> scalar (12 B/token)": (lambda: SF.masked_mean(lpd, mk), 12),
+            "masked_mean(values, mask, axis=-1) -> [B] (12 B/token)": (lambda: SF.masked_mean(lpd, mk, axis=-1), 12),
+            "kl_penalty low_var_kl forward (12 B/token)": (lambda: CA.kl_penalty(lpd, ref, "low_var_kl"), 12),
+            "apply_kl_penalty: rewards = scores - beta * kl * mask, batch KL, one host sync (24 B/token)":
+                (lambda: CA.apply_kl_penalty(td, kl_ctrl, "low_var_kl"), 24),
+            "agg_loss seq-mean-token-mean forward + backward (28 B/token)": (agg_fb, 28),
+            # per kept token: the int64 mask and the fp32 rewards, read and written once each (the uids are B values)
+            "filter_tensordict: the kept trajectories of response_mask, token_level_rewards and uid selected (24 B/token)":
+                (lambda: DF.filter_tensordict({"response_mask": mask, "token_level_rewards": rewards, "uid": uid}, kept_list), 24),
+        }
+        block_ms = {}
+        for name, (fn, bpt) in blocks.items():
+            ms = timed_ms(fn)
+            block_ms[name] = {"ms": ms, "GB/s": tokens * bpt / ms / 1e6}
     out = {
         "metric": "DAPO loss path (filter + GRPO advantage + clipped loss fwd+bwd) tokens/sec @[B,L] fp32",
         "value": tokens * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
@@ -258,10 +261,10 @@ def bench_config3(args, dev):
         out["cpu_baseline"] = {"value": n_s * L / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
                                "sample": f"first {n_s} kept trajectories (of {Bk}) x {L} tokens, filter over {2 * n_s} "
                                          f"trajectories; median of 3 passes ({med:.2f} s each)"}
-    print(json.dumps(out), flush=True)
+    return out
 
 
-def bench_config5(args, dev):
+def bench_config5(args, dev, quick=False):
     """Fused lm_head + log-prob/entropy (MFMA path): hidden [16384, 3584] ~ N(0,1), W [152064, 3584] ~ N(0, 0.02),
     bf16, uniform labels, forward + backward to hidden and W.  Not the headline; same JSON shape."""
     import torch
@@ -312,40 +315,60 @@ def bench_config5(args, dev):
     # the opt-in route that parks the fp32 logit tiles between forward and backward is reported beside it
     FL.set_saved_logits_limit(0)
     wall, fwd_ms, bwd_ms = timed()
-    FL.set_saved_logits_limit(16 << 30)
-    p_wall, p_fwd_ms, p_bwd_ms = timed()
-    FL.set_saved_logits_limit(0)
-    saved_gb = FL._saved_logits_bytes(T, V) / 1e9
     gemm = 2.0 * T * H * V
-    # the same tensors as a packed batch of 8 sequences of 2048 tokens whose first 512 are prompt tokens: their rows
-    # arrive with zero gradients and the backward leaves them out of its GEMMs
-    live = (torch.arange(T, device=dev) % 2048 >= 512).float()
-    dense_g = (g_lp, g_h)
-    g_lp, g_h = dense_g[0] * live, dense_g[1] * live
-    r_wall, r_fwd_ms, r_bwd_ms = timed()
-    g_lp, g_h = dense_g
-    n_live = int(live.sum().item())
     tf_step = 3 * gemm / (wall / steps) / 1e12
+    extras = {}
+    if not quick:
+        FL.set_saved_logits_limit(16 << 30)
+        p_wall, p_fwd_ms, p_bwd_ms = timed()
+        FL.set_saved_logits_limit(0)
+        saved_gb = FL._saved_logits_bytes(T, V) / 1e9
+        # the same tensors as a packed batch of 8 sequences of 2048 tokens whose first 512 are prompt tokens: their
+        # rows arrive with zero gradients and the backward leaves them out of its GEMMs
+        live = (torch.arange(T, device=dev) % 2048 >= 512).float()
+        dense_g = (g_lp, g_h)
+        g_lp, g_h = dense_g[0] * live, dense_g[1] * live
+        r_wall, r_fwd_ms, r_bwd_ms = timed()
+        g_lp, g_h = dense_g
+        n_live = int(live.sum().item())
 
-    # the same forward launch on quiet operands (all zeros): identical instruction stream, fewer wires toggling.
-    # The gap to the timing on the configuration's random operands is what the power limit costs.
-    def forward_ms(hh, ww, n=5):
-        with torch.no_grad():
-            for _ in range(2):
-                fused_linear_logprob_entropy(hh, ww, y)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(n):
-                fused_linear_logprob_entropy(hh, ww, y)
-            e1.record()
-            torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / n
+        # the same forward launch on quiet operands (all zeros): identical instruction stream, fewer wires toggling.
+        # The gap to the timing on the configuration's random operands is what the power limit costs.
+        def forward_ms(hh, ww, n=5):
+            with torch.no_grad():
+                for _ in range(2):
+                    fused_linear_logprob_entropy(hh, ww, y)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(n):
+                    fused_linear_logprob_entropy(hh, ww, y)
+                e1.record()
+                torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / n
 
-    fwd_random_ms = forward_ms(h.detach(), w.detach())
-    hz, wz = torch.zeros_like(h), torch.zeros_like(w)
-    fwd_zero_ms = forward_ms(hz, wz)
-    del hz, wz
+        fwd_random_ms = forward_ms(h.detach(), w.detach())
+        hz, wz = torch.zeros_like(h), torch.zeros_like(w)
+        fwd_zero_ms = forward_ms(hz, wz)
+        del hz, wz
+        extras = {
+            "parked_variant": {"what": "set_saved_logits_limit(16 GiB): the forward parks its fp32 logit tiles "
+                                       f"({saved_gb:.2f} GB) and the backward reads them back instead of recomputing; "
+                                       "opt-in, NOT the configuration's route",
+                               "ms_per_step": p_wall * 1e3 / steps, "tokens_per_s": T * steps / p_wall,
+                               "forward_ms": p_fwd_ms, "backward_ms": p_bwd_ms,
+                               "algorithmic_TFLOP/s": 3 * gemm / (p_wall / steps) / 1e12,
+                               "frac_of_peak": 3 * gemm / (p_wall / steps) / 1e12 / 2500.0},
+            "response_rows_variant": {"what": "8 packed sequences of 2048 tokens, the first 512 of each prompt tokens "
+                                              "with zero upstream gradients: the backward runs its GEMMs over the "
+                                              f"{n_live} response rows only (set_skip_zero_rows, on by default)",
+                                      "ms_per_step": r_wall * 1e3 / steps, "tokens_per_s": T * steps / r_wall,
+                                      "forward_ms": r_fwd_ms, "backward_ms": r_bwd_ms, "rows_with_gradient": n_live},
+            "power_limit_probe": {"what": "the forward alone (no grad) on the configuration's random operands and on "
+                                          "all-zero operands: same instructions, quieter data",
+                                  "forward_ms_random_operands": fwd_random_ms, "TFLOP/s_random": gemm / fwd_random_ms / 1e9,
+                                  "forward_ms_zero_operands": fwd_zero_ms, "TFLOP/s_zero": gemm / fwd_zero_ms / 1e9},
+        }
     out = {
         "metric": "fused lm_head+logprob/entropy fwd+bwd tokens/sec @vocab152k bf16; % MFMA roofline",
         "value": T * steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warm,
@@ -357,22 +380,7 @@ def bench_config5(args, dev):
         "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
                     "backward (recompute + dlogits per slab, d hidden and d weight per 65536 columns)":
                         {"ms": bwd_ms, "TFLOP/s executed": 3 * gemm / bwd_ms / 1e9}},
-        "parked_variant": {"what": "set_saved_logits_limit(16 GiB): the forward parks its fp32 logit tiles "
-                                   f"({saved_gb:.2f} GB) and the backward reads them back instead of recomputing; "
-                                   "opt-in, NOT the configuration's route",
-                           "ms_per_step": p_wall * 1e3 / steps, "tokens_per_s": T * steps / p_wall,
-                           "forward_ms": p_fwd_ms, "backward_ms": p_bwd_ms,
-                           "algorithmic_TFLOP/s": 3 * gemm / (p_wall / steps) / 1e12,
-                           "frac_of_peak": 3 * gemm / (p_wall / steps) / 1e12 / 2500.0},
-        "response_rows_variant": {"what": "8 packed sequences of 2048 tokens, the first 512 of each prompt tokens with "
-                                          "zero upstream gradients: the backward runs its GEMMs over the "
-                                          f"{n_live} response rows only (set_skip_zero_rows, on by default)",
-                                  "ms_per_step": r_wall * 1e3 / steps, "tokens_per_s": T * steps / r_wall,
-                                  "forward_ms": r_fwd_ms, "backward_ms": r_bwd_ms, "rows_with_gradient": n_live},
-        "power_limit_probe": {"what": "the forward alone (no grad) on the configuration's random operands and on "
-                                      "all-zero operands: same instructions, quieter data",
-                              "forward_ms_random_operands": fwd_random_ms, "TFLOP/s_random": gemm / fwd_random_ms / 1e9,
-                              "forward_ms_zero_operands": fwd_zero_ms, "TFLOP/s_zero": gemm / fwd_zero_ms / 1e9},
+        **extras,
         "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel", "achieved": tf_step, "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": tf_step / 2500.0, "traffic": None,
                      "note": "algorithmic flops = 3 GEMMs x 2*T*H*V per step (forward, d hidden, d weight); the "
@@ -396,10 +404,10 @@ def bench_config5(args, dev):
         out["cpu_baseline"] = {"value": n_s / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
                                "sample": f"first {n_s} of {T} tokens against the full [{V}, {H}] weight in fp32; "
                                          f"median of 2 fwd+bwd passes ({med:.2f} s each)"}
-    print(json.dumps(out), flush=True)
+    return out
 
 
-def bench_config1(args, dev):
+def bench_config1(args, dev, quick=False):
     """Config 1, the CPU-runnable GRPO step in fp32: 64 prompts x 8 responses, L = 256, V = 32000.  One step =
     group-normalised advantages over the 512 trajectories, then 64 micro-batches of 8 sequences, each
     logits [2048, 32000] fp32 -> log-prob -> clipped loss (eps 0.2, token-mean) + 0.001 * low_var_kl -> backward to
@@ -453,58 +461,60 @@ def bench_config1(args, dev):
     tokens = B * L
     step_bytes = tokens * V * 4 * 3  # fp32 logits: forward reads the row, backward reads it and writes the gradient
 
-    def fused_step():  # the same step with the single-pass logits -> loss -> dlogits kernel per micro-batch
-        adv, _ = CA.compute_grpo_outcome_advantage(rewards, mask, uid)
-        for mb in range(B // MB):
-            rows = slice(mb * MB, mb * MB + MB)
-            CA.fused_actor_step(logits.detach(), labels[rows], old[rows], adv[rows], mask[rows], cfg,
-                                ref_log_prob=ref[rows], loss_scale_factor=scale)
-
-    for _ in range(warm):
-        fused_step()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    for _ in range(steps):
-        fused_step()
-    torch.cuda.synchronize()
-    fused_wall = time.perf_counter() - t1
-
-    # the same 64 single-pass micro-batch steps recorded once into a HIP graph and replayed: one submission per step
-    graph_ms = None
-    try:
-        losses = []
-
-        def graph_body():
+    fused_wall, graph_ms = None, None
+    if not quick:
+        def fused_step():  # the same step with the single-pass logits -> loss -> dlogits kernel per micro-batch
             adv, _ = CA.compute_grpo_outcome_advantage(rewards, mask, uid)
             for mb in range(B // MB):
                 rows = slice(mb * MB, mb * MB + MB)
-                losses.append(CA.fused_actor_step(logits.detach(), labels[rows], old[rows], adv[rows], mask[rows], cfg,
-                                                  ref_log_prob=ref[rows], loss_scale_factor=scale).loss)
+                CA.fused_actor_step(logits.detach(), labels[rows], old[rows], adv[rows], mask[rows], cfg,
+                                    ref_log_prob=ref[rows], loss_scale_factor=scale)
 
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            graph_body()
-        torch.cuda.current_stream().wait_stream(side)
+        for _ in range(warm):
+            fused_step()
         torch.cuda.synchronize()
-        eager_total = float(torch.stack(losses).sum())
-        losses.clear()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            graph_body()
-        for _ in range(warm + 1):
-            graph.replay()
-        torch.cuda.synchronize()
-        t2 = time.perf_counter()
+        t1 = time.perf_counter()
         for _ in range(steps):
-            graph.replay()
+            fused_step()
         torch.cuda.synchronize()
-        graph_ms = (time.perf_counter() - t2) * 1e3 / steps
-        replay_total = float(torch.stack(losses).sum())
-        if replay_total != eager_total:
-            raise RuntimeError(f"graph replay gives loss {replay_total}, eager {eager_total}")
-    except Exception as e:  # reported, never hidden: the eager figures above stand by themselves
-        graph_ms = f"failed: {type(e).__name__}: {e}"
+        fused_wall = time.perf_counter() - t1
+
+        # the same 64 single-pass micro-batch steps recorded once into a HIP graph and replayed: one submission per step
+        graph_ms = None
+        try:
+            losses = []
+
+            def graph_body():
+                adv, _ = CA.compute_grpo_outcome_advantage(rewards, mask, uid)
+                for mb in range(B // MB):
+                    rows = slice(mb * MB, mb * MB + MB)
+                    losses.append(CA.fused_actor_step(logits.detach(), labels[rows], old[rows], adv[rows], mask[rows], cfg,
+                                                      ref_log_prob=ref[rows], loss_scale_factor=scale).loss)
+
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                graph_body()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            eager_total = float(torch.stack(losses).sum())
+            losses.clear()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                graph_body()
+            for _ in range(warm + 1):
+                graph.replay()
+            torch.cuda.synchronize()
+            t2 = time.perf_counter()
+            for _ in range(steps):
+                graph.replay()
+            torch.cuda.synchronize()
+            graph_ms = (time.perf_counter() - t2) * 1e3 / steps
+            replay_total = float(torch.stack(losses).sum())
+            if replay_total != eager_total:
+                raise RuntimeError(f"graph replay gives loss {replay_total}, eager {eager_total}")
+        except Exception as e:  # reported, never hidden: the eager figures above stand by themselves
+            graph_ms = f"failed: {type(e).__name__}: {e}"
     gbs = step_bytes * steps / wall / 1e9
     out = {
         "metric": "GRPO loss step (advantages + 64 micro-batches of logprob fwd, clipped loss + KL, bwd) tokens/sec @vocab32k fp32",
@@ -517,9 +527,10 @@ def bench_config1(args, dev):
                      "achieved": gbs, "peak": 8000.0, "unit": "GB/s", "frac": gbs / 8000.0, "traffic": None,
                      "note": "64 micro-batches of 262 MB each; per micro-batch two logits passes (0.12 ms at the "
                              "config 2 rates) and the [8, 256] loss kernels, issued through the C++ torch.library layer"},
-        "fused_step_variant": {"what": "siirl_actor_step_fused per micro-batch (one pass over the logits)",
-                               "ms_per_step": fused_wall * 1e3 / steps, "tokens_per_s": tokens * steps / fused_wall,
-                               "ms_per_step_as_one_hip_graph": graph_ms},
+        "fused_step_variant": None if quick else {
+            "what": "siirl_actor_step_fused per micro-batch (one pass over the logits)",
+            "ms_per_step": fused_wall * 1e3 / steps, "tokens_per_s": tokens * steps / fused_wall,
+            "ms_per_step_as_one_hip_graph": graph_ms},
         "cpu_baseline": None,
     }
     if not args.no_cpu_baseline:  # the CPU-runnable case: the oracle on a sample of 8 of the 64 micro-batches
@@ -541,10 +552,10 @@ def bench_config1(args, dev):
         out["cpu_baseline"] = {"value": n_mb * MB * L / el, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(),
                                "kind": "port", "sample": f"advantages over all {B} trajectories + the first {n_mb} of "
                                                          f"{B // MB} micro-batches, one pass ({el:.1f} s)"}
-    print(json.dumps(out), flush=True)
+    return out
 
 
-def bench_config4(args, dev):
+def bench_config4(args, dev, quick=False):
     """Config 4, GSPO long context: sequences of 32768 response tokens, bf16 logits at V = 151936 (Qwen3), one
     sequence per micro-batch.  One step = one sequence: log-prob forward, GSPO loss (sequence-level ratio, clip
     3e-4 / 4e-4, seq-mean-token-mean, scaled by 1/32) forward + backward, log-prob backward to the logits.  The
@@ -617,7 +628,7 @@ def bench_config4(args, dev):
         out["cpu_baseline"] = {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
                                "sample": f"first {rows} of {L} tokens of the sequence, upcast to fp32; median of 2 "
                                          f"passes ({med:.2f} s each)"}
-    print(json.dumps(out), flush=True)
+    return out
 
 
 def bench_critic(args, dev):
@@ -1030,6 +1041,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="default workload only: leave out the short runs of configs 1, 3, 4 and 5")
     ap.add_argument("--with-row-skip", action="store_true",
                     help="also time the variant that writes zeros, unread, on rows whose gradients are zero")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -1063,14 +1076,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    if args.workload == "config5":
-        return bench_config5(args, dev)
-    if args.workload == "config3":
-        return bench_config3(args, dev)
-    if args.workload == "config1":
-        return bench_config1(args, dev)
-    if args.workload == "config4":
-        return bench_config4(args, dev)
+    by_name = {"config1": bench_config1, "config3": bench_config3, "config4": bench_config4, "config5": bench_config5}
+    if args.workload in by_name:
+        print(json.dumps(by_name[args.workload](args, dev)), flush=True)
+        return
     if args.workload == "critic":
         return bench_critic(args, dev)
     if args.workload == "glue":
@@ -1231,6 +1240,50 @@ def main():
         return (time.perf_counter() - t3) * 1e3 / 5
 
     division_ms, folded_ms = temperature_flow(False), temperature_flow(True)
+
+    # The headline once more through the reference's two names, as the actor calls them when the entropy bonus is on
+    # (siirl/engine/actor/dp_actor.py:182-195): logprobs_from_logits(logits, labels, inplace_backward=False), then
+    # entropy_from_logits(logits), then backward through both.  The second call is served by the first one's pass, so
+    # this must cost what the headline's one call costs.
+    def named_flow():
+        lp = SF.logprobs_from_logits(x, labels, inplace_backward=False)
+        ent = SF.entropy_from_logits(x)
+        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+        x.grad = None
+
+    for _ in range(args.warmup):
+        named_flow()
+    torch.cuda.synchronize()
+    t4 = time.perf_counter()
+    for _ in range(args.steps):
+        named_flow()
+    torch.cuda.synchronize()
+    named_ms = (time.perf_counter() - t4) * 1e3 / args.steps
+
+    # A copy yardstick from the library's own row mover: siirl_gather_rows with the identity index over the same
+    # tensor reads and writes the backward's bytes (16-byte non-temporal accesses, no arithmetic).
+    from siirl_amd import _lib
+
+    ident = torch.arange(T, device=dev, dtype=torch.int64)
+    dst = torch.empty_like(logits)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def copy_rows():
+        rc = _lib.lib().siirl_gather_rows(_lib.ptr(logits), _lib.ptr(ident), T, V * es, T, _lib.ptr(dst),
+                                          _lib.current_stream(dev))
+        _lib.check(rc, "siirl_gather_rows")
+
+    for _ in range(2):
+        copy_rows()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(10):
+        copy_rows()
+    e1.record()
+    torch.cuda.synchronize()
+    copy_ms = e0.elapsed_time(e1) / 10
+    copy_gbs = 2 * es * V * T / copy_ms / 1e6
+    del dst, ident
     torch.cuda.empty_cache()
 
     out = {
@@ -1260,6 +1313,16 @@ def main():
                                        "(profiles/lpe_config2_hbm_traffic.md); a constant here, not read in this process"},
         "row_skip_variant": row_skip,
         "fused_step_variant": fused_step,
+        "reference_named_flow_ms": named_ms,
+        "reference_named_flow": {"what": "logprobs_from_logits(logits, labels, inplace_backward=False) + "
+                                         "entropy_from_logits(logits) + backward, the actor's own calls "
+                                         "(dp_actor.py:182-195), timed like the headline",
+                                 "ms_per_step": named_ms, "over_headline": named_ms / ms_per_step},
+        "copy_yardstick_GBs": copy_gbs,
+        "copy_yardstick": {"what": "siirl_gather_rows with the identity index over the same [T, V] tensor: the "
+                                   "library's plain row mover reading and writing the backward's bytes",
+                           "ms": copy_ms, "GB/s": copy_gbs, "backward_GB/s": bwd_gbs,
+                           "backward_over_copy": bwd_gbs / copy_gbs},
         "temperature_flow": {"what": f"temperature {temp}: `logits / T`, logprobs_from_logits, entropy_from_logits, "
                                      "backward (the reference's lines) against logprobs_and_entropy_from_logits("
                                      "logits, labels, temperature=T), backward",
@@ -1269,6 +1332,24 @@ def main():
         out["cpu_baseline"] = cpu_baseline(logits.detach(), labels, g_lp, g_ent)
     else:
         out["cpu_baseline"] = None
+    if not args.no_other_configs and args.seqs == SEQS:
+        # the other four configurations of the baseline, each a short run of its own workload (`--workload configN`
+        # gives the full line with its variants): step time, roofline fraction and the CPU oracle beside it
+        del x, logits, labels, g_lp, g_ent, mask, x3, lp_now, old_lp, ref_lp, adv, m2, lp, ent, dx
+        torch.cuda.empty_cache()
+        quick_steps = {"config1": (5, 2), "config3": (10, 2), "config4": (5, 2), "config5": (4, 1)}
+        fns = {"config1": bench_config1, "config3": bench_config3, "config4": bench_config4, "config5": bench_config5}
+        out["configs"] = {}
+        for name, fn in fns.items():
+            sub = argparse.Namespace(**vars(args))
+            sub.steps, sub.warmup = quick_steps[name]
+            r = fn(sub, dev, quick=True)
+            out["configs"][name] = {k: r[k] for k in ("metric", "value", "unit", "ms_per_step", "steps", "warmup", "dtype")}
+            out["configs"][name]["workload"] = r["config"]["workload"]
+            out["configs"][name]["roofline"] = {k: r["roofline"][k] for k in ("bound", "kernel", "achieved", "peak", "unit", "frac")}
+            out["configs"][name]["cpu_baseline"] = r["cpu_baseline"]
+            del r
+            torch.cuda.empty_cache()
     print(json.dumps(out), flush=True)
 
 

@@ -75,7 +75,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1008
+#define SIIRL_HIP_ABI_VERSION 1009
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -631,21 +631,29 @@ int siirl_marft_gae(const float* const* token_level_rewards, const float* const*
 
 /* ------------------------------------------------- lm_head projection fused with log-prob / entropy */
 
-/* Bytes of scratch for the two entry points below. */
+/* Bytes of scratch for the two entry points below, for 16-bit operands (SIIRL_BF16, SIIRL_F16) and, `_dtype`, for
+ * the operand dtype given (SIIRL_F32 operands are staged as three bf16 terms per element: 6 more bytes per element of
+ * hidden and of weight). */
 size_t siirl_fused_linear_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V);
 size_t siirl_fused_linear_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int want_d_hidden, int want_d_weight);
+size_t siirl_fused_linear_fwd_workspace_bytes_dtype(int dtype, int64_t T, int64_t H, int64_t V);
+size_t siirl_fused_linear_bwd_workspace_bytes_dtype(int dtype, int64_t T, int64_t H, int64_t V, int want_d_hidden,
+                                                    int want_d_weight);
 /* Bytes of the optional saved_logits buffer of the two entry points below: 4 bytes per logit, whole 256 x 256 tiles. */
 size_t siirl_fused_linear_saved_logits_bytes(int64_t T, int64_t V);
 
 /*
  * Forward: z = (hidden[T, H] . weight[V, H]^T) * inv_temperature is formed tile by tile on the matrix cores
- * (bf16 operands, fp32 accumulation) and reduced in the epilogue; no [T, V] tensor is needed.
+ * (fp32 accumulation) and reduced in the epilogue; no [T, V] tensor is needed.
+ * dtype of hidden and weight: SIIRL_BF16 or SIIRL_F16 (exact products of the operands on the bf16 / fp16 matrix
+ * instructions), or SIIRL_F32: each operand is first staged in the workspace as three bf16 terms per element
+ * (x = hi + lo, a.b ~ hi.hi + hi.lo + lo.hi, relative error 2^-16 per product) and the same bf16 kernels run over
+ * K = 3 H -- the reference's matmul in the input dtype (experimental/torch_functional.py:21) to better than TF32.
  * Outputs as siirl_logprob_entropy_fwd: logprob[T] (with labels), entropy[T], lse[T], ex[T], all fp32.
  * saved_logits (may be NULL): siirl_fused_linear_saved_logits_bytes(T, V) bytes, 16-byte aligned, into which the
  * fp32 accumulator tiles are parked in the kernel's own lane order for the backward; an opaque buffer, trading
  * memory for the backward's recomputation.
- * dtype must be SIIRL_BF16; H a multiple of 64; hidden and weight row-major, contiguous, 16-byte aligned;
- * workspace 256-byte aligned.
+ * H a multiple of 64; hidden and weight row-major, contiguous, 16-byte aligned; workspace 256-byte aligned.
  * Replaces: FusedLinearForPPO.forward  siirl/utils/experimental/torch_functional.py:20-32,70-133
  *           linear_cross_entropy fwd   siirl/utils/kernel/linear_cross_entropy.py:40-88 ->
  *                                      siirl/utils/kernel/kernels.py:507-696 (reduction "none", no TP group)
@@ -657,11 +665,15 @@ int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const void* weigh
 
 /*
  * Backward: for upstream gradients g_logprob[T] / g_entropy[T] (either may be NULL) writes
- * d_hidden[T, H] and / or d_weight[V, H] in bf16 (either may be NULL).  The vocabulary is walked in slabs of
- * 8192 columns: the slab's logits are recomputed -- or, when saved_logits holds what the forward call with the
- * same hidden, weight and inv_temperature parked there, read back --, dlogits = inv_T * (g_lp (onehot - p)
- * - g_H p (z - ex)) is written to scratch in both layouts, then d_hidden += dlogits . W_slab (fp32 accumulation
- * across slabs, rounded once) and d_weight_slab = dlogits^T . hidden.  Both routes give the same bits.
+ * d_hidden[T, H] and / or d_weight[V, H] in the operands' dtype (either may be NULL).  The vocabulary is walked in
+ * slabs of 8192 columns: the slab's logits are recomputed -- or, when saved_logits holds what the forward call with
+ * the same hidden, weight and inv_temperature parked there, read back --, dlogits = inv_T * (g_lp (onehot - p)
+ * - g_H p (z - ex)) is written to scratch as bf16 (token-major, one layout for both consumers), then
+ * d_hidden += dlogits . W_slab (fp32 accumulation across slabs, rounded once) and d_weight_slab = dlogits^T . hidden.
+ * Both routes give the same bits.  For SIIRL_F16 and SIIRL_F32 operands the logits are recomputed as in the forward;
+ * the two gradient GEMMs multiply the bf16 dlogits (bf16 for its range: a softmax gradient underflows fp16) with
+ * hidden and W rounded to bf16, so the gradients carry one more 2^-9 rounding than with bf16 operands; the reference
+ * rounds dlogits to the operands' dtype at the same place (experimental/torch_functional.py:62).
  * Replaces: FusedLinearForPPO.backward siirl/utils/experimental/torch_functional.py:35-67,135-188
  *           linear_cross_entropy bwd   siirl/utils/kernel/kernels.py:1378-1586 (the split-N d_logits strategy
  *                                      :1263-1375,1523-1581)
@@ -688,6 +700,8 @@ int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const void* weigh
  */
 size_t siirl_fused_linear_bwd_rows_workspace_bytes(int64_t n_rows, int64_t H, int64_t V, int want_d_hidden,
                                                    int want_d_weight);
+size_t siirl_fused_linear_bwd_rows_workspace_bytes_dtype(int dtype, int64_t n_rows, int64_t H, int64_t V,
+                                                         int want_d_hidden, int want_d_weight);
 int siirl_fused_linear_logprob_entropy_bwd_rows(const void* hidden, const void* weight, int dtype, const int64_t* labels,
                                                 int64_t T, int64_t H, int64_t V, float inv_temperature, const float* lse,
                                                 const float* ex, const float* g_logprob, const float* g_entropy,

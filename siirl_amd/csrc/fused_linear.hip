@@ -31,6 +31,7 @@ namespace siirl {
 namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 // Rows of the workgroup tile: 256 (8 waves, one workgroup per CU) or 128 (4 waves, 64 KB ring, two independent
@@ -121,7 +122,8 @@ __device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (N
 // m0 (the DMA's LDS base) is a reserved register: naming it in a clobber list is right but draws a warning
 #pragma clang diagnostic push
 #pragma clang diagnostic ignored "-Winline-asm"
-template <class Epi, bool AT = false>
+// F16: the 16-bit operands are IEEE half instead of bf16 (the same data movement, the other MFMA)
+template <class Epi, bool AT = false, bool F16 = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void gemm_nt_kernel(GemmArgs g, Epi epi) {
   static_assert(!AT || (BM == 256 && WN == 4), "the K-major-rows form of A is written for the 256-row tile and 8 waves");
   extern __shared__ __align__(16) char smem[];
@@ -260,7 +262,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
     for (int i = 0; i < MI; ++i)
 #pragma unroll
       for (int j = 0; j < NJ; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], __builtin_bit_cast(bf16x8, bc[j][kk]), acc[i][j], 0, 0, 0);
+        if constexpr (F16)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[i]), __builtin_bit_cast(f16x8, bc[j][kk]),
+                                                             acc[i][j], 0, 0, 0);
+        else
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], __builtin_bit_cast(bf16x8, bc[j][kk]), acc[i][j], 0, 0, 0);
   };
   fread(afa, 0, 0);
   // One K-step.  The vector-memory instructions (12 with 8 waves) are spread over the step (B for one N-tile before each of the
@@ -531,10 +537,10 @@ struct AccumF32Epi {  // C_s[row][col] = (beta ? C_s : 0) + acc, one fp32 buffer
   }
 };
 
-struct StoreBf16Epi {  // C[row][col] = bf16(acc)
-  uint16_t* C;
+struct StoreEpi {  // C[row][col] = acc, rounded to the output type (out_dtype: SIIRL_BF16, SIIRL_F16 or SIIRL_F32)
+  void* C;
   int64_t ldc;
-  int M, N;
+  int M, N, out_dtype;
   __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn, int lane, int tid,
                              char* smem) const {
 #pragma unroll
@@ -547,7 +553,13 @@ struct StoreBf16Epi {  // C[row][col] = bf16(acc)
         for (int j = 0; j < NJ; ++j) {
           const int col = n0 + acc_col(wn, j, lane);
           if (col >= N) continue;
-          C[(int64_t)row * ldc + col] = (uint16_t)(pack_bf16(acc[i][j][r], 0.f) & 0xffffu);
+          const int64_t at = (int64_t)row * ldc + col;
+          if (out_dtype == SIIRL_BF16)
+            reinterpret_cast<uint16_t*>(C)[at] = (uint16_t)(pack_bf16(acc[i][j][r], 0.f) & 0xffffu);
+          else if (out_dtype == SIIRL_F16)
+            reinterpret_cast<uint16_t*>(C)[at] = (uint16_t)(pack_f16(acc[i][j][r], 0.f) & 0xffffu);
+          else
+            reinterpret_cast<float*>(C)[at] = acc[i][j][r];
         }
       }
   }
@@ -573,8 +585,10 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const uint16_t* __restrict_
 
 // The same packing of the transpose: B[n][k] = in[k][n] with in of shape [R = K][C = N].  A workgroup stages a
 // 64 x 64 tile through LDS and emits its 512 chunks.
+// from_f16: the input holds IEEE halves, the packed output bf16 (round to nearest even).
+__device__ __forceinline__ uint32_t half2_to_bf16x2(uint32_t w) { return pack_bf16(f16_lo(w), f16_hi(w)); }
 __global__ __launch_bounds__(256) void transpose_pack_b_kernel(const uint16_t* __restrict__ in, int64_t ld_in, int R,
-                                                               int C, u32x4* __restrict__ out, int64_t KB) {
+                                                               int C, u32x4* __restrict__ out, int64_t KB, int from_f16) {
   __shared__ __align__(16) uint16_t tile[64][72];  // 144-byte rows: 16-byte aligned, 36 dwords (column reads spread)
   const int r0 = blockIdx.x * 64, c0 = blockIdx.y * 64;  // r = k, c = n
   // 16 bytes (8 columns) per thread and pass, 8 threads per row, 32 rows per pass; ld_in and c0 are multiples of 8
@@ -593,6 +607,7 @@ __global__ __launch_bounds__(256) void transpose_pack_b_kernel(const uint16_t* _
                   (uint32_t)t[4] | ((uint32_t)t[5] << 16), (uint32_t)t[6] | ((uint32_t)t[7] << 16)};
       }
     }
+    if (from_f16) v = u32x4{half2_to_bf16x2(v.x), half2_to_bf16x2(v.y), half2_to_bf16x2(v.z), half2_to_bf16x2(v.w)};
     *reinterpret_cast<u32x4*>(&tile[rr][cc]) = v;
   }
   __syncthreads();
@@ -611,7 +626,7 @@ __global__ __launch_bounds__(256) void transpose_pack_b_kernel(const uint16_t* _
 __global__ __launch_bounds__(256) void label_logit_kernel(const uint16_t* __restrict__ hidden,
                                                           const uint16_t* __restrict__ W,
                                                           const int64_t* __restrict__ labels, int T, int H, int64_t V,
-                                                          float inv_T, float* __restrict__ out) {
+                                                          float inv_T, float* __restrict__ out, int f16) {
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= T) return;
@@ -625,9 +640,13 @@ __global__ __launch_bounds__(256) void label_logit_kernel(const uint16_t* __rest
   float s = 0.f;
   for (int i = lane; i < H / 8; i += kWave) {
     const u32x4 u = a[i], v = b[i];
-    s += bf16_lo(u.x) * bf16_lo(v.x) + bf16_hi(u.x) * bf16_hi(v.x) + bf16_lo(u.y) * bf16_lo(v.y) +
-         bf16_hi(u.y) * bf16_hi(v.y) + bf16_lo(u.z) * bf16_lo(v.z) + bf16_hi(u.z) * bf16_hi(v.z) +
-         bf16_lo(u.w) * bf16_lo(v.w) + bf16_hi(u.w) * bf16_hi(v.w);
+    if (f16)
+      s += f16_lo(u.x) * f16_lo(v.x) + f16_hi(u.x) * f16_hi(v.x) + f16_lo(u.y) * f16_lo(v.y) + f16_hi(u.y) * f16_hi(v.y) +
+           f16_lo(u.z) * f16_lo(v.z) + f16_hi(u.z) * f16_hi(v.z) + f16_lo(u.w) * f16_lo(v.w) + f16_hi(u.w) * f16_hi(v.w);
+    else
+      s += bf16_lo(u.x) * bf16_lo(v.x) + bf16_hi(u.x) * bf16_hi(v.x) + bf16_lo(u.y) * bf16_lo(v.y) +
+           bf16_hi(u.y) * bf16_hi(v.y) + bf16_lo(u.z) * bf16_lo(v.z) + bf16_hi(u.z) * bf16_hi(v.z) +
+           bf16_lo(u.w) * bf16_lo(v.w) + bf16_hi(u.w) * bf16_hi(v.w);
   }
   s = wave_sum(s);
   if (lane == 0) out[row] = s * inv_T;
@@ -684,10 +703,40 @@ __global__ __launch_bounds__(256) void merge_partials_kernel(const float* __rest
   if (logprob) logprob[row] = label_logit[row] - lse;
 }
 
-__global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restrict__ in, const float* __restrict__ in2,
-                                                          uint16_t* __restrict__ out, int64_t n) {
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
-    out[i] = (uint16_t)(pack_bf16(in2 ? in[i] + in2[i] : in[i], 0.f) & 0xffffu);
+// out = in (+ in2), rounded to out_dtype (SIIRL_BF16, SIIRL_F16 or SIIRL_F32)
+__global__ __launch_bounds__(256) void sum_convert_kernel(const float* __restrict__ in, const float* __restrict__ in2,
+                                                          void* __restrict__ out, int64_t n, int out_dtype) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const float v = in2 ? in[i] + in2[i] : in[i];
+    if (out_dtype == SIIRL_BF16)
+      reinterpret_cast<uint16_t*>(out)[i] = (uint16_t)(pack_bf16(v, 0.f) & 0xffffu);
+    else if (out_dtype == SIIRL_F16)
+      reinterpret_cast<uint16_t*>(out)[i] = (uint16_t)(pack_f16(v, 0.f) & 0xffffu);
+    else
+      reinterpret_cast<float*>(out)[i] = v;
+  }
+}
+
+// fp32 operands are staged as three bf16 terms per element so that the bf16 matrix cores reproduce the product to
+// 2^-16: x = hi + lo + O(2^-16 x) with hi = bf16(x), lo = bf16(x - hi), and
+//   a . b ~ a_hi . b_hi + a_hi . b_lo + a_lo . b_hi .
+// A row of K floats becomes a row of 3 K bf16: [hi | hi | lo] for the A operand (role 0), [hi | lo | hi] for the B
+// operand (role 1); the GEMM then simply runs over K' = 3 K.  The first K columns are bf16(x): what the two gradient
+// GEMMs use.  Four elements per thread.
+__global__ __launch_bounds__(256) void split3_kernel(const float* __restrict__ in, int64_t rows, int64_t K,
+                                                     uint16_t* __restrict__ out, int role) {
+  const int64_t q = (int64_t)blockIdx.x * 256 + threadIdx.x;  // quad index
+  const int64_t kq = K / 4;
+  if (q >= rows * kq) return;
+  const int64_t r = q / kq, k = (q - r * kq) * 4;
+  const float4 x = *reinterpret_cast<const float4*>(in + r * K + k);
+  const uint32_t h01 = pack_bf16(x.x, x.y), h23 = pack_bf16(x.z, x.w);
+  const uint32_t l01 = pack_bf16(x.x - bf16_lo(h01), x.y - bf16_hi(h01));
+  const uint32_t l23 = pack_bf16(x.z - bf16_lo(h23), x.w - bf16_hi(h23));
+  uint16_t* o = out + r * 3 * K + k;
+  *reinterpret_cast<uint2*>(o) = make_uint2(h01, h23);
+  *reinterpret_cast<uint2*>(o + K) = role == 0 ? make_uint2(h01, h23) : make_uint2(l01, l23);
+  *reinterpret_cast<uint2*>(o + 2 * K) = role == 0 ? make_uint2(l01, l23) : make_uint2(h01, h23);
 }
 
 // ------------------------------------------------------------------------------ host
@@ -695,14 +744,14 @@ __global__ __launch_bounds__(256) void f32_to_bf16_kernel(const float* __restric
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
 // AT: A is given by its K-rows (A[K][M], M contiguous, row pitch lda >= tiles_m * BM, K readable rows)
-template <class Epi, bool AT = false>
+template <class Epi, bool AT = false, bool F16 = false>
 int launch_gemm(const uint16_t* A, int64_t lda, const u32x4* Bp, int64_t kb_total, int M, int N, int K, const Epi& epi,
                 hipStream_t st, const char* what, int splits = 1) {
-  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi, AT>), kSmemBytes)) return rc;
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi, AT, F16>), kSmemBytes)) return rc;
   GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN, splits};
   if (AT && lda < (int64_t)g.tiles_m * BM) return fail(SIIRL_ERR_INVALID_ARGUMENT, "%s: row pitch %lld is shorter than %d tiles", what, (long long)lda, g.tiles_m);
   const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n * splits);
-  gemm_nt_kernel<Epi, AT><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
+  gemm_nt_kernel<Epi, AT, F16><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
   SIIRL_LAUNCH_CHECK(what);
   return SIIRL_OK;
 }
@@ -716,13 +765,18 @@ inline int pick_splits(int M, int N, int K) {
   return eff(2 * tiles) > eff(tiles) * 1.05 ? 2 : 1;
 }
 
+// K of the logits GEMM for operands of `dtype`: the hidden size, or three bf16 terms per fp32 element (split3_kernel)
+inline int64_t logits_k(int dtype, int64_t H) { return dtype == SIIRL_F32 ? 3 * H : H; }
+
 int check_fused(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V, float inv_T, int dtype) {
-  SIIRL_REQUIRE(dtype == SIIRL_BF16, "fused lm_head path takes bf16 operands (dtype %d given)", dtype);
-  // 32-bit byte offsets inside a 256-row tile bound the row pitch of every A operand (W: H, D: group of slabs + pad)
+  SIIRL_REQUIRE(dtype == SIIRL_BF16 || dtype == SIIRL_F16 || dtype == SIIRL_F32,
+                "fused lm_head path takes bf16, fp16 or fp32 operands (dtype %d given)", dtype);
+  // 32-bit byte offsets inside a 256-row tile bound the row pitch of every A operand (W: K, D: group of slabs + pad)
   SIIRL_REQUIRE(T >= 1 && T < (1LL << 22) && V >= 1 && V < (1LL << 30), "T=%lld (< 4194304) V=%lld out of range",
                 (long long)T, (long long)V);
-  SIIRL_REQUIRE(H >= BK && H % BK == 0 && H < (1 << 22), "hidden size %lld must be a positive multiple of %d",
-                (long long)H, BK);
+  SIIRL_REQUIRE(H >= BK && H % BK == 0 && logits_k(dtype, H) < (1 << 22),
+                "hidden size %lld must be a positive multiple of %d (below %d)", (long long)H, BK,
+                (1 << 22) / (dtype == SIIRL_F32 ? 3 : 1));
   SIIRL_REQUIRE(hidden && weight, "NULL operand");
   SIIRL_REQUIRE(((uintptr_t)hidden & 15) == 0 && ((uintptr_t)weight & 15) == 0, "operands must be 16-byte aligned");
   SIIRL_REQUIRE(inv_T > 0.f && inv_T < 1e30f, "inv_temperature must be positive and finite");
@@ -733,38 +787,55 @@ int check_ws_align(const void* ws) {
   return SIIRL_OK;
 }
 
+// hs / wsp: the three-term bf16 copies of fp32 operands ([T][3 H], [V][3 H]); absent for 16-bit operands
 struct FwdWs {
-  size_t part, label, hp, total;
+  size_t part, label, hp, hs, wsp, total;
 };
-FwdWs fwd_ws(int64_t T, int64_t H, int64_t V) {
+FwdWs fwd_ws(int64_t T, int64_t H, int64_t V, int dtype) {
   FwdWs w;
-  const int64_t tiles_v = (V + BM - 1) / BM;
+  const int64_t tiles_v = (V + BM - 1) / BM, Kc = logits_k(dtype, H);
   size_t off = 0;
   w.part = off; off += round_up((size_t)tiles_v * 3 * T * 4, 256);
   w.label = off; off += round_up((size_t)T * 4, 256);
-  w.hp = off; off += (size_t)round_up(T, BN) * H * 2;
+  w.hp = off; off += (size_t)round_up(T, BN) * Kc * 2;
+  w.hs = off; off += dtype == SIIRL_F32 ? round_up((size_t)T * Kc * 2, 256) : 0;
+  w.wsp = off; off += dtype == SIIRL_F32 ? round_up((size_t)V * Kc * 2, 256) : 0;
   w.total = off;
   return w;
 }
 
 struct BwdWs {
-  size_t hp, wtp, htp, d, dh32, total;
+  size_t hp, wtp, htp, d, dh32, hs, wsp, total;
   int64_t ldwt, ldt, hpad, ldd_row;  // ldt: token count padded to BK (the K of the d-weight GEMM); ldd_row: pitch of D
 };
-BwdWs bwd_ws(int64_t T, int64_t H, int64_t V, bool want_dh, bool want_dw) {
+BwdWs bwd_ws(int64_t T, int64_t H, int64_t V, bool want_dh, bool want_dw, int dtype) {
   BwdWs w;
+  const int64_t Kc = logits_k(dtype, H);
   w.ldwt = round_up(V, BK);
   w.ldt = round_up(T, BK);
   w.ldd_row = (int64_t)kDhGroup * kSlab + kLdPad;
   w.hpad = round_up(H, BN);
   size_t off = 0;
-  w.hp = off; off += (size_t)round_up(T, BN) * H * 2;
+  w.hp = off; off += (size_t)round_up(T, BN) * Kc * 2;
   w.wtp = off; off += want_dh ? (size_t)w.hpad * w.ldwt * 2 : 0;
   w.htp = off; off += want_dw ? (size_t)w.hpad * w.ldt * 2 : 0;
   w.d = off; off += round_up((size_t)w.ldt * w.ldd_row * 2, 256);  // rows [T, ldt) are K-padding of d weight: zeros
   w.dh32 = off; off += want_dh ? 2 * round_up((size_t)T * H * 4, 256) : 0;  // one buffer per K run
+  w.hs = off; off += dtype == SIIRL_F32 ? round_up((size_t)T * Kc * 2, 256) : 0;
+  w.wsp = off; off += dtype == SIIRL_F32 ? round_up((size_t)V * Kc * 2, 256) : 0;
   w.total = off;
   return w;
+}
+
+// fp32 operands -> their three-term bf16 copies (hidden in the B role, weight in the A role)
+int stage_f32(const void* hidden, const void* weight, int64_t T, int64_t H, int64_t V, uint16_t* hs, uint16_t* wsp,
+              hipStream_t st) {
+  const int64_t qh = T * (H / 4), qw = V * (H / 4);
+  split3_kernel<<<dim3((unsigned)((qh + 255) / 256)), dim3(256), 0, st>>>((const float*)hidden, T, H, hs, 1);
+  SIIRL_LAUNCH_CHECK("split3_kernel(hidden)");
+  split3_kernel<<<dim3((unsigned)((qw + 255) / 256)), dim3(256), 0, st>>>((const float*)weight, V, H, wsp, 0);
+  SIIRL_LAUNCH_CHECK("split3_kernel(weight)");
+  return SIIRL_OK;
 }
 
 __global__ __launch_bounds__(256) void zero_fill_kernel(u32x4* __restrict__ p, int64_t n16) {
@@ -803,7 +874,8 @@ __global__ __launch_bounds__(256) void gather_token_operands_kernel(const int64_
 struct RowsWs {
   size_t hidden, labels, lse, ex, g_lp, g_ent, dh, inner, inner_bytes, total;
 };
-RowsWs rows_ws(int64_t n, int64_t H, int64_t V, bool want_dh, bool want_dw) {
+RowsWs rows_ws(int64_t n, int64_t H, int64_t V, bool want_dh, bool want_dw, int dtype) {
+  const size_t es = dtype_size(dtype);
   RowsWs w;
   size_t off = 0;
   auto take = [&off](size_t bytes) {
@@ -811,15 +883,15 @@ RowsWs rows_ws(int64_t n, int64_t H, int64_t V, bool want_dh, bool want_dw) {
     off += round_up(bytes, 256);
     return at;
   };
-  w.hidden = take((size_t)n * H * 2);
+  w.hidden = take((size_t)n * H * es);
   w.labels = take((size_t)n * 8);
   w.lse = take((size_t)n * 4);
   w.ex = take((size_t)n * 4);
   w.g_lp = take((size_t)n * 4);
   w.g_ent = take((size_t)n * 4);
-  w.dh = take(want_dh ? (size_t)n * H * 2 : 0);
+  w.dh = take(want_dh ? (size_t)n * H * es : 0);
   w.inner = off;
-  w.inner_bytes = n > 0 ? bwd_ws(n, H, V, want_dh, want_dw).total : 0;
+  w.inner_bytes = n > 0 ? bwd_ws(n, H, V, want_dh, want_dw, dtype).total : 0;
   w.total = off + w.inner_bytes;
   return w;
 }
@@ -829,15 +901,22 @@ RowsWs rows_ws(int64_t n, int64_t H, int64_t V, bool want_dh, bool want_dw) {
 
 using namespace siirl;
 
+extern "C" size_t siirl_fused_linear_fwd_workspace_bytes_dtype(int dtype, int64_t T, int64_t H, int64_t V) {
+  if (T < 1 || V < 1 || H < 1 || dtype_size(dtype) == 0) return 0;
+  return fwd_ws(T, H, V, dtype).total;
+}
 extern "C" size_t siirl_fused_linear_fwd_workspace_bytes(int64_t T, int64_t H, int64_t V) {
-  if (T < 1 || V < 1) return 0;
-  return fwd_ws(T, H, V).total;
+  return siirl_fused_linear_fwd_workspace_bytes_dtype(SIIRL_BF16, T, H, V);
 }
 
+extern "C" size_t siirl_fused_linear_bwd_workspace_bytes_dtype(int dtype, int64_t T, int64_t H, int64_t V,
+                                                               int want_d_hidden, int want_d_weight) {
+  if (T < 1 || V < 1 || H < 1 || dtype_size(dtype) == 0) return 0;
+  return bwd_ws(T, H, V, want_d_hidden != 0, want_d_weight != 0, dtype).total;
+}
 extern "C" size_t siirl_fused_linear_bwd_workspace_bytes(int64_t T, int64_t H, int64_t V, int want_d_hidden,
                                                          int want_d_weight) {
-  if (T < 1 || V < 1 || H < 1) return 0;
-  return bwd_ws(T, H, V, want_d_hidden != 0, want_d_weight != 0).total;
+  return siirl_fused_linear_bwd_workspace_bytes_dtype(SIIRL_BF16, T, H, V, want_d_hidden, want_d_weight);
 }
 
 extern "C" size_t siirl_fused_linear_saved_logits_bytes(int64_t T, int64_t V) {
@@ -855,7 +934,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   SIIRL_REQUIRE(((uintptr_t)saved_logits & 15) == 0, "saved_logits must be 16-byte aligned");
   SIIRL_REQUIRE((logprob == nullptr) == (labels == nullptr), "labels and logprob must be given together");
   SIIRL_REQUIRE(entropy == nullptr || ex != nullptr, "ex is required when entropy is requested");
-  const FwdWs ws = fwd_ws(T, H, V);
+  const FwdWs ws = fwd_ws(T, H, V, dtype);
   if (workspace == nullptr || workspace_bytes < ws.total)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, ws.total);
   if (int rc = check_ws_align(workspace)) return rc;
@@ -864,15 +943,27 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   float* label_logit = reinterpret_cast<float*>((char*)workspace + ws.label);
   const uint16_t* h = (const uint16_t*)hidden;
   const uint16_t* w = (const uint16_t*)weight;
+  const int64_t Kc = logits_k(dtype, H);
+  const bool f16 = dtype == SIIRL_F16;
+  if (dtype == SIIRL_F32) {
+    uint16_t* hs = (uint16_t*)((char*)workspace + ws.hs);
+    uint16_t* wsp = (uint16_t*)((char*)workspace + ws.wsp);
+    if (int rc = stage_f32(hidden, weight, T, H, V, hs, wsp, st)) return rc;
+    h = hs;
+    w = wsp;
+  }
   if (labels) {
-    label_logit_kernel<<<dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st>>>(h, w, labels, (int)T, (int)H, V,
-                                                                          inv_temperature, label_logit);
+    label_logit_kernel<<<dim3((unsigned)((T + 3) / 4)), dim3(256), 0, st>>>(h, w, labels, (int)T, (int)Kc, V,
+                                                                          inv_temperature, label_logit, (int)f16);
     SIIRL_LAUNCH_CHECK("label_logit_kernel");
   }
   u32x4* hp = reinterpret_cast<u32x4*>((char*)workspace + ws.hp);
-  if (int rc = pack_hidden(h, T, H, hp, st)) return rc;
+  if (int rc = pack_hidden(h, T, Kc, hp, st)) return rc;
   SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part, saved_logits, (int)((T + BN - 1) / BN)};
-  if (int rc = launch_gemm(w, H, hp, H / 16, (int)V, (int)T, (int)H, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>")) return rc;
+  if (int rc = f16 ? launch_gemm<SoftmaxPartialsEpi, false, true>(w, Kc, hp, Kc / 16, (int)V, (int)T, (int)Kc, epi, st,
+                                                                  "gemm_nt_kernel<SoftmaxPartialsEpi, f16>")
+                   : launch_gemm(w, Kc, hp, Kc / 16, (int)V, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>"))
+    return rc;
   const int tiles_v = (int)((V + BM - 1) / BM);
   merge_partials_kernel<<<dim3((unsigned)((T + kMergeTok - 1) / kMergeTok)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
                                                                                logprob, entropy, lse, ex);
@@ -894,30 +985,42 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
   SIIRL_REQUIRE(g_entropy == nullptr || ex != nullptr, "ex is required with g_entropy");
   SIIRL_REQUIRE(d_hidden != nullptr || d_weight != nullptr, "neither d_hidden nor d_weight requested");
   const bool want_dh = d_hidden != nullptr, want_dw = d_weight != nullptr;
-  const BwdWs ws = bwd_ws(T, H, V, want_dh, want_dw);
+  const BwdWs ws = bwd_ws(T, H, V, want_dh, want_dw, dtype);
   if (workspace == nullptr || workspace_bytes < ws.total)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, ws.total);
   if (int rc = check_ws_align(workspace)) return rc;
   hipStream_t st = (hipStream_t)stream;
   char* base = (char*)workspace;
-  u32x4* hp = (u32x4*)(base + ws.hp);          // packed hidden: B[n = token][k = H]
+  u32x4* hp = (u32x4*)(base + ws.hp);          // packed hidden: B[n = token][k = K of the logits GEMM]
   u32x4* Wtp = (u32x4*)(base + ws.wtp);        // packed W^T:    B[n = H][k = vocabulary]
   u32x4* Htp = (u32x4*)(base + ws.htp);        // packed hidden^T: B[n = H][k = token]
   uint16_t* D = (uint16_t*)(base + ws.d);      // [ldt][ldd_row]: kDhGroup slabs side by side
   float* dH32 = (float*)(base + ws.dh32);      // [T][H]
   const uint16_t* h = (const uint16_t*)hidden;
   const uint16_t* w = (const uint16_t*)weight;
+  // The logits are recomputed from the operands as given (fp16: the half MFMA; fp32: three bf16 terms per element,
+  // K = 3 H).  The two gradient GEMMs multiply the bf16 dlogits with bf16 copies of hidden and W (for fp16 and fp32
+  // operands: rounded to bf16 while they are transposed and packed) and write their fp32 sums in the operands' dtype.
+  const int64_t Kc = logits_k(dtype, H);
+  const bool f16 = dtype == SIIRL_F16;
+  if (dtype == SIIRL_F32) {
+    uint16_t* hs = (uint16_t*)(base + ws.hs);
+    uint16_t* wsp = (uint16_t*)(base + ws.wsp);
+    if (int rc = stage_f32(hidden, weight, T, H, V, hs, wsp, st)) return rc;
+    h = hs;
+    w = wsp;
+  }
 
   if (!saved_logits)
-    if (int rc = pack_hidden(h, T, H, hp, st)) return rc;
+    if (int rc = pack_hidden(h, T, Kc, hp, st)) return rc;
   if (want_dh) {
     transpose_pack_b_kernel<<<dim3((unsigned)(ws.ldwt / 64), (unsigned)(ws.hpad / 64)), dim3(256), 0, st>>>(
-        w, H, (int)V, (int)H, Wtp, ws.ldwt / 16);
+        w, Kc, (int)V, (int)H, Wtp, ws.ldwt / 16, (int)f16);
     SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(W)");
   }
   if (want_dw) {
     transpose_pack_b_kernel<<<dim3((unsigned)(ws.ldt / 64), (unsigned)(ws.hpad / 64)), dim3(256), 0, st>>>(
-        h, H, (int)T, (int)H, Htp, ws.ldt / 16);
+        h, Kc, (int)T, (int)H, Htp, ws.ldt / 16, (int)f16);
     SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(hidden)");
   }
   if (want_dw && ws.ldt > T) {  // the token rows that only pad the K of the d-weight GEMM (ldd_row * 2 % 16 == 0)
@@ -937,7 +1040,10 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
     if (!saved_logits) {
       DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
                      D + (int64_t)gs * kSlab, ws.ldd_row};
-      if (int rc = launch_gemm(w + v0 * H, H, hp, H / 16, N, (int)T, (int)H, epi, st, "gemm_nt_kernel<DlogitsEpi>")) return rc;
+      if (int rc = f16 ? launch_gemm<DlogitsEpi, false, true>(w + v0 * Kc, Kc, hp, Kc / 16, N, (int)T, (int)Kc, epi, st,
+                                                              "gemm_nt_kernel<DlogitsEpi, f16>")
+                       : launch_gemm(w + v0 * Kc, Kc, hp, Kc / 16, N, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<DlogitsEpi>"))
+        return rc;
     } else if (gs == 0) {
       // the whole group's dlogits in one pass over the tiles the forward parked
       const int64_t left = V - v0, cap = (int64_t)kDhGroup * kSlab;
@@ -969,26 +1075,30 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
       // by its K-rows (tokens)
       const int64_t g0 = v0 - (int64_t)gs * kSlab;
       const int M = gs * kSlab + N;
-      StoreBf16Epi sto{(uint16_t*)d_weight + g0 * H, H, M, (int)H};
-      if (int rc = launch_gemm<StoreBf16Epi, true>(D, ws.ldd_row, Htp, ws.ldt / 16, M, (int)H, (int)ws.ldt, sto, st,
-                                                   "gemm_nt_kernel<StoreBf16Epi, A by K-rows>"))
+      StoreEpi sto{(char*)d_weight + g0 * H * (int64_t)dtype_size(dtype), H, M, (int)H, dtype};
+      if (int rc = launch_gemm<StoreEpi, true>(D, ws.ldd_row, Htp, ws.ldt / 16, M, (int)H, (int)ws.ldt, sto, st,
+                                               "gemm_nt_kernel<StoreEpi, A by K-rows>"))
         return rc;
     }
   }
   if (want_dh) {
     const int64_t n = T * H;
     const unsigned blocks = (unsigned)((n + 255) / 256 < 16384 ? (n + 255) / 256 : 16384);
-    f32_to_bf16_kernel<<<dim3(blocks), dim3(256), 0, st>>>(dH32, dh_splits > 1 ? dH32 + dh32_stride : nullptr,
-                                                           (uint16_t*)d_hidden, n);
-    SIIRL_LAUNCH_CHECK("f32_to_bf16_kernel");
+    sum_convert_kernel<<<dim3(blocks), dim3(256), 0, st>>>(dH32, dh_splits > 1 ? dH32 + dh32_stride : nullptr, d_hidden, n,
+                                                           dtype);
+    SIIRL_LAUNCH_CHECK("sum_convert_kernel");
   }
   return SIIRL_OK;
 }
 
+extern "C" size_t siirl_fused_linear_bwd_rows_workspace_bytes_dtype(int dtype, int64_t n_rows, int64_t H, int64_t V,
+                                                                    int want_d_hidden, int want_d_weight) {
+  if (n_rows < 0 || H <= 0 || V <= 0 || dtype_size(dtype) == 0) return 0;
+  return rows_ws(n_rows, H, V, want_d_hidden != 0, want_d_weight != 0, dtype).total;
+}
 extern "C" size_t siirl_fused_linear_bwd_rows_workspace_bytes(int64_t n_rows, int64_t H, int64_t V, int want_d_hidden,
                                                               int want_d_weight) {
-  if (n_rows < 0 || H <= 0 || V <= 0) return 0;
-  return rows_ws(n_rows, H, V, want_d_hidden != 0, want_d_weight != 0).total;
+  return siirl_fused_linear_bwd_rows_workspace_bytes_dtype(SIIRL_BF16, n_rows, H, V, want_d_hidden, want_d_weight);
 }
 
 extern "C" int siirl_fused_linear_logprob_entropy_bwd_rows(const void* hidden, const void* weight, int dtype,
@@ -1009,12 +1119,13 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd_rows(const void* hidden, c
   const bool want_dh = d_hidden != nullptr, want_dw = d_weight != nullptr;
   if (n_rows == 0) {  // no row carries a gradient: both results are zero
     if (want_dh)
-      if (int rc = siirl_scatter_rows(nullptr, nullptr, 0, H * 2, T, d_hidden, stream)) return rc;
+      if (int rc = siirl_scatter_rows(nullptr, nullptr, 0, H * (int64_t)dtype_size(dtype), T, d_hidden, stream)) return rc;
     if (want_dw)
-      if (int rc = siirl_scatter_rows(nullptr, nullptr, 0, H * 2, V, d_weight, stream)) return rc;
+      if (int rc = siirl_scatter_rows(nullptr, nullptr, 0, H * (int64_t)dtype_size(dtype), V, d_weight, stream)) return rc;
     return SIIRL_OK;
   }
-  const RowsWs ws = rows_ws(n_rows, H, V, want_dh, want_dw);
+  const RowsWs ws = rows_ws(n_rows, H, V, want_dh, want_dw, dtype);
+  const int64_t row_bytes = H * (int64_t)dtype_size(dtype);
   if (workspace == nullptr || workspace_bytes < ws.total)
     return fail(SIIRL_ERR_WORKSPACE, "workspace of %zu bytes is smaller than the %zu needed", workspace_bytes, ws.total);
   if (int rc = check_ws_align(workspace)) return rc;
@@ -1027,7 +1138,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd_rows(const void* hidden, c
   float* g_lp_c = (float*)(base + ws.g_lp);
   float* g_ent_c = (float*)(base + ws.g_ent);
   void* dh_c = base + ws.dh;
-  if (int rc = siirl_gather_rows(hidden, rows, n_rows, H * 2, T, hidden_c, stream)) return rc;
+  if (int rc = siirl_gather_rows(hidden, rows, n_rows, row_bytes, T, hidden_c, stream)) return rc;
   gather_token_operands_kernel<<<dim3((unsigned)((n_rows + 255) / 256)), dim3(256), 0, st>>>(
       rows, n_rows, T, labels, lse, ex, g_logprob, g_entropy, labels_c, lse_c, ex_c, g_lp_c, g_ent_c);
   SIIRL_LAUNCH_CHECK("gather_token_operands_kernel");
@@ -1037,6 +1148,6 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd_rows(const void* hidden, c
                                                       base + ws.inner, ws.inner_bytes, stream))
     return rc;
   if (want_dh)
-    if (int rc = siirl_scatter_rows(dh_c, rows, n_rows, H * 2, T, d_hidden, stream)) return rc;
+    if (int rc = siirl_scatter_rows(dh_c, rows, n_rows, row_bytes, T, d_hidden, stream)) return rc;
   return SIIRL_OK;
 }

@@ -1070,17 +1070,24 @@ Tensor kl_penalty(const Tensor& logprob, const Tensor& ref_logprob, int64_t kl_m
 
 // ------------------------------------------------------------------ lm_head fused with log-prob / entropy
 
-void require_bf16_2d(const Tensor& t, const char* name) {
-  require_gpu(t, name);
-  TORCH_CHECK_TYPE(t.scalar_type() == at::kBFloat16 && t.dim() == 2 && t.is_contiguous(), "siirl_amd: `", name,
-                   "` must be a contiguous 2-D bfloat16 tensor");
+// hidden states and weights: bfloat16, float16 or float32, both of one dtype
+int fused_operand_dtype(const Tensor& hidden, const Tensor& weight) {
+  for (const Tensor* t : {&hidden, &weight}) {
+    require_gpu(*t, t == &hidden ? "hidden" : "weight");
+    TORCH_CHECK_TYPE(t->dim() == 2 && t->is_contiguous() &&
+                         (t->scalar_type() == at::kBFloat16 || t->scalar_type() == at::kHalf || t->scalar_type() == at::kFloat),
+                     "siirl_amd: `", t == &hidden ? "hidden" : "weight",
+                     "` must be a contiguous 2-D bfloat16, float16 or float32 tensor");
+  }
+  TORCH_CHECK_TYPE(hidden.scalar_type() == weight.scalar_type(), "siirl_amd: hidden (", hidden.scalar_type(),
+                   ") and weight (", weight.scalar_type(), ") must have one dtype");
+  return hidden.scalar_type() == at::kBFloat16 ? SIIRL_BF16 : hidden.scalar_type() == at::kHalf ? SIIRL_F16 : SIIRL_F32;
 }
 
 std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> fused_linear_fwd(const Tensor& hidden, const Tensor& weight,
                                                                     const Tensor& labels, double inv_temperature,
                                                                     bool save_logits) {
-  require_bf16_2d(hidden, "hidden");
-  require_bf16_2d(weight, "weight");
+  const int dt = fused_operand_dtype(hidden, weight);
   const int64_t T = hidden.size(0), H = hidden.size(1), V = weight.size(0);
   TORCH_CHECK_VALUE(weight.size(1) == H && labels.dim() == 1 && labels.size(0) == T && labels.scalar_type() == at::kLong,
                     "shape mismatch: hidden ", hidden.sizes(), ", weight ", weight.sizes(), ", labels ", labels.sizes());
@@ -1096,11 +1103,11 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> fused_linear_fwd(const Tensor
       save_logits = false;  // no room to keep the logits: the backward recomputes them
     }
   }
-  const size_t nws = siirl_fused_linear_fwd_workspace_bytes(T, H, V);
+  const size_t nws = siirl_fused_linear_fwd_workspace_bytes_dtype(dt, T, H, V);
   Tensor ws = at::empty({(int64_t)std::max<size_t>(nws, 256)}, hidden.options().dtype(at::kByte));
   Tensor y = labels.contiguous();
   DeviceGuard guard(hidden.device());
-  check_rc(siirl_fused_linear_logprob_entropy_fwd(ptr(hidden), ptr(weight), SIIRL_BF16, ptr<int64_t>(y), T, H, V,
+  check_rc(siirl_fused_linear_logprob_entropy_fwd(ptr(hidden), ptr(weight), dt, ptr<int64_t>(y), T, H, V,
                                                   (float)inv_temperature, ptr<float>(lp), ptr<float>(ent),
                                                   ptr<float>(lse), ptr<float>(ex),
                                                   save_logits ? ptr<float>(saved) : nullptr, ptr(ws), nws,
@@ -1114,8 +1121,7 @@ std::tuple<Tensor, Tensor> fused_linear_bwd(const Tensor& hidden, const Tensor& 
                                             const optional<Tensor>& g_lp, const optional<Tensor>& g_ent,
                                             bool need_hidden, bool need_weight, const optional<Tensor>& saved_in,
                                             bool skip_zero_rows) {
-  require_bf16_2d(hidden, "hidden");
-  require_bf16_2d(weight, "weight");
+  const int dt = fused_operand_dtype(hidden, weight);
   require_f32c(g_lp, "g_logprob");
   require_f32c(g_ent, "g_entropy");
   const int64_t T = hidden.size(0), H = hidden.size(1), V = weight.size(0);
@@ -1150,19 +1156,19 @@ std::tuple<Tensor, Tensor> fused_linear_bwd(const Tensor& hidden, const Tensor& 
     Tensor rows = at::nonzero(live).reshape({-1});
     const int64_t n = rows.size(0);
     if (n < T) {
-      const size_t nws = siirl_fused_linear_bwd_rows_workspace_bytes(n, H, V, (int)need_hidden, (int)need_weight);
+      const size_t nws = siirl_fused_linear_bwd_rows_workspace_bytes_dtype(dt, n, H, V, (int)need_hidden, (int)need_weight);
       Tensor ws = at::empty({(int64_t)std::max<size_t>(nws, 256)}, hidden.options().dtype(at::kByte));
       check_rc(siirl_fused_linear_logprob_entropy_bwd_rows(
-                   ptr(hidden), ptr(weight), SIIRL_BF16, ptr<int64_t>(y), T, H, V, (float)inv_temperature, ptr<float>(lse),
+                   ptr(hidden), ptr(weight), dt, ptr<int64_t>(y), T, H, V, (float)inv_temperature, ptr<float>(lse),
                    ptr<float>(ex), ptr<float>(g_lp), ptr<float>(g_ent), ptr<int64_t>(rows), n,
                    need_hidden ? ptr(d_h) : nullptr, need_weight ? ptr(d_w) : nullptr, ptr(ws), nws, stream_of(hidden)),
                "siirl_fused_linear_logprob_entropy_bwd_rows");
       return {d_h, d_w};
     }
   }
-  const size_t nws = siirl_fused_linear_bwd_workspace_bytes(T, H, V, (int)need_hidden, (int)need_weight);
+  const size_t nws = siirl_fused_linear_bwd_workspace_bytes_dtype(dt, T, H, V, (int)need_hidden, (int)need_weight);
   Tensor ws = at::empty({(int64_t)std::max<size_t>(nws, 256)}, hidden.options().dtype(at::kByte));
-  check_rc(siirl_fused_linear_logprob_entropy_bwd(ptr(hidden), ptr(weight), SIIRL_BF16, ptr<int64_t>(y), T, H, V,
+  check_rc(siirl_fused_linear_logprob_entropy_bwd(ptr(hidden), ptr(weight), dt, ptr<int64_t>(y), T, H, V,
                                                   (float)inv_temperature, ptr<float>(lse), ptr<float>(ex),
                                                   ptr<float>(saved), ptr<float>(g_lp), ptr<float>(g_ent),
                                                   need_hidden ? ptr(d_h) : nullptr, need_weight ? ptr(d_w) : nullptr,
@@ -1177,8 +1183,11 @@ struct FusedLinearFn : public torch::autograd::Function<FusedLinearFn> {
     at::AutoDispatchBelowADInplaceOrView below;
     require_gpu(hidden, "hidden");
     require_gpu(weight, "weight");
-    TORCH_CHECK_TYPE(hidden.scalar_type() == at::kBFloat16 && weight.scalar_type() == at::kBFloat16,
-                     "siirl_amd: the fused lm_head path takes bfloat16 hidden states and weights");
+    TORCH_CHECK_TYPE(hidden.scalar_type() == weight.scalar_type() &&
+                         (hidden.scalar_type() == at::kBFloat16 || hidden.scalar_type() == at::kHalf ||
+                          hidden.scalar_type() == at::kFloat),
+                     "siirl_amd: the fused lm_head path takes hidden states and weights of one dtype, bfloat16, "
+                     "float16 or float32 (got ", hidden.scalar_type(), " and ", weight.scalar_type(), ")");
     Tensor h = hidden.detach().contiguous(), w = weight.detach().contiguous();
     Tensor y = labels.detach();
     if (y.device() != h.device()) y = y.to(h.device());

@@ -6,7 +6,9 @@
 * ``linear_cross_entropy`` -- mirror of ``siirl/utils/kernel/linear_cross_entropy.py:40-117``:
   ``(hidden, weight, labels, temperature, reduction, dist_process_group) -> (logprobs, entropy)``.
 
-Both run the MFMA kernels of ``csrc/fused_linear.hip`` through the C ABI.  Operands are bf16 on the GPU.  Neither
+Both run the MFMA kernels of ``csrc/fused_linear.hip`` through the C ABI.  Operands are bf16, fp16 or fp32 on the GPU (fp16: the half matrix instruction; fp32: three bf16
+terms per element, products good to 2^-16; the gradient GEMMs always multiply bf16 dlogits with bf16-rounded
+operands and return the operands' dtype).  Neither
 pass holds a ``[T, V]`` tensor: the backward recomputes the logits slab by slab, which is the reference's memory
 behaviour.  Opt-in trade of memory for time: with ``set_saved_logits_limit(nbytes)`` (or
 ``SIIRL_AMD_SAVED_LOGITS_LIMIT`` bytes in the environment; default 0 = never), a forward that a backward will follow

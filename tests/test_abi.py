@@ -48,7 +48,7 @@ def test_every_entry_point_cites_the_reference():
             continue
         if n in ("siirl_hip_abi_version", "siirl_hip_last_error", "siirl_agg_loss_bwd", "siirl_actor_loss_bwd",
                  "siirl_kl_penalty_bwd", "siirl_masked_reduce_bwd", "siirl_actor_loss_cov_bwd",
-                 "siirl_range_select_write") or n.endswith("_workspace_bytes") or n.endswith("_logits_bytes"):
+                 "siirl_range_select_write") or n.endswith("_workspace_bytes") or n.endswith("_workspace_bytes_dtype") or n.endswith("_logits_bytes"):
             continue  # utilities and backward halves documented with their forward
         pos = text.index(n + "(")
         comment = text[text.rfind("/*", 0, pos):pos]

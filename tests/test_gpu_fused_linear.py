@@ -405,3 +405,57 @@ def test_zero_gradient_rows_with_one_gradient_requested(dev, wrt):
     else:
         assert hd.grad is None
         _check_grad(wd.grad, dw64, "d_weight")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("T,H,V", [(5, 64, 33), (300, 128, 1000), (513, 256, 8200), (64, 3584, 2048), (130, 128, 65537)])
+def test_fp16_and_fp32_operands(dev, dtype, T, H, V):
+    """hidden and W in float16 / float32 (the reference multiplies in whatever dtype they arrive,
+    ``experimental/torch_functional.py:20-23``): log-prob and entropy against the oracle on the same values -- exact
+    fp16 products on the half matrix instruction; three bf16 terms per fp32 element, good to 2^-16 per product --,
+    gradients in the operands' dtype at the fused path's bar (bf16 dlogits times bf16-rounded operands, no more
+    roundings than with bf16 operands once the outputs are fp16 / fp32).  Upstream gradients of order 1 here: a
+    softmax gradient of order 1e-2 / V underflows an fp16 *result*, which is what loss scaling is for."""
+    from siirl_amd.fused_linear import FusedLinearForPPO, linear_cross_entropy
+
+    g = torch.Generator().manual_seed(7 * T + H + V)
+    h = torch.randn(T, H, generator=g).to(dtype)
+    w = (torch.randn(V, H, generator=g) * (2.0 / H ** 0.5)).to(dtype)
+    y = torch.randint(0, V, (T,), generator=g)
+    g_lp, g_h = torch.randn(T, generator=g), torch.randn(T, generator=g)
+    hd, wd = h.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    lp, ent = FusedLinearForPPO()(hd, wd, y.to(dev), temperature=0.8)
+    assert lp.dtype == torch.float32 and ent.dtype == torch.float32
+    lp64, ent64 = OFL.fused_linear_for_ppo_fwd(h, w, y, 0.8, dtype=torch.float64)
+    e_lp, e_ent = (lp.cpu().double() - lp64).abs().max().item(), (ent.cpu().double() - ent64).abs().max().item()
+    print(f"[operands {dtype}] ({T}, {H}, {V}): logprob err {e_lp:.2e}, entropy err {e_ent:.2e}", flush=True)
+    assert e_lp < 1e-4 and e_ent < 1e-4, (e_lp, e_ent)
+    torch.autograd.backward([lp, ent], [g_lp.to(dev), g_h.to(dev)])
+    assert hd.grad.dtype == dtype and wd.grad.dtype == dtype
+    dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp, g_h, h, w, y, 0.8, dtype=torch.float64)
+    _check_grad(hd.grad, dh64, f"d_hidden {dtype}", floor=1e-6)
+    _check_grad(wd.grad, dw64, f"d_weight {dtype}", floor=1e-6)
+    # the Triton-shaped interface and the row-subset backward take the same operands
+    lp2, ent2 = linear_cross_entropy(h.to(dev), w.to(dev), y.to(dev), 0.8, "none", None)
+    assert torch.equal(lp2, lp.detach()) and torch.equal(ent2, ent.detach())
+    if T >= 64:
+        live = (torch.arange(T) % 3 != 0).float()
+        hd2, wd2 = h.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+        lp3, ent3 = FusedLinearForPPO()(hd2, wd2, y.to(dev), temperature=0.8)
+        torch.autograd.backward([lp3, ent3], [(g_lp * live).to(dev), (g_h * live).to(dev)])
+        dh64s, dw64s = OFL.fused_linear_for_ppo_bwd(g_lp * live, g_h * live, h, w, y, 0.8, dtype=torch.float64)
+        _check_grad(hd2.grad, dh64s, f"d_hidden {dtype}, rows without gradient left out", floor=1e-6)
+        _check_grad(wd2.grad, dw64s, f"d_weight {dtype}, rows without gradient left out", floor=1e-6)
+        assert torch.count_nonzero(hd2.grad[live == 0]) == 0
+
+
+def test_mixed_operand_dtypes_are_refused(dev):
+    from siirl_amd.fused_linear import fused_linear_logprob_entropy
+
+    h = torch.randn(8, 64, device=dev)
+    w = torch.randn(16, 64, device=dev).to(torch.bfloat16)
+    y = torch.zeros(8, dtype=torch.int64, device=dev)
+    with pytest.raises(TypeError, match="one dtype"):
+        fused_linear_logprob_entropy(h, w, y)
+    with pytest.raises(TypeError):
+        fused_linear_logprob_entropy(h.double(), w.double(), y)

@@ -75,7 +75,7 @@ typedef enum siirl_kl_mode {
 
 /* ABI version of this header (major * 1000 + minor); siirl_hip_abi_version() returns the one the library was built
  * from.  A host compiled against another version must not call the library. */
-#define SIIRL_HIP_ABI_VERSION 1009
+#define SIIRL_HIP_ABI_VERSION 1010
 int siirl_hip_abi_version(void);
 
 /* Message of the last failing call on this thread ("" if none).  Host pointer, valid until the
@@ -89,8 +89,8 @@ const char* siirl_hip_last_error(void);
  * its logits, siirl_logprob_entropy_bwd counts both upstream gradients of the row as zero: with
  * SIIRL_BWD_SKIP_ZERO_ROWS the row's gradient is written as zeros unread; without that flag it is zero as well unless
  * the row holds +inf or NaN logits (contiguous rows are then still read, with their probabilities forced to 0).  The
- * single-launch step entry points (siirl_logprob_entropy_fwd_bwd, siirl_actor_step_fused) treat it as an ignored
- * label (log-prob 0, no log-prob gradient) and still read the row; the lm_head entry points know no special labels
+ * single-launch step entry points (siirl_logprob_entropy_fwd_bwd, siirl_actor_step_fused) do the same in one go:
+ * log-prob and entropy 0 and a gradient of zeros, the row unread.  The lm_head entry points know no special labels
  * (any label outside [0, V) gives NaN there). */
 #define SIIRL_LABEL_SKIP_ROW (-101)
 
@@ -254,22 +254,26 @@ int siirl_actor_loss_fwd(const float* old_log_prob, const float* log_prob, const
 /*
  * siirl_actor_loss_fwd for callers that cannot allocate or bring a workspace (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc): same operands, same kernels, same results bit for bit,
- * with the scratch taken from a buffer of SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES that is part of the library's
- * device image (one copy per GPU, held until the process ends).  The call allocates nothing and frees nothing.
- * A [B, L] problem whose siirl_loss_workspace_bytes(B, L) exceeds the buffer (64 bytes per 2048-token segment of a
- * row: about 65 000 segments) is refused with SIIRL_ERR_WORKSPACE.  All calls on one GPU share the buffer: calls
- * that overlap in time on one GPU (different streams or threads) race; calls on one stream do not.  The first
- * call on each GPU looks the buffer's address up (hipGetSymbolAddress) and must happen outside stream capture.
+ * with the scratch taken from a buffer that is part of the library's device image (one copy per GPU, held until the
+ * process ends): SIIRL_ACTOR_LOSS_STATIC_SLOTS slices of SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES each.  The call
+ * allocates nothing and frees nothing.  `slot` in [0, SIIRL_ACTOR_LOSS_STATIC_SLOTS) names the slice this call uses
+ * (anything else is refused with SIIRL_ERR_INVALID_ARGUMENT): calls that may overlap in time on one GPU -- different
+ * streams or threads -- must be given different slots and then do not touch each other's scratch; calls that share
+ * a slot and overlap race; calls on one stream may share a slot.  A [B, L] problem whose
+ * siirl_loss_workspace_bytes(B, L) exceeds a slice (64 bytes per 2048-token segment of a row: about 65 000
+ * segments) is refused with SIIRL_ERR_WORKSPACE.  The first call on each GPU looks the buffer's address up
+ * (hipGetSymbolAddress) and must happen outside stream capture.
  * This entry point has no counterpart in the reference.
  */
 #define SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES (4u << 20)
+#define SIIRL_ACTOR_LOSS_STATIC_SLOTS 4
 int siirl_actor_loss_fwd_static(const float* old_log_prob, const float* log_prob, const float* advantages,
                                 const void* mask, int mask_dtype, const float* is_weights, const float* entropy,
                                 const float* ref_log_prob, int64_t B, int64_t L, int loss_mode, float clip_low,
                                 float clip_high, float clip_c, float log_ratio_clamp, int agg_mode,
                                 float entropy_coeff, int kl_mode, int kl_straight_through, float kl_coef,
                                 float policy_drift_coeff, float loss_scale, float* out16, float* row_msum,
-                                float* row_s, siirl_stream_t stream);
+                                float* row_s, int slot, siirl_stream_t stream);
 
 /*
  * Backward of siirl_actor_loss_fwd for an upstream gradient g_loss[0] (device scalar) on out16[SIIRL_OUT_LOSS]:

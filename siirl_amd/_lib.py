@@ -16,7 +16,7 @@ MARFT_MAX_AGENTS = 16  # SIIRL_MARFT_MAX_AGENTS
 LABEL_SKIP_ROW = -101  # SIIRL_LABEL_SKIP_ROW
 MARFT_STORE_FLOAT, MARFT_STORE_TRUNCATED, MARFT_STORE_NONZERO = range(3)  # siirl_marft_store
 MAX_EOS_TOKENS = 16  # SIIRL_MAX_EOS_TOKENS
-ABI_VERSION = 1009  # SIIRL_HIP_ABI_VERSION of include/siirl_hip.h that SIGNATURES below transcribes
+ABI_VERSION = 1010  # SIIRL_HIP_ABI_VERSION of include/siirl_hip.h that SIGNATURES below transcribes
 BWD_SKIP_ZERO_ROWS = 1
 
 _p, _i64, _i32, _f32, _u32, _sz, _f64 = (C.c_void_p, C.c_int64, C.c_int, C.c_float, C.c_uint32, C.c_size_t,
@@ -38,7 +38,7 @@ SIGNATURES = {
     "siirl_actor_loss_fwd": (_i32, [_p, _p, _p, _p, _i32, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _f32, _f32, _i32,
                                     _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _p, _sz, _p]),
     "siirl_actor_loss_fwd_static": (_i32, [_p, _p, _p, _p, _i32, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _f32, _f32,
-                                           _i32, _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _p]),
+                                           _i32, _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _i32, _p]),
     "siirl_actor_loss_bwd": (_i32, [_p, _p, _p, _p, _p, _i32, _p, _p, _p, _i64, _i64, _i32, _f32, _f32, _f32, _f32,
                                     _i32, _f32, _i32, _i32, _f32, _f32, _f32, _p, _p, _p, _p, _p, _p]),
     "siirl_cov_workspace_bytes": (_sz, []),

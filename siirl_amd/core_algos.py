@@ -375,9 +375,7 @@ def _marft_walk(rewards, values, masks, chains, gamma, lam, out_dtype=None):
     if walked and mdt not in _MARFT_INT_MASKS:
         # the reference's range(mask row sum) (:410-412)
         raise TypeError("only integer tensors of a single element can be converted to an index")
-    for first, n in walked:
-        if first < 0 or first + n > B:
-            raise IndexError(f"index {first + n - 1} is out of bounds for dimension 0 with size {B}")
+    _check_marft_chains(walked, B)
     out_dtypes = [out_dtype or m.dtype for m in masks]
     if any(d != out_dtypes[0] for d in out_dtypes):
         raise NotImplementedError("siirl_amd: the agents' outputs must share one dtype")
@@ -415,6 +413,23 @@ def _marft_walk(rewards, values, masks, chains, gamma, lam, out_dtype=None):
     adv = [a.to(d) for a, d in zip(adv, out_dtypes)]
     ret = [a.to(d) for a, d in zip(ret, out_dtypes)]
     return adv, ret, [m.detach().to(dev) for m in masks], back
+
+
+def _check_marft_chains(walked, B):
+    """The requests' row ranges ``(first row, trajectory length)`` must lie inside the batch (the reference's own
+    ``IndexError``) and must not overlap: the reference walks requests one after the other, so where a ``traj_len``
+    runs into the next request's rows the later walk overwrites the earlier one's results and reads its values
+    (``core_algos.py:400-448``); here every request is walked by a wave of its own at the same time, which has no
+    such order -- refused instead of answered differently from run to run."""
+    for first, n in walked:
+        if first < 0 or first + n > B:
+            raise IndexError(f"index {first + n - 1} is out of bounds for dimension 0 with size {B}")
+    ordered = sorted(walked)
+    for (a, na), (b, _) in zip(ordered, ordered[1:]):
+        if a + na > b:
+            raise NotImplementedError(f"siirl_amd: the request that starts at row {a} with traj_len {na} runs into the "
+                                      f"request that starts at row {b}; overlapping requests are walked one after "
+                                      "the other by the reference and are not supported here")
 
 
 def compute_marft_gae_advantage_return(data, pre_agent_group_ids, gamma, lam):

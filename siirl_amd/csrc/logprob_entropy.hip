@@ -547,6 +547,21 @@ __global__ __launch_bounds__(kFusedThreads) void lpe_fused_kernel(const typename
   u32x4* dv = reinterpret_cast<u32x4*>(d + sp.head);
   constexpr int kTile = kFusedThreads * kFusedUnroll;
 
+  // A row labelled "skip" (a packed token outside the response window) is not read at all, as in the two-launch
+  // kernels: log-prob and entropy 0, a gradient of zeros whatever the upstream coefficients would be.  The label is
+  // the same for the whole workgroup, so every thread leaves here, before the first barrier.
+  if (labels && labels[row] == kSkipRow) {
+    if (tid == 0) {
+      if (logprob) logprob[row] = 0.f;
+      if (ENT && entropy) entropy[row] = 0.f;
+    }
+    for (int i = tid; i < sp.head; i += kFusedThreads) E::store1(d + i, 0.f);
+    for (int i = sp.tail0 + tid; i < V; i += kFusedThreads) E::store1(d + i, 0.f);
+    const u32x4 z = u32x4{0u, 0u, 0u, 0u};
+    for (int i = tid; i < sp.nvec; i += kFusedThreads) st16<true>(z, dv + i);
+    return;
+  }
+
   // the first `cap` 16-byte vectors of the row are kept in LDS between the passes
   extern __shared__ __align__(16) char row_lds[];
   u32x4* keep = reinterpret_cast<u32x4*>(row_lds);
@@ -595,7 +610,7 @@ __global__ __launch_bounds__(kFusedThreads) void lpe_fused_kernel(const typename
   {
     const int64_t yl = labels ? labels[row] : -1;
     if (yl >= 0 && yl < (int64_t)V) y = (int)yl;
-    ignored = labels && (yl == kIgnoreIndex || yl == kSkipRow);
+    ignored = labels && yl == kIgnoreIndex;
   }
   if (tid == 0) {
     for (int w = 1; w < kFusedThreads / kWave; ++w) merge(st, sm[w * 3], sm[w * 3 + 1], sm[w * 3 + 2], k);

@@ -19,10 +19,12 @@
 
 // Scratch of siirl_actor_loss_fwd_static, the entry point that allocates nothing: the segment partials, the row
 // pre-pass sums and the finish records that the other forward entry points take from the caller's workspace.  One
-// copy per GPU, held until the process ends.  In host code this name is only a handle for hipGetSymbolAddress;
-// kernels receive the device address that call returns.
-constexpr size_t kStaticScratchBytes = SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES;
-static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+// copy per GPU, held until the process ends, cut into slices ("slots") so that calls on different streams can each
+// have their own.  In host code this name is only a handle for hipGetSymbolAddress; kernels receive the device
+// address that call returns.
+constexpr size_t kStaticScratchBytes = SIIRL_ACTOR_LOSS_STATIC_SCRATCH_BYTES;  // per slot
+constexpr int kStaticSlots = SIIRL_ACTOR_LOSS_STATIC_SLOTS;
+static __device__ __align__(256) unsigned char scratch[kStaticSlots * kStaticScratchBytes];
 
 namespace siirl {
 namespace {
@@ -1046,24 +1048,26 @@ extern "C" int siirl_actor_loss_fwd_static(const float* old_log_prob, const floa
                                            float log_ratio_clamp, int agg_mode, float entropy_coeff, int kl_mode,
                                            int kl_straight_through, float kl_coef, float policy_drift_coeff,
                                            float loss_scale, float* out16, float* row_msum, float* row_s,
-                                           siirl_stream_t stream) {
+                                           int slot, siirl_stream_t stream) {
   LossArgs a{};
   if (int rc = fill_actor_args(a, old_log_prob, log_prob, advantages, mask, mask_dtype, is_weights, entropy,
                                ref_log_prob, B, L, loss_mode, clip_low, clip_high, clip_c, log_ratio_clamp, agg_mode,
                                entropy_coeff, kl_mode, kl_straight_through, kl_coef, policy_drift_coeff, loss_scale))
     return rc;
+  SIIRL_REQUIRE(slot >= 0 && slot < kStaticSlots, "slot %d is outside [0, %d)", slot, kStaticSlots);
   SIIRL_REQUIRE(out16 && (B == 0 || row_msum), "NULL output");
   SIIRL_REQUIRE(B == 0 || (loss_mode != SIIRL_LOSS_GSPO && loss_mode != SIIRL_LOSS_GEO_MEAN) || row_s,
                 "row_s is required for the gspo and geo_mean losses");
   const size_t need = B == 0 ? 0 : ws_bytes_of(B, L);
   if (need > kStaticScratchBytes)
     return fail(SIIRL_ERR_WORKSPACE,
-                "B=%lld x L=%lld needs %zu bytes of scratch, the static buffer holds %zu: use siirl_actor_loss_fwd "
+                "B=%lld x L=%lld needs %zu bytes of scratch, a slot of the static buffer holds %zu: use siirl_actor_loss_fwd "
                 "with a workspace of the caller's", (long long)B, (long long)L, need, kStaticScratchBytes);
   void* ws = nullptr;
   if (int rc = static_scratch_address(&ws)) return rc;
-  // every scratch slot that the finish kernels read is written by this call's earlier kernels: nothing to clear
-  return run_forward(a, out16, row_msum, row_s, ws, kStaticScratchBytes, (hipStream_t)stream);
+  // every scratch word that the finish kernels read is written by this call's earlier kernels: nothing to clear
+  return run_forward(a, out16, row_msum, row_s, (unsigned char*)ws + (size_t)slot * kStaticScratchBytes,
+                     kStaticScratchBytes, (hipStream_t)stream);
 }
 
 extern "C" int siirl_actor_loss_bwd(const float* g_loss, const float* old_log_prob, const float* log_prob,

@@ -14,7 +14,7 @@ Differences a caller can observe, all deliberate:
   by one backward kernel.  ``set_pairing(False)`` turns this off;
 * a label of ``-101`` (``siirl_amd.padding.LABEL_SKIP_ROW``, set by ``unpad_ids_and_labels(..., response_length=L)``
   on the packed tokens outside the response window) makes both passes skip the row: log-prob and entropy 0, zero
-  gradient, the logits of the row are never read;
+  gradient, the logits of the row are never read (the single-launch step, ``fused_actor_step``, does the same);
 * the backward writes zeros, without reading the row, where both upstream gradients of a row are zero
   (``set_skip_zero_rows``): a NaN or Inf in a padded row's logits therefore does not reach ``dlogits`` as it would
   through the reference's autograd.

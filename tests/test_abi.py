@@ -84,8 +84,12 @@ def test_argument_validation_without_gpu():
                                   0.0, 1.0, p, p, None, p, 1 << 20, None) == -1  # geo_mean needs row_s
     # the allocation-free variant refuses what its fixed buffer cannot hold, before any device call
     assert h.siirl_actor_loss_fwd_static(p, p, p, p, L.F32, None, None, None, 1 << 20, 4096, 0, 0.2, 0.2, 3.0, 20.0, 0,
-                                         0.0, 0, 0, 0.0, 0.0, 1.0, p, p, p, None) == -4
+                                         0.0, 0, 0, 0.0, 0.0, 1.0, p, p, p, 0, None) == -4
     assert b"static buffer" in h.siirl_hip_last_error()
+    for bad_slot in (-1, 4):  # and a slot outside its slices
+        assert h.siirl_actor_loss_fwd_static(p, p, p, p, L.F32, None, None, None, 2, 4, 0, 0.2, 0.2, 3.0, 20.0, 0, 0.0, 0,
+                                             0, 0.0, 0.0, 1.0, p, p, p, bad_slot, None) == -1
+        assert b"slot" in h.siirl_hip_last_error()
     # the covariance losses: their two modes go through their own entry points and nowhere else
     assert h.siirl_actor_loss_fwd(p, p, p, p, L.F32, None, None, None, 2, 4, 5, 0.2, 0.2, 3.0, 20.0, 0, 0.0, 0, 0, 0.0,
                                   0.0, 1.0, p, p, p, p, 1 << 20, None) == -1

@@ -155,6 +155,46 @@ def test_fwd_bwd_entry_equals_two_launches(dev, T, V, dtype):
                                            _lib.ptr(x), V, st) == -1  # no in-place mode
 
 
+@pytest.mark.parametrize("V,dtype", [(1000, torch.float32), (50257, torch.bfloat16)])
+def test_skip_labelled_rows_agree_between_the_paths(dev, V, dtype):
+    """Rows labelled LABEL_SKIP_ROW (packed tokens outside the response window): the single-launch entry and the
+    two-launch kernels give the same answer -- log-prob and entropy 0, a gradient of zeros whatever the upstream
+    gradients are -- and neither reads the row (it holds NaN here)."""
+    from siirl_amd import _lib
+    from siirl_amd.padding import LABEL_SKIP_ROW
+
+    h = _lib.lib()
+    T = 9
+    g = torch.Generator().manual_seed(V)
+    x = (torch.randn(T, V, generator=g) * 3).to(dtype)
+    y = torch.randint(0, V, (T,), generator=g)
+    skipped = torch.tensor([1, 4, 8])
+    y[skipped] = LABEL_SKIP_ROW
+    x[skipped] = float("nan")
+    x, y = x.to(dev), y.to(dev)
+    g1 = (torch.randn(T, generator=g) * 1e-2).to(dev)  # non-zero on the skipped rows as well
+    g2 = (torch.randn(T, generator=g) * 1e-2).to(dev)
+    code, st = _lib.dtype_code(dtype), _lib.current_stream(dev)
+    lp, ent, lse, ex, lp2, ent2 = (torch.full((T,), 7.0, device=dev) for _ in range(6))
+    d, d2 = torch.full_like(x, 7.0), torch.full_like(x, 7.0)
+    _lib.check(h.siirl_logprob_entropy_fwd_bwd(_lib.ptr(x), code, T, V, V, _lib.ptr(y), 1.0, _lib.ptr(g1), _lib.ptr(g2),
+                                               _lib.ptr(lp), _lib.ptr(ent), _lib.ptr(d), V, st), "fwd_bwd")
+    _lib.check(h.siirl_logprob_entropy_fwd(_lib.ptr(x), code, T, V, V, _lib.ptr(y), 1.0, _lib.ptr(lp2), _lib.ptr(ent2),
+                                           _lib.ptr(lse), _lib.ptr(ex), st), "fwd")
+    _lib.check(h.siirl_logprob_entropy_bwd(_lib.ptr(x), code, T, V, V, _lib.ptr(y), 1.0, _lib.ptr(lse), _lib.ptr(ex),
+                                           _lib.ptr(g1), _lib.ptr(g2), _lib.ptr(d2), V, 1, st), "bwd")
+    sk = skipped.to(dev)
+    for t in (lp, ent, lp2, ent2):
+        assert torch.count_nonzero(t[sk]) == 0
+    assert torch.count_nonzero(d[sk]) == 0 and torch.count_nonzero(d2[sk]) == 0
+    live = torch.ones(T, dtype=torch.bool, device=dev)
+    live[sk] = False
+    assert (lp[live] - lp2[live]).abs().max() < 1e-5 and (ent[live] - ent2[live]).abs().max() < 1e-4
+    diff = (d[live].float() - d2[live].float()).abs()
+    assert bool((diff <= 1e-9 + 2 * ULP[dtype] * d2[live].float().abs()).all()), diff.max()
+    assert bool(torch.isfinite(d.float()).all()) and bool(torch.isfinite(d2.float()).all())
+
+
 def test_fused_step_random_sweep(dev):
     """Seeded random shapes, dtypes, loss modes, aggregation modes, coefficients and temperatures through the
     single-pass step, each against the oracle's micro-batch step (tolerances of _check).  ``SIIRL_TEST_SEED=<int>`` in

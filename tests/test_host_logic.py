@@ -201,3 +201,19 @@ def test_uid_codes_for_keys_that_are_not_int64():
     assert DF._uid_tensor(np.asarray([3, 3, 1]), "cpu").tolist() == [3, 3, 1]
     with pytest.raises(ValueError):
         DF._uid_tensor(np.asarray(["a", "b"]), "cpu")  # numpy strings have .item: int() as in the reference
+
+
+def test_marft_requests_must_not_overlap():
+    """Requests whose row ranges overlap are refused on the host, before anything is launched (the reference walks
+    them sequentially, last writer wins; concurrent waves would race); ranges that touch are fine."""
+    from siirl_amd.core_algos import _check_marft_chains
+
+    _check_marft_chains([(0, 4), (4, 4), (8, 2)], 10)
+    _check_marft_chains([(4, 4), (0, 4)], 8)  # any order
+    _check_marft_chains([], 0)
+    with pytest.raises(NotImplementedError, match="runs into"):
+        _check_marft_chains([(0, 5), (4, 4)], 10)
+    with pytest.raises(NotImplementedError, match="runs into"):
+        _check_marft_chains([(4, 4), (0, 6)], 10)
+    with pytest.raises(IndexError):
+        _check_marft_chains([(0, 4), (4, 7)], 10)

@@ -101,3 +101,35 @@ def test_split_then_restore_round_trip(seed):
     per_row = torch.cat([mb["input_ids"][:, 0] for mb in mbs[0]])
     restored = SB.restore_dynamic_batch(per_row, idx)
     assert torch.equal(restored, batch["input_ids"][:, 0])
+
+
+def test_ties_follow_the_reference_heap_order_worked_by_hand():
+    """Equal sums everywhere, so every decision is a tie-break.  Expected assignments are worked by hand from the
+    reference's comparison keys (``siirl/utils/model_utils/seqlen_balancing.py:41-142``): a set compares by
+    (sum, number of items, list of (index, value) items); a state's sets are kept in descending order; the heap pops
+    the state with the largest spread first and, among equal spreads, the one whose largest set is larger; a merge
+    pairs set i of the first popped state with set k - 1 - i of the second and re-sorts.
+
+    [1, 1, 1, 1], k = 2.  Four singleton states of spread 1; among equal spreads the larger first set wins, and the
+    sets differ only in their index, so index 3 pops first, then 2: {3} | {2}, spread 0.  Then 1 and 0: {1} | {0}.
+    Both have spread 0; {3} > {1}, so {3} | {2} pops first and merges with {1} | {0} crosswise: {3, 0} | {2, 1}.
+    Sums and sizes tie; the item lists [(3, 1), (0, 1)] > [(2, 1), (1, 1)] keep that order.
+
+    [4, 3, 3, 2, 2, 2], k = 2 (indices 0..5).  Spreads 4, 3, 3, 2, 2, 2.  Pop index 0 (spread 4), then of the two
+    3s the larger item list: index 2.  -> {0} | {2}, sums 4 | 3, spread 1.  Pop index 1 (spread 3), then of the 2s
+    the largest index, 5 -> {1} | {5}, sums 3 | 2, spread 1.  Pop 4, then 3 -> {4} | {3}, spread 0.  The two spread-1
+    states: first sets {0} (sum 4) > {1} (sum 3), so {0} | {2} pops first and takes {1} | {5} crosswise:
+    {0, 5} (6) and {2, 1} (6); equal sums and sizes, item lists [(2, 3), (1, 3)] > [(0, 4), (5, 2)], so the order
+    becomes {2, 1} | {0, 5}.  Last merge: its first set (sum 6) > {4} (sum 2), so it pops first and takes {4} | {3}
+    crosswise: {2, 1, 3} (8) | {0, 5, 4} (8); [(2, 3), ...] > [(0, 4), ...] keeps the order."""
+    assert SB.karmarkar_karp([1, 1, 1, 1], 2, False) == [[3, 0], [2, 1]]
+    assert SB.karmarkar_karp([4, 3, 3, 2, 2, 2], 2, False) == [[2, 1, 3], [0, 5, 4]]
+    assert SB.get_seqlen_balanced_partitions([4, 3, 3, 2, 2, 2], 2, False) == [[1, 2, 3], [0, 4, 5]]
+    # equal_size seeds the heap with groups of k neighbours of the sorted list.
+    # [2, 2, 1, 1], k = 2: groups (indices 2, 3) and (0, 1); inside a group the larger index sorts first:
+    # {3} | {2} and {1} | {0}, both spread 0; {1} (sum 2) > {3} (sum 1) pops first and takes the other crosswise:
+    # {1, 2} (3) | {0, 3} (3); (1, 2) > (0, 2) keeps the order.
+    assert SB.karmarkar_karp([2, 2, 1, 1], 2, True) == [[1, 2], [0, 3]]
+    # [5] * 6, k = 3: groups {2} | {1} | {0} and {5} | {4} | {3}; the second has the larger first set, pops first and
+    # takes the first crosswise: {5, 0} | {4, 1} | {3, 2}, already in descending item order.
+    assert SB.karmarkar_karp([5, 5, 5, 5, 5, 5], 3, True) == [[5, 0], [4, 1], [3, 2]]

@@ -6,8 +6,10 @@
 // (siirl/utils/kernel/linear_cross_entropy.py:40-117 -> siirl/utils/kernel/kernels.py:507-696,1378-1586); the
 // per-tile online-softmax state (max, sum exp, sum x*exp) is the one of kernels.py:254-266,343-350.
 //
-// One GEMM core, C[M,N] = A[M,K] . B[N,K]^T, bf16 operands, fp32 accumulation, 256 x 256 x 64 workgroup tile,
-// 8 waves (2 x 4) of 128 x 64 (4 x 2 MFMA 32x32x16 bf16 tiles, 128 accumulator registers each):
+// One GEMM core, C[M,N] = A[M,K] . B[N,K]^T, 16-bit operands, fp32 accumulation, 256 x 256 x 64 workgroup tile,
+// 8 waves (2 x 4) of 128 x 64 (8 x 4 MFMA 16x16x32 tiles, 128 accumulator registers each).  The 16x16x32 shape moves
+// half the accumulator data per flop of the 32x32x16 one; with random operand bits the matrix cores then sustain
+// 1.79 instead of 1.62 PFLOP/s in an LDS-fed loop at this part's power limit, which is what sets these kernels' time.
 //   * A (K-major rows) goes global -> LDS by DMA (global_load_lds_dwordx4, no staging registers, no ds_write)
 //     into a ring of four 32 KB stages.  Rows are unpadded; 16-byte chunks are XOR-swizzled by (row / 2) % 8 so
 //     that the ds_read_b128 fragment reads are conflict-free.  A stage is issued three K-steps before it is read
@@ -32,28 +34,18 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-// Rows of the workgroup tile: 256 (8 waves, one workgroup per CU) or 128 (4 waves, 64 KB ring, two independent
-// workgroups per CU whose prologues and epilogues overlap each other's main loop).  Measured at T=16384, H=3584,
-// V=152064: 128 is 1.5 % slower forward and 4 % slower backward, so the overlap is not what the core lacks.
-#ifndef SIIRL_GEMM_BM
-#define SIIRL_GEMM_BM 256
-#endif
-static_assert(SIIRL_GEMM_BM == 256 || SIIRL_GEMM_BM == 128, "the workgroup tile has 256 or 128 rows");
-constexpr int BM = SIIRL_GEMM_BM, BN = 256, BK = 64;
-// Waves along N: 4 (8 waves of 128 x 64, two per SIMD) or 2 (4 waves of 128 x 128, one per SIMD, accumulators in
-// the AGPRs).  Measured at T=16384, H=3584, V=152064: the 4-wave grid is 5 % slower in the d-weight GEMM, 9 % in the
-// forward and 14 % in d-hidden: its matrix cores are busy 0.67 of the cycles at 1.74 GHz against 0.76 at 1.66 GHz, so
-// halving the operand fetches per MFMA frees little power and does not pay for losing the second wave per SIMD.
-#ifndef SIIRL_GEMM_WAVES_N
-#define SIIRL_GEMM_WAVES_N 4
-#endif
-constexpr int WM = BM / 128, WN = SIIRL_GEMM_WAVES_N;  // wave grid over the workgroup tile
+// Workgroup tile 256 x 256 x 64, 8 waves as 2 (M) x 4 (N), two per SIMD, one workgroup per CU (the LDS ring).
+// (Measured alternatives at T=16384, H=3584, V=152064, with the 32x32x16 MFMA: 128-row tiles with two workgroups per
+// CU 1.5-4 % slower; 4 waves of 128 x 128, one per SIMD, 5-14 % slower.)
+constexpr int BM = 256, BN = 256, BK = 64;
+constexpr int WM = 2, WN = 4;  // wave grid over the workgroup tile
 constexpr int kThreads = WM * WN * 64;
-constexpr int kWavesPerSimd = kThreads / 256;  // one workgroup per CU (the LDS ring), four SIMDs
-static_assert(kThreads == 256 || kThreads == 512, "4 or 8 waves per workgroup");
-constexpr int MI = BM / (WM * 32), NJ = BN / (WN * 32);  // 32x32 MFMA tiles per wave
+constexpr int kWavesPerSimd = kThreads / 256;
+constexpr int MI = BM / (WM * 16), NJ = BN / (WN * 16);  // 16x16 MFMA tiles per wave: 8 x 4
+constexpr int KS = BK / 32;                              // K = 32 slices per K-step
+static_assert(MI == 8 && NJ == 4 && KS == 2, "the K-step schedule is written for 8 x 4 tiles and two K slices");
 constexpr int kRowBytes = BK * 2;             // unpadded rows, 16-byte chunks XOR-swizzled by (row / 2) % 8
 constexpr int kTileBytes = BM * kRowBytes;    // 32768
 constexpr int kStageBytes = kTileBytes;       // A tile only: B goes global -> registers
@@ -80,7 +72,7 @@ struct GemmArgs {
   const uint16_t* A;
   int64_t lda;
   const u32x4* Bp;  // fragment-packed B (see pack layout), already offset to the first K block of this GEMM
-  int64_t kb_total; // 16-wide K blocks per 32-row block of the packed buffer
+  int64_t kb_total; // 32-wide K blocks per 16-row block of the packed buffer
   int M, N, K;  // K is a multiple of BK; rows beyond M are clamped on load and masked by the epilogue
   int tiles_m, tiles_n;
   int splits;  // K is cut into `splits` runs of K-steps; run s is tile column tn + s * tiles_n of the raster
@@ -98,7 +90,7 @@ struct TileCoord {
 // which keeps a strip's B-tiles hot across the 8 XCDs.  (Sweeping N fastest instead, which would stream the big
 // operand from memory once rather than once per strip, measured 4 % slower forward and 8-17 % slower backward GEMMs
 // at T=16384, H=3584, V=152064: the L2 reuse inside a strip matters more than the bytes from memory.)
-constexpr int kXcd = 8, kBlkM = 8 * 256 / BM, kBlkN = 4;
+constexpr int kXcd = 8, kBlkM = 8, kBlkN = 4;
 __host__ __device__ inline int64_t raster_grid(int tiles_m, int tiles_n) {
   const int64_t blocks = (int64_t)((tiles_m + kBlkM - 1) / kBlkM) * ((tiles_n + kBlkN - 1) / kBlkN);
   return (blocks + kXcd - 1) / kXcd * kXcd * (kBlkM * kBlkN);
@@ -112,12 +104,12 @@ __device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int id) {
   return {tm, tn, tm < g.tiles_m && tn < g.tiles_n * g.splits};
 }
 
-// Accumulator coordinates of lane `lane` in wave (wm, wn): element r of acc[i][j] is
-//   row = wm*MI*32 + i*32 + (r/4)*8 + (lane/32)*4 + r%4 ,  col = wn*NJ*32 + j*32 + lane%32   (tile-relative)
+// Accumulator coordinates of lane `lane` in wave (wm, wn): element r (0..3) of acc[i][j] is
+//   row = wm*128 + i*16 + (lane/16)*4 + r ,  col = wn*64 + j*16 + lane%16   (tile-relative)
 __device__ __forceinline__ int acc_row(int wm, int i, int r, int lane) {
-  return wm * (MI * 32) + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+  return wm * (MI * 16) + i * 16 + (lane >> 4) * 4 + r;
 }
-__device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (NJ * 32) + j * 32 + (lane & 31); }
+__device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (NJ * 16) + j * 16 + (lane & 15); }
 
 // m0 (the DMA's LDS base) is a reserved register: naming it in a clobber list is right but draws a warning
 #pragma clang diagnostic push
@@ -125,7 +117,6 @@ __device__ __forceinline__ int acc_col(int wn, int j, int lane) { return wn * (N
 // F16: the 16-bit operands are IEEE half instead of bf16 (the same data movement, the other MFMA)
 template <class Epi, bool AT = false, bool F16 = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void gemm_nt_kernel(GemmArgs g, Epi epi) {
-  static_assert(!AT || (BM == 256 && WN == 4), "the K-major-rows form of A is written for the 256-row tile and 8 waves");
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int wm = w / WN, wn = w % WN;
@@ -166,22 +157,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
     }
   }
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
-  // B: fragment-packed, one 16-byte load per lane per MFMA operand, no LDS
+  // B: fragment-packed, one 16-byte load per lane per MFMA operand, no LDS.  N-tile j of the wave, K slice s of the
+  // K-step: chunk ((n0 / 16 + wn * NJ + j) * kb_total + kt * KS + s) * 64 + lane.
   const char* gB =
-      reinterpret_cast<const char*>(g.Bp + ((int64_t)(n0 >> 5) * g.kb_total + (int64_t)kt_first * (BK / 16)) * 64);
+      reinterpret_cast<const char*>(g.Bp + ((int64_t)(n0 >> 4) * g.kb_total + (int64_t)kt_first * KS) * 64);
   uint32_t offB[NJ];
 #pragma unroll
   for (int j = 0; j < NJ; ++j) offB[j] = (uint32_t)(((wn * NJ + j) * g.kb_total * 64 + lane) * 16);
 
-  floatx16 acc[MI][NJ];
+  floatx4 acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < NJ; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
-  u32x4 b0[NJ][BK / 16], b1[NJ][BK / 16];
+  u32x4 b0[NJ][KS], b1[NJ][KS];
   auto dma = [&](int stage, int kt, int i0 = 0, int i1 = kDmaPerWave) {
     const char* base = gA + (int64_t)kt * a_step;
 #pragma unroll
@@ -190,26 +182,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(dst), "v"(offA[i]), "s"(base) : "m0", "memory");
     }
   };
-  auto bload = [&](u32x4 (&b)[NJ][BK / 16], int kt, int j) {
-    const char* base = gB + (int64_t)kt * (BK / 16 * 1024);
+  auto bload = [&](u32x4 (&b)[NJ][KS], int kt, int j) {
+    const char* base = gB + (int64_t)kt * (KS * 1024);
     asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(b[j][0]) : "v"(offB[j]), "s"(base));
     asm volatile("global_load_dwordx4 %0, %1, %2 offset:1024" : "=v"(b[j][1]) : "v"(offB[j]), "s"(base));
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:2048" : "=v"(b[j][2]) : "v"(offB[j]), "s"(base));
-    asm volatile("global_load_dwordx4 %0, %1, %2 offset:3072" : "=v"(b[j][3]) : "v"(offB[j]), "s"(base));
   };
   // waits until only this wave's last kDmaPerWave loads (one stage of DMA) are in flight and ties the B registers
-  // to the wait (at most 30 asm operands: the registers of N-tiles 2 and 3 are tied by a second, empty statement)
-  static_assert((NJ == 2 || NJ == 4) && BK == 64 && kDmaPerWave % 2 == 0, "see the load schedule of a K-step");
-  auto bwait = [&](u32x4 (&b)[NJ][BK / 16]) {
+  // to the wait
+  static_assert(NJ * KS == 8 && kDmaPerWave % 2 == 0, "see the load schedule of a K-step");
+  auto bwait = [&](u32x4 (&b)[NJ][KS]) {
     asm volatile("s_waitcnt vmcnt(%[n])"
-                 : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[0][2]), "+v"(b[0][3]), "+v"(b[1][0]), "+v"(b[1][1]),
-                   "+v"(b[1][2]), "+v"(b[1][3])
+                 : "+v"(b[0][0]), "+v"(b[0][1]), "+v"(b[1][0]), "+v"(b[1][1]), "+v"(b[2][0]), "+v"(b[2][1]),
+                   "+v"(b[3][0]), "+v"(b[3][1])
                  : [n] "n"(kDmaPerWave)
                  : "memory");
-    if constexpr (NJ == 4)
-      asm volatile(""
-                   : "+v"(b[NJ - 2][0]), "+v"(b[NJ - 2][1]), "+v"(b[NJ - 2][2]), "+v"(b[NJ - 2][3]), "+v"(b[NJ - 1][0]),
-                     "+v"(b[NJ - 1][1]), "+v"(b[NJ - 1][2]), "+v"(b[NJ - 1][3])::"memory");
   };
 
 #pragma unroll
@@ -220,64 +206,69 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
   bwait(b0);
   __syncthreads();
 
-  // A fragments.  AT = false: lane (m = lane % 32, k-group lane / 32) reads its 8 consecutive K entries as one
-  // 16-byte chunk of row m.  AT = true: the stage holds K-rows, so the 8 entries come from two transposing reads
-  // (ds_read_b64_tr_b16): in each block of 16 lanes, lane 4 e + c addresses the 8 bytes of K-row e, M-chunk c, and
-  // receives the entries of K-rows 0..3 at M = its own index in the block.
-  const int m31 = lane & 31, gsel = lane >> 5, sw = (m31 >> 1) & 7;
-  const int frag_row = (wm * (MI * 32) + m31) * kRowBytes;
-  int xk[BK / 16];
+  // A fragments of MFMA group gq = 2 * s + hf: K slice s (32 columns), row blocks hf * 4 .. hf * 4 + 3 of the wave's
+  // eight 16-row blocks.  AT = false: lane (m = lane % 16, 8-column chunk lane / 16 of the slice) reads its 8
+  // consecutive K entries as one 16-byte chunk of row m.  AT = true: the stage holds K-rows, so the 8 entries come
+  // from two transposing reads (ds_read_b64_tr_b16): in each block of 16 lanes, lane 4 e + c addresses the 8 bytes of
+  // K-row e, M-chunk c, and receives the entries of K-rows 0..3 at M = its own index in the block; block lane / 16
+  // takes the 8 K-rows lane / 16 * 8 .. + 7 of the slice.
+  const int m15 = lane & 15, kq = lane >> 4, sw = m15 >> 1;
+  const int frag_row = (wm * (MI * 16) + m15) * kRowBytes;
+  int xk[KS];
 #pragma unroll
-  for (int kk = 0; kk < BK / 16; ++kk) xk[kk] = frag_row + (((kk * 2 + gsel) ^ sw) << 4);
-  const int tq = (lane & 15) >> 2, tmb = (lane >> 4) & 1;
-  const int xt0 = (gsel * 8 + tq) * 512 + wm * 256 + (lane & 3) * 8 + ((tmb ^ tq) << 5);  // M-tiles 0 and 2
-  const int xt1 = xt0 ^ 64;                                                                // M-tiles 1 and 3
+  for (int s = 0; s < KS; ++s) xk[s] = frag_row + (((s * 4 + kq) ^ sw) << 4);
+  const int tq = m15 >> 2;
+  const int xt0 = (kq * 8 + tq) * 512 + wm * 256 + (lane & 3) * 8 + (tq << 5);  // row block ii: xt0 ^ (ii << 5)
 
   // step kt: stage kt % 4 is read; B(kt + 1) and DMA(kt + 3) are issued (K-steps past the end are clamped to the
   // last one: they land in stages that are not read again); the barrier at the end publishes stage
   // (kt + 2) % 4, whose DMA was issued one step earlier, and frees stage kt % 4 for DMA(kt + 4).
-  // A fragments are read one MFMA K-slice ahead; the slice after the last one of a step is the first of the next
+  // A fragments are read one MFMA group ahead; the group after the last one of a step is the first of the next
   // step, whose stage was published by the previous barrier, so the reads cross the barrier.
-  bf16x8 afa[MI], afb[MI];
-  auto fread = [&](bf16x8 (&af)[MI], int stage, int kk) {
+  bf16x8 afa[4], afb[4];
+  auto fread = [&](bf16x8 (&af)[4], int stage, int gq) {
     const char* cur = smem + stage * kStageBytes;
+    const int s = gq >> 1, hf = gq & 1;
     if constexpr (AT) {
       typedef short s16x4 __attribute__((ext_vector_type(4)));
-      typedef short s16x8 __attribute__((ext_vector_type(8)));
       typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
 #pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        const char* at = cur + ((i & 1) ? xt1 : xt0) + kk * (16 * 512) + (i >> 1) * 128;
+      for (int ii = 0; ii < 4; ++ii) {
+        const char* at = cur + (xt0 ^ (ii << 5)) + s * (32 * 512) + hf * 128;
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(at + 4 * 512));
-        af[i] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        af[ii] = __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < MI; ++i) af[i] = *reinterpret_cast<const bf16x8*>(cur + xk[kk] + i * 32 * kRowBytes);
+      for (int ii = 0; ii < 4; ++ii)
+        af[ii] = *reinterpret_cast<const bf16x8*>(cur + xk[s] + (hf * 4 + ii) * 16 * kRowBytes);
     }
   };
-  auto mma = [&](bf16x8 (&af)[MI], u32x4 (&bc)[NJ][BK / 16], int kk) {
+  auto mma = [&](bf16x8 (&af)[4], u32x4 (&bc)[NJ][KS], int gq) {
+    const int s = gq >> 1, hf = gq & 1;
 #pragma unroll
-    for (int i = 0; i < MI; ++i)
+    for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
-      for (int j = 0; j < NJ; ++j)
+      for (int j = 0; j < NJ; ++j) {
+        floatx4& c = acc[hf * 4 + ii][j];
         if constexpr (F16)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, af[i]), __builtin_bit_cast(f16x8, bc[j][kk]),
-                                                             acc[i][j], 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[ii]), __builtin_bit_cast(f16x8, bc[j][s]), c, 0, 0, 0);
         else
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], __builtin_bit_cast(bf16x8, bc[j][kk]), acc[i][j], 0, 0, 0);
+          c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[ii], __builtin_bit_cast(bf16x8, bc[j][s]), c, 0, 0, 0);
+      }
   };
   fread(afa, 0, 0);
-  // One K-step.  The vector-memory instructions (12 with 8 waves) are spread over the step (B for one N-tile before each of the
-  // first two MFMA groups, half of the DMA before each of the last two) instead of being issued in one burst, and
-  // the wave raises its priority while it issues MFMAs so that its SIMD partner's loads do not delay them.
-  auto mma_prio = [&](bf16x8 (&af)[MI], u32x4 (&bc)[NJ][BK / 16], int kk) {
+  // One K-step: four groups of 16 MFMAs.  The 12 vector-memory instructions are spread over the step (B for two
+  // N-tiles before each of the first two groups, half of the DMA before each of the last two) instead of being issued
+  // in one burst, and the wave raises its priority while it issues MFMAs so that its SIMD partner's loads do not
+  // delay them.
+  auto mma_prio = [&](bf16x8 (&af)[4], u32x4 (&bc)[NJ][KS], int gq) {
     __builtin_amdgcn_s_setprio(1);
-    mma(af, bc, kk);
+    mma(af, bc, gq);
     __builtin_amdgcn_s_setprio(0);
   };
-  auto step = [&](int kt, u32x4 (&bc)[NJ][BK / 16], u32x4 (&bn)[NJ][BK / 16]) {
+  auto step = [&](int kt, u32x4 (&bc)[NJ][KS], u32x4 (&bn)[NJ][KS]) {
     const int stage = kt & 3;
     const int ktb = kt + 1 < KT ? kt + 1 : KT - 1, kta = kt + 3 < KT ? kt + 3 : KT - 1;
 #pragma unroll
@@ -312,22 +303,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
 
 // ------------------------------------------------------------------------------ parked accumulator tiles
 
-// Tile (tm, tn) of the forward GEMM occupies kQuads * kThreads 16-byte slots; slot c * kThreads + tid holds
-// elements 4q .. 4q + 3 of thread tid's acc[i][j], c = (i * NJ + j) * 4 + q.  A wave instruction therefore moves
-// one contiguous KB, and the tile can be handed to any epilogue exactly as the main loop would have left it.
+// Tile (tm, tn) of the forward GEMM occupies kQuads * kThreads 16-byte slots; slot c * kThreads + tid holds thread
+// tid's acc[i][j] (four registers), c = i * NJ + j.  A wave instruction therefore moves one contiguous KB, and the
+// tile can be handed to any epilogue exactly as the main loop would have left it.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
-constexpr int kQuads = MI * NJ * 4;
+constexpr int kQuads = MI * NJ;
 constexpr int64_t kSavedTileBytes = (int64_t)kQuads * kThreads * 16;  // BM * BN * 4
 __device__ __forceinline__ f32x4* saved_tile(float* base, int tm, int tn, int tiles_n) {
   return reinterpret_cast<f32x4*>(base) + ((int64_t)tm * tiles_n + tn) * (kQuads * kThreads);
 }
 
 // Runs an epilogue over parked tiles: workgroup b takes tile (tm_first + b / tiles_n, b % tiles_n) and calls the
-// epilogue with vocabulary row m0 counted from the first tile row of the launch.  (Measured at T=16384, V=152064:
-// 0.87 ms per 32768 columns (launches take 65536), 4.9 TB/s of its 8 bytes per logit, arithmetic and LDS writes about level with the
-// memory time; splitting the workgroup into its two rows of waves, each with half the LDS image so that two share
-// a CU, was 15 % slower, and 256 persistent workgroups that issue the next tile's loads before draining the LDS
-// image were 17-27 % slower, with full barriers or with barriers that order the LDS only.)
+// epilogue with vocabulary row m0 counted from the first tile row of the launch.
 template <class Epi>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd, kWavesPerSimd))) void replay_tiles_kernel(
     const float* __restrict__ saved, int tiles_n, int tm_first, Epi epi) {
@@ -336,19 +323,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
   const int wm = w / WN, wn = w % WN;
   const int tml = blockIdx.x / tiles_n, tn = blockIdx.x - tml * tiles_n;
   const f32x4* src = saved_tile(const_cast<float*>(saved), tm_first + tml, tn, tiles_n) + tid;
-  floatx16 acc[MI][NJ];
+  floatx4 acc[MI][NJ];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < NJ; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const f32x4 v = __builtin_nontemporal_load(src + ((i * NJ + j) * 4 + q) * kThreads);
-        acc[i][j][q * 4] = v.x;
-        acc[i][j][q * 4 + 1] = v.y;
-        acc[i][j][q * 4 + 2] = v.z;
-        acc[i][j][q * 4 + 3] = v.w;
-      }
+    for (int j = 0; j < NJ; ++j) acc[i][j] = __builtin_nontemporal_load(src + (i * NJ + j) * kThreads);
   epi(acc, tml * BM, tn * BN, tml, 0, wm, wn, lane, tid, smem);
 }
 
@@ -356,8 +335,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
 
 // The two fused GEMMs run "transposed": M is the vocabulary (A = W), N the tokens (B = hidden).  In the MFMA
 // accumulator layout a lane then owns one token (column) and its registers run over vocabulary rows, so the
-// softmax reductions over the vocabulary are in-register, followed by one exchange between the two lane halves
-// and a merge of the WM waves through LDS -- no 32-lane butterfly per row.
+// softmax reductions over the vocabulary are in-register, followed by two exchanges between the four lanes that
+// share a token and a merge of the WM waves through LDS -- no 16-lane butterfly per row.
 //
 // Per token of the tile: mx = max_v z, s = sum exp(z - mx), t = sum z * exp(z - mx) over the tile's 256
 // vocabulary rows, z = acc * inv_T; one (mx, s, t) per token is written to part[tm][.][token].
@@ -367,22 +346,15 @@ struct SoftmaxPartialsEpi {
   float* part;  // [tiles_m][3][T]
   float* save;  // null, or the parked accumulator tiles (see saved_tile)
   int tiles_n;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
+  __device__ __forceinline__ void operator()(floatx4 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
                                              int lane, int tid, char* smem) const {
-    // Parking costs about 11 us per tile (256 KB per workgroup).  Starting the first workgroup of each CU in one of
-    // eight phases of a tile's duration, so that the stores of a round do not arrive together, changed nothing:
-    // the time is the workgroup's own drain, not a burst.  Non-temporal stores measured the same as plain ones.
+    // Parking costs about 11 us per tile (256 KB per workgroup): the workgroup's own drain, not a burst of the round.
     if (save) {
       f32x4* dst = saved_tile(save, tm, n0 / BN, tiles_n) + tid;
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int j = 0; j < NJ; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const f32x4 v = {acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]};
-            dst[((i * NJ + j) * 4 + q) * kThreads] = v;
-          }
+        for (int j = 0; j < NJ; ++j) dst[(i * NJ + j) * kThreads] = acc[i][j];
     }
     float* sh = reinterpret_cast<float*>(smem);  // [WM][BN][3]; the main loop's last barrier freed the LDS
     const float k = kLog2e;
@@ -394,10 +366,11 @@ struct SoftmaxPartialsEpi {
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
+        for (int r = 0; r < 4; ++r) {
           const bool ok = full || (m0 + acc_row(wm, i, r, lane) < V);
           mx = fmaxf(mx, ok ? acc[i][j][r] * inv_T : ninf);
         }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
       float s = 0.f, t = 0.f;
       if (mx > ninf) {
@@ -405,7 +378,7 @@ struct SoftmaxPartialsEpi {
 #pragma unroll
         for (int i = 0; i < MI; ++i)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
+          for (int r = 0; r < 4; ++r) {
             const bool ok = full || (m0 + acc_row(wm, i, r, lane) < V);
             const float x = acc[i][j][r] * inv_T;
             const float e = ok ? fast_exp2(fmaf(x, k, nmk)) : 0.f;
@@ -413,9 +386,11 @@ struct SoftmaxPartialsEpi {
             t = fmaf(ok ? x : 0.f, e, t);
           }
       }
+      s += __shfl_xor(s, 16, kWave);
+      t += __shfl_xor(t, 16, kWave);
       s += __shfl_xor(s, 32, kWave);
       t += __shfl_xor(t, 32, kWave);
-      if (lane < 32) {
+      if (lane < 16) {
         float* d = sh + (wm * BN + acc_col(wn, j, lane)) * 3;
         d[0] = mx;
         d[1] = s;
@@ -468,7 +443,7 @@ struct DlogitsEpi {
   // two fused multiply-adds, one exp2 and one multiply per logit.  FULL: every vocabulary row of the tile is inside
   // the slab.
   template <bool FULL>
-  __device__ __forceinline__ void tile(floatx16 (&acc)[MI][NJ], int m0, int n0, int wm, int wn, int lane) const {
+  __device__ __forceinline__ void tile(floatx4 (&acc)[MI][NJ], int m0, int n0, int wm, int wn, int lane) const {
     const float ek = inv_T * kLog2e;
 #pragma unroll
     for (int j = 0; j < NJ; ++j) {
@@ -486,24 +461,23 @@ struct DlogitsEpi {
       }
       uint16_t* drow = D + (int64_t)tok * ldd;
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+      for (int i = 0; i < MI; ++i) {
+        const int v = m0 + acc_row(wm, i, 0, lane);  // 4 consecutive vocabulary rows of the slab
+        float d[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int v = m0 + acc_row(wm, i, q * 4, lane);  // 4 consecutive vocabulary rows of the slab
-          float d[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float a = acc[i][j][q * 4 + e];
-            const float p = fast_exp2(fmaf(a, ek, nl));
-            float g = p * fmaf(a, c1, c0);
-            if (v + e == y) g += cy;
-            d[e] = (FULL || v + e < Vs) ? g : 0.f;
-          }
-          if (FULL || v < Vpad) *reinterpret_cast<uint2*>(drow + v) = make_uint2(pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3]));
+        for (int e = 0; e < 4; ++e) {
+          const float a = acc[i][j][e];
+          const float p = fast_exp2(fmaf(a, ek, nl));
+          float g = p * fmaf(a, c1, c0);
+          if (v + e == y) g += cy;
+          d[e] = (FULL || v + e < Vs) ? g : 0.f;
         }
+        // the four lanes that share the token hold 16 consecutive rows: 32 contiguous bytes per token and store
+        if (FULL || v < Vpad) *reinterpret_cast<uint2*>(drow + v) = make_uint2(pack_bf16(d[0], d[1]), pack_bf16(d[2], d[3]));
+      }
     }
   }
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
+  __device__ __forceinline__ void operator()(floatx4 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn,
                                              int lane, int tid, char* smem) const {
     if (m0 + BM <= Vs)
       tile<true>(acc, m0, n0, wm, wn, lane);
@@ -518,12 +492,12 @@ struct AccumF32Epi {  // C_s[row][col] = (beta ? C_s : 0) + acc, one fp32 buffer
   float* C;
   int64_t ldc, split_stride;
   int M, N, beta;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn, int lane, int tid,
+  __device__ __forceinline__ void operator()(floatx4 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn, int lane, int tid,
                              char* smem) const {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int r = 0; r < 4; ++r) {
         const int row = m0 + acc_row(wm, i, r, lane);
         if (row >= M) continue;
 #pragma unroll
@@ -541,12 +515,12 @@ struct StoreEpi {  // C[row][col] = acc, rounded to the output type (out_dtype: 
   void* C;
   int64_t ldc;
   int M, N, out_dtype;
-  __device__ __forceinline__ void operator()(floatx16 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn, int lane, int tid,
+  __device__ __forceinline__ void operator()(floatx4 (&acc)[MI][NJ], int m0, int n0, int tm, int split, int wm, int wn, int lane, int tid,
                              char* smem) const {
 #pragma unroll
     for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
+      for (int r = 0; r < 4; ++r) {
         const int row = m0 + acc_row(wm, i, r, lane);
         if (row >= M) continue;
 #pragma unroll
@@ -567,9 +541,9 @@ struct StoreEpi {  // C[row][col] = acc, rounded to the output type (out_dtype: 
 
 // ------------------------------------------------------------------------------ small kernels
 
-// Fragment-packed B operand.  For a K-major matrix B[n][k] the packed buffer holds, for each block of 32 rows nb
-// and each block of 16 columns kb, the 64 x 16 bytes that one 32x32x16 MFMA takes as its B operand, in lane order:
-//   chunk index ((nb * KB + kb) * 64 + l),  l = (n % 32) + 32 * ((k % 16) / 8),  8 consecutive k per chunk.
+// Fragment-packed B operand.  For a K-major matrix B[n][k] the packed buffer holds, for each block of 16 rows nb
+// and each block of 32 columns kb, the 64 x 16 bytes that one 16x16x32 MFMA takes as its B operand, in lane order:
+//   chunk index ((nb * KB + kb) * 64 + l),  l = (n % 16) + 16 * ((k % 32) / 8),  8 consecutive k per chunk.
 // Rows n >= N and columns k >= K are zero.  One thread per chunk.
 __global__ __launch_bounds__(256) void pack_b_kernel(const uint16_t* __restrict__ in, int64_t ld_in, int N, int K,
                                                      u32x4* __restrict__ out, int64_t KB, int64_t chunks) {
@@ -577,7 +551,7 @@ __global__ __launch_bounds__(256) void pack_b_kernel(const uint16_t* __restrict_
   if (ch >= chunks) return;
   const int l = (int)(ch & 63);
   const int64_t blk = ch >> 6, kb = blk % KB, nb = blk / KB;
-  const int64_t n = nb * 32 + (l & 31), k = kb * 16 + (l >> 5) * 8;
+  const int64_t n = nb * 16 + (l & 15), k = kb * 32 + (l >> 4) * 8;
   u32x4 v = {0u, 0u, 0u, 0u};
   if (n < N && k < K) v = *reinterpret_cast<const u32x4*>(in + n * ld_in + k);  // K % 8 == 0
   out[ch] = v;
@@ -617,7 +591,7 @@ __global__ __launch_bounds__(256) void transpose_pack_b_kernel(const uint16_t* _
 #pragma unroll
     for (int e = 0; e < 4; ++e) w[e] = (uint32_t)tile[kc * 8 + 2 * e][nl] | ((uint32_t)tile[kc * 8 + 2 * e + 1][nl] << 16);
     const int64_t n = c0 + nl, k = r0 + kc * 8;
-    const int64_t ch = ((n >> 5) * KB + (k >> 4)) * 64 + (n & 31) + 32 * ((k >> 3) & 1);
+    const int64_t ch = ((n >> 4) * KB + (k >> 5)) * 64 + (n & 15) + 16 * ((k >> 3) & 3);
     out[ch] = u32x4{w[0], w[1], w[2], w[3]};
   }
 }
@@ -844,7 +818,7 @@ __global__ __launch_bounds__(256) void zero_fill_kernel(u32x4* __restrict__ p, i
 
 int pack_hidden(const uint16_t* h, int64_t T, int64_t H, u32x4* out, hipStream_t st) {
   const int64_t chunks = round_up(T, BN) * H / 8;
-  pack_b_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(h, H, (int)T, (int)H, out, H / 16, chunks);
+  pack_b_kernel<<<dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st>>>(h, H, (int)T, (int)H, out, H / 32, chunks);
   SIIRL_LAUNCH_CHECK("pack_b_kernel");
   return SIIRL_OK;
 }
@@ -960,9 +934,9 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   u32x4* hp = reinterpret_cast<u32x4*>((char*)workspace + ws.hp);
   if (int rc = pack_hidden(h, T, Kc, hp, st)) return rc;
   SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part, saved_logits, (int)((T + BN - 1) / BN)};
-  if (int rc = f16 ? launch_gemm<SoftmaxPartialsEpi, false, true>(w, Kc, hp, Kc / 16, (int)V, (int)T, (int)Kc, epi, st,
+  if (int rc = f16 ? launch_gemm<SoftmaxPartialsEpi, false, true>(w, Kc, hp, Kc / 32, (int)V, (int)T, (int)Kc, epi, st,
                                                                   "gemm_nt_kernel<SoftmaxPartialsEpi, f16>")
-                   : launch_gemm(w, Kc, hp, Kc / 16, (int)V, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>"))
+                   : launch_gemm(w, Kc, hp, Kc / 32, (int)V, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>"))
     return rc;
   const int tiles_v = (int)((V + BM - 1) / BM);
   merge_partials_kernel<<<dim3((unsigned)((T + kMergeTok - 1) / kMergeTok)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
@@ -1015,12 +989,12 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
     if (int rc = pack_hidden(h, T, Kc, hp, st)) return rc;
   if (want_dh) {
     transpose_pack_b_kernel<<<dim3((unsigned)(ws.ldwt / 64), (unsigned)(ws.hpad / 64)), dim3(256), 0, st>>>(
-        w, Kc, (int)V, (int)H, Wtp, ws.ldwt / 16, (int)f16);
+        w, Kc, (int)V, (int)H, Wtp, ws.ldwt / 32, (int)f16);
     SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(W)");
   }
   if (want_dw) {
     transpose_pack_b_kernel<<<dim3((unsigned)(ws.ldt / 64), (unsigned)(ws.hpad / 64)), dim3(256), 0, st>>>(
-        h, Kc, (int)T, (int)H, Htp, ws.ldt / 16, (int)f16);
+        h, Kc, (int)T, (int)H, Htp, ws.ldt / 32, (int)f16);
     SIIRL_LAUNCH_CHECK("transpose_pack_b_kernel(hidden)");
   }
   if (want_dw && ws.ldt > T) {  // the token rows that only pad the K of the d-weight GEMM (ldd_row * 2 % 16 == 0)
@@ -1040,9 +1014,9 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
     if (!saved_logits) {
       DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
                      D + (int64_t)gs * kSlab, ws.ldd_row};
-      if (int rc = f16 ? launch_gemm<DlogitsEpi, false, true>(w + v0 * Kc, Kc, hp, Kc / 16, N, (int)T, (int)Kc, epi, st,
+      if (int rc = f16 ? launch_gemm<DlogitsEpi, false, true>(w + v0 * Kc, Kc, hp, Kc / 32, N, (int)T, (int)Kc, epi, st,
                                                               "gemm_nt_kernel<DlogitsEpi, f16>")
-                       : launch_gemm(w + v0 * Kc, Kc, hp, Kc / 16, N, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<DlogitsEpi>"))
+                       : launch_gemm(w + v0 * Kc, Kc, hp, Kc / 32, N, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<DlogitsEpi>"))
         return rc;
     } else if (gs == 0) {
       // the whole group's dlogits in one pass over the tiles the forward parked
@@ -1066,7 +1040,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
       if (g0 == 0) dh_splits = pick_splits((int)T, (int)H, K);
       const int splits = (K / BK >= 2) ? dh_splits : 1;
       AccumF32Epi acc{dH32, H, dh32_stride, (int)T, (int)H, g0 > 0 ? 1 : 0};
-      if (int rc = launch_gemm(D, ws.ldd_row, Wtp + (g0 / 16) * 64, ws.ldwt / 16, (int)T, (int)H, K, acc, st,
+      if (int rc = launch_gemm(D, ws.ldd_row, Wtp + (g0 / 32) * 64, ws.ldwt / 32, (int)T, (int)H, K, acc, st,
                                "gemm_nt_kernel<AccumF32Epi>", splits))
         return rc;
     }
@@ -1076,7 +1050,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
       const int64_t g0 = v0 - (int64_t)gs * kSlab;
       const int M = gs * kSlab + N;
       StoreEpi sto{(char*)d_weight + g0 * H * (int64_t)dtype_size(dtype), H, M, (int)H, dtype};
-      if (int rc = launch_gemm<StoreEpi, true>(D, ws.ldd_row, Htp, ws.ldt / 16, M, (int)H, (int)ws.ldt, sto, st,
+      if (int rc = launch_gemm<StoreEpi, true>(D, ws.ldd_row, Htp, ws.ldt / 32, M, (int)H, (int)ws.ldt, sto, st,
                                                "gemm_nt_kernel<StoreEpi, A by K-rows>"))
         return rc;
     }

@@ -76,6 +76,7 @@ struct GemmArgs {
   int M, N, K;  // K is a multiple of BK; rows beyond M are clamped on load and masked by the epilogue
   int tiles_m, tiles_n;
   int splits;  // K is cut into `splits` runs of K-steps; run s is tile column tn + s * tiles_n of the raster
+  int blk_m;   // tiles along M of an XCD's block of 32 tiles
 };
 
 struct TileCoord {
@@ -84,23 +85,25 @@ struct TileCoord {
 };
 // XCD-aware rasterisation.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2, so
 // workgroup id runs on XCD id % 8 as that XCD's (id / 8)-th workgroup.  The tile grid is cut into blocks of
-// kBlkM x kBlkN tiles (32 tiles: one XCD's resident set); block b goes to XCD b % 8 and its tiles to 32
-// consecutive workgroups of that XCD, so the workgroups sharing an L2 at any time share 8 A-tiles and 4
-// B-tiles instead of streaming 32 different A-tiles.  Blocks sweep M fastest inside a strip of kBlkN N-tiles,
-// which keeps a strip's B-tiles hot across the 8 XCDs.  (Sweeping N fastest instead, which would stream the big
+// blk_m x blk_n tiles (32 tiles: one XCD's resident set; blk_m is the launch's choice among 2, 4, 8, 16); block b
+// goes to XCD b % 8 and its tiles to 32 consecutive workgroups of that XCD, so the workgroups sharing an L2 at any
+// time share blk_m A-tiles and blk_n B-tiles instead of streaming 32 different A-tiles.  Blocks sweep M fastest
+// inside a strip of blk_n N-tiles, which keeps a strip's B-tiles hot across the 8 XCDs.  (Sweeping N fastest instead, which would stream the big
 // operand from memory once rather than once per strip, measured 4 % slower forward and 8-17 % slower backward GEMMs
 // at T=16384, H=3584, V=152064: the L2 reuse inside a strip matters more than the bytes from memory.)
-constexpr int kXcd = 8, kBlkM = 8, kBlkN = 4;
-__host__ __device__ inline int64_t raster_grid(int tiles_m, int tiles_n) {
-  const int64_t blocks = (int64_t)((tiles_m + kBlkM - 1) / kBlkM) * ((tiles_n + kBlkN - 1) / kBlkN);
-  return (blocks + kXcd - 1) / kXcd * kXcd * (kBlkM * kBlkN);
+constexpr int kXcd = 8, kBlkTiles = 32;
+__host__ __device__ inline int64_t raster_grid(int tiles_m, int tiles_n, int blk_m) {
+  const int blk_n = kBlkTiles / blk_m;
+  const int64_t blocks = (int64_t)((tiles_m + blk_m - 1) / blk_m) * ((tiles_n + blk_n - 1) / blk_n);
+  return (blocks + kXcd - 1) / kXcd * kXcd * kBlkTiles;
 }
 __device__ __forceinline__ TileCoord tile_of(const GemmArgs& g, int id) {
+  const int blk_m = g.blk_m, blk_n = kBlkTiles / blk_m;
   const int xcd = id % kXcd, l = id / kXcd;
-  const int blk = (l / (kBlkM * kBlkN)) * kXcd + xcd, j = l % (kBlkM * kBlkN);
-  const int mb = (g.tiles_m + kBlkM - 1) / kBlkM;
-  const int tm = (blk % mb) * kBlkM + j % kBlkM;
-  const int tn = (blk / mb) * kBlkN + j / kBlkM;
+  const int blk = (l / kBlkTiles) * kXcd + xcd, j = l % kBlkTiles;
+  const int mb = (g.tiles_m + blk_m - 1) / blk_m;
+  const int tm = (blk % mb) * blk_m + j % blk_m;
+  const int tn = (blk / mb) * blk_n + j / blk_m;
   return {tm, tn, tm < g.tiles_m && tn < g.tiles_n * g.splits};
 }
 
@@ -250,7 +253,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWaves
 #pragma unroll
     for (int ii = 0; ii < 4; ++ii)
 #pragma unroll
-      for (int j = 0; j < NJ; ++j) {
+      for (int jj = 0; jj < NJ; ++jj) {
+        // boustrophedon over the N-tiles: consecutive MFMAs always share one operand (0.5-0.8 % faster at T=16384,
+        // H=3584, V=152064 than restarting at N-tile 0 for every row block: fewer operand wires toggle)
+        const int j = (ii & 1) ? NJ - 1 - jj : jj;
         floatx4& c = acc[hf * 4 + ii][j];
         if constexpr (F16)
           c = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, af[ii]), __builtin_bit_cast(f16x8, bc[j][s]), c, 0, 0, 0);
@@ -720,15 +726,22 @@ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 // AT: A is given by its K-rows (A[K][M], M contiguous, row pitch lda >= tiles_m * BM, K readable rows)
 template <class Epi, bool AT = false, bool F16 = false>
 int launch_gemm(const uint16_t* A, int64_t lda, const u32x4* Bp, int64_t kb_total, int M, int N, int K, const Epi& epi,
-                hipStream_t st, const char* what, int splits = 1) {
+                hipStream_t st, const char* what, int splits = 1, int blk_m = 8) {
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_nt_kernel<Epi, AT, F16>), kSmemBytes)) return rc;
-  GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN, splits};
+  GemmArgs g{A, lda, Bp, kb_total, M, N, K, (M + BM - 1) / BM, (N + BN - 1) / BN, splits, blk_m};
   if (AT && lda < (int64_t)g.tiles_m * BM) return fail(SIIRL_ERR_INVALID_ARGUMENT, "%s: row pitch %lld is shorter than %d tiles", what, (long long)lda, g.tiles_m);
-  const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n * splits);
+  const int64_t tiles = raster_grid(g.tiles_m, g.tiles_n * splits, blk_m);
   gemm_nt_kernel<Epi, AT, F16><<<dim3((unsigned)tiles), dim3(kThreads), kSmemBytes, st>>>(g, epi);
   SIIRL_LAUNCH_CHECK(what);
   return SIIRL_OK;
 }
+
+// Tiles along M of an XCD's block, per GEMM of the fused path.  Measured at T=16384, H=3584, V=152064 (ms per step
+// for blocks of 2 x 16 / 4 x 8 / 8 x 4 / 16 x 2 tiles): forward 13.34 / 13.32 / 13.67 / 15.16; recompute + dlogits
+// 13.97 / 14.17 / 14.30 / 14.90 (1 x 32: slower again); d hidden 13.49 / 13.31 / 13.50 / 13.74; d weight 13.77 /
+// 13.50 / 13.40 / 14.24.  The A operand of the first two is W, streamed from memory once per strip of blk_n token
+// tiles: wider strips read it less often.
+constexpr int kBlkFwd = 4, kBlkRecompute = 2, kBlkDHidden = 4, kBlkDWeight = 8;
 
 // Two K runs when that fills the 256 compute units' last round noticeably better (896 tiles = 3.5 rounds become
 // 1792 = 7) and the GEMM is deep enough for the second fp32 buffer's extra pass not to matter.
@@ -935,8 +948,9 @@ extern "C" int siirl_fused_linear_logprob_entropy_fwd(const void* hidden, const 
   if (int rc = pack_hidden(h, T, Kc, hp, st)) return rc;
   SoftmaxPartialsEpi epi{inv_temperature, (int)T, (int)V, part, saved_logits, (int)((T + BN - 1) / BN)};
   if (int rc = f16 ? launch_gemm<SoftmaxPartialsEpi, false, true>(w, Kc, hp, Kc / 32, (int)V, (int)T, (int)Kc, epi, st,
-                                                                  "gemm_nt_kernel<SoftmaxPartialsEpi, f16>")
-                   : launch_gemm(w, Kc, hp, Kc / 32, (int)V, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>"))
+                                                                  "gemm_nt_kernel<SoftmaxPartialsEpi, f16>", 1, kBlkFwd)
+                   : launch_gemm(w, Kc, hp, Kc / 32, (int)V, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<SoftmaxPartialsEpi>", 1,
+                                 kBlkFwd))
     return rc;
   const int tiles_v = (int)((V + BM - 1) / BM);
   merge_partials_kernel<<<dim3((unsigned)((T + kMergeTok - 1) / kMergeTok)), dim3(256), 0, st>>>(part, tiles_v, (int)T, label_logit,
@@ -1015,8 +1029,9 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
       DlogitsEpi epi{inv_temperature, (int)T, N, Npad, v0, lse, ex, g_logprob, g_entropy, labels,
                      D + (int64_t)gs * kSlab, ws.ldd_row};
       if (int rc = f16 ? launch_gemm<DlogitsEpi, false, true>(w + v0 * Kc, Kc, hp, Kc / 32, N, (int)T, (int)Kc, epi, st,
-                                                              "gemm_nt_kernel<DlogitsEpi, f16>")
-                       : launch_gemm(w + v0 * Kc, Kc, hp, Kc / 32, N, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<DlogitsEpi>"))
+                                                              "gemm_nt_kernel<DlogitsEpi, f16>", 1, kBlkRecompute)
+                       : launch_gemm(w + v0 * Kc, Kc, hp, Kc / 32, N, (int)T, (int)Kc, epi, st, "gemm_nt_kernel<DlogitsEpi>", 1,
+                                     kBlkRecompute))
         return rc;
     } else if (gs == 0) {
       // the whole group's dlogits in one pass over the tiles the forward parked
@@ -1041,7 +1056,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
       const int splits = (K / BK >= 2) ? dh_splits : 1;
       AccumF32Epi acc{dH32, H, dh32_stride, (int)T, (int)H, g0 > 0 ? 1 : 0};
       if (int rc = launch_gemm(D, ws.ldd_row, Wtp + (g0 / 32) * 64, ws.ldwt / 32, (int)T, (int)H, K, acc, st,
-                               "gemm_nt_kernel<AccumF32Epi>", splits))
+                               "gemm_nt_kernel<AccumF32Epi>", splits, kBlkDHidden))
         return rc;
     }
     if (want_dw && (gs == kDhGroup - 1 || v0 + kSlab >= V)) {
@@ -1051,7 +1066,7 @@ extern "C" int siirl_fused_linear_logprob_entropy_bwd(const void* hidden, const 
       const int M = gs * kSlab + N;
       StoreEpi sto{(char*)d_weight + g0 * H * (int64_t)dtype_size(dtype), H, M, (int)H, dtype};
       if (int rc = launch_gemm<StoreEpi, true>(D, ws.ldd_row, Htp, ws.ldt / 32, M, (int)H, (int)ws.ldt, sto, st,
-                                               "gemm_nt_kernel<StoreEpi, A by K-rows>"))
+                                               "gemm_nt_kernel<StoreEpi, A by K-rows>", 1, kBlkDWeight))
         return rc;
     }
   }

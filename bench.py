@@ -38,7 +38,7 @@ SEED = 20250602
 # rocprofv3 --pmc runs, FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what the same
 # counter reads for a plain 2 GiB device copy (FETCH_SIZE reads half the bytes fetched: factor 2.0;
 # WRITE_SIZE factor 1.0).  Figures and commands: profiles/lpe_config2_hbm_traffic.md
-MEASURED_TRAFFIC_BYTES = int((4872295.36 * 2.0 + 9733447.5) * 1024)
+MEASURED_TRAFFIC_BYTES = int((4872246.35 * 2.0 + 9733599.87) * 1024)
 # The same for loss_partials_kernel + loss_bwd_kernel at config 3 with 5488 kept trajectories
 # (profiles/loss_path_config3_hbm_traffic.md)
 MEASURED_TRAFFIC_BYTES_CONFIG3 = int(((526927.5 + 527223.3) * 2.0 + 1372.0 + 176093.0) * 1024)
@@ -100,6 +100,11 @@ def cpu_baseline(logits, labels, g_lp, g_ent, rows=4096, iters=5):
     return {"value": rows / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "cpu": cpu_model(), "kind": "port",
             "sample": f"first {rows} of {logits.shape[0]} rows of the same tensor, upcast to fp32; "
                       f"median of {iters} fwd+bwd passes ({med:.2f} s each)"}
+
+
+def gemm_rate(config5_line):
+    """TFLOP/s of the forward GEMM of a config 5 line."""
+    return next(v["TFLOP/s"] for k, v in config5_line["kernels"].items() if k.startswith("forward"))
 
 
 def bench_config3(args, dev, quick=False):
@@ -317,6 +322,33 @@ def bench_config5(args, dev, quick=False):
     wall, fwd_ms, bwd_ms = timed()
     gemm = 2.0 * T * H * V
     tf_step = 3 * gemm / (wall / steps) / 1e12
+
+    # yardstick: the vendor library's plain bf16 GEMMs (torch.mm -> hipBLASLt / rocBLAS) of the shapes and operand
+    # layouts of the fused path's GEMMs, no epilogue, results written out; reported beside the fused kernels' rates,
+    # never part of `value`
+    def mm_ms(a, b, out_shape, n=5):
+        with torch.no_grad():
+            out_buf = torch.empty(out_shape, dtype=torch.bfloat16, device=dev)
+            for _ in range(2):
+                torch.mm(a, b, out=out_buf)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(n):
+                torch.mm(a, b, out=out_buf)
+            e1.record()
+            torch.cuda.synchronize()
+            del out_buf
+        return e0.elapsed_time(e1) / n
+
+    Vg = 65536  # one group of dlogits columns, as the backward updates d hidden and d weight
+    with torch.no_grad():
+        dl = (torch.randn(T, Vg, device=dev, generator=gen) * 1e-3).to(torch.bfloat16)
+        lib_ms = mm_ms(w.detach(), h.detach().t(), (V, T))                 # logits^T = W . hidden^T
+        lib_dh_ms = mm_ms(dl, w.detach()[:Vg], (T, H))                     # d hidden += dlogits . W_group
+        lib_dw_ms = mm_ms(dl.t(), h.detach(), (Vg, H))                     # d weight_group = dlogits^T . hidden
+        del dl
+    torch.cuda.empty_cache()
     extras = {}
     if not quick:
         FL.set_saved_logits_limit(16 << 30)
@@ -380,6 +412,14 @@ def bench_config5(args, dev, quick=False):
         "kernels": {"forward (gemm_nt_kernel<SoftmaxPartialsEpi> + merge)": {"ms": fwd_ms, "TFLOP/s": gemm / fwd_ms / 1e9},
                     "backward (recompute + dlogits per slab, d hidden and d weight per 65536 columns)":
                         {"ms": bwd_ms, "TFLOP/s executed": 3 * gemm / bwd_ms / 1e9}},
+        "library_gemm_yardstick": {"what": f"torch.mm in bf16 through the vendor library, no epilogue: W [{V}, {H}] . "
+                                           f"hidden^T (the forward's and the recompute's GEMM), dlogits [{T}, {Vg}] . "
+                                           f"W[:{Vg}] (d hidden of one 65536-column group), dlogits^T . hidden (d weight "
+                                           "of one group)",
+                                   "ms": lib_ms, "TFLOP/s": gemm / lib_ms / 1e9,
+                                   "fused_forward_over_library": (gemm / fwd_ms / 1e9) / (gemm / lib_ms / 1e9),
+                                   "d_hidden_shape_TFLOP/s": 2.0 * T * H * Vg / lib_dh_ms / 1e9,
+                                   "d_weight_shape_TFLOP/s": 2.0 * T * H * Vg / lib_dw_ms / 1e9},
         **extras,
         "roofline": {"bound": "mfma", "kernel": "gemm_nt_kernel", "achieved": tf_step, "peak": 2500.0, "unit": "TFLOP/s",
                      "frac": tf_step / 2500.0, "traffic": None,
@@ -1348,6 +1388,9 @@ def main():
             out["configs"][name]["workload"] = r["config"]["workload"]
             out["configs"][name]["roofline"] = {k: r["roofline"][k] for k in ("bound", "kernel", "achieved", "peak", "unit", "frac")}
             out["configs"][name]["cpu_baseline"] = r["cpu_baseline"]
+            if "library_gemm_yardstick" in r:
+                out["configs"][name]["library_gemm_yardstick_TFLOPs"] = r["library_gemm_yardstick"]["TFLOP/s"]
+                out["configs"][name]["forward_TFLOPs"] = gemm_rate(r)
             del r
             torch.cuda.empty_cache()
     print(json.dumps(out), flush=True)

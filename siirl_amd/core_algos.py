@@ -568,10 +568,11 @@ def apply_kl_penalty(data, kl_ctrl, kl_penalty="kl", multi_turn=False):
 
 def compute_advantage(data, adv_estimator, gamma=1.0, lam=1.0, norm_adv_by_std_in_grpo=True,
                       weight_factor_in_cpgd="STD_weight", **kwargs):
-    """Dispatcher (reference ``core_algos.py:1400-1492``).  The GAE (``:1424-1439``, without the PF-PPO
-    reweighting), GRPO (``:1440-1471``) and multi-agent GAE (``:1483-1489``, ``data`` then needs ``.batch`` and
-    ``.non_tensor_batch``) branches are built; the CPGD branch fails with the reference's own ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a
-    keyword it does not take, ``:1475-1480``); ``compute_cpgd_outcome_advantage`` is there to be called directly."""
+    """Dispatcher (reference ``core_algos.py:1400-1492``).  The GAE (``:1424-1439``, with the PF-PPO resampling
+    of ``use_pf_ppo``, ``:1434-1439``), GRPO (``:1440-1471``) and multi-agent GAE (``:1483-1489``, ``data`` then needs
+    ``.batch`` and ``.non_tensor_batch``) branches are built; the CPGD branch fails with the reference's own
+    ``TypeError`` (it hands ``compute_grpo_outcome_advantage`` a keyword it does not take, ``:1475-1480``);
+    ``compute_cpgd_outcome_advantage`` is there to be called directly."""
     if "response_mask" not in data.keys():
         _td_set(data, "response_mask", compute_response_mask(data))
     est = adv_estimator.value if isinstance(adv_estimator, Enum) else adv_estimator

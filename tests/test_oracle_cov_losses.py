@@ -36,6 +36,33 @@ def test_kl_cov_worked_case():
     assert float(z1) == 0.0 and float(z2) == 0.0
 
 
+def test_kl_cov_cut_moves_only_among_near_ties_when_the_means_are_rounded_differently():
+    """The reference centres with float32 ``.mean()`` (``core_algos.py:1055``); the device path sums the means in
+    double and rounds once.  The two means can differ in the last bits, so can the covariances, and with them the
+    membership exactly at the cut of ``topk`` -- and only there: every token chosen by one and not by the other
+    has a covariance within a few float32 spacings of the k-th value."""
+    g = torch.Generator().manual_seed(11)
+    for n, ratio in ((4096, 0.01), (50000, 0.002), (200000, 0.0002)):
+        a = torch.randn(n, generator=g)
+        lp = -1.5 + torch.randn(n, generator=g)
+        k = max(1, int(n * ratio))
+        cov_ref = (a - a.mean()) * (lp - lp.mean())                                   # the reference's arithmetic
+        ma, ml = a.double().mean().float(), lp.double().mean().float()                 # double sum, one rounding
+        cov_dev = (a - ma) * (lp - ml)
+        top_ref = set(torch.topk(cov_ref, k).indices.tolist())
+        top_dev = set(torch.topk(cov_dev, k).indices.tolist())
+        cut = torch.topk(cov_ref, k).values[-1]
+        # a changed mean moves every cov by at most delta = |mean shift| * |other factor| (+ rounding); the cut moves by
+        # at most delta as well, so a token that changes sides lies within 2 delta of it
+        eps = float(torch.finfo(torch.float32).eps)
+        delta = (abs(float(a.mean() - ma)) * float((lp - ml).abs().max())
+                 + abs(float(lp.mean() - ml)) * float((a - ma).abs().max()) + 4 * eps * float(cov_ref.abs().max()))
+        slack = 2 * delta
+        for i in top_ref ^ top_dev:
+            assert abs(float(cov_ref[i]) - float(cut)) <= slack, (n, i, float(cov_ref[i]), float(cut), slack)
+        assert len(top_ref ^ top_dev) <= max(2, k // 50)
+
+
 def test_kl_cov_ignores_masked_tokens_and_counts():
     g = torch.Generator().manual_seed(3)
     B, L = 7, 50

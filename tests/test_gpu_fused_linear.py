@@ -449,6 +449,54 @@ def test_fp16_and_fp32_operands(dev, dtype, T, H, V):
         assert torch.count_nonzero(hd2.grad[live == 0]) == 0
 
 
+def test_fp16_and_fp32_random_shapes_sweep(dev):
+    """Seeded random shapes with float16 / float32 operands on both backward routes (recompute and parked logits),
+    around the same tile, slab and group boundaries as the bf16 sweep.  ``SIIRL_TEST_SEED=<int>`` shifts the seeds."""
+    import random
+
+    from siirl_amd import fused_linear as FL
+
+    shift = 100003 * int(os.environ.get("SIIRL_TEST_SEED", "0"))
+    edges = (1, 2, 255, 256, 257, 513, 8191, 8192, 8193, 16385)
+    try:
+        for case in range(12):
+            rnd = random.Random(5200 + case + shift)
+            dtype = (torch.float16, torch.float32)[case % 2]
+            T = rnd.choice((1, 7, 63, 64, 65, 255, 256, 257, rnd.randint(1, 600)))
+            H = 64 * rnd.choice((1, 2, 3, 5))
+            V = rnd.choice(edges) if case % 3 else rnd.randint(1, 20000)
+            if case == 7:
+                T, H, V = 100, 64, 65536 + rnd.choice((-1, 0, 1, 300))
+            temperature = rnd.choice((1.0, 0.6, 1.9))
+            which = rnd.choice(("both", "both", "logprob", "entropy"))
+            g = torch.Generator().manual_seed(5200 + case + shift)
+            h = torch.randn(T, H, generator=g).to(dtype)
+            w = (torch.randn(V, H, generator=g) * (2.0 / H ** 0.5)).to(dtype)
+            y = torch.randint(0, V, (T,), generator=g)
+            g_lp, g_h = torch.randn(T, generator=g), torch.randn(T, generator=g)
+            FL.set_saved_logits_limit((1 << 34) if case % 4 < 2 else 0)
+            hd, wd = h.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+            lp, ent = FL.FusedLinearForPPO()(hd, wd, y.to(dev), temperature=temperature)
+            lp64, ent64 = OFL.fused_linear_for_ppo_fwd(h, w, y, temperature, dtype=torch.float64)
+            what = (case, dtype, T, H, V, temperature, which)
+            assert (lp.cpu().double() - lp64).abs().max() < 1e-4 and (ent.cpu().double() - ent64).abs().max() < 1e-4, what
+            outs, grads = [], []
+            if which != "entropy":
+                outs.append(lp), grads.append(g_lp.to(dev))
+            if which != "logprob":
+                outs.append(ent), grads.append(g_h.to(dev))
+            torch.autograd.backward(outs, grads)
+            zero = torch.zeros_like(g_lp)
+            dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp if which != "entropy" else zero,
+                                                      g_h if which != "logprob" else zero, h, w, y, temperature,
+                                                      dtype=torch.float64)
+            assert hd.grad.dtype == dtype and wd.grad.dtype == dtype
+            _check_grad(hd.grad, dh64, f"d_hidden {what}", floor=1e-5)
+            _check_grad(wd.grad, dw64, f"d_weight {what}", floor=1e-5)
+    finally:
+        FL.set_saved_logits_limit(0)
+
+
 def test_mixed_operand_dtypes_are_refused(dev):
     from siirl_amd.fused_linear import fused_linear_logprob_entropy
 

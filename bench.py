@@ -1377,7 +1377,7 @@ def main():
         # gives the full line with its variants): step time, roofline fraction and the CPU oracle beside it
         del x, logits, labels, g_lp, g_ent, mask, x3, lp_now, old_lp, ref_lp, adv, m2, lp, ent, dx
         torch.cuda.empty_cache()
-        quick_steps = {"config1": (5, 2), "config3": (10, 2), "config4": (5, 2), "config5": (4, 1)}
+        quick_steps = {"config1": (5, 2), "config3": (10, 2), "config4": (5, 2), "config5": (8, 2)}
         fns = {"config1": bench_config1, "config3": bench_config3, "config4": bench_config4, "config5": bench_config5}
         out["configs"] = {}
         for name, fn in fns.items():

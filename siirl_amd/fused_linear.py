@@ -42,16 +42,17 @@ def set_saved_logits_limit(nbytes: int) -> None:
     _SAVED_LOGITS_LIMIT = int(nbytes)
 
 
-_SKIP_ZERO_ROWS = True
+_SKIP_ZERO_ROWS = False
 
 
 def set_skip_zero_rows(flag: bool) -> None:
-    """Backward leaves token rows whose upstream gradients are both zero out of its three GEMMs (the prompt tokens
-    of a packed batch: the actor keeps only the response slice of the log-probs, reference
-    ``siirl/engine/actor/dp_actor.py:170-172,228-231``).  On by default.  Costs one host synchronisation per backward
-    (the count of such rows), so it is skipped under stream capture and when the logits were parked; ``d_hidden``
-    of a skipped row is zero even where its hidden state holds NaN or Inf; ``d_weight`` is summed over the remaining
-    rows, which changes its rounding order, not its value."""
+    """``True``: the backward leaves token rows whose upstream gradients are both zero out of its three GEMMs (the
+    prompt tokens of a packed batch: the actor keeps only the response slice of the log-probs, reference
+    ``siirl/engine/actor/dp_actor.py:170-172,228-231``).  Off by default, because it departs from the reference's
+    autograd in two ways: it costs one host synchronisation per backward (the count of such rows; it is therefore
+    not applied under stream capture, nor when the logits were parked), and ``d_hidden`` of a skipped row is zero even
+    where its hidden state holds NaN or Inf.  ``d_weight`` is summed over the remaining rows, which changes its
+    rounding order, not its value."""
     global _SKIP_ZERO_ROWS
     _SKIP_ZERO_ROWS = bool(flag)
 

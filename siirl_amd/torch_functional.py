@@ -15,9 +15,9 @@ Differences a caller can observe, all deliberate:
 * a label of ``-101`` (``siirl_amd.padding.LABEL_SKIP_ROW``, set by ``unpad_ids_and_labels(..., response_length=L)``
   on the packed tokens outside the response window) makes both passes skip the row: log-prob and entropy 0, zero
   gradient, the logits of the row are never read (the single-launch step, ``fused_actor_step``, does the same);
-* the backward writes zeros, without reading the row, where both upstream gradients of a row are zero
-  (``set_skip_zero_rows``): a NaN or Inf in a padded row's logits therefore does not reach ``dlogits`` as it would
-  through the reference's autograd.
+* opt-in (``set_skip_zero_rows(True)``): the backward writes zeros, without reading the row, where both upstream
+  gradients of a row are zero; a NaN or Inf in a padded row's logits then does not reach ``dlogits`` as it would
+  through the reference's autograd, so the default leaves it off.
 """
 
 from __future__ import annotations
@@ -35,12 +35,13 @@ _bwd = _OPS.logprob_entropy_bwd
 _bwd_ = _OPS.logprob_entropy_bwd_
 _lpe = _OPS.logprob_entropy.default
 
-_SKIP_ZERO_ROWS = True
+_SKIP_ZERO_ROWS = False
 
 
 def set_skip_zero_rows(flag: bool) -> None:
-    """Backward writes zeros, without reading the row, where both upstream gradients are zero
-    (padding rows).  On by default; identical results for finite logits."""
+    """``True``: the backward writes zeros, without reading the row, where both upstream gradients are zero
+    (padding rows).  Identical results for finite logits; a NaN or Inf in such a row then no longer reaches
+    ``dlogits`` as it does through the reference's autograd (``0 * NaN``), which is why it is off by default."""
     global _SKIP_ZERO_ROWS
     _SKIP_ZERO_ROWS = bool(flag)
 

@@ -564,7 +564,7 @@ def test_packed_rows_outside_the_response_window_are_skipped(dev, dtype, inplace
         assert torch.equal(skipped.cpu(), (pos < S - L - 1) | (pos > S - 2))
         labels1, lp1, ent1, lpw1, entw1, dx1 = flow(L, skipped)
     finally:
-        TF.set_skip_zero_rows(True)
+        TF.set_skip_zero_rows(False)
     assert torch.equal(lpw1, lpw0) and torch.equal(entw1, entw0)
     assert torch.equal(lp1[~skipped], lp0[~skipped]) and torch.equal(ent1[~skipped], ent0[~skipped])
     assert not lp1[skipped].any() and not ent1[skipped].any()

@@ -229,6 +229,16 @@ def test_parked_logits_allocation_failure_falls_back_to_recompute(dev):
         assert torch.equal(a, b)
 
 
+@pytest.fixture
+def rows_left_out():
+    """The opt-in backward that leaves rows without upstream gradient out of its GEMMs (off by default)."""
+    import siirl_amd.fused_linear as FL
+
+    FL.set_skip_zero_rows(True)
+    yield
+    FL.set_skip_zero_rows(False)
+
+
 def _live_rows(T, pattern, seed):
     g = torch.Generator().manual_seed(seed)
     if pattern == "packed":  # sequences of prompt + response tokens: only the response rows carry a gradient
@@ -274,7 +284,7 @@ def test_zero_gradient_rows_left_out_of_backward(dev, T, H, V, pattern):
             lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y.to(dev), 0.9)
             torch.autograd.backward([lp, ent], [g_lp.to(dev), g_h.to(dev)])
         finally:
-            FL.set_skip_zero_rows(True)
+            FL.set_skip_zero_rows(False)
         _check_grad(hd.grad, dh64, f"d_hidden skip={skip}")
         _check_grad(wd.grad, dw64, f"d_weight skip={skip}")
         out[skip] = (hd.grad, wd.grad)
@@ -296,7 +306,7 @@ def test_zero_gradient_rows_left_out_of_backward(dev, T, H, V, pattern):
         assert not out[True][1].any()
 
 
-def test_zero_gradient_rows_hide_nan_hidden_states(dev):
+def test_zero_gradient_rows_hide_nan_hidden_states(dev, rows_left_out):
     import siirl_amd.fused_linear as FL
 
     T, H, V = 200, 64, 700
@@ -311,6 +321,23 @@ def test_zero_gradient_rows_hide_nan_hidden_states(dev):
     dh64, dw64 = OFL.fused_linear_for_ppo_bwd(g_lp[60:], g_h[60:], h[60:], w, y[60:], 1.0, dtype=torch.float64)
     _check_grad(hd.grad[60:], dh64, "d_hidden")
     _check_grad(wd.grad, dw64, "d_weight")
+
+
+def test_default_backward_lets_nan_of_a_zero_gradient_row_through(dev):
+    """Without the opt-in the backward is dense: a NaN hidden state in a row whose upstream gradients are zero reaches
+    d_weight and that row of d_hidden, as ``0 * NaN`` does through the reference's autograd
+    (``experimental/torch_functional.py:49-67``)."""
+    import siirl_amd.fused_linear as FL
+
+    T, H, V = 200, 64, 700
+    h, w, y, g_lp, g_h = _inputs(T, H, V, seed=11)
+    live = torch.arange(T) >= 60
+    h[:60] = float("nan")
+    hd, wd = h.to(dev).requires_grad_(True), w.to(dev).requires_grad_(True)
+    lp, ent = FL.fused_linear_logprob_entropy(hd, wd, y.to(dev), 1.0)
+    torch.autograd.backward([lp, ent], [(g_lp * live).to(dev), (g_h * live).to(dev)])
+    assert torch.isnan(wd.grad).any() and torch.isnan(hd.grad[:60]).any()
+    assert torch.isfinite(hd.grad[60:]).all()
 
 
 def test_backward_rows_through_the_c_abi(dev):
@@ -363,7 +390,7 @@ def test_backward_rows_through_the_c_abi(dev):
     assert call(picked, n=-1)[0] == -1
 
 
-def test_zero_gradient_rows_sweep(dev):
+def test_zero_gradient_rows_sweep(dev, rows_left_out):
     """Seeded random shapes and row patterns (``SIIRL_TEST_SEED`` shifts the seed): the backward that leaves rows out
     against the oracle, and zero rows of d_hidden exactly zero."""
     import siirl_amd.fused_linear as FL
@@ -385,7 +412,7 @@ def test_zero_gradient_rows_sweep(dev):
 
 
 @pytest.mark.parametrize("wrt", ["hidden", "weight"])
-def test_zero_gradient_rows_with_one_gradient_requested(dev, wrt):
+def test_zero_gradient_rows_with_one_gradient_requested(dev, wrt, rows_left_out):
     """The row-subset backward when only d_hidden or only d_weight is asked for."""
     import siirl_amd.fused_linear as FL
 

@@ -196,6 +196,37 @@ def test_special_rows(dev):
     assert torch.isnan(bad[1]) and torch.isnan(bad[2]) and not torch.isnan(bad[0])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_nan_in_a_row_without_upstream_gradient(dev, dtype):
+    """By default the backward is dense, and ``0 * NaN`` reaches ``dlogits`` as it does through the reference's
+    autograd (``torch_functional.py:99-132`` under ``backward()``); with ``set_skip_zero_rows(True)`` such a row is
+    written as zeros unread.  Rows with a gradient are the same bits either way."""
+    import siirl_amd.torch_functional as TF
+
+    T, V = 37, 1000
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(T, V, generator=g) * 2).to(dtype)
+    x[3, 17] = float("nan")
+    y = torch.randint(0, V, (T,), generator=g)
+    g_lp, g_ent = torch.randn(T, generator=g), torch.randn(T, generator=g)
+    g_lp[3] = 0.0
+    g_ent[3] = 0.0
+    grads = {}
+    for skip in (False, True):
+        TF.set_skip_zero_rows(skip)
+        try:
+            xd = x.to(dev).requires_grad_(True)
+            lp, ent = TF.logprobs_and_entropy_from_logits(xd, y.to(dev))
+            torch.autograd.backward([lp, ent], [g_lp.to(dev), g_ent.to(dev)])
+        finally:
+            TF.set_skip_zero_rows(False)
+        grads[skip] = xd.grad
+    assert torch.isnan(grads[False][3]).any() and not grads[True][3].any()
+    keep = torch.arange(T) != 3
+    assert torch.equal(grads[False][keep.to(dev)], grads[True][keep.to(dev)])
+    assert torch.isfinite(grads[False][keep.to(dev)]).all()
+
+
 def test_no_cpu_fallback():
     import siirl_amd.torch_functional as SF
 
